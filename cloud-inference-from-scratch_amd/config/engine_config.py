@@ -1,0 +1,60 @@
+"""Engine options: the knobs of the reference's ``EngineConfig``
+(src/cloud_engine/config.py:24-48, engine_config.json:26-40) that concern one
+GPU's engine, under names that say what they bound.  Unknown overrides raise,
+as in ``build_config`` (src/cloud_engine/config.py:107-109).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, fields, replace
+from typing import Any
+
+DTYPES = ("bfloat16", "float32")
+_DTYPE_ALIASES = {"bf16": "bfloat16", "fp32": "float32", "bfloat16": "bfloat16", "float32": "float32"}
+
+
+def canonical_dtype(name: str) -> str:
+    try:
+        return _DTYPE_ALIASES[str(name).replace("torch.", "")]
+    except KeyError:
+        raise ValueError(f"dtype must be one of {DTYPES} (or bf16/fp32), got {name!r}") from None
+
+
+@dataclass(frozen=True)
+class EngineConfig:
+    dtype: str = "bfloat16"
+    max_model_len: int = 4096
+    max_output_tokens: int = 256
+    eos_token_id: int | None = None
+    max_running: int = 16  # reference: max_active_sequences
+    max_queue_size: int = 64
+    token_budget: int = 2048  # reference: max_batched_tokens
+    prefill_chunk: int = 256  # reference: prefill_chunk_size
+    page_size: int = 16  # reference: block_size, fixed at 16 there
+    kv_tokens: int | None = None  # pool size in tokens; None: from kv_cache_bytes
+    kv_cache_bytes: int = 4 << 30
+    prefix_cache_pages: int = 256  # reference: prefix_cache_max_blocks
+    graph_decode: bool = True  # reference: cuda_graph_decode
+    seed: int = 0
+
+    def validated(self) -> "EngineConfig":
+        config = replace(self, dtype=canonical_dtype(self.dtype))
+        for name in ("max_model_len", "max_output_tokens", "max_running", "max_queue_size",
+                     "token_budget", "prefill_chunk", "page_size"):
+            if getattr(config, name) < 1:
+                raise ValueError(f"{name} must be positive")
+        if config.page_size & (config.page_size - 1):
+            raise ValueError(f"page_size must be a power of two, got {config.page_size}")
+        if config.prefix_cache_pages < 0:
+            raise ValueError("prefix_cache_pages must be non-negative")
+        if config.kv_tokens is not None and config.kv_tokens < config.page_size:
+            raise ValueError("kv_tokens too small for even one page")
+        return config
+
+
+def build_engine_config(base: EngineConfig | None = None, **overrides: Any) -> EngineConfig:
+    known = {item.name for item in fields(EngineConfig)}
+    unknown = set(overrides) - known
+    if unknown:
+        raise ValueError(f"unknown config overrides: {sorted(unknown)}")
+    return replace(base or EngineConfig(), **overrides).validated()

@@ -1,0 +1,95 @@
+// Shared device helpers for the gfx950 kernels: storage types, bf16 conversion,
+// wave64 and workgroup reductions, launch-error reporting.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define CIE_API extern "C" __attribute__((visibility("default")))
+
+// Return codes of every entry point.  0 is success; the Python side turns the
+// others into exceptions that name the entry point.
+enum {
+    CIE_OK = 0,
+    CIE_BAD_ARGUMENT = 1,   // a size or option the kernel does not take
+    CIE_LAUNCH_FAILED = 2,  // hipGetLastError() after the launch
+};
+
+constexpr int kWave = 64;
+
+// Activation / weight storage.  dtype codes used across the C ABI.
+enum { CIE_F32 = 0, CIE_BF16 = 1 };
+
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16_t x) {
+    return __uint_as_float(static_cast<uint32_t>(x.bits) << 16);
+}
+
+// Round to nearest even; NaN stays NaN.
+__device__ __forceinline__ uint16_t bf16_bits_from_float(float x) {
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_float(float x);
+template <>
+__device__ __forceinline__ float from_float<float>(float x) {
+    return x;
+}
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float x) {
+    bf16_t r;
+    r.bits = bf16_bits_from_float(x);
+    return r;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, kWave));
+    return v;
+}
+
+// Sum over a workgroup of up to 16 waves; every thread gets the result.
+// `scratch` is at least 16 floats of LDS; the call contains barriers.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int waves = (blockDim.x + kWave - 1) / kWave;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < waves; ++w) total += scratch[w];
+    return total;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int waves = (blockDim.x + kWave - 1) / kWave;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = scratch[0];
+    for (int w = 1; w < waves; ++w) total = fmaxf(total, scratch[w]);
+    return total;
+}
+
+static inline int cie_after_launch() {
+    return hipGetLastError() == hipSuccess ? CIE_OK : CIE_LAUNCH_FAILED;
+}

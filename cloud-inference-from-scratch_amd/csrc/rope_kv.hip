@@ -1,0 +1,82 @@
+// Fused rotary position encoding (half-split pairing: element i rotates with
+// element i + D/2) of q and k, and the write of rotated k and of v into the
+// paged cache.
+//
+//   qkv  [tokens, (Hq + 2*Hkv) * D]   q rotated in place
+//   pool [pages, Hkv, page_size, D]   one for keys, one for values
+//   slot of token t: page = block_table[seq_slot[seq_of_token[t]], pos / P], row = pos % P
+//
+// Angles come from a float32 cos/sin table [max_position, D/2]; the rotation is
+// computed in float32 and rounded once.  One workgroup per (token, head).
+#include "common.h"
+
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restrict__ cos_table,
+                                     const float* __restrict__ sin_table,
+                                     const int* __restrict__ positions,
+                                     const int* __restrict__ seq_of_token,
+                                     const int* __restrict__ seq_slot,
+                                     const int* __restrict__ block_table, int table_width,
+                                     T* __restrict__ k_pool, T* __restrict__ v_pool, int q_heads,
+                                     int kv_heads, int head_dim, int page_size, int rotate,
+                                     int write_kv) {
+    const int token = blockIdx.x;
+    const int head = blockIdx.y;  // [0,Hq): q   [Hq,Hq+Hkv): k   [Hq+Hkv,Hq+2Hkv): v
+    const int half = head_dim / 2;
+    const int pos = positions[token];
+    T* src = qkv + (static_cast<size_t>(token) * (q_heads + 2 * kv_heads) + head) * head_dim;
+
+    T* dst = nullptr;
+    if (head >= q_heads) {
+        if (!write_kv) return;
+        const int kv_head = (head - q_heads) % kv_heads;
+        const int slot = seq_slot[seq_of_token[token]];
+        const int page = block_table[static_cast<size_t>(slot) * table_width + pos / page_size];
+        if (page < 0) return;  // the host never schedules a token without a page
+        T* pool = head < q_heads + kv_heads ? k_pool : v_pool;
+        dst = pool + ((static_cast<size_t>(page) * kv_heads + kv_head) * page_size + pos % page_size) * head_dim;
+    }
+    const bool is_value = head >= q_heads + kv_heads;
+    if (is_value || !rotate) {
+        if (dst)
+            for (int i = threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
+        return;
+    }
+    const float* cos_row = cos_table + static_cast<size_t>(pos) * half;
+    const float* sin_row = sin_table + static_cast<size_t>(pos) * half;
+    T* target = dst ? dst : src;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        const float x1 = to_float(src[i]);
+        const float x2 = to_float(src[i + half]);
+        const float c = cos_row[i];
+        const float s = sin_row[i];
+        target[i] = from_float<T>(x1 * c - x2 * s);
+        target[i + half] = from_float<T>(x2 * c + x1 * s);
+    }
+}
+
+CIE_API int cie_rope_kv_write(void* stream, int dtype, void* qkv, const float* cos_table,
+                              const float* sin_table, const int* positions, const int* seq_of_token,
+                              const int* seq_slot, const int* block_table, int table_width,
+                              void* k_pool, void* v_pool, int tokens, int q_heads, int kv_heads,
+                              int head_dim, int page_size, int rotate, int write_kv) {
+    if (tokens < 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 2 || page_size <= 0 ||
+        table_width <= 0)
+        return CIE_BAD_ARGUMENT;
+    if (tokens == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    dim3 grid(tokens, q_heads + 2 * kv_heads);
+    if (dtype == CIE_F32)
+        rope_kv_write_kernel<float><<<grid, 64, 0, s>>>(
+            static_cast<float*>(qkv), cos_table, sin_table, positions, seq_of_token, seq_slot, block_table,
+            table_width, static_cast<float*>(k_pool), static_cast<float*>(v_pool), q_heads, kv_heads,
+            head_dim, page_size, rotate, write_kv);
+    else if (dtype == CIE_BF16)
+        rope_kv_write_kernel<bf16_t><<<grid, 64, 0, s>>>(
+            static_cast<bf16_t*>(qkv), cos_table, sin_table, positions, seq_of_token, seq_slot, block_table,
+            table_width, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads,
+            head_dim, page_size, rotate, write_kv);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}

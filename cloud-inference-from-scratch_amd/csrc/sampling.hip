@@ -1,0 +1,108 @@
+// Sampling over float32 logits [rows, vocab]; one workgroup per row.
+//
+// Greedy: the first index of the maximum (ties go to the lower index).
+// Temperature: p_i = exp((l_i - max) / T); with the row's uniform number u in
+// [0, 1) the token is the first i whose running sum of p exceeds u * sum(p).
+// u is made on the host from (seed, request, step), so a draw depends neither
+// on the batch nor on the thread layout.  T <= 0 means greedy.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ void argmax_block(const float* row, int vocab, float* s_val, int* s_idx,
+                                             float& best_out, int& idx_out) {
+    float best = -INFINITY;
+    int best_idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < vocab; i += kThreads) {
+        const float v = row[i];
+        if (v > best || (v == best && i < best_idx)) {
+            best = v;
+            best_idx = i;
+        }
+    }
+    s_val[threadIdx.x] = best;
+    s_idx[threadIdx.x] = best_idx;
+    __syncthreads();
+    for (int stride = kThreads / 2; stride > 0; stride >>= 1) {
+        if (threadIdx.x < stride) {
+            const float v = s_val[threadIdx.x + stride];
+            const int i = s_idx[threadIdx.x + stride];
+            if (v > s_val[threadIdx.x] || (v == s_val[threadIdx.x] && i < s_idx[threadIdx.x])) {
+                s_val[threadIdx.x] = v;
+                s_idx[threadIdx.x] = i;
+            }
+        }
+        __syncthreads();
+    }
+    best_out = s_val[0];
+    idx_out = s_idx[0] == 0x7fffffff ? 0 : s_idx[0];
+    __syncthreads();
+}
+
+__global__ void __launch_bounds__(kThreads)
+sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+              const float* __restrict__ uniform, int* __restrict__ out, int vocab, int ld) {
+    __shared__ float s_val[kThreads];
+    __shared__ int s_idx[kThreads];
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const float* row = logits + static_cast<size_t>(r) * ld;
+    float best;
+    int best_idx;
+    argmax_block(row, vocab, s_val, s_idx, best, best_idx);
+    const float temp = temperature ? temperature[r] : 0.f;
+    if (!(temp > 0.f)) {
+        if (threadIdx.x == 0) out[r] = best_idx;
+        return;
+    }
+    // Each thread owns one contiguous span of the row, so the running sum has a fixed order.
+    const int span = (vocab + kThreads - 1) / kThreads;
+    const int begin = min(threadIdx.x * span, vocab);
+    const int end = min(begin + span, vocab);
+    const float inv_t = 1.0f / temp;
+    float local = 0.f;
+    for (int i = begin; i < end; ++i) local += expf((row[i] - best) * inv_t);
+    s_val[threadIdx.x] = local;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float running = 0.f;
+        for (int t = 0; t < kThreads; ++t) {  // exclusive prefix over the spans
+            const float v = s_val[t];
+            s_val[t] = running;
+            running += v;
+        }
+        const float target = uniform[r] * running;
+        int owner = 0;  // the last non-empty span that starts at or below the target
+        for (int t = 1; t < kThreads; ++t)
+            if (t * span < vocab && s_val[t] <= target) owner = t;
+        scratch[0] = target;
+        s_idx[0] = owner;
+    }
+    __syncthreads();
+    if (threadIdx.x != s_idx[0]) return;
+    const float target = scratch[0];
+    float running = s_val[threadIdx.x];
+    int pick = end - 1;  // if rounding leaves the target unreached inside the span: its last token
+    for (int i = begin; i < end; ++i) {
+        running += expf((row[i] - best) * inv_t);
+        if (running > target) {
+            pick = i;
+            break;
+        }
+    }
+    out[r] = pick;
+}
+
+}  // namespace
+
+CIE_API int cie_sample(void* stream, const float* logits, const float* temperature,
+                       const float* uniform, int* out, int rows, int vocab, int ld) {
+    if (rows < 0 || vocab <= 0 || ld < vocab) return CIE_BAD_ARGUMENT;
+    if (temperature && !uniform) return CIE_BAD_ARGUMENT;
+    if (rows == 0) return CIE_OK;
+    sample_kernel<<<rows, kThreads, 0, static_cast<hipStream_t>(stream)>>>(logits, temperature, uniform,
+                                                                           out, vocab, ld);
+    return cie_after_launch();
+}

@@ -1,0 +1,78 @@
+"""Device side of the cache: page pools, block tables and state rows.
+
+For every group of the :class:`~cie_amd.cache.manager.CacheManager` one pool
+``[units, 2, pages, kv_heads, page_size, head_dim]`` (keys at index 0, values at
+index 1 of the second axis; a page of one head is contiguous so that a kernel
+streams ``page_size * head_dim`` elements per page and head) and one int32 block
+table ``[max_running, width]`` whose row ``slot`` mirrors the request's host
+table.  The reference keeps ``[layers, pages, page_size, kv_heads, head_dim]``
+pools (src/cloud_engine/cache.py:266-274) and uploads padded tables every step
+(src/cloud_engine/engine.py:264-278); here only rows that changed are copied.
+"""
+
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+from ..cache.manager import CacheManager, FixedState
+from .batch import PagedView, StateView
+
+_STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
+
+
+class DeviceCache:
+    def __init__(self, manager: CacheManager, dtype: torch.dtype, device: torch.device) -> None:
+        self.manager = manager
+        self.dtype = dtype
+        self.device = device
+        self.pools: list[torch.Tensor] = []
+        self.tables: list[torch.Tensor] = []
+        self.host_tables: list[torch.Tensor] = []
+        for group in manager.groups:
+            spec = group.spec
+            shape = (len(group.units), 2, group.allocator.total_pages, spec.kv_heads, manager.page_size,
+                     spec.head_dim)
+            self.pools.append(torch.zeros(shape, dtype=dtype, device=device))
+            self.tables.append(torch.zeros((manager.max_running, manager.table_width), dtype=torch.int32,
+                                           device=device))
+            self.host_tables.append(torch.zeros((manager.max_running, manager.table_width), dtype=torch.int32,
+                                                pin_memory=device.type == "cuda"))
+        self.states: dict[int, torch.Tensor] = {}
+        for unit, spec in manager.state_units.items():
+            assert isinstance(spec, FixedState)
+            self.states[unit] = torch.zeros((manager.max_running, *spec.shape),
+                                            dtype=_STATE_DTYPES[spec.dtype], device=device)
+        self._views: dict[int, Any] = {}
+        for unit in range(len(manager.unit_specs)):
+            if unit in manager.unit_group:
+                index = manager.unit_group[unit]
+                local = manager.groups[index].units.index(unit)
+                pool = self.pools[index]
+                self._views[unit] = PagedView(pool[local, 0], pool[local, 1], self.tables[index],
+                                              manager.page_size)
+            elif unit in self.states:
+                self._views[unit] = StateView(self.states[unit])
+            else:
+                self._views[unit] = None
+
+    def view(self, unit: int) -> Any:
+        return self._views[unit]
+
+    def bytes(self) -> int:
+        return sum(p.numel() * p.element_size() for p in self.pools)
+
+    def sync(self) -> None:
+        """Bring the device block tables up to the host's; clear the state of
+        slots that were handed to a new request."""
+        for group, slot, table in self.manager.take_dirty_rows():
+            host = self.host_tables[group]
+            row = host[slot]
+            if table:
+                row[: len(table)] = torch.tensor([max(p, 0) for p in table], dtype=torch.int32)
+            self.tables[group][slot].copy_(row, non_blocking=True)
+        fresh = self.manager.take_fresh_slots()
+        if fresh and self.states:
+            for state in self.states.values():
+                state[fresh] = 0

@@ -1,0 +1,173 @@
+"""The step function: a batch of (request, its next tokens) in, logits out.
+
+Counterpart of the reference's ``RaggedRunner`` (src/cloud_engine/engine.py:193-488):
+``admit`` / ``release`` / ``allocated_tokens`` are what the scheduler calls;
+:meth:`Runner.run` grows the cache all-or-nothing, packs the step's tokens on
+one flat axis (prompt portions beside single decode tokens, cut anywhere), runs
+the model once on exactly these tokens against the cache earlier steps left,
+commits the lengths and returns float32 logits at the wanted places.  Unlike
+the reference it returns logits at *any* wanted position and leaves sampling to
+the caller, so trace replay and generation drive the same function.
+"""
+
+from __future__ import annotations
+
+from collections import deque
+from collections.abc import Sequence
+from dataclasses import dataclass, field
+from typing import Any
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..config.engine_config import EngineConfig
+from ..profiling import trace_range
+from .batch import StepBatch
+from .device_cache import DeviceCache
+
+
+@dataclass(frozen=True)
+class StepEntry:
+    """One request's share of a step: its next ``tokens`` starting at
+    ``start_pos`` (which must equal what the cache holds for it) and the places
+    among these tokens whose logits are wanted."""
+
+    request_id: str
+    tokens: Sequence[int]
+    start_pos: int
+    want: Sequence[int] = field(default_factory=tuple)
+
+
+class Runner:
+    def __init__(self, model: Any, config: EngineConfig, device: str | torch.device = "cuda:0") -> None:
+        if not torch.cuda.is_available():
+            raise RuntimeError("the engine runs on the GPU only; no GPU is visible")
+        self.model = model
+        self.config = config
+        self.device = torch.device(device)
+        self.dtype = model.dtype
+        needs = model.cache_needs()
+        max_position = model.spec.max_position
+        if config.max_model_len > max_position:
+            raise ValueError(f"max_model_len {config.max_model_len} exceeds the model's {max_position} positions")
+        kv_tokens = config.kv_tokens if config.kv_tokens is not None else self._tokens_from_bytes(needs)
+        self.cache = CacheManager(
+            needs, config.page_size, kv_tokens, config.max_running, config.max_model_len,
+            prefill_chunk=config.prefill_chunk, prefix_cache_pages=config.prefix_cache_pages,
+        )
+        self.device_cache = DeviceCache(self.cache, self.dtype, self.device)
+        self.forward_invocations = 0
+        self.max_forward_request_count = 0
+        self.forward_plans: deque[tuple[tuple[str, int, int, int], ...]] = deque(maxlen=256)
+        self._staging = [None, None]
+        self._staging_turn = 0
+
+    def _tokens_from_bytes(self, needs: list[Any]) -> int:
+        element = torch.tensor([], dtype=self.dtype).element_size()
+        per_token = sum(2 * n.kv_heads * n.head_dim * element for n in needs if hasattr(n, "kv_heads"))
+        if per_token == 0:
+            return self.config.page_size
+        tokens = self.config.kv_cache_bytes // per_token
+        return max(self.config.page_size, tokens // self.config.page_size * self.config.page_size)
+
+    # -- what the scheduler calls ------------------------------------------------
+    def admit(self, request: Any) -> None:
+        request.tokens_fed = self.cache.admit(request.request_id, request.prompt_token_ids)
+
+    def release(self, request: Any, preempted: bool = False) -> None:
+        self.cache.release(request.request_id, None if preempted else request.prompt_token_ids)
+
+    def allocated_tokens(self, request: Any) -> int:
+        return self.cache.allocated_tokens(request.request_id)
+
+    # -- packing -----------------------------------------------------------------
+    def _stage(self, count: int) -> tuple[torch.Tensor, torch.Tensor]:
+        turn = self._staging_turn
+        self._staging_turn ^= 1
+        pair = self._staging[turn]
+        if pair is None or pair[0].numel() < count:
+            size = max(1024, 1 << (count - 1).bit_length())
+            pair = (torch.empty(size, dtype=torch.int32, pin_memory=True),
+                    torch.empty(size, dtype=torch.int32, device=self.device))
+            self._staging[turn] = pair
+        return pair
+
+    def pack(self, entries: Sequence[StepEntry]) -> StepBatch:
+        vocab = self.model.spec.vocab_size
+        ids: list[int] = []
+        positions: list[int] = []
+        seq_of_token: list[int] = []
+        slots: list[int] = []
+        starts: list[int] = []
+        q_lens: list[int] = []
+        q_start_loc = [0]
+        logit_rows: list[int] = []
+        seen: set[str] = set()
+        for index, entry in enumerate(entries):
+            if entry.request_id in seen:
+                raise ValueError(f"request {entry.request_id} appears twice in one step")
+            seen.add(entry.request_id)
+            count = len(entry.tokens)
+            if count == 0:
+                raise ValueError(f"request {entry.request_id} brings no tokens")
+            held = self.cache.length(entry.request_id)
+            if entry.start_pos != held:
+                raise ValueError(
+                    f"request {entry.request_id} continues at {entry.start_pos} but the cache holds {held} tokens"
+                )
+            for token in entry.tokens:
+                if not 0 <= token < vocab:
+                    raise ValueError(f"token id {token} outside the vocabulary of {vocab}")
+            base = len(ids)
+            ids.extend(entry.tokens)
+            positions.extend(range(entry.start_pos, entry.start_pos + count))
+            seq_of_token.extend([index] * count)
+            slots.append(self.cache.slot(entry.request_id))
+            starts.append(entry.start_pos)
+            q_lens.append(count)
+            q_start_loc.append(base + count)
+            for place in entry.want:
+                if not 0 <= place < count:
+                    raise ValueError(f"wanted place {place} outside the {count} tokens of {entry.request_id}")
+                logit_rows.append(base + place)
+        parts = [ids, positions, seq_of_token, slots, starts, q_lens, q_start_loc, logit_rows]
+        flat = [value for part in parts for value in part]
+        host, dev = self._stage(len(flat))
+        host[: len(flat)] = torch.tensor(flat, dtype=torch.int32)
+        dev[: len(flat)].copy_(host[: len(flat)], non_blocking=True)
+        views = []
+        offset = 0
+        for part in parts:
+            views.append(dev[offset: offset + len(part)])
+            offset += len(part)
+        return StepBatch(
+            tokens=len(ids), sequences=len(entries), token_ids=views[0], positions=views[1],
+            seq_of_token=views[2], seq_slot=views[3], seq_start=views[4], seq_q_len=views[5],
+            q_start_loc=views[6], logit_rows=views[7], host_slots=slots, host_starts=starts,
+            host_q_lens=q_lens, request_ids=tuple(e.request_id for e in entries),
+        )
+
+    # -- the step ------------------------------------------------------------------
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """One step.  Returns float32 logits ``[sum(len(e.want)), vocab]`` on the
+        device, in the order of the entries and of their ``want``.  Raises
+        ``CacheCapacityFull`` before anything changes if pages run out."""
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        required = {e.request_id: e.start_pos + len(e.tokens) for e in entries}
+        with trace_range("ragged.kv.ensure_capacity"):
+            self.cache.ensure_capacity_batch(required)
+            self.device_cache.sync()
+        batch = self.pack(entries)
+        self.forward_invocations += 1
+        self.max_forward_request_count = max(self.max_forward_request_count, len(entries))
+        self.forward_plans.append(
+            tuple((e.request_id, e.start_pos, len(e.tokens), len(e.want)) for e in entries)
+        )
+        phase = "decode" if batch.all_decode else "mixed"
+        with trace_range(f"ragged.forward.{phase}.requests_{batch.sequences}.tokens_{batch.tokens}"):
+            logits = self.model.forward(batch, self.device_cache)
+        with trace_range("ragged.kv.commit"):
+            self.cache.commit_lengths(required)
+            self.device_cache.sync()
+        return logits

@@ -1,0 +1,161 @@
+"""Build and load the HIP kernel library (``csrc/*.hip`` -> one shared object).
+
+The library is plain ``extern "C"`` entry points compiled by ``hipcc`` for
+gfx950 and loaded with ``ctypes``; it links neither Python nor torch.  It is
+built in-tree under ``csrc/_build`` (or, where the tree is read-only, in a
+per-user folder under the temporary directory).  A stamp of the sources' hash
+lies beside the built file; a stale or missing library is rebuilt at the first
+call, each source printing a line as it finishes.  There is no fallback: if
+the library can be neither loaded nor built, :func:`load_library` raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+CSRC = Path(__file__).resolve().parent.parent / "csrc"
+LIB_NAME = "libcie_kernels.so"
+ARCH = "gfx950"
+# Packed float32 instructions are switched off for every kernel of this library.
+HIPCC_FLAGS = [
+    "-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-fvisibility=hidden",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+_lock = threading.Lock()
+_library: ctypes.CDLL | None = None
+
+
+class KernelLibraryError(RuntimeError):
+    """The HIP kernel library is missing and could not be built."""
+
+
+def sources() -> list[Path]:
+    return sorted(CSRC.glob("*.hip"))
+
+
+def source_hash() -> str:
+    digest = hashlib.sha256()
+    for path in sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h"))):
+        digest.update(path.name.encode())
+        digest.update(path.read_bytes())
+    digest.update(" ".join(HIPCC_FLAGS).encode())
+    return digest.hexdigest()
+
+
+def _hipcc() -> str | None:
+    found = shutil.which("hipcc")
+    if found:
+        return found
+    candidate = Path(os.environ.get("ROCM_PATH", "/opt/rocm")) / "bin" / "hipcc"
+    return str(candidate) if candidate.is_file() else None
+
+
+def _build_dirs() -> list[Path]:
+    fallback = Path(tempfile.gettempdir()) / f"cie_amd_build_{os.getuid()}"
+    return [CSRC / "_build", fallback]
+
+
+def _log(message: str) -> None:
+    print(f"[cie_amd build] {message}", file=sys.stderr, flush=True)
+
+
+def _writable(folder: Path) -> bool:
+    try:
+        folder.mkdir(parents=True, exist_ok=True)
+        probe = folder / f".probe_{os.getpid()}"
+        probe.write_text("")
+        probe.unlink()
+        return True
+    except OSError:
+        return False
+
+
+def build_library(force: bool = True) -> Path:
+    """Compile every ``.hip`` source for gfx950 and link the shared object.
+
+    Works without a GPU (hipcc cross-compiles).  Returns the library's path."""
+    hipcc = _hipcc()
+    if hipcc is None:
+        raise KernelLibraryError("hipcc not found (looked on PATH and under $ROCM_PATH/bin)")
+    folder = next((d for d in _build_dirs() if _writable(d)), None)
+    if folder is None:
+        raise KernelLibraryError(f"no writable build folder among {[str(d) for d in _build_dirs()]}")
+    wanted = source_hash()
+    target = folder / LIB_NAME
+    stamp = folder / "sources.sha256"
+    if not force and target.is_file() and stamp.is_file() and stamp.read_text().strip() == wanted:
+        return target
+    env = dict(os.environ)
+    if not env.get("HOME") or not os.access(env["HOME"], os.W_OK):
+        env["HOME"] = str(folder)  # hipcc wants a writable home for its temporary files
+    files = sources()
+    _log(f"compiling {len(files)} HIP sources for {ARCH} into {folder}")
+    started = time.time()
+
+    def compile_one(path: Path) -> Path:
+        obj = folder / (path.stem + ".o")
+        cmd = [hipcc, *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(path), "-o", str(obj)]
+        done = subprocess.run(cmd, env=env, capture_output=True, text=True)
+        if done.returncode != 0:
+            raise KernelLibraryError(f"hipcc failed on {path.name}:\n{done.stderr[-4000:]}")
+        _log(f"  {path.name} done ({time.time() - started:.0f}s)")
+        return obj
+
+    workers = max(1, min(len(files), os.cpu_count() or 4, 8))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        objects = list(pool.map(compile_one, files))
+    scratch = folder / f"{LIB_NAME}.{os.getpid()}.tmp"
+    link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(scratch), *map(str, objects)]
+    done = subprocess.run(link, env=env, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise KernelLibraryError(f"linking {LIB_NAME} failed:\n{done.stderr[-4000:]}")
+    os.replace(scratch, target)
+    stamp.write_text(wanted + "\n")
+    _log(f"built {target} in {time.time() - started:.0f}s")
+    return target
+
+
+def find_built(check_stamp: bool = True) -> Path | None:
+    wanted = source_hash() if check_stamp else None
+    for folder in _build_dirs():
+        target = folder / LIB_NAME
+        stamp = folder / "sources.sha256"
+        if target.is_file():
+            if not check_stamp or (stamp.is_file() and stamp.read_text().strip() == wanted):
+                return target
+    return None
+
+
+def load_library() -> ctypes.CDLL:
+    """The loaded kernel library; built first if nothing current is there."""
+    global _library
+    with _lock:
+        if _library is not None:
+            return _library
+        path = find_built(check_stamp=True)
+        if path is None:
+            stale = find_built(check_stamp=False)
+            try:
+                path = build_library(force=False)
+            except KernelLibraryError:
+                if stale is None:
+                    raise
+                _log(f"sources changed but rebuilding failed; loading the stale {stale}")
+                path = stale
+        try:
+            _library = ctypes.CDLL(str(path))
+        except OSError as exc:
+            raise KernelLibraryError(f"cannot load {path}: {exc}") from exc
+        _library.cie_path = str(path)  # type: ignore[attr-defined]
+        return _library

@@ -1,0 +1,267 @@
+"""Python faces of the HIP entry points.
+
+Every function checks on the host what the kernel and its grid assume (device,
+dtype, contiguity, shapes, index ranges that are known on the host) and raises
+``ValueError`` with the offending value otherwise: a kernel is never launched
+on operands it was not written for.  Kernels run on torch's current stream.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .library import load_library
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+_ERRORS = {1: "bad argument (a size or option the kernel does not take)", 2: "kernel launch failed"}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _CODES[dtype]
+    except KeyError:
+        raise ValueError(f"kernels take float32 or bfloat16, got {dtype}") from None
+
+
+def _require(condition: bool, message: str) -> None:
+    if not condition:
+        raise ValueError(message)
+
+
+def _gpu(name: str, tensor: torch.Tensor, dtype: Optional[torch.dtype] = None, dims: Optional[int] = None) -> None:
+    _require(tensor.is_cuda, f"{name} must live on the GPU, is on {tensor.device}")
+    _require(tensor.is_contiguous(), f"{name} must be contiguous")
+    if dtype is not None:
+        _require(tensor.dtype == dtype, f"{name} must be {dtype}, is {tensor.dtype}")
+    if dims is not None:
+        _require(tensor.dim() == dims, f"{name} must have {dims} dims, has shape {tuple(tensor.shape)}")
+
+
+def _ptr(tensor: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _run(name: str, code: int) -> None:
+    if code != 0:
+        raise KernelError(f"{name}: {_ERRORS.get(code, f'error {code}')}")
+
+
+def _i(value: int) -> ctypes.c_int:
+    return ctypes.c_int(int(value))
+
+
+def _f(value: float) -> ctypes.c_float:
+    return ctypes.c_float(float(value))
+
+
+# ---------------------------------------------------------------------------
+def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t] = float32(table[ids[t]])``; ids int32 [T] (already checked against the vocabulary)."""
+    _gpu("table", table, dims=2)
+    _gpu("ids", ids, torch.int32, 1)
+    vocab, hidden = table.shape
+    tokens = ids.shape[0]
+    if out is None:
+        out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
+    _gpu("out", out, torch.float32, 2)
+    _require(out.shape == (tokens, hidden), f"out must be {(tokens, hidden)}, is {tuple(out.shape)}")
+    _run("cie_embed", load_library().cie_embed(_stream(), _i(_code(table.dtype)), _ptr(table), _ptr(ids),
+                                               _ptr(out), _i(tokens), _i(hidden), _i(vocab)))
+    return out
+
+
+def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``residual += branch`` (if given; written back unless ``rows``), then RMS-normalise.
+
+    residual float32 [T, H]; branch and the result in ``out_dtype``; weight [H]
+    in ``out_dtype`` or float32.  With ``rows`` (int32 [n]) only those rows are
+    produced, in that order, and the residual is left as it is."""
+    _gpu("residual", residual, torch.float32, 2)
+    tokens, hidden = residual.shape
+    _gpu("weight", weight, dims=1)
+    _require(weight.shape[0] == hidden, f"weight must be [{hidden}], is {tuple(weight.shape)}")
+    _require(weight.dtype in (out_dtype, torch.float32), f"weight dtype {weight.dtype} does not fit {out_dtype}")
+    _require(hidden * 4 <= 64 * 1024, f"hidden size {hidden} exceeds the norm kernel's 16384")
+    _require(eps > 0, f"eps must be positive, is {eps}")
+    if branch is not None:
+        _gpu("branch", branch, out_dtype, 2)
+        _require(branch.shape == residual.shape, f"branch {tuple(branch.shape)} vs residual {tuple(residual.shape)}")
+    if rows is not None:
+        _gpu("rows", rows, torch.int32, 1)
+        n_out = rows.shape[0]
+    else:
+        n_out = tokens
+    if out is None:
+        out = torch.empty((n_out, hidden), dtype=out_dtype, device=residual.device)
+    _gpu("out", out, out_dtype, 2)
+    _require(out.shape == (n_out, hidden), f"out must be {(n_out, hidden)}, is {tuple(out.shape)}")
+    _run("cie_add_rmsnorm", load_library().cie_add_rmsnorm(
+        _stream(), _i(_code(out_dtype)), _i(_code(weight.dtype)), _ptr(residual), _ptr(branch), _ptr(weight),
+        _ptr(out), _ptr(rows), _i(n_out), _i(hidden), _f(eps), _i(0 if rows is not None else 1)))
+    return out
+
+
+def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                  seq_of_token: torch.Tensor, seq_slot: torch.Tensor, block_table: torch.Tensor,
+                  k_pool: torch.Tensor, v_pool: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int,
+                  rotate: bool = True, write_kv: bool = True) -> None:
+    """Rotate q (in place) and k, write k and v of every token into its cache slot.
+
+    qkv [T, (Hq+2Hkv)*D]; cos/sin float32 [max_position, D/2]; pools
+    [pages, Hkv, page_size, D] in qkv's dtype; block_table int32 [slots, width]."""
+    _gpu("qkv", qkv, dims=2)
+    tokens = qkv.shape[0]
+    _require(qkv.shape[1] == (q_heads + 2 * kv_heads) * head_dim,
+             f"qkv row is {qkv.shape[1]}, heads say {(q_heads + 2 * kv_heads) * head_dim}")
+    _require(head_dim % 2 == 0, f"head_dim must be even, is {head_dim}")
+    for name, table in (("cos", cos), ("sin", sin)):
+        _gpu(name, table, torch.float32, 2)
+        _require(table.shape[1] == head_dim // 2, f"{name} must be [max_position, {head_dim // 2}]")
+    _require(cos.shape == sin.shape, "cos and sin tables differ in shape")
+    for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
+        _gpu(name, meta, torch.int32, 1)
+        _require(meta.shape[0] >= tokens, f"{name} has {meta.shape[0]} entries for {tokens} tokens")
+    _gpu("seq_slot", seq_slot, torch.int32, 1)
+    _gpu("block_table", block_table, torch.int32, 2)
+    for name, pool in (("k_pool", k_pool), ("v_pool", v_pool)):
+        _gpu(name, pool, qkv.dtype, 4)
+        _require(pool.shape[1] == kv_heads and pool.shape[3] == head_dim,
+                 f"{name} {tuple(pool.shape)} does not match Hkv={kv_heads}, D={head_dim}")
+    _require(k_pool.shape == v_pool.shape, "key and value pools differ in shape")
+    page_size = k_pool.shape[2]
+    _run("cie_rope_kv_write", load_library().cie_rope_kv_write(
+        _stream(), _i(_code(qkv.dtype)), _ptr(qkv), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(seq_of_token),
+        _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]), _ptr(k_pool), _ptr(v_pool), _i(tokens),
+        _i(q_heads), _i(kv_heads), _i(head_dim), _i(page_size), _i(1 if rotate else 0), _i(1 if write_kv else 0)))
+
+
+def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for gate_up [T, 2I]."""
+    _gpu("gate_up", gate_up, dims=2)
+    tokens, twice = gate_up.shape
+    _require(twice % 2 == 0, f"gate_up row must be even, is {twice}")
+    inter = twice // 2
+    if out is None:
+        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
+    _gpu("out", out, gate_up.dtype, 2)
+    _require(out.shape == (tokens, inter), f"out must be {(tokens, inter)}, is {tuple(out.shape)}")
+    _run("cie_silu_mul", load_library().cie_silu_mul(_stream(), _i(_code(gate_up.dtype)), _ptr(gate_up),
+                                                     _ptr(out), _i(tokens), _i(inter)))
+    return out
+
+
+def paged_attention_generic(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                            block_table: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor,
+                            seq_slot: torch.Tensor, tokens: int, q_heads: int, kv_heads: int, head_dim: int,
+                            window: Optional[int], scale: float,
+                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention of each token over its request's cached keys (its own included).
+
+    ``q`` is any tensor whose row ``t`` holds the token's q heads in its first
+    ``q_heads*head_dim`` elements, rows ``q_row_stride`` elements apart (the
+    fused qkv buffer qualifies).  Returns [tokens, q_heads*head_dim]."""
+    _require(q.is_cuda and q.dim() == 2 and q.stride(1) == 1 and q.stride(0) == q_row_stride,
+             f"q must be 2-d on the GPU with unit inner stride and row stride {q_row_stride}")
+    _require(q.shape[0] >= tokens and q.shape[1] >= q_heads * head_dim, f"q {tuple(q.shape)} too small")
+    _require(q_heads % kv_heads == 0, f"{q_heads} query heads are no multiple of {kv_heads} key heads")
+    _require(head_dim % 8 == 0 and head_dim <= 256, f"head_dim must be a multiple of 8 up to 256, is {head_dim}")
+    _require(q_row_stride % 8 == 0, f"q row stride must be a multiple of 8, is {q_row_stride}")
+    for name, pool in (("k_pool", k_pool), ("v_pool", v_pool)):
+        _gpu(name, pool, q.dtype, 4)
+        _require(pool.shape[1] == kv_heads and pool.shape[3] == head_dim,
+                 f"{name} {tuple(pool.shape)} does not match Hkv={kv_heads}, D={head_dim}")
+    _gpu("block_table", block_table, torch.int32, 2)
+    for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
+        _gpu(name, meta, torch.int32, 1)
+        _require(meta.shape[0] >= tokens, f"{name} has {meta.shape[0]} entries for {tokens} tokens")
+    _gpu("seq_slot", seq_slot, torch.int32, 1)
+    if out is None:
+        out = torch.empty((tokens, q_heads * head_dim), dtype=q.dtype, device=q.device)
+    _gpu("out", out, q.dtype, 2)
+    _require(out.shape == (tokens, q_heads * head_dim), f"out is {tuple(out.shape)}")
+    _run("cie_paged_attention_generic", load_library().cie_paged_attention_generic(
+        _stream(), _i(_code(q.dtype)), _ptr(q), _i(q_row_stride), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
+        _i(block_table.shape[1]), _ptr(positions), _ptr(seq_of_token), _ptr(seq_slot), _ptr(out), _i(tokens),
+        _i(q_heads), _i(kv_heads), _i(head_dim), _i(k_pool.shape[2]), _i(window or 0), _f(scale)))
+    return out
+
+
+def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """True float32 ``a @ weight.T + bias``; a [M, K] (rows may be strided), weight [N, K]."""
+    _require(a.is_cuda and a.dtype == torch.float32 and a.dim() == 2 and a.stride(1) == 1,
+             "a must be a float32 GPU matrix with unit inner stride")
+    _gpu("weight", weight, torch.float32, 2)
+    m, k = a.shape
+    n = weight.shape[0]
+    _require(weight.shape[1] == k, f"a is [{m},{k}] but weight is {tuple(weight.shape)}")
+    if bias is not None:
+        _gpu("bias", bias, torch.float32, 1)
+        _require(bias.shape[0] == n, f"bias must be [{n}]")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    _gpu("out", out, torch.float32, 2)
+    _require(out.shape == (m, n), f"out must be {(m, n)}")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    _run("cie_gemm_f32", load_library().cie_gemm_f32(_stream(), _ptr(a), _ptr(weight), _ptr(bias), _ptr(out),
+                                                     _i(m), _i(n), _i(k), _i(lda), _i(n)))
+    return out
+
+
+def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+              out_dtype: torch.dtype = torch.bfloat16, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Matrix-core ``a @ weight.T + bias`` for few rows: bf16 operands, float32
+    accumulation, float32 or bf16 result.  K must be a multiple of 8."""
+    _require(a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1,
+             "a must be a bfloat16 GPU matrix with unit inner stride")
+    _gpu("weight", weight, torch.bfloat16, 2)
+    m, k = a.shape
+    n = weight.shape[0]
+    _require(weight.shape[1] == k, f"a is [{m},{k}] but weight is {tuple(weight.shape)}")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    _require(k % 8 == 0 and lda % 8 == 0, f"K and the row stride must be multiples of 8, are {k} and {lda}")
+    _require(a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+    if bias is not None:
+        _gpu("bias", bias, torch.bfloat16, 1)
+        _require(bias.shape[0] == n, f"bias must be [{n}]")
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    _gpu("out", out, out_dtype, 2)
+    _require(out.shape == (m, n), f"out must be {(m, n)}")
+    _run("cie_gemm_bf16", load_library().cie_gemm_bf16(_stream(), _ptr(a), _ptr(weight), _ptr(bias), _ptr(out),
+                                                       _i(_code(out_dtype)), _i(m), _i(n), _i(k), _i(lda), _i(n)))
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+           uniform: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row of float32 logits: argmax where the row's temperature
+    is 0 (or none is given), else a draw with the row's uniform number."""
+    _gpu("logits", logits, torch.float32, 2)
+    rows, vocab = logits.shape
+    if temperature is not None:
+        _gpu("temperature", temperature, torch.float32, 1)
+        _require(uniform is not None, "temperature sampling needs the uniform numbers")
+        _gpu("uniform", uniform, torch.float32, 1)
+        _require(temperature.shape[0] == rows and uniform.shape[0] == rows, "one temperature and one uniform per row")
+    if out is None:
+        out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    _gpu("out", out, torch.int32, 1)
+    _require(out.shape[0] == rows, f"out must be [{rows}]")
+    _run("cie_sample", load_library().cie_sample(_stream(), _ptr(logits), _ptr(temperature), _ptr(uniform),
+                                                 _ptr(out), _i(rows), _i(vocab), _i(vocab)))
+    return out

@@ -1,0 +1,43 @@
+"""Gated feed-forward (SwiGLU): ``down(act(gate(x)) * up(x))`` without biases.
+
+Reference: ``Qwen2MLP`` (src/cloud_engine/model.py:86-100).  Gate and up are
+one fused product here, the activation and the multiply one kernel.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.tensors import TensorSpec
+from .base import Part, register_part
+from .linear import linear
+
+
+class GatedMLP(Part):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
+        if activation != "silu":
+            raise ValueError(f"gated feed-forward runs silu only, got {activation!r}")
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        return {
+            prefix + "gate_proj.weight": TensorSpec((self.intermediate_size, self.hidden_size)),
+            prefix + "up_proj.weight": TensorSpec((self.intermediate_size, self.hidden_size)),
+            prefix + "down_proj.weight": TensorSpec((self.hidden_size, self.intermediate_size)),
+        }
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        self.w_gate_up = torch.cat(
+            [tensors[prefix + "gate_proj.weight"], tensors[prefix + "up_proj.weight"]], dim=0
+        ).contiguous()
+        self.w_down = tensors[prefix + "down_proj.weight"].contiguous()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        gate_up = linear(x, self.w_gate_up)
+        return linear(ops.silu_mul(gate_up), self.w_down)
+
+
+register_part("feed_forward", "gated_mlp", GatedMLP)

@@ -1,0 +1,40 @@
+"""RMSNorm, fused with the residual add that precedes it.
+
+Formula of the reference's ``rms_norm`` (src/cloud_engine/attention.py:52-57):
+``x * rsqrt(mean(x^2) + eps) * weight`` with float32 statistics.  The reference
+rounds the normalised value to the model dtype before the weight multiply; here
+the multiply is float32 too and the result is rounded once.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from ..weights.tensors import TensorSpec
+from .base import Part, register_part
+
+
+class RMSNorm(Part):
+    def __init__(self, size: int, eps: float) -> None:
+        if size <= 0 or not eps > 0:
+            raise ValueError(f"RMSNorm needs a positive size and eps, got {size}, {eps}")
+        self.size = size
+        self.eps = eps
+        self.weight: Optional[torch.Tensor] = None
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        return {prefix + "weight": TensorSpec((self.size,), init="norm", keeps_float32=True)}
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        self.weight = tensors[prefix + "weight"].contiguous()
+
+    def forward(self, residual: torch.Tensor, branch: Optional[torch.Tensor], out_dtype: torch.dtype,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.add_rmsnorm(residual, branch, self.weight, self.eps, out_dtype, rows=rows)
+
+
+register_part("norm", "rms_norm", RMSNorm)

@@ -1,0 +1,158 @@
+"""Schedules for replay tests, in the line format ``bin/trace_run`` reads, and
+helpers that drive a Runner with them and sort the logits by request and position."""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+
+def whole(requests: dict[str, list[int]]) -> list[dict]:
+    """Each request alone and whole: one step, every position wanted."""
+    steps = []
+    for rid, tokens in requests.items():
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": tokens, "want": list(range(len(tokens)))}],
+                      "end": [rid]})
+    return steps
+
+
+def tail_one_by_one(requests: dict[str, list[int]], tail: int = 32) -> list[dict]:
+    """Most of the request in one step, the last ``tail`` tokens one by one."""
+    steps = []
+    for rid, tokens in requests.items():
+        head = max(len(tokens) - tail, 1)
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": tokens[:head], "want": list(range(head))}],
+                      "end": []})
+        for i in range(head, len(tokens)):
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": [tokens[i]], "want": [0]}],
+                          "end": [rid] if i == len(tokens) - 1 else []})
+        if head == len(tokens):
+            steps[-1]["end"] = [rid]
+    return steps
+
+
+def portions(requests: dict[str, list[int]], sizes=(7, 2, 16, 3, 2, 5, 33, 2, 9, 17)) -> list[dict]:
+    """Portions of changing size, down to two tokens, crossing pages at odd offsets."""
+    steps = []
+    for rid, tokens in requests.items():
+        fed = 0
+        turn = 0
+        while fed < len(tokens):
+            size = min(sizes[turn % len(sizes)], len(tokens) - fed)
+            if len(tokens) - fed - size == 1:  # never leave a one-token rest: portions have two tokens or more
+                size += 1
+            turn += 1
+            chunk = tokens[fed:fed + size]
+            fed += size
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": chunk, "want": list(range(size))}],
+                          "end": [rid] if fed == len(tokens) else []})
+    return steps
+
+
+def mixed(requests: dict[str, list[int]], live: int = 4, chunk_sizes=(5, 12, 2, 9, 3), decode_tail: int = 6,
+          seed: int = 0) -> list[dict]:
+    """Up to ``live`` requests at a time; each step holds portions of some beside
+    single tokens of others; a finished request's pages go back and the next
+    waiting request starts, so pages are used again."""
+    rng = np.random.default_rng(seed)
+    waiting = list(requests.items())
+    active: list[list] = []  # [rid, tokens, fed]
+    steps = []
+    turn = 0
+    while waiting or active:
+        while waiting and len(active) < live:
+            rid, tokens = waiting.pop(0)
+            active.append([rid, tokens, 0])
+        entries = []
+        ended = []
+        for state in active:
+            rid, tokens, fed = state
+            if rng.random() < 0.25 and len(active) > 1 and len(entries) > 0:
+                continue  # this request sits the step out
+            left = len(tokens) - fed
+            if left <= decode_tail:
+                size = 1
+            else:
+                size = min(chunk_sizes[turn % len(chunk_sizes)], left - decode_tail)
+                size = max(size, 1)
+            turn += 1
+            chunk = tokens[fed:fed + size]
+            state[2] = fed + size
+            entries.append({"id": rid, "tokens": chunk, "want": list(range(size))})
+            if state[2] == len(tokens):
+                ended.append(rid)
+        active = [s for s in active if s[2] < len(s[1])]
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+    return steps
+
+
+def max_live_tokens(steps: list[dict], page: int = 64) -> int:
+    """Most tokens live requests hold at any time, each rounded up to ``page``."""
+    held: dict[str, int] = {}
+    peak = 0
+    for step in steps:
+        for entry in step["entries"]:
+            held[entry["id"]] = held.get(entry["id"], 0) + len(entry["tokens"])
+        peak = max(peak, sum(-(-n // page) * page for n in held.values()))
+        for rid in step["end"]:
+            held.pop(rid, None)
+    return peak
+
+
+def drive_runner(runner, steps: list[dict]) -> dict[int, np.ndarray]:
+    """What bin/trace_run does, in-process."""
+    from cie_amd.engine.runner import StepEntry
+
+    out = {}
+    for step in steps:
+        entries = []
+        for item in step["entries"]:
+            if not runner.cache.has(item["id"]):
+                runner.cache.admit(item["id"])
+            entries.append(StepEntry(item["id"], item["tokens"], runner.cache.length(item["id"]), item["want"]))
+        if entries:
+            logits = runner.run(entries)
+            if logits.shape[0]:
+                out[step["step"]] = logits.float().cpu().numpy()
+        for rid in step["end"]:
+            runner.cache.release(rid)
+        runner.cache.assert_invariants()
+    return out
+
+
+def by_position(steps: list[dict], outputs: dict[int, np.ndarray]) -> dict[str, dict[int, np.ndarray]]:
+    """{request: {position: logits row}} from the per-step arrays."""
+    fed: dict[str, int] = {}
+    rows: dict[str, dict[int, np.ndarray]] = {}
+    for step in steps:
+        data = outputs.get(step["step"])
+        cursor = 0
+        for entry in step["entries"]:
+            base = fed.get(entry["id"], 0)
+            for place in entry["want"]:
+                rows.setdefault(entry["id"], {})[base + place] = data[cursor]
+                cursor += 1
+            fed[entry["id"]] = base + len(entry["tokens"])
+        if data is not None:
+            assert cursor == data.shape[0], "logits rows and wanted places disagree"
+    return rows
+
+
+def compare(rows: dict[str, dict[int, np.ndarray]], plain: dict[str, torch.Tensor], rtol: float, atol: float) -> float:
+    """Assert every position of every request against the plain logits; returns the worst abs difference."""
+    worst = 0.0
+    for rid, expected in plain.items():
+        got = rows[rid]
+        assert sorted(got) == list(range(expected.shape[0])), f"{rid}: positions {sorted(got)[:5]}..."
+        stacked = np.stack([got[p] for p in range(expected.shape[0])])
+        want = expected.numpy()
+        diff = np.abs(stacked - want)
+        worst = max(worst, float(diff.max()))
+        bad = diff > atol + rtol * np.abs(want)
+        if bad.any():
+            pos = int(np.argwhere(bad.any(axis=1))[0][0])
+            raise AssertionError(
+                f"request {rid}: first wrong position {pos} of {expected.shape[0]}, "
+                f"max |diff| there {diff[pos].max():.3e}, overall {diff.max():.3e}"
+            )
+    return worst

@@ -1,0 +1,296 @@
+"""GPU: each HIP kernel alone against a plain float32 torch reference of the same
+operation, at sizes other than the tiny models' (odd widths, many heads and
+groups, head sizes in steps of 16)."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+import plain_qwen2
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-2)
+
+
+def rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from cie_amd.kernels import ops as module
+
+    return module
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(ops, dtype):
+    table = rand((1000, 72), dtype, 1)
+    ids = torch.tensor([0, 999, 5, 5, 321], dtype=torch.int32).cuda()
+    out = ops.embed(table, ids)
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out, table.float()[ids.long()], rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [72, 1000, 4104])
+def test_add_rmsnorm(ops, dtype, hidden):
+    residual = rand((7, hidden), torch.float32, 2, 3.0)
+    branch = rand((7, hidden), dtype, 3)
+    weight = rand((hidden,), dtype, 4) + 1
+    eps = 1e-5
+    expect_res = residual + branch.float()
+    expect = plain_qwen2.rms_norm(expect_res, weight.float(), eps)
+    out = ops.add_rmsnorm(residual, branch, weight, eps, dtype)
+    torch.testing.assert_close(residual, expect_res, rtol=0, atol=0)  # the float32 sum is written back
+    torch.testing.assert_close(out.float(), expect, **tol(dtype))
+    # no branch, selected rows only, float32 weight beside bf16 activations
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32).cuda()
+    before = residual.clone()
+    out = ops.add_rmsnorm(residual, None, weight.float(), eps, dtype, rows=rows)
+    torch.testing.assert_close(residual, before, rtol=0, atol=0)
+    torch.testing.assert_close(out.float(), expect[rows.long()], **tol(dtype))
+
+
+def test_rmsnorm_invariants(ops):
+    """weight 1, tiny eps: every output row has RMS 1; scaling the input changes nothing."""
+    x = rand((4, 200), torch.float32, 5, 2.0)
+    ones = torch.ones(200, device="cuda")
+    out = ops.add_rmsnorm(x.clone(), None, ones, 1e-12, torch.float32)
+    torch.testing.assert_close(out.pow(2).mean(-1), torch.ones(4, device="cuda"), rtol=1e-5, atol=1e-5)
+    out2 = ops.add_rmsnorm(x * 7.5, None, ones, 1e-12, torch.float32)
+    torch.testing.assert_close(out, out2, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(ops, dtype):
+    gate_up = rand((5, 2 * 333), dtype, 6, 2.0)
+    g, u = gate_up.float()[:, :333], gate_up.float()[:, 333:]
+    out = ops.silu_mul(gate_up)
+    torch.testing.assert_close(out.float(), torch.nn.functional.silu(g) * u, **tol(dtype))
+    zero_gate = torch.cat([torch.zeros(5, 333), torch.randn(5, 333)], dim=1).to(dtype).cuda()
+    assert ops.silu_mul(zero_gate).abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("shape", [(1, 40, 24), (5, 515, 96), (70, 130, 200), (130, 64, 17)])
+def test_gemm_f32(ops, shape):
+    m, n, k = shape
+    a, w, b = rand((m, k), torch.float32, 7), rand((n, k), torch.float32, 8), rand((n,), torch.float32, 9)
+    expect = (a.double() @ w.double().t() + b.double()).float()
+    torch.testing.assert_close(ops.gemm_f32(a, w, b), expect, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(ops.gemm_f32(a, w), (a.double() @ w.double().t()).float(), rtol=1e-5, atol=1e-5)
+    # a row's result does not depend on the other rows of the batch (bitwise)
+    assert torch.equal(ops.gemm_f32(a[:1].contiguous(), w, b), ops.gemm_f32(a, w, b)[:1])
+
+
+@pytest.mark.parametrize("shape", [(1, 40, 24), (5, 515, 96), (16, 64, 128), (17, 130, 200), (33, 70, 1032),
+                                   (64, 256, 264), (150, 99, 72)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_gemm_bf16(ops, shape, out_dtype):
+    m, n, k = shape
+    a, w, b = rand((m, k), torch.bfloat16, 10), rand((n, k), torch.bfloat16, 11), rand((n,), torch.bfloat16, 12)
+    expect = a.double() @ w.double().t()
+    out = ops.gemm_bf16(a, w, None, out_dtype)
+    assert out.dtype == out_dtype
+    if out_dtype == torch.float32:
+        torch.testing.assert_close(out.double(), expect, rtol=1e-4, atol=1e-4 * math.sqrt(k))
+    else:
+        torch.testing.assert_close(out.double(), expect, rtol=1e-2, atol=1e-2 * math.sqrt(k))
+    out = ops.gemm_bf16(a, w, b, torch.float32)
+    torch.testing.assert_close(out.double(), expect + b.double(), rtol=1e-4, atol=1e-4 * math.sqrt(k))
+
+
+def build_cache(dtype, lengths, kv_heads, head_dim, page_size, seed, shuffle=True):
+    """Random keys/values for sequences of the given lengths, scattered over the
+    pages of a pool in a shuffled order.  Returns pools, block table and the
+    dense per-sequence tensors."""
+    g = torch.Generator().manual_seed(seed)
+    pages_per = [-(-n // page_size) for n in lengths]
+    total = sum(pages_per) + 3
+    order = torch.randperm(total, generator=g).tolist() if shuffle else list(range(total))
+    width = max(pages_per) + 2
+    table = torch.zeros((len(lengths) + 2, width), dtype=torch.int32)
+    slots = list(range(len(lengths), 0, -1))  # slot != sequence index, on purpose
+    k_pool = torch.zeros((total, kv_heads, page_size, head_dim))
+    v_pool = torch.zeros_like(k_pool)
+    dense = []
+    cursor = 0
+    for s, n in enumerate(lengths):
+        k = torch.randn((n, kv_heads, head_dim), generator=g)
+        v = torch.randn((n, kv_heads, head_dim), generator=g)
+        k, v = k.to(dtype).float(), v.to(dtype).float()
+        dense.append((k, v))
+        for p in range(pages_per[s]):
+            page = order[cursor]
+            cursor += 1
+            table[slots[s], p] = page
+            rows = slice(p * page_size, min((p + 1) * page_size, n))
+            count = rows.stop - rows.start
+            k_pool[page, :, :count] = k[rows].transpose(0, 1)
+            v_pool[page, :, :count] = v[rows].transpose(0, 1)
+    return k_pool.to(dtype).cuda(), v_pool.to(dtype).cuda(), table.cuda(), slots, dense
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geometry", [(4, 2, 16, 16), (16, 2, 128, 16), (6, 6, 48, 8), (8, 1, 64, 32), (5, 5, 80, 4)])
+def test_paged_attention_generic(ops, dtype, geometry):
+    """Ragged batch: a long prompt portion with context, a fresh prompt, single
+    decode tokens at page edges.  Context/query sizes follow the reference's
+    matrix (tests/remote_ragged_gpu_tests.py:118-121) scaled down."""
+    q_heads, kv_heads, head_dim, page_size = geometry
+    contexts = [0, 15, 16, 17, 127, 300, 1]
+    q_lens = [7, 1, 1, 2, 16, 1, 33]
+    lengths = [c + q for c, q in zip(contexts, q_lens)]
+    k_pool, v_pool, table, slots, dense = build_cache(dtype, lengths, kv_heads, head_dim, page_size, seed=20)
+    scale = 1.0 / math.sqrt(head_dim)
+    g = torch.Generator().manual_seed(21)
+    positions, seq_of_token, expected, qs = [], [], [], []
+    for s, (c, n) in enumerate(zip(contexts, q_lens)):
+        q = (torch.randn((n, q_heads, head_dim), generator=g) * 2).to(dtype).float()
+        qs.append(q)
+        positions += list(range(c, c + n))
+        seq_of_token += [s] * n
+        k, v = dense[s]
+        expected.append(plain_qwen2.causal_attention(q, k, v, scale, past_len=c))
+    q_all = torch.cat(qs).reshape(len(positions), q_heads * head_dim)
+    stride = (q_heads + 2 * kv_heads) * head_dim  # as if q sat inside a fused qkv buffer
+    buffer = torch.zeros((len(positions), stride))
+    buffer[:, : q_heads * head_dim] = q_all
+    buffer = buffer.to(dtype).cuda()
+    out = ops.paged_attention_generic(
+        buffer, stride, k_pool, v_pool, table, torch.tensor(positions, dtype=torch.int32).cuda(),
+        torch.tensor(seq_of_token, dtype=torch.int32).cuda(), torch.tensor(slots, dtype=torch.int32).cuda(),
+        len(positions), q_heads, kv_heads, head_dim, None, scale)
+    torch.testing.assert_close(out.float().cpu(), torch.cat(expected), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_far_key_and_window(ops, dtype):
+    """One far key is made to dominate: the output must be its value row.  With a
+    window that excludes it, it must vanish; the window's edge is exact."""
+    q_heads, kv_heads, head_dim, page_size = 4, 2, 32, 8
+    length, far = 400, 37
+    k_pool, v_pool, table, slots, dense = build_cache(dtype, [length], kv_heads, head_dim, page_size, seed=30)
+    k, v = dense[0]
+    q = torch.zeros((1, q_heads, head_dim))
+    for h in range(q_heads):
+        q[0, h] = k[far, h // 2] * 4.0  # aligned with the far key, far larger score than any other
+    q = q.to(dtype).float()
+    scale = 1.0 / math.sqrt(head_dim)
+    args = (k_pool, v_pool, table, torch.tensor([length - 1], dtype=torch.int32).cuda(),
+            torch.tensor([0], dtype=torch.int32).cuda(), torch.tensor(slots, dtype=torch.int32).cuda(),
+            1, q_heads, kv_heads, head_dim)
+    qd = q.reshape(1, -1).to(dtype).cuda()
+    full = ops.paged_attention_generic(qd, q_heads * head_dim, *args, None, scale).float().cpu()
+    expect_full = plain_qwen2.causal_attention(q, k, v, scale, past_len=length - 1)
+    torch.testing.assert_close(full, expect_full, **tol(dtype))
+    # the far key carries nearly all the weight
+    torch.testing.assert_close(full.reshape(q_heads, head_dim), v[far].repeat_interleave(2, dim=0), rtol=0.1, atol=0.1)
+    for window in (length - far, length - far - 1):  # far key just inside / just outside
+        got = ops.paged_attention_generic(qd, q_heads * head_dim, *args, window, scale).float().cpu()
+        expect = plain_qwen2.causal_attention(q, k, v, scale, past_len=length - 1, window=window)
+        torch.testing.assert_close(got, expect, **tol(dtype))
+    assert (got - full).abs().max() > 0.1  # outside the window the answer changes
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geometry", [(4, 2, 16, 16), (3, 1, 48, 8), (16, 2, 128, 16)])
+def test_rope_kv_write(ops, dtype, geometry):
+    q_heads, kv_heads, head_dim, page_size = geometry
+    theta, max_pos = 10000.0, 512
+    lengths = [40, 3, 100]
+    starts = [30, 0, 99]  # tokens of this step: positions start..length-1
+    k_pool, v_pool, table, slots, _ = build_cache(dtype, lengths, kv_heads, head_dim, page_size, seed=40)
+    k_before, v_before = k_pool.clone(), v_pool.clone()
+    positions, seq_of_token = [], []
+    for s, (start, n) in enumerate(zip(starts, lengths)):
+        positions += list(range(start, n))
+        seq_of_token += [s] * (n - start)
+    t = len(positions)
+    qkv = rand((t, (q_heads + 2 * kv_heads) * head_dim), dtype, 41)
+    original = qkv.float().cpu()
+    cos, sin = plain_qwen2.rope_tables(head_dim, max_pos, theta)
+    half = head_dim // 2
+    pos_t = torch.tensor(positions)
+    ops.rope_kv_write(qkv, cos[:, :half].contiguous().cuda(), sin[:, :half].contiguous().cuda(),
+                      torch.tensor(positions, dtype=torch.int32).cuda(),
+                      torch.tensor(seq_of_token, dtype=torch.int32).cuda(),
+                      torch.tensor(slots, dtype=torch.int32).cuda(), table, k_pool, v_pool,
+                      q_heads, kv_heads, head_dim)
+    q_in = original[:, : q_heads * head_dim].view(t, q_heads, head_dim)
+    k_in = original[:, q_heads * head_dim: (q_heads + kv_heads) * head_dim].view(t, kv_heads, head_dim)
+    v_in = original[:, (q_heads + kv_heads) * head_dim:].view(t, kv_heads, head_dim)
+    q_expect = plain_qwen2.apply_rope(q_in, cos, sin, pos_t)
+    k_expect = plain_qwen2.apply_rope(k_in, cos, sin, pos_t)
+    torch.testing.assert_close(qkv.float().cpu()[:, : q_heads * head_dim].view(t, q_heads, head_dim), q_expect, **tol(dtype))
+    table_h = table.cpu()
+    touched = torch.zeros(k_pool.shape[:3], dtype=torch.bool)  # [page, head, row]
+    for i, (pos, s) in enumerate(zip(positions, seq_of_token)):
+        page = int(table_h[slots[s], pos // page_size])
+        row = pos % page_size
+        torch.testing.assert_close(k_pool[page, :, row].float().cpu(), k_expect[i], **tol(dtype))
+        torch.testing.assert_close(v_pool[page, :, row].float().cpu(), v_in[i], rtol=0, atol=0)
+        touched[page, :, row] = True
+    # nothing else in the pools moved
+    untouched = ~touched.cuda()
+    assert torch.equal(k_pool[untouched], k_before[untouched])
+    assert torch.equal(v_pool[untouched], v_before[untouched])
+
+
+def test_rope_shift_invariance():
+    """Scores of rotated q and k depend on the distance of their positions only
+    (pins sign and pairing of the rotation in the plain implementation)."""
+    head_dim = 32
+    cos, sin = plain_qwen2.rope_tables(head_dim, 600, 10000.0)
+    g = torch.Generator().manual_seed(50)
+    q = torch.randn((1, 1, head_dim), generator=g, dtype=torch.float64)
+    k = torch.randn((1, 1, head_dim), generator=g, dtype=torch.float64)
+    cos, sin = cos.double(), sin.double()
+
+    def score(m, n):
+        qm = plain_qwen2.apply_rope(q, cos, sin, torch.tensor([m]))
+        kn = plain_qwen2.apply_rope(k, cos, sin, torch.tensor([n]))
+        return (qm * kn).sum()
+
+    assert abs(score(10, 3) - score(210, 203)) < 1e-3  # float32 tables limit the agreement
+    assert abs(score(10, 3) - score(10, 4)) > 1e-3
+
+
+def test_sample_greedy_and_temperature(ops):
+    g = torch.Generator().manual_seed(60)
+    logits = torch.randn((6, 1003), generator=g).cuda() * 3
+    logits[2, 500] = logits[2, 17] = logits[2].max() + 1  # a tie: the lower index wins
+    out = ops.sample(logits)
+    assert out.tolist() == torch.argmax(logits, dim=-1).tolist()
+    assert out[2].item() == 17
+    temperature = torch.tensor([0.0, 0.7, 1.0, 1.3, 0.7, 2.0]).cuda()
+    uniform = torch.tensor([0.3, 0.0, 0.999999, 0.5, 0.25, 0.75]).cuda()
+    got = ops.sample(logits, temperature, uniform).tolist()
+    assert got[0] == out[0].item()  # temperature 0 is greedy
+    for r in range(1, 6):
+        p = torch.softmax(logits[r].double() / temperature[r].double(), dim=-1).cpu()
+        cdf = torch.cumsum(p, dim=0)
+        u = float(uniform[r])
+        lo = cdf[got[r] - 1].item() if got[r] > 0 else 0.0
+        assert lo - 1e-5 <= u <= cdf[got[r]].item() + 1e-5, (r, got[r], lo, u, cdf[got[r]].item())
+
+
+def test_sample_frequencies(ops):
+    """Empirical frequencies on a four-token vocabulary follow softmax(l / T)."""
+    logits = torch.tensor([[0.0, 1.0, 2.0, -1.0]]).repeat(4000, 1).cuda()
+    g = torch.Generator().manual_seed(61)
+    uniform = torch.rand(4000, generator=g).cuda()
+    temperature = torch.full((4000,), 0.8).cuda()
+    got = ops.sample(logits, temperature, uniform)
+    freq = torch.bincount(got.long().cpu(), minlength=4).double() / 4000
+    expect = torch.softmax(torch.tensor([0.0, 1.0, 2.0, -1.0]).double() / 0.8, dim=0)
+    assert (freq - expect).abs().max() < 0.03
