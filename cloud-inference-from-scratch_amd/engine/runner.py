@@ -22,6 +22,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..config.engine_config import EngineConfig
 from ..profiling import trace_range
+from ..sampling.sampler import Sampler
 from .batch import StepBatch
 from .device_cache import DeviceCache
 
@@ -59,6 +60,7 @@ class Runner:
         self.forward_invocations = 0
         self.max_forward_request_count = 0
         self.forward_plans: deque[tuple[tuple[str, int, int, int], ...]] = deque(maxlen=256)
+        self.sampler = Sampler(config.seed)
         self._staging = [None, None]
         self._staging_turn = 0
 
@@ -79,6 +81,32 @@ class Runner:
 
     def allocated_tokens(self, request: Any) -> int:
         return self.cache.allocated_tokens(request.request_id)
+
+    def free_tokens(self) -> int:
+        """Tokens the pool could take now (free pages of the scarcest group)."""
+        return min((g.allocator.free_count for g in self.cache.groups), default=0) * self.cache.page_size
+
+    def execute_batch(self, plan: Any) -> dict[str, int]:
+        """Run a scheduler's plan and sample where it asks to (the reference's
+        ``execute_batch``, src/cloud_engine/engine.py:439-488)."""
+        entries = [
+            StepEntry(item.request.request_id, item.token_ids, item.start_pos,
+                      (item.query_length - 1,) if item.sample else ())
+            for item in plan.items
+        ]
+        logits = self.run(entries)
+        for item in plan.items:
+            item.request.tokens_fed = item.end_pos
+        sampled = [item.request for item in plan.items if item.sample]
+        if not sampled:
+            return {}
+        with trace_range("ragged.sample"):
+            tokens = self.sampler.sample(
+                logits,
+                [r.config.temperature for r in sampled],
+                [self.sampler.uniform(r.config.seed, r.serial, r.generated_count) for r in sampled],
+            )
+        return {r.request_id: token for r, token in zip(sampled, tokens)}
 
     # -- packing -----------------------------------------------------------------
     def _stage(self, count: int) -> tuple[torch.Tensor, torch.Tensor]:
