@@ -67,6 +67,10 @@ class Engine:
                 self.model_config = config
             else:
                 raise ValueError("give a model folder or a configuration for random weights")
+            # a request can never be longer than the model's position table
+            positions = self.model.spec.max_position
+            if self.engine_config.max_model_len > positions:
+                self.engine_config = build_engine_config(self.engine_config, max_model_len=positions)
             self.runner = Runner(self.model, self.engine_config, device)
         self.metrics = Metrics()
         self.scheduler = Scheduler(self.engine_config, self.runner, self.metrics,

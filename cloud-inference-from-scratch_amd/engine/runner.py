@@ -69,8 +69,11 @@ class Runner:
         per_token = sum(2 * n.kv_heads * n.head_dim * element for n in needs if hasattr(n, "kv_heads"))
         if per_token == 0:
             return self.config.page_size
+        page = self.config.page_size
         tokens = self.config.kv_cache_bytes // per_token
-        return max(self.config.page_size, tokens // self.config.page_size * self.config.page_size)
+        # more than every slot full plus the prefix index can never be used
+        useful = (self.config.max_running * -(-self.config.max_model_len // page) + self.config.prefix_cache_pages) * page
+        return max(page, min(tokens, useful) // page * page)
 
     # -- what the scheduler calls ------------------------------------------------
     def admit(self, request: Any) -> None:

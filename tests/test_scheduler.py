@@ -1,0 +1,265 @@
+"""CPU: the scheduler's decisions, with a fake runner in the manner of the
+reference's tests/test_ragged_scheduler.py (FakePackedRunner :32-69: a token
+capacity, a capacity error that carries ``is_capacity_error``, token
+``100 + generated_count``)."""
+
+import pytest
+
+from cie_amd.config import build_engine_config
+from cie_amd.engine.scheduler import (
+    GenerationConfig, RejectedError, RejectionReason, RequestState, Scheduler,
+)
+from cie_amd.metrics import Metrics
+
+
+class FakeRunner:
+    def __init__(self, token_capacity: int = 10_000, eos_at: dict | None = None) -> None:
+        self.token_capacity = token_capacity
+        self.resident: dict[str, int] = {}
+        self.traces: list[tuple[tuple[str, ...], tuple[int, ...]]] = []
+        self.plans = []
+        self.released: list[tuple[str, bool]] = []
+        self.fail_next: Exception | None = None
+
+    def admit(self, request) -> None:
+        if request.request_id in self.resident:
+            raise RuntimeError("duplicate admission")
+        self.resident[request.request_id] = 0
+        request.tokens_fed = 0
+
+    def release(self, request, preempted: bool = False) -> None:
+        if request.request_id in self.resident:
+            self.released.append((request.request_id, preempted))
+        self.resident.pop(request.request_id, None)
+
+    def allocated_tokens(self, request) -> int:
+        return self.resident.get(request.request_id, 0)
+
+    def free_tokens(self) -> int:
+        return self.token_capacity - sum(self.resident.values())
+
+    def execute_batch(self, plan):
+        if self.fail_next is not None:
+            error, self.fail_next = self.fail_next, None
+            raise error
+        required = dict(self.resident)
+        for item in plan.items:
+            required[item.request.request_id] = max(required[item.request.request_id], item.end_pos)
+        if sum(required.values()) > self.token_capacity:
+            error = RuntimeError("fake KV capacity exhausted")
+            error.is_capacity_error = True
+            raise error
+        self.resident = required
+        self.plans.append(plan)
+        self.traces.append((plan.request_ids, tuple(item.query_length for item in plan.items)))
+        outputs = {}
+        for item in plan.items:
+            assert item.start_pos == item.request.tokens_fed, "a portion must start where the cache ends"
+            item.request.tokens_fed = item.end_pos
+            if item.sample:
+                outputs[item.request.request_id] = 100 + item.request.generated_count
+        return outputs
+
+
+def make(runner, **overrides):
+    options = dict(max_model_len=128, max_running=4, max_queue_size=8, token_budget=16, prefill_chunk=4)
+    options.update(overrides)
+    return Scheduler(build_engine_config(**options), runner, Metrics())
+
+
+def test_requests_share_one_forward():
+    runner = FakeRunner()
+    scheduler = make(runner)
+    requests = [scheduler.submit([i + 1] * 3, GenerationConfig(max_output_tokens=2)) for i in range(3)]
+    scheduler.run_until_done(100)
+    assert [r.generated_token_ids for r in requests] == [[100, 101]] * 3
+    assert any(len(ids) == 3 for ids, _ in runner.traces)
+    assert all(r.state is RequestState.COMPLETED and r.finish_reason == "max_output_tokens_reached" for r in requests)
+    assert not runner.resident
+
+
+def test_prefill_is_cut_into_portions_under_the_budget():
+    runner = FakeRunner()
+    scheduler = make(runner, token_budget=5, prefill_chunk=4)
+    request = scheduler.submit(list(range(11)), GenerationConfig(max_output_tokens=1))
+    scheduler.run_until_done(100)
+    assert request.generated_token_ids == [100]
+    assert [lengths[0] for _, lengths in runner.traces][:3] == [4, 4, 3]
+    samples = [item.sample for plan in runner.plans for item in plan.items]
+    assert samples == [False, False, True]  # logits only where the portion reaches the tail
+
+
+def test_decode_goes_first_and_budget_is_shared():
+    runner = FakeRunner()
+    scheduler = make(runner, token_budget=6, prefill_chunk=4)
+    first = scheduler.submit([1] * 2, GenerationConfig(max_output_tokens=4))
+    scheduler.step()  # first: whole prompt, gets a token, now decoding
+    late = scheduler.submit([2] * 20, GenerationConfig(max_output_tokens=1))
+    scheduler.step()
+    plan = runner.plans[-1]
+    assert plan.request_ids == (first.request_id, late.request_id)
+    assert [item.query_length for item in plan.items] == [1, 4] and plan.items[0].is_decode
+    assert not plan.items[1].is_decode and plan.token_count <= 6
+    scheduler.run_until_done(100)
+    for plan in runner.plans:
+        assert plan.token_count <= 6 and len(set(plan.request_ids)) == len(plan.request_ids)
+        phases = [item.is_decode for item in plan.items]
+        assert phases == sorted(phases, reverse=True), "decode items come before prefill items"
+
+
+def test_custom_priority_reorders_but_cannot_exceed_budget():
+    runner = FakeRunner()
+    scheduler = make(runner, token_budget=4)
+    scheduler.scheduling_priority = lambda candidate: (candidate.remaining_tokens,)
+    long = scheduler.submit([1] * 8, GenerationConfig(max_output_tokens=1))
+    short = scheduler.submit([2] * 2, GenerationConfig(max_output_tokens=1))
+    scheduler._admit_waiting()
+    plan = scheduler._build_batch_plan()
+    assert plan.request_ids == (short.request_id, long.request_id) and plan.token_count == 4
+
+
+def test_pressure_preempts_then_recomputes_without_token_drift():
+    runner = FakeRunner(token_capacity=10)
+    scheduler = make(runner, token_budget=8, prefill_chunk=4)
+    requests = [scheduler.submit([i + 1] * 4, GenerationConfig(max_output_tokens=3)) for i in range(2)]
+    scheduler.run_until_done(200)
+    assert [r.generated_token_ids for r in requests] == [[100, 101, 102]] * 2
+    assert sum(r.preemption_count for r in requests) > 0 and sum(r.recomputed_tokens for r in requests) > 0
+    snapshot = scheduler.metrics.snapshot()
+    assert snapshot["requests"]["preempted_total"] > 0 and snapshot["tokens"]["recomputed_total"] > 0
+    assert snapshot["requests"]["completed_total"] == 2
+    assert not runner.resident
+    assert any(flag for _, flag in runner.released), "a preemption releases without storing a prefix"
+
+
+def test_preempted_request_keeps_generated_tokens_and_its_place():
+    runner = FakeRunner(token_capacity=12)
+    scheduler = make(runner, token_budget=16, prefill_chunk=8)
+    a = scheduler.submit([1] * 5, GenerationConfig(max_output_tokens=4))
+    b = scheduler.submit([2] * 5, GenerationConfig(max_output_tokens=4))
+    c = scheduler.submit([3] * 2, GenerationConfig(max_output_tokens=1))
+    scheduler.config = build_engine_config(scheduler.config, max_running=2)
+    scheduler.step()  # a and b prefilled: 10 resident; each has its first token
+    scheduler.step()  # 12 resident
+    assert (a.generated_count, b.generated_count) == (2, 2)
+    scheduler.step()  # 14 > 12: the larger one (tie: the later arrival) is preempted
+    assert b.state is RequestState.WAITING and b.preemption_count == 1 and b.tokens_fed == 0
+    assert b.generated_token_ids == [100, 101] and b.recompute_until == 6
+    assert scheduler.waiting[0] is b, "the preempted request waits at the head, before the newcomer"
+    scheduler.step()  # a decodes alone: 7 resident, 5 free; b needs 5 + 2 + 1 = 8: still waiting, c behind it
+    assert b.state is RequestState.WAITING and c.state is RequestState.WAITING
+    scheduler.run_until_done(200)
+    assert [r.generated_token_ids for r in (a, b, c)] == [[100, 101, 102, 103]] * 2 + [[100]]
+    # the recompute fed prompt and generated tokens as prompt portions and sampled only at the tail
+    recompute = [item for plan in runner.plans for item in plan.items
+                 if item.request is b and item.start_pos == 0 and item.query_length > 5]
+    assert recompute and recompute[0].token_ids == (2, 2, 2, 2, 2, 100, 101) and recompute[0].sample
+
+
+def test_custom_preemption_policy_selects_victim():
+    runner = FakeRunner(token_capacity=10)
+    scheduler = make(runner, token_budget=8, prefill_chunk=4)
+    scheduler.preemption_priority = lambda candidate: (-candidate.arrival_ns,)
+    requests = [scheduler.submit([i + 1] * 4, GenerationConfig(max_output_tokens=3)) for i in range(2)]
+    scheduler._admit_waiting()
+    runner.resident = {r.request_id: 4 for r in requests}
+    assert scheduler._preempt_for_capacity(scheduler._build_batch_plan())
+    assert (requests[0].preemption_count, requests[1].preemption_count) == (1, 0)
+
+
+def test_single_request_that_cannot_fit_is_rejected():
+    runner = FakeRunner(token_capacity=6)
+    scheduler = make(runner, token_budget=16, prefill_chunk=16)
+    request = scheduler.submit([1] * 8, GenerationConfig(max_output_tokens=2))
+    scheduler.run_until_done(10)
+    assert request.state is RequestState.FAILED and request.rejected
+    assert "KV capacity cannot fit one runnable sequence" in request.error_detail
+    assert scheduler.metrics.snapshot()["requests"]["rejected_total"] == 1 and not runner.resident
+
+
+def test_submit_time_rejections():
+    scheduler = make(FakeRunner(), max_queue_size=2, max_model_len=16)
+    with pytest.raises(RejectedError) as caught:
+        scheduler.submit([], GenerationConfig(max_output_tokens=1))
+    assert caught.value.reason is RejectionReason.CONTEXT_OVERFLOW
+    with pytest.raises(RejectedError) as caught:
+        scheduler.submit([1] * 10, GenerationConfig(max_output_tokens=7))
+    assert caught.value.reason is RejectionReason.CONTEXT_OVERFLOW
+    scheduler.submit([1] * 10, GenerationConfig(max_output_tokens=6))
+    scheduler.submit([1], GenerationConfig(max_output_tokens=1))
+    with pytest.raises(RejectedError) as caught:
+        scheduler.submit([1], GenerationConfig(max_output_tokens=1))
+    assert caught.value.reason is RejectionReason.QUEUE_FULL
+    assert [r.request_id for r in scheduler.waiting] == ["req-00000001", "req-00000002"]
+
+
+def test_generation_config_validation():
+    assert GenerationConfig(max_output_tokens=1, temperature=0.8).temperature == 0.8
+    with pytest.raises(ValueError):
+        GenerationConfig(max_output_tokens=1, temperature=-1.0)
+    with pytest.raises(ValueError):
+        GenerationConfig(max_output_tokens=0)
+
+
+def test_eos_finishes_and_is_kept_but_not_streamed():
+    runner = FakeRunner()
+    scheduler = make(runner)
+    streamed = []
+    request = scheduler.submit([1, 2], GenerationConfig(max_output_tokens=10, eos_token_id=102),
+                               on_token=lambda r, t: streamed.append(t))
+    ignoring = scheduler.submit([1, 2], GenerationConfig(max_output_tokens=4, eos_token_id=None))
+    scheduler.run_until_done(100)
+    assert request.generated_token_ids == [100, 101, 102] and request.finish_reason == "eos_token_reached"
+    assert streamed == [100, 101]
+    assert ignoring.generated_token_ids == [100, 101, 102, 103]
+
+
+def test_active_limit_and_fifo_admission():
+    runner = FakeRunner()
+    scheduler = make(runner, max_running=2)
+    requests = [scheduler.submit([1] * 2, GenerationConfig(max_output_tokens=2)) for _ in range(4)]
+    scheduler.step()
+    assert [r.state for r in requests[:2]] == [RequestState.DECODING] * 2
+    assert [r.state for r in requests[2:]] == [RequestState.WAITING] * 2
+    scheduler.run_until_done(100)
+    assert max(len(ids) for ids, _ in runner.traces) == 2
+    order = [rid for rid, _ in runner.released]
+    assert order == [r.request_id for r in requests]
+
+
+def test_cancel_is_idempotent_and_frees():
+    runner = FakeRunner()
+    scheduler = make(runner)
+    request = scheduler.submit([1] * 3, GenerationConfig(max_output_tokens=5))
+    waiting = scheduler.submit([1] * 3, GenerationConfig(max_output_tokens=5))
+    scheduler.step()
+    scheduler.cancel(request)
+    scheduler.cancel(request)
+    scheduler.cancel(waiting)
+    assert request.state is RequestState.CANCELLED and not runner.resident and not scheduler.has_work()
+    assert scheduler.metrics.snapshot()["requests"]["cancelled_total"] == 2
+
+
+def test_forward_failure_fails_the_plan_and_the_loop_goes_on():
+    runner = FakeRunner()
+    scheduler = make(runner)
+    doomed = scheduler.submit([1] * 3, GenerationConfig(max_output_tokens=2))
+    runner.fail_next = RuntimeError("kernel exploded")
+    scheduler.step()
+    assert doomed.state is RequestState.FAILED and not doomed.rejected and "kernel exploded" in doomed.error_detail
+    later = scheduler.submit([1] * 3, GenerationConfig(max_output_tokens=2))
+    scheduler.run_until_done(100)
+    assert later.generated_token_ids == [100, 101] and not runner.resident
+
+
+def test_admission_failure_is_counted():
+    class Refusing(FakeRunner):
+        def admit(self, request):
+            error = RuntimeError("no slot")
+            error.is_capacity_error = True
+            raise error
+
+    scheduler = make(Refusing())
+    request = scheduler.submit([1], GenerationConfig(max_output_tokens=1))
+    scheduler.step()
+    assert request.state is RequestState.FAILED and request.rejected and "admission refused" in request.error_detail
