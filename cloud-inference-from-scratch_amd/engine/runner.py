@@ -123,18 +123,13 @@ class Runner:
             self._staging[turn] = pair
         return pair
 
-    def pack(self, entries: Sequence[StepEntry]) -> StepBatch:
+    def check(self, entries: Sequence[StepEntry]) -> None:
+        """Refuse a step the kernels were not written for, before anything changes."""
+        if not entries:
+            raise ValueError("a step needs at least one entry")
         vocab = self.model.spec.vocab_size
-        ids: list[int] = []
-        positions: list[int] = []
-        seq_of_token: list[int] = []
-        slots: list[int] = []
-        starts: list[int] = []
-        q_lens: list[int] = []
-        q_start_loc = [0]
-        logit_rows: list[int] = []
         seen: set[str] = set()
-        for index, entry in enumerate(entries):
+        for entry in entries:
             if entry.request_id in seen:
                 raise ValueError(f"request {entry.request_id} appears twice in one step")
             seen.add(entry.request_id)
@@ -149,6 +144,21 @@ class Runner:
             for token in entry.tokens:
                 if not 0 <= token < vocab:
                     raise ValueError(f"token id {token} outside the vocabulary of {vocab}")
+            for place in entry.want:
+                if not 0 <= place < count:
+                    raise ValueError(f"wanted place {place} outside the {count} tokens of {entry.request_id}")
+
+    def pack(self, entries: Sequence[StepEntry]) -> StepBatch:
+        ids: list[int] = []
+        positions: list[int] = []
+        seq_of_token: list[int] = []
+        slots: list[int] = []
+        starts: list[int] = []
+        q_lens: list[int] = []
+        q_start_loc = [0]
+        logit_rows: list[int] = []
+        for index, entry in enumerate(entries):
+            count = len(entry.tokens)
             base = len(ids)
             ids.extend(entry.tokens)
             positions.extend(range(entry.start_pos, entry.start_pos + count))
@@ -157,10 +167,7 @@ class Runner:
             starts.append(entry.start_pos)
             q_lens.append(count)
             q_start_loc.append(base + count)
-            for place in entry.want:
-                if not 0 <= place < count:
-                    raise ValueError(f"wanted place {place} outside the {count} tokens of {entry.request_id}")
-                logit_rows.append(base + place)
+            logit_rows.extend(base + place for place in entry.want)
         parts = [ids, positions, seq_of_token, slots, starts, q_lens, q_start_loc, logit_rows]
         flat = [value for part in parts for value in part]
         host, dev = self._stage(len(flat))
@@ -183,8 +190,7 @@ class Runner:
         """One step.  Returns float32 logits ``[sum(len(e.want)), vocab]`` on the
         device, in the order of the entries and of their ``want``.  Raises
         ``CacheCapacityFull`` before anything changes if pages run out."""
-        if not entries:
-            raise ValueError("a step needs at least one entry")
+        self.check(entries)
         required = {e.request_id: e.start_pos + len(e.tokens) for e in entries}
         with trace_range("ragged.kv.ensure_capacity"):
             self.cache.ensure_capacity_batch(required)

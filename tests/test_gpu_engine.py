@@ -1,0 +1,199 @@
+"""GPU: the whole engine through its entry points: greedy generation against the
+plain implementation, long decoding, the first tokens of a sequence, temperature
+sampling, cache pressure with recompute preemption, prefix reuse, the command line."""
+
+from __future__ import annotations
+
+import json
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+from conftest import ROOT, TINY, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+
+def float_weights(tensors):
+    return {k: v.float() for k, v in tensors.items()}
+
+
+def make_engine(folder, dtype="float32", **options):
+    from cie_amd import Engine
+
+    defaults = dict(page_size=8, kv_tokens=1024, max_running=8, prefill_chunk=16, token_budget=48,
+                    prefix_cache_pages=0)
+    defaults.update(options)
+    return Engine(folder, dtype=dtype, **defaults)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(tiny_folders, name):
+    """Engine.generate in float32: chunked prefill mixed with decoding of other
+    requests yields exactly the plain implementation's greedy tokens."""
+    from cie_amd import GenerationConfig
+
+    folder, raw, tensors = tiny_folders[name]
+    lengths = [5, 17, 33] if name == "A" else [1, 9, 40, 64, 100]
+    prompts = [random_tokens(n, raw["vocab_size"], 200 + i) for i, n in enumerate(lengths)]
+    engine = make_engine(folder, page_size=16 if name == "A" else 8)
+    results = engine.generate(prompts, GenerationConfig(max_output_tokens=8, eos_token_id=None))
+    weights = float_weights(tensors)
+    for prompt, result in zip(prompts, results):
+        expected = plain.generate_greedy(raw, weights, prompt, 8)
+        assert result.token_ids == expected, f"prompt of {len(prompt)} tokens"
+        assert (result.input_tokens, result.output_tokens) == (len(prompt), 8)
+        assert result.finish_reason == "max_output_tokens_reached" and result.ttft_ms is not None
+    metrics = engine.snapshot_metrics()
+    assert metrics["requests"]["completed_total"] == len(prompts) and metrics["kv_cache"]["pages_used"] == 0
+    assert metrics["runner"]["max_forward_request_count"] > 1, "requests shared forwards"
+    assert metrics["tokens"]["output_total"] == 8 * len(prompts)
+
+
+def test_eos_stops_generation(tiny_folders):
+    from cie_amd import GenerationConfig
+
+    folder, raw, tensors = tiny_folders["A"]
+    prompt = random_tokens(12, raw["vocab_size"], 300)
+    expected = plain.generate_greedy(raw, float_weights(tensors), prompt, 6)
+    engine = make_engine(folder)
+    result = engine.generate([prompt], GenerationConfig(max_output_tokens=6, eos_token_id=expected[2]))[0]
+    stop = expected.index(expected[2])
+    assert result.token_ids == expected[: stop + 1] and result.finish_reason == "eos_token_reached"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(tiny_folders, dtype):
+    """A prompt of one token, then 150 decode steps: every step's logits against
+    the plain implementation run on the whole generated sequence (teacher forced
+    on the engine's own tokens); positions 0..7 are checked on their own."""
+    from cie_amd.engine.runner import StepEntry
+
+    folder, raw, tensors = tiny_folders["B"]
+    engine = make_engine(folder, dtype=dtype, kv_tokens=160, max_model_len=160)
+    runner = engine.runner
+    runner.cache.admit("long")
+    tokens = [3]
+    rows = []
+    for step in range(150):
+        logits = runner.run([StepEntry("long", [tokens[-1]], step, [0])])
+        rows.append(logits[0].float().cpu())
+        tokens.append(int(logits[0].argmax()))
+    expected = plain.forward(raw, float_weights(tensors), tokens[:-1])
+    got = torch.stack(rows)
+    tol = dict(rtol=1e-4, atol=2e-5) if dtype == "float32" else dict(rtol=2e-2, atol=2e-2)
+    torch.testing.assert_close(got[:8], expected[:8], **tol)
+    torch.testing.assert_close(got, expected, **tol)
+    if dtype == "float32":
+        assert tokens[1:] == [int(r.argmax()) for r in expected]
+    runner.cache.release("long")
+    assert runner.cache.stats().pages_used == 0
+
+
+def test_temperature_sampling_is_seeded_and_independent_of_the_batch(tiny_folders):
+    from cie_amd import GenerationConfig
+
+    folder, raw, _ = tiny_folders["B"]
+    prompts = [random_tokens(n, raw["vocab_size"], 400 + n) for n in (9, 40, 64)]
+    gen = [GenerationConfig(max_output_tokens=12, temperature=0.8, eos_token_id=None, seed=50 + i) for i in range(3)]
+    together = make_engine(folder, token_budget=48).generate(prompts, gen)
+    alone = [make_engine(folder, token_budget=7, prefill_chunk=5).generate([p], [g])[0] for p, g in zip(prompts, gen)]
+    assert [r.token_ids for r in together] == [r.token_ids for r in alone]
+    other_seed = make_engine(folder).generate(prompts[:1], GenerationConfig(max_output_tokens=12, temperature=0.8, seed=7))
+    assert other_seed[0].token_ids != together[0].token_ids
+    greedy = make_engine(folder).generate(prompts[:1], GenerationConfig(max_output_tokens=12, eos_token_id=None))
+    assert greedy[0].token_ids != together[0].token_ids  # the draws are not all argmax
+
+
+def test_pressure_preempts_and_recomputes_to_the_same_tokens(tiny_folders):
+    """A pool too small for two requests at once (reference
+    tests/remote_ragged_gpu_tests.py:294-332): preemptions > 0, recomputed tokens
+    > 0, outputs identical to the unpressured run, allocator drained."""
+    from cie_amd import GenerationConfig
+
+    folder, raw, _ = tiny_folders["A"]
+    prompts = [random_tokens(56, raw["vocab_size"], 500 + i) for i in range(2)]
+    gen = GenerationConfig(max_output_tokens=12, eos_token_id=None)
+    roomy = make_engine(folder, page_size=16, kv_tokens=512).generate(prompts, gen)
+    tight = make_engine(folder, page_size=16, kv_tokens=128)  # 8 pages; each request ends at 68 tokens = 5 pages
+    results = tight.generate(prompts, gen)
+    assert [r.token_ids for r in results] == [r.token_ids for r in roomy]
+    metrics = tight.snapshot_metrics()
+    assert metrics["requests"]["preempted_total"] > 0 and metrics["tokens"]["recomputed_total"] > 0
+    assert metrics["kv_cache"]["pages_used"] == 0
+    tight.runner.cache.assert_invariants()
+
+
+def test_prefix_reuse_keeps_tokens_and_saves_work(tiny_folders):
+    """reference tests/remote_ragged_gpu_tests.py:335-377: the same prompt twice
+    gives identical tokens, the warm run feeds at least a page less, hits >= 1,
+    request pages 0 and prefix pages > 0 afterwards.  Beyond it: a prompt that
+    shares only the first pages and then differs also hits."""
+    from cie_amd import GenerationConfig
+
+    folder, raw, tensors = tiny_folders["A"]
+    prompt = random_tokens(45, raw["vocab_size"], 600)
+    sibling = prompt[:32] + random_tokens(9, raw["vocab_size"], 601)
+    gen = GenerationConfig(max_output_tokens=6, eos_token_id=None)
+    engine = make_engine(folder, page_size=16, prefix_cache_pages=8)
+    cold = engine.generate([prompt], gen)[0]
+    cold_work = engine.snapshot_metrics()["tokens"]["input_total"]
+    warm = engine.generate([prompt], gen)[0]
+    warm_work = engine.snapshot_metrics()["tokens"]["input_total"] - cold_work
+    assert warm.token_ids == cold.token_ids
+    assert warm_work + 16 <= cold_work
+    third = engine.generate([sibling], gen)[0]
+    assert third.token_ids == plain.generate_greedy(raw, float_weights(tensors), sibling, 6)
+    cache = engine.snapshot_metrics()["kv_cache"]
+    assert cache["prefix_cache_hits"] >= 2 and cache["request_pages_used"] == 0 and cache["prefix_pages_used"] > 0
+    engine.runner.cache.assert_invariants()
+
+
+def test_step_refuses_what_it_cannot_run(tiny_folders):
+    from cie_amd.cache import CacheCapacityFull
+    from cie_amd.engine.runner import StepEntry
+
+    folder, raw, _ = tiny_folders["A"]
+    runner = make_engine(folder, page_size=16, kv_tokens=32, max_model_len=32).runner
+    runner.cache.admit("a"), runner.cache.admit("b")
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        runner.run([StepEntry("a", [raw["vocab_size"]], 0, [0])])
+    with pytest.raises(ValueError, match="continues at 3"):
+        runner.run([StepEntry("a", [1], 3, [0])])
+    with pytest.raises(ValueError, match="twice"):
+        runner.run([StepEntry("a", [1], 0, []), StepEntry("a", [2], 1, [])])
+    with pytest.raises(ValueError, match="wanted place"):
+        runner.run([StepEntry("a", [1, 2], 0, [2])])
+    runner.run([StepEntry("a", list(range(20)), 0, [])])
+    with pytest.raises(CacheCapacityFull):
+        runner.run([StepEntry("b", list(range(20)), 0, [])])  # 2 pages needed, none free
+    assert runner.cache.length("a") == 20 and runner.cache.length("b") == 0
+    assert runner.cache.block_table(0, "b") == []  # nothing changed
+
+
+def test_command_line_generates(tiny_folders, tmp_path):
+    folder, raw, tensors = tiny_folders["A"]
+    prompt = [7, 8, 9, 10, 11]
+    expected = plain.generate_greedy(raw, float_weights(tensors), prompt, 5)
+    done = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "cie"), "generate", "--token-ids", " ".join(map(str, prompt)),
+         "--model", str(folder), "--max-output-tokens", "5", "--dtype", "fp32", "--no-stream", "--ignore-eos",
+         "--max-model-len", "64", "--kv-tokens", "256"],
+        capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert done.stdout.split() == [str(t) for t in expected]
+    config_path = tmp_path / "config.json"
+    config_path.write_text(json.dumps(TINY["B"]))
+    out_dir = tmp_path / "model"
+    done = subprocess.run([sys.executable, str(ROOT / "bin" / "cie"), "init-model", "--config", str(config_path),
+                           "--out", str(out_dir), "--seed", "4"], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0 and (out_dir / "model.safetensors").is_file() and (out_dir / "config.json").is_file()
+    done = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "cie"), "generate", "--token-ids", "1,2,3", "--model", str(out_dir),
+         "--max-output-tokens", "4", "--temperature", "0.8", "--seed", "3", "--metrics", "--max-model-len", "64"],
+        capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert '"completed_total": 1' in done.stdout

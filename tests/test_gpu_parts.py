@@ -1,0 +1,308 @@
+"""GPU: each part of a layer alone against the plain implementation, and a toy
+mixer with state of its own that is registered, built and stepped from the test
+without any change to the package."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+import plain_qwen2 as plain
+import replay_util
+from conftest import random_tokens
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+
+
+def check(got, expect, dtype):
+    """float32: rounding of float32 sums.  bfloat16: every intermediate is rounded
+    to 8 mantissa bits (relative 2^-9), so the error of an element scales with the
+    magnitude of the tensor it was summed from, not with the element itself: the
+    absolute allowance is tied to the tensor's largest value."""
+    if dtype == "float32":
+        torch.testing.assert_close(got, expect, rtol=1e-4, atol=2e-5)
+    else:
+        scale = float(expect.abs().max())
+        torch.testing.assert_close(got, expect, rtol=2e-2, atol=1e-2 * max(scale, 1.0))
+
+
+
+def harness(needs, lengths, page_size=8, dtype=torch.float32):
+    """A cache with one unit per need and live requests of the given lengths (nothing committed yet)."""
+    from cie_amd.cache import CacheManager
+    from cie_amd.engine.device_cache import DeviceCache
+
+    manager = CacheManager(needs, page_size, kv_tokens=512, max_running=4, max_model_len=256)
+    device_cache = DeviceCache(manager, dtype, torch.device("cuda:0"))
+    for i, n in enumerate(lengths):
+        manager.admit(f"r{i}")
+    manager.ensure_capacity_batch({f"r{i}": n for i, n in enumerate(lengths)})
+    device_cache.sync()
+    return manager, device_cache
+
+
+def batch_of(manager, portions):
+    """StepBatch for portions [(request index, start, count)], built by hand."""
+    from cie_amd.engine.batch import StepBatch
+
+    positions, seq_of_token, slots, starts, q_lens, loc = [], [], [], [], [], [0]
+    for s, (index, start, count) in enumerate(portions):
+        positions += list(range(start, start + count))
+        seq_of_token += [s] * count
+        slots.append(manager.slot(f"r{index}"))
+        starts.append(start)
+        q_lens.append(count)
+        loc.append(loc[-1] + count)
+    as_dev = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")  # noqa: E731
+    total = len(positions)
+    return StepBatch(tokens=total, sequences=len(portions), token_ids=as_dev([0] * total), positions=as_dev(positions),
+                     seq_of_token=as_dev(seq_of_token), seq_slot=as_dev(slots), seq_start=as_dev(starts),
+                     seq_q_len=as_dev(q_lens), q_start_loc=as_dev(loc), logit_rows=as_dev(list(range(total))),
+                     host_slots=slots, host_starts=starts, host_q_lens=q_lens)
+
+
+def bound(part, prefix, dtype, seed, scale=0.2):
+    from cie_amd.weights import RandomSource
+
+    expected = part.expected_tensors(prefix)
+    tensors = RandomSource(seed, std=scale).load(expected, dtype, "cuda:0")
+    part.bind(tensors, prefix, torch.float32 if dtype == "float32" else torch.bfloat16, torch.device("cuda:0"))
+    return {k: v.float().cpu() for k, v in tensors.items()}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_part(dtype):
+    from cie_amd.parts.norm import RMSNorm
+
+    norm = RMSNorm(size=200, eps=3e-5)
+    weights = bound(norm, "n.", dtype, 1)
+    act = norm.dtype
+    residual = torch.randn((6, 200), device="cuda") * 2
+    branch = torch.randn((6, 200), device="cuda").to(act)
+    expect_sum = residual.cpu() + branch.float().cpu()
+    out = norm.forward(residual, branch, act)
+    torch.testing.assert_close(residual.cpu(), expect_sum, rtol=0, atol=0)
+    check(out.float().cpu(), plain.rms_norm(expect_sum, weights["n.weight"], 3e-5), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_feed_forward_part(dtype):
+    from cie_amd.parts.feed_forward import GatedMLP
+
+    mlp = GatedMLP(hidden_size=72, intermediate_size=200)
+    w = bound(mlp, "m.", dtype, 2)
+    x = torch.randn((9, 72), device="cuda").to(mlp.dtype)
+    expect = plain.swiglu(x.float().cpu(), w["m.gate_proj.weight"], w["m.up_proj.weight"], w["m.down_proj.weight"])
+    check(mlp.forward(x).float().cpu(), expect, dtype)
+    with pytest.raises(ValueError, match="silu"):
+        GatedMLP(8, 8, activation="gelu")
+
+
+def test_position_part_tables_and_no_position():
+    from cie_amd.parts.position import NoPosition, RotaryHalf
+
+    rotary = RotaryHalf(head_dim=48, theta=5e5, max_position=77)
+    cos, sin = rotary.tables(torch.device("cuda:0"))
+    ref_cos, ref_sin = plain.rope_tables(48, 77, 5e5)
+    assert cos.shape == (77, 24) and cos.dtype == torch.float32
+    torch.testing.assert_close(cos.cpu(), ref_cos[:, :24], rtol=0, atol=0)
+    torch.testing.assert_close(sin.cpu(), ref_sin[:, :24], rtol=0, atol=0)
+    assert not NoPosition().rotates
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rotary", [True, False])
+def test_attention_part_whole_and_in_portions(dtype, rotary):
+    """The mixer alone: one request whole, another cut into a portion and single
+    tokens, in one batch with it.  Without rotation it reduces to plain masked
+    attention (library routine, see tests/test_plain.py)."""
+    from cie_amd.config import PartSpec
+    from cie_amd.parts.attention import Attention
+
+    hidden, heads, kv_heads, head_dim = 40, 6, 2, 16
+    position = (PartSpec.of("rotary_half", head_dim=head_dim, theta=1e4, max_position=256) if rotary
+                else PartSpec.of("none", head_dim=head_dim, max_position=256))
+    attention = Attention(hidden, heads, kv_heads, head_dim, qkv_bias=True, out_bias=False, position=position)
+    # float32 takes very peaked softmaxes (scores of order 10); in bfloat16 the rounding of q and k alone
+    # moves such scores by tenths, so that case runs at a scale where the softmax is still well conditioned
+    w = bound(attention, "a.", dtype, 3, scale=0.5 if dtype == "float32" else 0.3)
+    lengths = [29, 21]
+    manager, device_cache = harness([attention.cache_need()], lengths,
+                                    dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    g = torch.Generator().manual_seed(4)
+    xs = [torch.randn((n, hidden), generator=g).to(attention.dtype) for n in lengths]
+    config = {"hidden_size": hidden, "num_attention_heads": heads, "head_dim": head_dim, "attention_bias": True}
+    expected = []
+    for x, n in zip(xs, lengths):
+        if rotary:
+            cos, sin = plain.rope_tables(head_dim, n, 1e4)
+        else:
+            cos, sin = torch.ones((n, head_dim)), torch.zeros((n, head_dim))
+        expected.append(plain.attention_layer(x.float(), w, "a.", config, cos, sin, torch.arange(n)))
+    view = device_cache.view(0)
+    # step 1: request 0 whole, first 10 tokens of request 1
+    got0 = {}
+    out = attention.forward(torch.cat([xs[0], xs[1][:10]]).cuda(), batch_of(manager, [(0, 0, 29), (1, 0, 10)]), view)
+    got0[0], first = out[:29], out[29:]
+    manager.commit_lengths({"r0": 29, "r1": 10})
+    # step 2: a 9-token portion of request 1; steps 3, 4: single tokens
+    second = attention.forward(xs[1][10:19].cuda(), batch_of(manager, [(1, 10, 9)]), view)
+    third = attention.forward(xs[1][19:20].cuda(), batch_of(manager, [(1, 19, 1)]), view)
+    fourth = attention.forward(xs[1][20:21].cuda(), batch_of(manager, [(1, 20, 1)]), view)
+    check(got0[0].float().cpu(), expected[0], dtype)
+    check(torch.cat([first, second, third, fourth]).float().cpu(), expected[1], dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_block_part(dtype):
+    """norm -> mixer -> add -> norm -> feed-forward, the add of the second branch left pending."""
+    from cie_amd.config import Qwen2Config
+    from cie_amd.parts.block import PreNormBlock
+
+    raw = dict(model_type="qwen2", hidden_size=48, num_hidden_layers=1, num_attention_heads=3,
+               num_key_value_heads=3, intermediate_size=88, vocab_size=32, rms_norm_eps=1e-5, rope_theta=1e4,
+               max_position_embeddings=64)
+    spec = Qwen2Config.from_hf_config(raw).model_spec().layers[0]
+    block = PreNormBlock(spec)
+    w = bound(block, "model.layers.0.", dtype, 5, scale=0.3)
+    manager, device_cache = harness([block.cache_need()], [13], dtype=block.dtype)
+    h = torch.randn((13, 48), generator=torch.Generator().manual_seed(6))
+    residual = h.clone().cuda()
+    out_residual, pending = block.forward(residual, None, batch_of(manager, [(0, 0, 13)]), device_cache.view(0))
+    p = "model.layers.0."
+    cos, sin = plain.rope_tables(16, 13, 1e4)
+    a = plain.rms_norm(h, w[p + "input_layernorm.weight"], 1e-5)
+    mid = h + plain.attention_layer(a, w, p + "self_attn.", raw, cos, sin, torch.arange(13))
+    m = plain.rms_norm(mid, w[p + "post_attention_layernorm.weight"], 1e-5)
+    branch = plain.swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    check(out_residual.cpu(), mid, dtype)
+    check(pending.float().cpu(), branch, dtype)
+
+
+# -- a toy mixer with state of its own -----------------------------------------------------
+def register_toy():
+    """A decaying running sum per request: s_t = decay * s_{t-1} + W x_t, y_t = s_t.
+    Its state lives in the cache's fixed-size slots; it is defined, registered
+    and wired into an architecture here, outside the package."""
+    from cie_amd.cache import FixedState
+    from cie_amd.config import LayerCall, LayerSpec, ModelSpec, PartSpec, Qwen2Config, register_architecture
+    from cie_amd.parts import Part, register_part
+    from cie_amd.weights import TensorSpec
+
+    class RunningSum(Part):
+        def __init__(self, hidden_size: int, decay: float) -> None:
+            self.hidden_size, self.decay = hidden_size, decay
+
+        def cache_need(self):
+            return FixedState((self.hidden_size,), "float32")
+
+        def expected_tensors(self, prefix):
+            return {prefix + "in_proj.weight": TensorSpec((self.hidden_size, self.hidden_size))}
+
+        def bind(self, tensors, prefix, dtype, device):
+            super().bind(tensors, prefix, dtype, device)
+            self.weight = tensors[prefix + "in_proj.weight"].float()
+
+        def forward(self, x, batch, view, writes=True):
+            projected = x.float() @ self.weight.t()
+            out = torch.empty_like(projected)
+            row = 0
+            for slot, count in zip(batch.host_slots, batch.host_q_lens):
+                state = view.state[slot].clone()
+                for _ in range(count):
+                    state = self.decay * state + projected[row]
+                    out[row] = state
+                    row += 1
+                if writes:
+                    view.state[slot] = state
+            return out.to(x.dtype)
+
+    class ToyConfig(Qwen2Config):
+        architecture = "ToyRunningSumForCausalLM"
+
+        def model_spec(self) -> ModelSpec:
+            base = super().model_spec()
+            attention_layer = base.layers[0]
+            toy_layer = LayerSpec(
+                mixer=PartSpec.of("running_sum", hidden_size=self.hidden_size, decay=0.75),
+                feed_forward=attention_layer.feed_forward, norm1=attention_layer.norm1, norm2=attention_layer.norm2,
+                names=(("norm1", "input_layernorm"), ("mixer", "toy"), ("norm2", "post_attention_layernorm"),
+                       ("feed_forward", "mlp")))
+            # layers: 0 toy, 1 attention; order: toy, attention, toy again (its own state unit)
+            return ModelSpec(
+                architecture=self.architecture, vocab_size=self.vocab_size, hidden_size=self.hidden_size,
+                layers=(toy_layer, attention_layer),
+                order=(LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2)),
+                final_norm=base.final_norm, tie_word_embeddings=True, max_position=self.max_position_embeddings)
+
+    register_part("mixer", "running_sum", RunningSum)
+    register_architecture("ToyRunningSumForCausalLM", ToyConfig)
+    return ToyConfig
+
+
+def toy_plain(raw, weights, tokens):
+    """Whole-sequence reference of the toy model, from the plain parts."""
+    eps = raw["rms_norm_eps"]
+    h = weights["model.embed_tokens.weight"][torch.tensor(tokens)]
+    cos, sin = plain.rope_tables(plain.head_dim_of(raw), len(tokens), raw["rope_theta"])
+
+    def toy(x, p):
+        projected = x @ weights[p + "toy.in_proj.weight"].t()
+        state = torch.zeros(raw["hidden_size"])
+        rows = []
+        for row in projected:
+            state = 0.75 * state + row
+            rows.append(state)
+        return torch.stack(rows)
+
+    def mlp(x, p):
+        return plain.swiglu(x, weights[p + "mlp.gate_proj.weight"], weights[p + "mlp.up_proj.weight"],
+                            weights[p + "mlp.down_proj.weight"])
+
+    for layer in (0, 1, 0):
+        p = f"model.layers.{layer}."
+        a = plain.rms_norm(h, weights[p + "input_layernorm.weight"], eps)
+        if layer == 0:
+            h = h + toy(a, p)
+        else:
+            h = h + plain.attention_layer(a, weights, p + "self_attn.", raw, cos, sin, torch.arange(len(tokens)))
+        h = h + mlp(plain.rms_norm(h, weights[p + "post_attention_layernorm.weight"], eps), p)
+    h = plain.rms_norm(h, weights["model.norm.weight"], eps)
+    return h @ weights["model.embed_tokens.weight"].t()
+
+
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
+    from cie_amd.config import build_engine_config, load_config
+    from cie_amd.engine import Runner, load_model
+    from cie_amd.parts.model import expected_tensors
+    from cie_amd.weights import RandomSource, write_tensors
+
+    register_toy()
+    raw = dict(architectures=["ToyRunningSumForCausalLM"], model_type="qwen2", hidden_size=32, num_hidden_layers=2,
+               num_attention_heads=2, num_key_value_heads=1, intermediate_size=56, vocab_size=64,
+               rms_norm_eps=1e-6, rope_theta=1e4, max_position_embeddings=128, tie_word_embeddings=True)
+    write_tensors(tmp_path, raw, {})  # config.json first, so that the registry picks the toy configuration
+    config = load_config(tmp_path)
+    spec = config.model_spec()
+    expected = expected_tensors(spec)
+    assert "model.layers.0.toy.in_proj.weight" in expected and "model.layers.1.self_attn.q_proj.weight" in expected
+    tensors = RandomSource(8, std=0.1).load(expected, "float32", "cpu")
+    write_tensors(tmp_path, raw, tensors)
+    model, _ = load_model(tmp_path, "float32")
+    engine_config = build_engine_config(dtype="float32", page_size=8, kv_tokens=128, max_running=4,
+                                        max_model_len=128, prefix_cache_pages=8)
+    runner = Runner(model, engine_config)
+    assert set(runner.cache.state_units) == {0, 2} and runner.cache.unit_group == {1: 0}
+    assert runner.cache.prefix_cache_pages == 0  # state cannot be taken over page by page
+    requests = {f"t{i}": random_tokens(n, 64, 70 + i) for i, n in enumerate([23, 40, 9, 31, 17])}
+    reference = {rid: toy_plain(raw, tensors, tokens) for rid, tokens in requests.items()}
+    for schedule in (replay_util.whole, replay_util.portions, lambda r: replay_util.mixed(r, live=3)):
+        steps = schedule(requests)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        replay_util.compare(rows, reference, rtol=1e-4, atol=2e-5)
+    # a slot handed to a new request starts from a cleared state (slots were reused above)
+    assert runner.cache.stats().slots_used == 0
