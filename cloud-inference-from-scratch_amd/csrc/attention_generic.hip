@@ -12,7 +12,8 @@
 //   s = (q . k) * scale;  p = exp(s - max);  out = sum(p * v) / sum(p)
 //
 //   q    [tokens, q_heads, D] with row stride q_row_stride (elements)
-//   pool [pages, kv_heads, page_size, D]
+//   keys   [pages, kv_heads, page_size, D]
+//   values [pages, kv_heads, D, page_size]  (transposed)
 //   out  [tokens, q_heads * D]
 #include "common.h"
 
@@ -74,11 +75,13 @@ paged_attention_generic_kernel(const T* __restrict__ q, int q_row_stride,
         const int key = base + lane;
         const bool valid = key < len;
         float s = -INFINITY;
-        uint32_t row = 0;
+        uint32_t head_block = 0;  // index of the (page, kv head) block of page_size * head_dim elements
+        uint32_t in_page = 0;
         if (valid) {
             const int page = table[key / page_size];
-            row = (static_cast<uint32_t>(page) * kv_heads + kv_head) * page_size + key % page_size;
-            const T* k_row = k_pool + static_cast<size_t>(row) * head_dim;
+            head_block = static_cast<uint32_t>(page) * kv_heads + kv_head;
+            in_page = key % page_size;
+            const T* k_row = k_pool + (static_cast<size_t>(head_block) * page_size + in_page) * head_dim;
             float dot = 0.f;
             for (int d = 0; d < head_dim; d += 8) {
                 float kk[8];
@@ -97,12 +100,13 @@ paged_attention_generic_kernel(const T* __restrict__ q, int q_row_stride,
         const int count = min(kWave, len - base);
         for (int j = 0; j < count; ++j) {
             const float pj = __shfl(p, j, kWave);
-            const uint32_t rj = __shfl(row, j, kWave);
-            const T* v_row = v_pool + static_cast<size_t>(rj) * head_dim;
+            const uint32_t block_j = __shfl(head_block, j, kWave);
+            const uint32_t in_page_j = __shfl(in_page, j, kWave);
+            const T* v_column = v_pool + static_cast<size_t>(block_j) * page_size * head_dim + in_page_j;
 #pragma unroll
             for (int i = 0; i < kMaxSlices; ++i) {
                 const int d = lane + kWave * i;
-                if (d < head_dim) acc[i] = fmaf(pj, to_float(v_row[d]), acc[i]);
+                if (d < head_dim) acc[i] = fmaf(pj, to_float(v_column[static_cast<size_t>(d) * page_size]), acc[i]);
             }
         }
         m = m_new;

@@ -1,0 +1,359 @@
+// Paged grouped-query attention on the matrix cores (bfloat16), for decode
+// tokens (with the context split over many waves) and for prompt portions.
+//
+// Cache layout: keys   [pages, kv_heads, page_size, D]   (a key row is contiguous)
+//               values [pages, kv_heads, D, page_size]   (transposed: a head
+//               dimension's page_size values are contiguous), so that both the
+//               K operand of Q.K^T and the V operand of P.V are plain vector loads.
+//
+// Work unit = one wave = (tile, kv head, split):
+//   tile   up to `tokens_per_tile` consecutive query tokens of one sequence; the
+//          rows of the tile are (token, head of the group): row = token * G + head,
+//          at most 16 * RT rows.  All rows share the KV head's keys and values.
+//   split  a contiguous part of the tile's key range; partial results of the
+//          splits are merged by `attention_merge_kernel`.
+//
+// Per block of 32 keys:
+//   S^T[key, row] = K[key, :] . Q[row, :]      v_mfma_f32_16x16x32_bf16, A = K, B = Q
+//   lane (r = lane % 16, g = lane / 16) then holds, for row r, the scores of keys
+//   g*4 .. g*4+3 of each 16-key tile: exactly the A-operand layout of P for
+//   O[row, d] += P[row, key] * V[key, d]       A = P (bf16), B = V^T rows
+//   The spread of a block's keys (and of a head's dimensions) over the lanes is
+//   the same for both operands of a product, which is all a dot product needs.
+// Scores, running maximum, sums and the output accumulator are float32.
+#include "common.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kKeysPerBlock = 32;
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return static_cast<uint32_t>(bf16_bits_from_float(lo)) | (static_cast<uint32_t>(bf16_bits_from_float(hi)) << 16);
+}
+
+struct AttentionArgs {
+    const bf16_t* q;
+    int q_row_stride;
+    const bf16_t* k_pool;
+    const bf16_t* v_pool;
+    const int* block_table;
+    int table_width;
+    const int* tile_seq;
+    const int* tile_q0;
+    const int* seq_slot;
+    const int* seq_start;
+    const int* seq_q_len;
+    const int* q_start_loc;
+    bf16_t* out;
+    float* part_o;   // [tiles, kv_heads, splits, rows, D]
+    float* part_ml;  // [tiles, kv_heads, splits, rows, 2]
+    int q_heads;
+    int kv_heads;
+    int page_shift;
+    int window;
+    float scale;
+    int n_splits;
+    int tokens_per_tile;
+    int keys_per_split;  // multiple of kKeysPerBlock; 0 with one split
+    const int* keys_per_split_dev;  // if set, read from the device instead (a captured graph's value changes per step)
+};
+
+template <int D, int RT>
+__global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs a) {
+    constexpr int NK = D / 32;   // matrix products per 16-key tile of Q.K^T
+    constexpr int ND = D / 16;   // 16-wide output tiles of the head dimension
+    constexpr int ROWS = 16 * RT;
+    const int lane = threadIdx.x;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int tile = blockIdx.x;
+    const int kv_head = blockIdx.y;
+    const int split = blockIdx.z;
+    const int group = a.q_heads / a.kv_heads;
+    const int seq = a.tile_seq[tile];
+    const int q0 = a.tile_q0[tile];
+    const int start = a.seq_start[seq];
+    const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
+    const int n_rows = n_tok * group;
+    const int first_row_token = a.q_start_loc[seq] + q0;
+    const int page_size = 1 << a.page_shift;
+    const int page_mask = page_size - 1;
+    const int* table = a.block_table + static_cast<size_t>(a.seq_slot[seq]) * a.table_width;
+
+    // keys this tile can see at all, and this split's share of them
+    const int hi = start + q0 + n_tok;
+    const int lo = (a.window > 0) ? max(0, start + q0 + 1 - a.window) : 0;
+    int range_begin = lo & ~(kKeysPerBlock - 1);
+    int range_end = hi;
+    if (a.n_splits > 1) {
+        const int per_split = a.keys_per_split_dev ? *a.keys_per_split_dev : a.keys_per_split;
+        range_begin += split * per_split;
+        range_end = min(hi, range_begin + per_split);
+    }
+
+    // Q fragments (B operand) and each lane's row facts
+    uint4 qf[RT][NK];
+    int row_pos[RT];   // position of the lane's row r of tile rt; -1 for a row that does not exist
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = rt * 16 + r;
+        const bool valid = row < n_rows;
+        const int tok = row / group;
+        const int head = row - tok * group;
+        row_pos[rt] = valid ? start + q0 + tok : -1;
+        const bf16_t* q_row = a.q + static_cast<size_t>(first_row_token + tok) * a.q_row_stride +
+                              static_cast<size_t>(kv_head * group + head) * D + g * (D / 4);
+#pragma unroll
+        for (int j = 0; j < NK; ++j)
+            qf[rt][j] = valid ? *reinterpret_cast<const uint4*>(q_row + j * 8) : uint4{0, 0, 0, 0};
+    }
+
+    float m_run[RT], l_run[RT];
+    floatx4 o[RT][ND];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        m_run[rt] = -INFINITY;
+        l_run[rt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) o[rt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    for (int kb = range_begin; kb < range_end; kb += kKeysPerBlock) {
+        // ---- S^T = K . Q^T for two 16-key tiles
+        floatx4 s[RT][2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            const int key = min(kb + kt * 16 + r, hi - 1);  // rows past the end are masked below
+            const int page = table[key >> a.page_shift];
+            const bf16_t* k_row = a.k_pool +
+                (((static_cast<size_t>(page) * a.kv_heads + kv_head) << a.page_shift) + (key & page_mask)) * D +
+                g * (D / 4);
+            uint4 kf[NK];
+#pragma unroll
+            for (int j = 0; j < NK; ++j) kf[j] = *reinterpret_cast<const uint4*>(k_row + j * 8);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < NK; ++j)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[j]),
+                                                                  __builtin_bit_cast(bf16x8, qf[rt][j]), acc, 0, 0, 0);
+                s[rt][kt] = acc;
+            }
+        }
+        // ---- V^T fragments of the block (B operand): for each 16-wide d tile, 4 keys of each 16-key tile
+        uint2 vf[ND][2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            const int key = min(kb + kt * 16 + g * 4, (hi - 1) & ~3);
+            const int page = table[key >> a.page_shift];
+            const bf16_t* v_base = a.v_pool +
+                ((static_cast<size_t>(page) * a.kv_heads + kv_head) * D << a.page_shift) + (key & page_mask);
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+                vf[dt][kt] = *reinterpret_cast<const uint2*>(v_base + (static_cast<size_t>(dt * 16 + r) << a.page_shift));
+        }
+        // ---- mask, running softmax, P as A operand, O += P . V
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const int pos = row_pos[rt];
+            const int row_lo = (a.window > 0) ? pos + 1 - a.window : 0;
+            float block_max = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = kb + kt * 16 + g * 4 + i;
+                    const bool seen = key <= pos && key >= row_lo && key < range_end;
+                    const float v = seen ? s[rt][kt][i] * a.scale : -INFINITY;
+                    s[rt][kt][i] = v;
+                    block_max = fmaxf(block_max, v);
+                }
+            }
+            block_max = fmaxf(block_max, __shfl_xor(block_max, 16, kWave));
+            block_max = fmaxf(block_max, __shfl_xor(block_max, 32, kWave));
+            const float m_new = fmaxf(m_run[rt], block_max);
+            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = __expf(m_run[rt] - m_safe);  // m_run = -inf: 0, and l, O are 0 anyway
+            m_run[rt] = m_new;
+            float p_sum = 0.f;
+            uint32_t pw[4];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                const float p0 = __expf(s[rt][kt][0] - m_safe);
+                const float p1 = __expf(s[rt][kt][1] - m_safe);
+                const float p2 = __expf(s[rt][kt][2] - m_safe);
+                const float p3 = __expf(s[rt][kt][3] - m_safe);
+                p_sum += (p0 + p1) + (p2 + p3);
+                pw[kt * 2] = pack_bf16(p0, p1);
+                pw[kt * 2 + 1] = pack_bf16(p2, p3);
+            }
+            l_run[rt] = l_run[rt] * alpha + p_sum;
+            // the accumulator's rows are g*4+i, the statistics' row is r: fetch alpha of those rows
+            float alpha_o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha, g * 4 + i, kWave);
+            const bf16x8 p_frag = __builtin_bit_cast(bf16x8, (uint4{pw[0], pw[1], pw[2], pw[3]}));
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                floatx4 acc = o[rt][dt];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] *= alpha_o[i];
+                const uint4 v = uint4{vf[dt][0].x, vf[dt][0].y, vf[dt][1].x, vf[dt][1].y};
+                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_frag, __builtin_bit_cast(bf16x8, v), acc, 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- finish: sums over the four lane groups, then normalise or hand the partial to the merge
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        float l = l_run[rt];
+        l += __shfl_xor(l, 16, kWave);
+        l += __shfl_xor(l, 32, kWave);
+        if (a.n_splits == 1) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = rt * 16 + g * 4 + i;
+                const float l_row = __shfl(l, g * 4 + i, kWave);
+                if (row < n_rows) {
+                    const int tok = row / group;
+                    const int head = row - tok * group;
+                    bf16_t* dst = a.out + static_cast<size_t>(first_row_token + tok) * a.q_heads * D +
+                                  static_cast<size_t>(kv_head * group + head) * D;
+                    const float inv = 1.0f / l_row;
+#pragma unroll
+                    for (int dt = 0; dt < ND; ++dt) dst[dt * 16 + r] = from_float<bf16_t>(o[rt][dt][i] * inv);
+                }
+            }
+        } else {
+            const size_t unit = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + split;
+            float* po = a.part_o + unit * ROWS * D;
+            float* pml = a.part_ml + unit * ROWS * 2;
+            if (g == 0) {
+                pml[(rt * 16 + r) * 2] = m_run[rt];
+                pml[(rt * 16 + r) * 2 + 1] = l;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = rt * 16 + g * 4 + i;
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt) po[static_cast<size_t>(row) * D + dt * 16 + r] = o[rt][dt][i];
+            }
+        }
+    }
+}
+
+// Merge the splits of every (tile, kv head): out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M).
+__global__ void __launch_bounds__(256)
+attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
+    const int tile = blockIdx.x;
+    const int kv_head = blockIdx.y;
+    const int group = a.q_heads / a.kv_heads;
+    const int seq = a.tile_seq[tile];
+    const int q0 = a.tile_q0[tile];
+    const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
+    const int n_rows = n_tok * group;
+    const int first_row_token = a.q_start_loc[seq] + q0;
+    const size_t unit0 = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits;
+    for (int idx = threadIdx.x; idx < n_rows * head_dim; idx += blockDim.x) {
+        const int row = idx / head_dim;
+        const int d = idx - row * head_dim;
+        float m_all = -INFINITY;
+        for (int s = 0; s < a.n_splits; ++s)
+            m_all = fmaxf(m_all, a.part_ml[((unit0 + s) * rows_per_tile + row) * 2]);
+        float num = 0.f, den = 0.f;
+        for (int s = 0; s < a.n_splits; ++s) {
+            const float* ml = a.part_ml + ((unit0 + s) * rows_per_tile + row) * 2;
+            const float w = (ml[0] == -INFINITY) ? 0.f : __expf(ml[0] - m_all);
+            num += a.part_o[((unit0 + s) * rows_per_tile + row) * head_dim + d] * w;
+            den += ml[1] * w;
+        }
+        const int tok = row / group;
+        const int head = row - tok * group;
+        a.out[static_cast<size_t>(first_row_token + tok) * a.q_heads * head_dim +
+              static_cast<size_t>(kv_head * group + head) * head_dim + d] = from_float<bf16_t>(num / den);
+    }
+}
+
+template <int D>
+int launch_for_dim(hipStream_t s, const AttentionArgs& a, int n_tiles, int row_tiles) {
+    dim3 grid(n_tiles, a.kv_heads, a.n_splits);
+    if (row_tiles == 1)
+        paged_attention_mfma_kernel<D, 1><<<grid, 64, 0, s>>>(a);
+    else if (row_tiles == 2)
+        paged_attention_mfma_kernel<D, 2><<<grid, 64, 0, s>>>(a);
+    else if (row_tiles == 4)
+        paged_attention_mfma_kernel<D, 4><<<grid, 64, 0, s>>>(a);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+}  // namespace
+
+// Workspace sizes (floats) the caller provides when n_splits > 1:
+//   part_o  n_tiles * kv_heads * n_splits * 16*row_tiles * head_dim
+//   part_ml n_tiles * kv_heads * n_splits * 16*row_tiles * 2
+CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stride, const void* k_pool,
+                                     const void* v_pool, const int* block_table, int table_width,
+                                     const int* tile_seq, const int* tile_q0, const int* seq_slot,
+                                     const int* seq_start, const int* seq_q_len, const int* q_start_loc,
+                                     void* out, float* part_o, float* part_ml, int n_tiles, int q_heads,
+                                     int kv_heads, int head_dim, int page_size, int window, float scale,
+                                     int n_splits, int tokens_per_tile, int row_tiles, int keys_per_split,
+                                     const int* keys_per_split_dev) {
+    if (n_tiles < 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || page_size < 4 ||
+        (page_size & (page_size - 1)) || table_width <= 0 || n_splits < 1 || n_splits > 65535 ||
+        kv_heads > 65535 || tokens_per_tile < 1 || q_row_stride % 8)
+        return CIE_BAD_ARGUMENT;
+    const int group = q_heads / kv_heads;
+    if (tokens_per_tile * group > 16 * row_tiles) return CIE_BAD_ARGUMENT;
+    if (n_splits > 1 && (!part_o || !part_ml ||
+                         (!keys_per_split_dev && (keys_per_split <= 0 || keys_per_split % kKeysPerBlock))))
+        return CIE_BAD_ARGUMENT;
+    if (n_tiles == 0) return CIE_OK;
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    AttentionArgs a;
+    a.q = static_cast<const bf16_t*>(q);
+    a.q_row_stride = q_row_stride;
+    a.k_pool = static_cast<const bf16_t*>(k_pool);
+    a.v_pool = static_cast<const bf16_t*>(v_pool);
+    a.block_table = block_table;
+    a.table_width = table_width;
+    a.tile_seq = tile_seq;
+    a.tile_q0 = tile_q0;
+    a.seq_slot = seq_slot;
+    a.seq_start = seq_start;
+    a.seq_q_len = seq_q_len;
+    a.q_start_loc = q_start_loc;
+    a.out = static_cast<bf16_t*>(out);
+    a.part_o = part_o;
+    a.part_ml = part_ml;
+    a.q_heads = q_heads;
+    a.kv_heads = kv_heads;
+    a.page_shift = page_shift;
+    a.window = window;
+    a.scale = scale;
+    a.n_splits = n_splits;
+    a.tokens_per_tile = tokens_per_tile;
+    a.keys_per_split = n_splits > 1 ? keys_per_split : 0;
+    a.keys_per_split_dev = n_splits > 1 ? keys_per_split_dev : nullptr;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int rc;
+    switch (head_dim) {
+        case 32: rc = launch_for_dim<32>(s, a, n_tiles, row_tiles); break;
+        case 64: rc = launch_for_dim<64>(s, a, n_tiles, row_tiles); break;
+        case 96: rc = launch_for_dim<96>(s, a, n_tiles, row_tiles); break;
+        case 128: rc = launch_for_dim<128>(s, a, n_tiles, row_tiles); break;
+        case 256: rc = launch_for_dim<256>(s, a, n_tiles, row_tiles); break;
+        default: return CIE_BAD_ARGUMENT;
+    }
+    if (rc != CIE_OK || n_splits == 1) return rc;
+    attention_merge_kernel<<<dim3(n_tiles, kv_heads), 256, 0, s>>>(a, head_dim, 16 * row_tiles);
+    return cie_after_launch();
+}

@@ -3,7 +3,8 @@
 // paged cache.
 //
 //   qkv  [tokens, (Hq + 2*Hkv) * D]   q rotated in place
-//   pool [pages, Hkv, page_size, D]   one for keys, one for values
+//   keys   [pages, Hkv, page_size, D]
+//   values [pages, Hkv, D, page_size]  (transposed, as the attention kernels read them)
 //   slot of token t: page = block_table[seq_slot[seq_of_token[t]], pos / P], row = pos % P
 //
 // Angles come from a float32 cos/sin table [max_position, D/2]; the rotation is
@@ -26,6 +27,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
     const int pos = positions[token];
     T* src = qkv + (static_cast<size_t>(token) * (q_heads + 2 * kv_heads) + head) * head_dim;
 
+    const bool is_value = head >= q_heads + kv_heads;
     T* dst = nullptr;
     if (head >= q_heads) {
         if (!write_kv) return;
@@ -33,11 +35,15 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
         const int slot = seq_slot[seq_of_token[token]];
         const int page = block_table[static_cast<size_t>(slot) * table_width + pos / page_size];
         if (page < 0) return;  // the host never schedules a token without a page
-        T* pool = head < q_heads + kv_heads ? k_pool : v_pool;
-        dst = pool + ((static_cast<size_t>(page) * kv_heads + kv_head) * page_size + pos % page_size) * head_dim;
+        const size_t head_base = (static_cast<size_t>(page) * kv_heads + kv_head) * page_size * head_dim;
+        if (is_value) {  // value element d of the token goes to [d, pos % page_size]
+            T* column = v_pool + head_base + pos % page_size;
+            for (int i = threadIdx.x; i < head_dim; i += blockDim.x) column[static_cast<size_t>(i) * page_size] = src[i];
+            return;
+        }
+        dst = k_pool + head_base + static_cast<size_t>(pos % page_size) * head_dim;
     }
-    const bool is_value = head >= q_heads + kv_heads;
-    if (is_value || !rotate) {
+    if (!rotate) {
         if (dst)
             for (int i = threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
         return;

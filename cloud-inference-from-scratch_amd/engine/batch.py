@@ -33,6 +33,9 @@ class StepBatch:
     host_starts: list[int] = field(default_factory=list)
     host_q_lens: list[int] = field(default_factory=list)
     request_ids: tuple[str, ...] = ()
+    # filled for a step that replays a captured graph: everything a kernel plan reads comes from the device
+    static_plan: Any = None
+    _tiles: dict = field(default_factory=dict)
 
     @property
     def all_decode(self) -> bool:
@@ -41,6 +44,28 @@ class StepBatch:
     @property
     def max_q_len(self) -> int:
         return max(self.host_q_lens, default=0)
+
+    def tiles(self, tokens_per_tile: int, decode: bool) -> tuple[torch.Tensor, torch.Tensor, int]:
+        """Query tiles of at most ``tokens_per_tile`` consecutive tokens of one
+        sequence, for the sequences that bring one token (``decode``) or more:
+        (sequence index of each tile, its first token within the sequence's
+        portion, number of tiles), the two lists as int32 device tensors."""
+        key = (tokens_per_tile, decode)
+        if key not in self._tiles:
+            seqs: list[int] = []
+            firsts: list[int] = []
+            for index, count in enumerate(self.host_q_lens):
+                if (count == 1) != decode:
+                    continue
+                for first in range(0, count, tokens_per_tile):
+                    seqs.append(index)
+                    firsts.append(first)
+            if seqs:
+                both = torch.tensor(seqs + firsts, dtype=torch.int32).to(self.token_ids.device, non_blocking=True)
+                self._tiles[key] = (both[: len(seqs)], both[len(seqs):], len(seqs))
+            else:
+                self._tiles[key] = (self.seq_slot, self.seq_slot, 0)
+        return self._tiles[key]
 
     @property
     def max_context(self) -> int:
@@ -52,7 +77,7 @@ class PagedView:
     """One cache unit of paged keys and values, as a mixer sees it."""
 
     k_pool: torch.Tensor         # [pages, kv_heads, page_size, head_dim]
-    v_pool: torch.Tensor
+    v_pool: torch.Tensor         # [pages, kv_heads, head_dim, page_size]  (transposed)
     block_table: torch.Tensor    # int32 [max_running, width] of the unit's group
     page_size: int
 

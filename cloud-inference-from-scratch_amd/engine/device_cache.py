@@ -1,9 +1,10 @@
 """Device side of the cache: page pools, block tables and state rows.
 
 For every group of the :class:`~cie_amd.cache.manager.CacheManager` one pool
-``[units, 2, pages, kv_heads, page_size, head_dim]`` (keys at index 0, values at
-index 1 of the second axis; a page of one head is contiguous so that a kernel
-streams ``page_size * head_dim`` elements per page and head) and one int32 block
+``[units, 2, pages, kv_heads, page_size * head_dim]`` (keys at index 0 of the
+second axis as ``[page_size, head_dim]``, values at index 1 transposed as
+``[head_dim, page_size]``, the layouts the matrix-core attention reads with plain
+vector loads; a page of one head is contiguous) and one int32 block
 table ``[max_running, width]`` whose row ``slot`` mirrors the request's host
 table.  The reference keeps ``[layers, pages, page_size, kv_heads, head_dim]``
 pools (src/cloud_engine/cache.py:266-274) and uploads padded tables every step
@@ -50,8 +51,10 @@ class DeviceCache:
                 index = manager.unit_group[unit]
                 local = manager.groups[index].units.index(unit)
                 pool = self.pools[index]
-                self._views[unit] = PagedView(pool[local, 0], pool[local, 1], self.tables[index],
-                                              manager.page_size)
+                spec = manager.groups[index].spec
+                pages = manager.groups[index].allocator.total_pages
+                values = pool[local, 1].view(pages, spec.kv_heads, spec.head_dim, manager.page_size)
+                self._views[unit] = PagedView(pool[local, 0], values, self.tables[index], manager.page_size)
             elif unit in self.states:
                 self._views[unit] = StateView(self.states[unit])
             else:

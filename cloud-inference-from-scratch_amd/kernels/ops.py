@@ -66,6 +66,19 @@ def _f(value: float) -> ctypes.c_float:
     return ctypes.c_float(float(value))
 
 
+def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, dtype: torch.dtype, kv_heads: int,
+                 head_dim: int) -> int:
+    """Keys [pages, Hkv, page_size, D], values transposed [pages, Hkv, D, page_size]; returns page_size."""
+    _gpu("k_pool", k_pool, dtype, 4)
+    _gpu("v_pool", v_pool, dtype, 4)
+    pages, heads, page_size, dim = k_pool.shape
+    _require(heads == kv_heads and dim == head_dim,
+             f"k_pool {tuple(k_pool.shape)} does not match Hkv={kv_heads}, D={head_dim}")
+    _require(tuple(v_pool.shape) == (pages, kv_heads, head_dim, page_size),
+             f"v_pool {tuple(v_pool.shape)} must be {(pages, kv_heads, head_dim, page_size)}")
+    return page_size
+
+
 # ---------------------------------------------------------------------------
 def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[t] = float32(table[ids[t]])``; ids int32 [T] (already checked against the vocabulary)."""
@@ -121,8 +134,9 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
                   rotate: bool = True, write_kv: bool = True) -> None:
     """Rotate q (in place) and k, write k and v of every token into its cache slot.
 
-    qkv [T, (Hq+2Hkv)*D]; cos/sin float32 [max_position, D/2]; pools
-    [pages, Hkv, page_size, D] in qkv's dtype; block_table int32 [slots, width]."""
+    qkv [T, (Hq+2Hkv)*D]; cos/sin float32 [max_position, D/2]; key pool
+    [pages, Hkv, page_size, D] and value pool [pages, Hkv, D, page_size] in qkv's
+    dtype; block_table int32 [slots, width]."""
     _gpu("qkv", qkv, dims=2)
     tokens = qkv.shape[0]
     _require(qkv.shape[1] == (q_heads + 2 * kv_heads) * head_dim,
@@ -137,12 +151,7 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
         _require(meta.shape[0] >= tokens, f"{name} has {meta.shape[0]} entries for {tokens} tokens")
     _gpu("seq_slot", seq_slot, torch.int32, 1)
     _gpu("block_table", block_table, torch.int32, 2)
-    for name, pool in (("k_pool", k_pool), ("v_pool", v_pool)):
-        _gpu(name, pool, qkv.dtype, 4)
-        _require(pool.shape[1] == kv_heads and pool.shape[3] == head_dim,
-                 f"{name} {tuple(pool.shape)} does not match Hkv={kv_heads}, D={head_dim}")
-    _require(k_pool.shape == v_pool.shape, "key and value pools differ in shape")
-    page_size = k_pool.shape[2]
+    page_size = _check_pools(k_pool, v_pool, qkv.dtype, kv_heads, head_dim)
     _run("cie_rope_kv_write", load_library().cie_rope_kv_write(
         _stream(), _i(_code(qkv.dtype)), _ptr(qkv), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(seq_of_token),
         _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]), _ptr(k_pool), _ptr(v_pool), _i(tokens),
@@ -180,10 +189,7 @@ def paged_attention_generic(q: torch.Tensor, q_row_stride: int, k_pool: torch.Te
     _require(q_heads % kv_heads == 0, f"{q_heads} query heads are no multiple of {kv_heads} key heads")
     _require(head_dim % 8 == 0 and head_dim <= 256, f"head_dim must be a multiple of 8 up to 256, is {head_dim}")
     _require(q_row_stride % 8 == 0, f"q row stride must be a multiple of 8, is {q_row_stride}")
-    for name, pool in (("k_pool", k_pool), ("v_pool", v_pool)):
-        _gpu(name, pool, q.dtype, 4)
-        _require(pool.shape[1] == kv_heads and pool.shape[3] == head_dim,
-                 f"{name} {tuple(pool.shape)} does not match Hkv={kv_heads}, D={head_dim}")
+    _check_pools(k_pool, v_pool, q.dtype, kv_heads, head_dim)
     _gpu("block_table", block_table, torch.int32, 2)
     for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
         _gpu(name, meta, torch.int32, 1)
@@ -198,6 +204,62 @@ def paged_attention_generic(q: torch.Tensor, q_row_stride: int, k_pool: torch.Te
         _i(block_table.shape[1]), _ptr(positions), _ptr(seq_of_token), _ptr(seq_slot), _ptr(out), _i(tokens),
         _i(q_heads), _i(kv_heads), _i(head_dim), _i(k_pool.shape[2]), _i(window or 0), _f(scale)))
     return out
+
+
+MFMA_HEAD_DIMS = (32, 64, 96, 128, 256)
+
+
+def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                         block_table: torch.Tensor, tile_seq: torch.Tensor, tile_q0: torch.Tensor, n_tiles: int,
+                         seq_slot: torch.Tensor, seq_start: torch.Tensor, seq_q_len: torch.Tensor,
+                         q_start_loc: torch.Tensor, out: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int,
+                         window: Optional[int], scale: float, tokens_per_tile: int, row_tiles: int,
+                         n_splits: int = 1, keys_per_split: int = 0,
+                         keys_per_split_dev: Optional[torch.Tensor] = None,
+                         part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None) -> None:
+    """Matrix-core attention (bf16) for the tiles ``(tile_seq[i], tile_q0[i])``: tile i
+    holds up to ``tokens_per_tile`` tokens of sequence ``tile_seq[i]`` from its
+    ``tile_q0[i]``-th token of this step on.  Rows of other tokens of ``out`` are left alone.
+    With ``n_splits > 1`` every tile's keys are cut into parts of ``keys_per_split``
+    (a multiple of 32, or read from ``keys_per_split_dev``) and merged through the workspaces."""
+    _require(q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 2 and q.stride(1) == 1
+             and q.stride(0) == q_row_stride, "q must be a bf16 GPU matrix with unit inner stride")
+    _require(q.shape[1] >= q_heads * head_dim and q_row_stride % 8 == 0, f"q {tuple(q.shape)} does not fit")
+    _require(head_dim in MFMA_HEAD_DIMS, f"head_dim must be one of {MFMA_HEAD_DIMS}, is {head_dim}")
+    _require(q_heads % kv_heads == 0, f"{q_heads} query heads are no multiple of {kv_heads} key heads")
+    group = q_heads // kv_heads
+    _require(row_tiles in (1, 2, 4) and 1 <= tokens_per_tile and tokens_per_tile * group <= 16 * row_tiles,
+             f"{tokens_per_tile} tokens of {group} heads do not fit {row_tiles} row tiles")
+    page_size = _check_pools(k_pool, v_pool, torch.bfloat16, kv_heads, head_dim)
+    _require(page_size >= 4 and page_size & (page_size - 1) == 0, f"page size must be a power of two >= 4, is {page_size}")
+    _gpu("block_table", block_table, torch.int32, 2)
+    for name, meta in (("tile_seq", tile_seq), ("tile_q0", tile_q0)):
+        _gpu(name, meta, torch.int32, 1)
+        _require(meta.shape[0] >= n_tiles, f"{name} has {meta.shape[0]} entries for {n_tiles} tiles")
+    for name, meta in (("seq_slot", seq_slot), ("seq_start", seq_start), ("seq_q_len", seq_q_len),
+                       ("q_start_loc", q_start_loc)):
+        _gpu(name, meta, torch.int32, 1)
+    _gpu("out", out, torch.bfloat16, 2)
+    _require(out.shape[1] == q_heads * head_dim and out.shape[0] <= q.shape[0], f"out is {tuple(out.shape)}")
+    _require(1 <= n_splits <= 65535, f"n_splits {n_splits} out of range")
+    if n_splits > 1:
+        rows = 16 * row_tiles
+        _require(part_o is not None and part_ml is not None, "split attention needs its workspaces")
+        _gpu("part_o", part_o, torch.float32)
+        _gpu("part_ml", part_ml, torch.float32)
+        units = n_tiles * kv_heads * n_splits
+        _require(part_o.numel() >= units * rows * head_dim and part_ml.numel() >= units * rows * 2,
+                 "attention workspaces are too small")
+        if keys_per_split_dev is not None:
+            _gpu("keys_per_split_dev", keys_per_split_dev, torch.int32)
+        else:
+            _require(keys_per_split > 0 and keys_per_split % 32 == 0, f"keys_per_split {keys_per_split} must be a multiple of 32")
+    _run("cie_paged_attention_mfma", load_library().cie_paged_attention_mfma(
+        _stream(), _ptr(q), _i(q_row_stride), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
+        _i(block_table.shape[1]), _ptr(tile_seq), _ptr(tile_q0), _ptr(seq_slot), _ptr(seq_start), _ptr(seq_q_len),
+        _ptr(q_start_loc), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_tiles), _i(q_heads), _i(kv_heads),
+        _i(head_dim), _i(page_size), _i(window or 0), _f(scale), _i(n_splits), _i(tokens_per_tile), _i(row_tiles),
+        _i(keys_per_split), _ptr(keys_per_split_dev)))
 
 
 def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,

@@ -90,12 +90,67 @@ class Attention(Part):
         return linear(context, self.w_o, self.b_o)
 
 
+def plan_splits(units: int, max_keys: int, target_waves: int = 1024, min_keys: int = 128) -> tuple[int, int]:
+    """How many parts to cut a decode tile's keys into so that the GPU is filled:
+    (number of splits, keys per split as a multiple of 32)."""
+    wanted = max(1, target_waves // max(units, 1))
+    splits = min(wanted, max(1, max_keys // min_keys))
+    if splits <= 1:
+        return 1, 0
+    per_split = -(-(-(-max_keys // splits)) // 32) * 32
+    return -(-max_keys // per_split), per_split
+
+
 def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, head_dim: int,
            window: Optional[int], scale: float) -> torch.Tensor:
-    """Pick the attention kernel for this step's rows."""
-    return ops.paged_attention_generic(
-        qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, batch.positions,
-        batch.seq_of_token, batch.seq_slot, batch.tokens, num_heads, num_kv_heads, head_dim, window, scale)
+    """Pick the attention kernel for this step's rows.
+
+    bfloat16 with a head size the matrix-core kernel takes: sequences that bring
+    one token go to the split-context decode form, prompt portions to the tiled
+    form with up to 64 rows per wave.  Everything else (float32, other head
+    sizes, groups of more than 16 heads, pages of fewer than 4 tokens): the
+    generic kernel."""
+    group = num_heads // num_kv_heads
+    page_size = view.page_size
+    if (qkv.dtype != torch.bfloat16 or head_dim not in ops.MFMA_HEAD_DIMS or group > 16 or page_size < 4
+            or page_size & (page_size - 1)):
+        return ops.paged_attention_generic(
+            qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, batch.positions,
+            batch.seq_of_token, batch.seq_slot, batch.tokens, num_heads, num_kv_heads, head_dim, window, scale)
+    out = torch.empty((batch.tokens, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    common = (batch.seq_slot, batch.seq_start, batch.seq_q_len, batch.q_start_loc, out, num_heads, num_kv_heads,
+              head_dim, window, scale)
+    max_keys = batch.max_context if window is None else min(batch.max_context, window + 32)
+    if batch.static_plan is not None:  # a captured decode step: the grid is fixed, lengths live on the device
+        plan = batch.static_plan
+        part_o, part_ml = _workspaces(qkv.device, batch.sequences * num_kv_heads * plan.n_splits, 16, head_dim)
+        ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, plan.tile_seq,
+                                 plan.tile_q0, batch.sequences, *common, tokens_per_tile=1, row_tiles=1,
+                                 n_splits=plan.n_splits, keys_per_split_dev=plan.keys_per_split,
+                                 part_o=part_o, part_ml=part_ml)
+        return out
+    tile_seq, tile_q0, n_tiles = batch.tiles(1, decode=True)
+    if n_tiles:
+        n_splits, per_split = plan_splits(n_tiles * num_kv_heads, max_keys)
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_o, part_ml = _workspaces(qkv.device, n_tiles * num_kv_heads * n_splits, 16, head_dim)
+        ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
+                                 n_tiles, *common, tokens_per_tile=1, row_tiles=1, n_splits=n_splits,
+                                 keys_per_split=per_split, part_o=part_o, part_ml=part_ml)
+    row_tiles = 4 if group <= 8 or group == 16 else 2 if group <= 10 else 1
+    row_tiles = max(row_tiles, -(-group // 16))
+    per_tile = (16 * row_tiles) // group
+    tile_seq, tile_q0, n_tiles = batch.tiles(per_tile, decode=False)
+    if n_tiles:
+        ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
+                                 n_tiles, *common, tokens_per_tile=per_tile, row_tiles=row_tiles)
+    return out
+
+
+def _workspaces(device: torch.device, units: int, rows: int, head_dim: int) -> tuple[torch.Tensor, torch.Tensor]:
+    return (torch.empty(units * rows * head_dim, dtype=torch.float32, device=device),
+            torch.empty(units * rows * 2, dtype=torch.float32, device=device))
 
 
 register_part("mixer", "attention", Attention)

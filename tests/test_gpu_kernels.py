@@ -137,6 +137,8 @@ def build_cache(dtype, lengths, kv_heads, head_dim, page_size, seed, shuffle=Tru
             count = rows.stop - rows.start
             k_pool[page, :, :count] = k[rows].transpose(0, 1)
             v_pool[page, :, :count] = v[rows].transpose(0, 1)
+    # values are cached transposed: [page, head, head_dim, page_size]
+    v_pool = v_pool.transpose(2, 3).contiguous()
     return k_pool.to(dtype).cuda(), v_pool.to(dtype).cuda(), table.cuda(), slots, dense
 
 
@@ -171,6 +173,135 @@ def test_paged_attention_generic(ops, dtype, geometry):
         torch.tensor(seq_of_token, dtype=torch.int32).cuda(), torch.tensor(slots, dtype=torch.int32).cuda(),
         len(positions), q_heads, kv_heads, head_dim, None, scale)
     torch.testing.assert_close(out.float().cpu(), torch.cat(expected), **tol(dtype))
+
+
+def run_mfma(ops, q_all, contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim, window,
+             scale, per_tile, row_tiles, n_splits=1, keys_per_split=0, decode_only=None):
+    """Drive the matrix-core kernel the way the attention part does: tiles of
+    ``per_tile`` tokens for the chosen sequences; returns [tokens, Hq*D] (rows of
+    sequences that were not chosen stay zero)."""
+    tokens = sum(q_lens)
+    as_dev = lambda values: torch.tensor(values, dtype=torch.int32).cuda()  # noqa: E731
+    loc = [0]
+    for n in q_lens:
+        loc.append(loc[-1] + n)
+    tile_seq, tile_q0 = [], []
+    for s, n in enumerate(q_lens):
+        if decode_only is not None and (n == 1) != decode_only:
+            continue
+        for first in range(0, n, per_tile):
+            tile_seq.append(s)
+            tile_q0.append(first)
+    stride = (q_heads + 2 * kv_heads) * head_dim
+    buffer = torch.zeros((tokens, stride))
+    buffer[:, : q_heads * head_dim] = q_all
+    buffer = buffer.to(torch.bfloat16).cuda()
+    out = torch.zeros((tokens, q_heads * head_dim), dtype=torch.bfloat16).cuda()
+    part_o = part_ml = None
+    if n_splits > 1:
+        units = len(tile_seq) * kv_heads * n_splits
+        part_o = torch.full((units * 16 * row_tiles * head_dim,), float("nan")).cuda()
+        part_ml = torch.full((units * 16 * row_tiles * 2,), float("nan")).cuda()
+    ops.paged_attention_mfma(buffer, stride, k_pool, v_pool, table, as_dev(tile_seq), as_dev(tile_q0), len(tile_seq),
+                             as_dev(slots), as_dev(contexts), as_dev(q_lens), as_dev(loc), out, q_heads, kv_heads,
+                             head_dim, window, scale, per_tile, row_tiles, n_splits=n_splits,
+                             keys_per_split=keys_per_split, part_o=part_o, part_ml=part_ml)
+    return out.float().cpu()
+
+
+MFMA_GEOMETRY = [(16, 2, 128, 16), (4, 2, 32, 8), (3, 1, 32, 8), (6, 6, 64, 4), (16, 1, 96, 32), (12, 4, 256, 16)]
+
+
+@pytest.mark.parametrize("geometry", MFMA_GEOMETRY)
+@pytest.mark.parametrize("row_tiles", [1, 2, 4])
+def test_paged_attention_mfma_ragged(ops, geometry, row_tiles):
+    """The tiled form on a ragged batch (reference matrix of contexts and query
+    lengths, tests/remote_ragged_gpu_tests.py:118-121): portions with and without
+    context, lengths that do not fill a tile, single tokens at page edges."""
+    q_heads, kv_heads, head_dim, page_size = geometry
+    group = q_heads // kv_heads
+    if group > 16 * row_tiles or (head_dim == 256 and row_tiles == 4):
+        pytest.skip("more heads per group than rows, or a variant the dispatcher never picks")
+    contexts = [0, 15, 16, 17, 127, 511, 1, 40]
+    q_lens = [7, 1, 2, 16, 1, 33, 64, 5]
+    lengths = [c + q for c, q in zip(contexts, q_lens)]
+    k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=70)
+    scale = 1.0 / math.sqrt(head_dim)
+    g = torch.Generator().manual_seed(71)
+    qs, expected = [], []
+    for s, (c, n) in enumerate(zip(contexts, q_lens)):
+        q = (torch.randn((n, q_heads, head_dim), generator=g) * 2).to(torch.bfloat16).float()
+        qs.append(q.reshape(n, -1))
+        expected.append(plain_qwen2.causal_attention(q, *dense[s], scale, past_len=c))
+    per_tile = (16 * row_tiles) // group
+    out = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
+                   None, scale, per_tile, row_tiles)
+    torch.testing.assert_close(out, torch.cat(expected), **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("geometry", MFMA_GEOMETRY)
+@pytest.mark.parametrize("splits", [(1, 0), (3, 704), (16, 128), (64, 32)])
+def test_paged_attention_mfma_decode_splits(ops, geometry, splits):
+    """Single tokens over contexts up to 2047 (boundary lengths of
+    tests/remote_gpu_tests.py:204), the keys cut into parts that are merged;
+    parts beyond a short context are empty."""
+    q_heads, kv_heads, head_dim, page_size = geometry
+    n_splits, per_split = splits
+    contexts = [0, 1, 15, 16, 17, 127, 128, 129, 1000, 2047]
+    q_lens = [1] * len(contexts)
+    lengths = [c + 1 for c in contexts]
+    k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=72)
+    scale = 1.0 / math.sqrt(head_dim)
+    g = torch.Generator().manual_seed(73)
+    qs, expected = [], []
+    for s, c in enumerate(contexts):
+        q = (torch.randn((1, q_heads, head_dim), generator=g) * 2).to(torch.bfloat16).float()
+        qs.append(q.reshape(1, -1))
+        expected.append(plain_qwen2.causal_attention(q, *dense[s], scale, past_len=c))
+    out = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
+                   None, scale, 1, 1, n_splits=n_splits, keys_per_split=per_split)
+    torch.testing.assert_close(out, torch.cat(expected), **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("window", [5, 32, 100])
+def test_paged_attention_mfma_window(ops, window):
+    q_heads, kv_heads, head_dim, page_size = 4, 2, 64, 8
+    contexts = [0, 90, 300, 33]
+    q_lens = [40, 1, 17, 1]
+    lengths = [c + q for c, q in zip(contexts, q_lens)]
+    k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=74)
+    scale = 1.0 / math.sqrt(head_dim)
+    g = torch.Generator().manual_seed(75)
+    qs, expected = [], []
+    for s, (c, n) in enumerate(zip(contexts, q_lens)):
+        q = (torch.randn((n, q_heads, head_dim), generator=g) * 2).to(torch.bfloat16).float()
+        qs.append(q.reshape(n, -1))
+        expected.append(plain_qwen2.causal_attention(q, *dense[s], scale, past_len=c, window=window))
+    want = torch.cat(expected)
+    tiled = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
+                     window, scale, 8, 1)
+    torch.testing.assert_close(tiled, want, **tol(torch.bfloat16))
+    split = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
+                     window, scale, 1, 1, n_splits=4, keys_per_split=32, decode_only=True)
+    rows = [40, 58]  # the two single-token sequences
+    torch.testing.assert_close(split[rows], want[rows], **tol(torch.bfloat16))
+
+
+def test_paged_attention_mfma_far_key(ops):
+    """One key among two thousand carries the weight: output = its value row, in
+    the tiled form and in every split layout."""
+    q_heads, kv_heads, head_dim, page_size = 16, 2, 128, 16
+    length, far = 2000, 1234
+    k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, [length], kv_heads, head_dim, page_size, seed=76)
+    k, v = dense[0]
+    q = torch.stack([k[far, h // 8] * 2.0 for h in range(q_heads)])[None].to(torch.bfloat16).float()
+    scale = 1.0 / math.sqrt(head_dim)
+    expect = plain_qwen2.causal_attention(q, k, v, scale, past_len=length - 1)
+    for n_splits, per_split in [(1, 0), (7, 288), (63, 32)]:
+        out = run_mfma(ops, q.reshape(1, -1), [length - 1], [1], k_pool, v_pool, table, slots, q_heads, kv_heads,
+                       head_dim, None, scale, 1, 1, n_splits=n_splits, keys_per_split=per_split)
+        torch.testing.assert_close(out, expect, **tol(torch.bfloat16))
+        torch.testing.assert_close(out.view(q_heads, head_dim), v[far].repeat_interleave(8, dim=0), rtol=0.05, atol=0.05)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -238,12 +369,12 @@ def test_rope_kv_write(ops, dtype, geometry):
         page = int(table_h[slots[s], pos // page_size])
         row = pos % page_size
         torch.testing.assert_close(k_pool[page, :, row].float().cpu(), k_expect[i], **tol(dtype))
-        torch.testing.assert_close(v_pool[page, :, row].float().cpu(), v_in[i], rtol=0, atol=0)
+        torch.testing.assert_close(v_pool[page, :, :, row].float().cpu(), v_in[i], rtol=0, atol=0)  # transposed
         touched[page, :, row] = True
     # nothing else in the pools moved
     untouched = ~touched.cuda()
     assert torch.equal(k_pool[untouched], k_before[untouched])
-    assert torch.equal(v_pool[untouched], v_before[untouched])
+    assert torch.equal(v_pool.transpose(2, 3)[untouched], v_before.transpose(2, 3)[untouched])
 
 
 def test_rope_shift_invariance():
