@@ -58,7 +58,8 @@ struct AttentionArgs {
     int n_splits;
     int tokens_per_tile;
     int keys_per_split;  // multiple of kKeysPerBlock; 0 with one split
-    const int* keys_per_split_dev;  // if set, read from the device instead (a captured graph's value changes per step)
+    const int* max_context_dev;  // if set (a captured graph replays with other lengths): keys per split are
+                                 // derived from this device value, the longest context of the step
 };
 
 template <int D, int RT>
@@ -89,7 +90,12 @@ __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs 
     int range_begin = lo & ~(kKeysPerBlock - 1);
     int range_end = hi;
     if (a.n_splits > 1) {
-        const int per_split = a.keys_per_split_dev ? *a.keys_per_split_dev : a.keys_per_split;
+        int per_split = a.keys_per_split;
+        if (a.max_context_dev) {
+            int most = *a.max_context_dev;
+            if (a.window > 0) most = min(most, a.window + 2 * kKeysPerBlock);
+            per_split = ((most + a.n_splits - 1) / a.n_splits + kKeysPerBlock - 1) & ~(kKeysPerBlock - 1);
+        }
         range_begin += split * per_split;
         range_end = min(hi, range_begin + per_split);
     }
@@ -305,7 +311,7 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
                                      void* out, float* part_o, float* part_ml, int n_tiles, int q_heads,
                                      int kv_heads, int head_dim, int page_size, int window, float scale,
                                      int n_splits, int tokens_per_tile, int row_tiles, int keys_per_split,
-                                     const int* keys_per_split_dev) {
+                                     const int* max_context_dev) {
     if (n_tiles < 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || page_size < 4 ||
         (page_size & (page_size - 1)) || table_width <= 0 || n_splits < 1 || n_splits > 65535 ||
         kv_heads > 65535 || tokens_per_tile < 1 || q_row_stride % 8)
@@ -313,7 +319,7 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     const int group = q_heads / kv_heads;
     if (tokens_per_tile * group > 16 * row_tiles) return CIE_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml ||
-                         (!keys_per_split_dev && (keys_per_split <= 0 || keys_per_split % kKeysPerBlock))))
+                         (!max_context_dev && (keys_per_split <= 0 || keys_per_split % kKeysPerBlock))))
         return CIE_BAD_ARGUMENT;
     if (n_tiles == 0) return CIE_OK;
     int page_shift = 0;
@@ -342,7 +348,7 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     a.n_splits = n_splits;
     a.tokens_per_tile = tokens_per_tile;
     a.keys_per_split = n_splits > 1 ? keys_per_split : 0;
-    a.keys_per_split_dev = n_splits > 1 ? keys_per_split_dev : nullptr;
+    a.max_context_dev = n_splits > 1 ? max_context_dev : nullptr;
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;
     switch (head_dim) {

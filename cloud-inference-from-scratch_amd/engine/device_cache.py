@@ -9,6 +9,12 @@ table ``[max_running, width]`` whose row ``slot`` mirrors the request's host
 table.  The reference keeps ``[layers, pages, page_size, kv_heads, head_dim]``
 pools (src/cloud_engine/cache.py:266-274) and uploads padded tables every step
 (src/cloud_engine/engine.py:264-278); here only rows that changed are copied.
+
+One page and one slot beyond the manager's are kept for padding: a captured
+decode graph runs a fixed number of rows, and the rows that no request fills
+use slot ``pad_slot``, whose block table points at page ``pad_page`` only.
+(The reference pads by repeating the last real row, which writes that row's
+cache slot twice, src/cloud_engine/engine.py:329-356.)
 """
 
 from __future__ import annotations
@@ -31,19 +37,21 @@ class DeviceCache:
         self.pools: list[torch.Tensor] = []
         self.tables: list[torch.Tensor] = []
         self.host_tables: list[torch.Tensor] = []
+        self.pad_slot = manager.max_running
         for group in manager.groups:
             spec = group.spec
-            shape = (len(group.units), 2, group.allocator.total_pages, spec.kv_heads, manager.page_size,
-                     spec.head_dim)
+            pad_page = group.allocator.total_pages
+            shape = (len(group.units), 2, pad_page + 1, spec.kv_heads, manager.page_size, spec.head_dim)
             self.pools.append(torch.zeros(shape, dtype=dtype, device=device))
-            self.tables.append(torch.zeros((manager.max_running, manager.table_width), dtype=torch.int32,
-                                           device=device))
+            table = torch.zeros((manager.max_running + 1, manager.table_width), dtype=torch.int32, device=device)
+            table[self.pad_slot] = pad_page
+            self.tables.append(table)
             self.host_tables.append(torch.zeros((manager.max_running, manager.table_width), dtype=torch.int32,
                                                 pin_memory=device.type == "cuda"))
         self.states: dict[int, torch.Tensor] = {}
         for unit, spec in manager.state_units.items():
             assert isinstance(spec, FixedState)
-            self.states[unit] = torch.zeros((manager.max_running, *spec.shape),
+            self.states[unit] = torch.zeros((manager.max_running + 1, *spec.shape),
                                             dtype=_STATE_DTYPES[spec.dtype], device=device)
         self._views: dict[int, Any] = {}
         for unit in range(len(manager.unit_specs)):
@@ -52,7 +60,7 @@ class DeviceCache:
                 local = manager.groups[index].units.index(unit)
                 pool = self.pools[index]
                 spec = manager.groups[index].spec
-                pages = manager.groups[index].allocator.total_pages
+                pages = manager.groups[index].allocator.total_pages + 1
                 values = pool[local, 1].view(pages, spec.kv_heads, spec.head_dim, manager.page_size)
                 self._views[unit] = PagedView(pool[local, 0], values, self.tables[index], manager.page_size)
             elif unit in self.states:

@@ -25,6 +25,7 @@ from ..profiling import trace_range
 from ..sampling.sampler import Sampler
 from .batch import StepBatch
 from .device_cache import DeviceCache
+from .graphs import DecodeGraphs
 
 
 @dataclass(frozen=True)
@@ -61,6 +62,7 @@ class Runner:
         self.max_forward_request_count = 0
         self.forward_plans: deque[tuple[tuple[str, int, int, int], ...]] = deque(maxlen=256)
         self.sampler = Sampler(config.seed)
+        self.graphs = DecodeGraphs(self) if config.graph_decode and getattr(model, "graph_safe", False) else None
         self._staging = [None, None]
         self._staging_turn = 0
 
@@ -84,6 +86,14 @@ class Runner:
 
     def allocated_tokens(self, request: Any) -> int:
         return self.cache.allocated_tokens(request.request_id)
+
+    @property
+    def graph_captures(self) -> int:
+        return self.graphs.captures if self.graphs is not None else 0
+
+    @property
+    def graph_replays(self) -> int:
+        return self.graphs.replays if self.graphs is not None else 0
 
     def free_tokens(self) -> int:
         """Tokens the pool could take now (free pages of the scarcest group)."""
@@ -195,15 +205,18 @@ class Runner:
         with trace_range("ragged.kv.ensure_capacity"):
             self.cache.ensure_capacity_batch(required)
             self.device_cache.sync()
-        batch = self.pack(entries)
         self.forward_invocations += 1
         self.max_forward_request_count = max(self.max_forward_request_count, len(entries))
         self.forward_plans.append(
             tuple((e.request_id, e.start_pos, len(e.tokens), len(e.want)) for e in entries)
         )
-        phase = "decode" if batch.all_decode else "mixed"
-        with trace_range(f"ragged.forward.{phase}.requests_{batch.sequences}.tokens_{batch.tokens}"):
-            logits = self.model.forward(batch, self.device_cache)
+        decode = all(len(e.tokens) == 1 for e in entries)
+        tokens = sum(len(e.tokens) for e in entries)
+        with trace_range(f"ragged.forward.{'decode' if decode else 'mixed'}.requests_{len(entries)}.tokens_{tokens}"):
+            if decode and self.graphs is not None and self.graphs.takes(len(entries)):
+                logits = self.graphs.run(entries)
+            else:
+                logits = self.model.forward(self.pack(entries), self.device_cache)
         with trace_range("ragged.kv.commit"):
             self.cache.commit_lengths(required)
             self.device_cache.sync()

@@ -215,13 +215,14 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
                          q_start_loc: torch.Tensor, out: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int,
                          window: Optional[int], scale: float, tokens_per_tile: int, row_tiles: int,
                          n_splits: int = 1, keys_per_split: int = 0,
-                         keys_per_split_dev: Optional[torch.Tensor] = None,
+                         max_context_dev: Optional[torch.Tensor] = None,
                          part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None) -> None:
     """Matrix-core attention (bf16) for the tiles ``(tile_seq[i], tile_q0[i])``: tile i
     holds up to ``tokens_per_tile`` tokens of sequence ``tile_seq[i]`` from its
     ``tile_q0[i]``-th token of this step on.  Rows of other tokens of ``out`` are left alone.
     With ``n_splits > 1`` every tile's keys are cut into parts of ``keys_per_split``
-    (a multiple of 32, or read from ``keys_per_split_dev``) and merged through the workspaces."""
+    (a multiple of 32; or, with ``max_context_dev``, derived on the device from the
+    step's longest context) and merged through the workspaces."""
     _require(q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 2 and q.stride(1) == 1
              and q.stride(0) == q_row_stride, "q must be a bf16 GPU matrix with unit inner stride")
     _require(q.shape[1] >= q_heads * head_dim and q_row_stride % 8 == 0, f"q {tuple(q.shape)} does not fit")
@@ -250,8 +251,8 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
         units = n_tiles * kv_heads * n_splits
         _require(part_o.numel() >= units * rows * head_dim and part_ml.numel() >= units * rows * 2,
                  "attention workspaces are too small")
-        if keys_per_split_dev is not None:
-            _gpu("keys_per_split_dev", keys_per_split_dev, torch.int32)
+        if max_context_dev is not None:
+            _gpu("max_context_dev", max_context_dev, torch.int32)
         else:
             _require(keys_per_split > 0 and keys_per_split % 32 == 0, f"keys_per_split {keys_per_split} must be a multiple of 32")
     _run("cie_paged_attention_mfma", load_library().cie_paged_attention_mfma(
@@ -259,7 +260,7 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
         _i(block_table.shape[1]), _ptr(tile_seq), _ptr(tile_q0), _ptr(seq_slot), _ptr(seq_start), _ptr(seq_q_len),
         _ptr(q_start_loc), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_tiles), _i(q_heads), _i(kv_heads),
         _i(head_dim), _i(page_size), _i(window or 0), _f(scale), _i(n_splits), _i(tokens_per_tile), _i(row_tiles),
-        _i(keys_per_split), _ptr(keys_per_split_dev)))
+        _i(keys_per_split), _ptr(max_context_dev)))
 
 
 def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,

@@ -25,6 +25,7 @@ from .linear import linear
 
 
 class Attention(Part):
+    graph_safe = True
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool, out_bias: bool, position: PartSpec, window: Optional[int] = None,
                  scale: Optional[float] = None) -> None:
@@ -120,14 +121,17 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     out = torch.empty((batch.tokens, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
     common = (batch.seq_slot, batch.seq_start, batch.seq_q_len, batch.q_start_loc, out, num_heads, num_kv_heads,
               head_dim, window, scale)
-    max_keys = batch.max_context if window is None else min(batch.max_context, window + 32)
+    max_keys = batch.max_context if window is None else min(batch.max_context, window + 64)
     if batch.static_plan is not None:  # a captured decode step: the grid is fixed, lengths live on the device
         plan = batch.static_plan
-        part_o, part_ml = _workspaces(qkv.device, batch.sequences * num_kv_heads * plan.n_splits, 16, head_dim)
+        bound = plan.max_keys if window is None else min(plan.max_keys, window + 64)
+        n_splits, _ = plan_splits(batch.sequences * num_kv_heads, bound)
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_o, part_ml = _workspaces(qkv.device, batch.sequences * num_kv_heads * n_splits, 16, head_dim)
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, plan.tile_seq,
                                  plan.tile_q0, batch.sequences, *common, tokens_per_tile=1, row_tiles=1,
-                                 n_splits=plan.n_splits, keys_per_split_dev=plan.keys_per_split,
-                                 part_o=part_o, part_ml=part_ml)
+                                 n_splits=n_splits, max_context_dev=plan.max_context, part_o=part_o, part_ml=part_ml)
         return out
     tile_seq, tile_q0, n_tiles = batch.tiles(1, decode=True)
     if n_tiles:
@@ -138,8 +142,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
                                  n_tiles, *common, tokens_per_tile=1, row_tiles=1, n_splits=n_splits,
                                  keys_per_split=per_split, part_o=part_o, part_ml=part_ml)
-    row_tiles = 4 if group <= 8 or group == 16 else 2 if group <= 10 else 1
-    row_tiles = max(row_tiles, -(-group // 16))
+    row_tiles = 2 if head_dim > 128 else 4  # 64 rows per wave; 32 where the accumulators would spill
     per_tile = (16 * row_tiles) // group
     tile_seq, tile_q0, n_tiles = batch.tiles(per_tile, decode=False)
     if n_tiles:

@@ -61,7 +61,14 @@ def build_part(role: str, spec: PartSpec) -> Any:
 
 
 class Part:
-    """Default behaviour of a part without tensors."""
+    """Default behaviour of a part without tensors.
+
+    ``graph_safe``: the part's ``forward`` reads everything that changes from
+    step to step (lengths, slots, positions) from device tensors of the batch,
+    never from its host lists, and launches the same kernels for the same batch
+    size: only then may a decode step that contains it be captured in a graph."""
+
+    graph_safe = False
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
         return {}

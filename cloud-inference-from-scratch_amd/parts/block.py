@@ -43,6 +43,10 @@ class PreNormBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False) for _, part in self._parts())
+
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], batch, view,
                 writes: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
         x = self.norm1.forward(residual, pending, self.dtype)

@@ -15,6 +15,7 @@ from .linear import linear
 
 
 class GatedMLP(Part):
+    graph_safe = True
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
         if activation != "silu":
             raise ValueError(f"gated feed-forward runs silu only, got {activation!r}")

@@ -69,6 +69,11 @@ class DecoderModel:
                 )
         return needs
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model may be captured in a graph."""
+        return all(getattr(block, "graph_safe", False) for block in self.blocks) and self.final_norm.graph_safe
+
     def load(self, source: Any, dtype: str, device: str | torch.device) -> "DecoderModel":
         """Bind weights from a source (``SafetensorsSource`` or ``RandomSource``)."""
         device = torch.device(device)

@@ -18,6 +18,7 @@ from .base import Part, register_part
 
 
 class RMSNorm(Part):
+    graph_safe = True
     def __init__(self, size: int, eps: float) -> None:
         if size <= 0 or not eps > 0:
             raise ValueError(f"RMSNorm needs a positive size and eps, got {size}, {eps}")

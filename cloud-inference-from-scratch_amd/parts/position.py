@@ -20,6 +20,7 @@ _TABLES: dict[tuple, tuple[torch.Tensor, torch.Tensor]] = {}
 
 
 class RotaryHalf(Part):
+    graph_safe = True
     rotates = True
 
     def __init__(self, head_dim: int, theta: float, max_position: int) -> None:
@@ -46,6 +47,7 @@ class RotaryHalf(Part):
 
 
 class NoPosition(Part):
+    graph_safe = True
     """Keys and queries enter the mixer as projected."""
 
     rotates = False

@@ -39,14 +39,14 @@ def plain_all(raw, tensors, requests):
     return {rid: plain_qwen2.forward(raw, weights, tokens) for rid, tokens in requests.items()}
 
 
-def make_runner(folder, dtype, kv_tokens, page_size, max_running=8):
+def make_runner(folder, dtype, kv_tokens, page_size, max_running=8, graph_decode=False):
     from cie_amd.config import build_engine_config
     from cie_amd.engine import Runner, load_model
 
     model, config = load_model(folder, dtype, "cuda:0")
     engine_config = build_engine_config(
         dtype=dtype, page_size=page_size, kv_tokens=kv_tokens, max_running=max_running,
-        max_model_len=min(config.max_position_embeddings, kv_tokens), prefix_cache_pages=0, graph_decode=False)
+        max_model_len=min(config.max_position_embeddings, kv_tokens), prefix_cache_pages=0, graph_decode=graph_decode)
     return Runner(model, engine_config, "cuda:0")
 
 
@@ -84,6 +84,28 @@ def test_replay_matches_plain(tiny_folders, plain, name, schedule, dtype):
     worst = replay_util.compare(rows, expected, **TOL[dtype])
     print(f"worst |diff| {worst:.3e}", flush=True)
     assert runner.cache.stats().pages_used == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_captured_decode_steps_match_plain(tiny_folders, plain, name, dtype):
+    """Decode steps replayed from captured graphs (buckets 1, 2 and 4, padded
+    rows on the pad slot), between eager prompt portions, every replay checked:
+    the tail schedule decodes one request at a time, the mixed one several."""
+    folder, raw, _ = tiny_folders[name]
+    requests, expected = plain[name]
+    page = 16 if name == "A" else 8
+    schedules = {"tail": replay_util.tail_one_by_one,
+                 "mixed": lambda r: replay_util.mixed(r, live=4, decode_tail=30, seed=5)}
+    for schedule, build in schedules.items():
+        steps = build(requests)
+        pool = replay_util.max_live_tokens(steps, page=page)
+        runner = make_runner(folder, dtype, pool, page, graph_decode=True)
+        assert runner.graphs is not None
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        replay_util.compare(rows, expected, **TOL[dtype])
+        assert runner.graph_replays >= 20 and runner.graph_captures >= (1 if schedule == "tail" else 2)
+        print(f"{name} {schedule} {dtype}: {runner.graph_captures} captures, {runner.graph_replays} replays", flush=True)
 
 
 def test_mixed_reuses_pages(tiny_folders, plain):
