@@ -254,34 +254,46 @@ __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs 
 }
 
 // Merge the splits of every (tile, kv head): out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M).
-__global__ void __launch_bounds__(256)
+// One workgroup per (tile, kv head, row); the splits' weights are made once in LDS, then every thread
+// sums its head dimensions over the splits with independent loads.
+constexpr int kMergeMaxSplits = 1024;
+
+__global__ void __launch_bounds__(128)
 attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
+    __shared__ float weight[kMergeMaxSplits];
+    __shared__ float scratch[16];
     const int tile = blockIdx.x;
     const int kv_head = blockIdx.y;
+    const int row = blockIdx.z;
     const int group = a.q_heads / a.kv_heads;
     const int seq = a.tile_seq[tile];
     const int q0 = a.tile_q0[tile];
     const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
-    const int n_rows = n_tok * group;
-    const int first_row_token = a.q_start_loc[seq] + q0;
+    if (row >= n_tok * group) return;
     const size_t unit0 = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits;
-    for (int idx = threadIdx.x; idx < n_rows * head_dim; idx += blockDim.x) {
-        const int row = idx / head_dim;
-        const int d = idx - row * head_dim;
-        float m_all = -INFINITY;
-        for (int s = 0; s < a.n_splits; ++s)
-            m_all = fmaxf(m_all, a.part_ml[((unit0 + s) * rows_per_tile + row) * 2]);
-        float num = 0.f, den = 0.f;
-        for (int s = 0; s < a.n_splits; ++s) {
-            const float* ml = a.part_ml + ((unit0 + s) * rows_per_tile + row) * 2;
-            const float w = (ml[0] == -INFINITY) ? 0.f : __expf(ml[0] - m_all);
-            num += a.part_o[((unit0 + s) * rows_per_tile + row) * head_dim + d] * w;
-            den += ml[1] * w;
-        }
-        const int tok = row / group;
-        const int head = row - tok * group;
-        a.out[static_cast<size_t>(first_row_token + tok) * a.q_heads * head_dim +
-              static_cast<size_t>(kv_head * group + head) * head_dim + d] = from_float<bf16_t>(num / den);
+    float m_local = -INFINITY;
+    for (int s = threadIdx.x; s < a.n_splits; s += blockDim.x)
+        m_local = fmaxf(m_local, a.part_ml[((unit0 + s) * rows_per_tile + row) * 2]);
+    const float m_all = block_max(m_local, scratch);
+    float den_local = 0.f;
+    for (int s = threadIdx.x; s < a.n_splits; s += blockDim.x) {
+        const float* ml = a.part_ml + ((unit0 + s) * rows_per_tile + row) * 2;
+        const float w = (ml[0] == -INFINITY) ? 0.f : __expf(ml[0] - m_all);
+        weight[s] = w;
+        den_local += ml[1] * w;
+    }
+    const float den = block_sum(den_local, scratch);  // its barriers also publish weight[]
+    const int tok = row / group;
+    const int head = row - tok * group;
+    bf16_t* dst = a.out + static_cast<size_t>(a.q_start_loc[seq] + q0 + tok) * a.q_heads * head_dim +
+                  static_cast<size_t>(kv_head * group + head) * head_dim;
+    const float inv = 1.0f / den;
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        const float* po = a.part_o + (unit0 * rows_per_tile + row) * head_dim + d;
+        const size_t stride = static_cast<size_t>(rows_per_tile) * head_dim;
+        float num = 0.f;
+        for (int s = 0; s < a.n_splits; ++s) num += po[s * stride] * weight[s];
+        dst[d] = from_float<bf16_t>(num * inv);
     }
 }
 
@@ -318,6 +330,7 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
         return CIE_BAD_ARGUMENT;
     const int group = q_heads / kv_heads;
     if (tokens_per_tile * group > 16 * row_tiles) return CIE_BAD_ARGUMENT;
+    if (n_splits > kMergeMaxSplits) return CIE_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml ||
                          (!max_context_dev && (keys_per_split <= 0 || keys_per_split % kKeysPerBlock))))
         return CIE_BAD_ARGUMENT;
@@ -360,6 +373,6 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
         default: return CIE_BAD_ARGUMENT;
     }
     if (rc != CIE_OK || n_splits == 1) return rc;
-    attention_merge_kernel<<<dim3(n_tiles, kv_heads), 256, 0, s>>>(a, head_dim, 16 * row_tiles);
+    attention_merge_kernel<<<dim3(n_tiles, kv_heads, tokens_per_tile * group), 128, 0, s>>>(a, head_dim, 16 * row_tiles);
     return cie_after_launch();
 }

@@ -48,6 +48,40 @@ static int launch_norm(hipStream_t s, float* residual, const void* branch, const
     return cie_after_launch();
 }
 
+// RMSNorm of rows whose partial sums of squares are already known (left by the product that wrote the
+// residual): no reduction over the row is needed, so a row is spread over several workgroups.
+template <typename T, typename W>
+__global__ void __launch_bounds__(256)
+rmsnorm_from_sumsq_kernel(const float* __restrict__ residual, const float* __restrict__ sumsq, int parts,
+                          const W* __restrict__ weight, T* __restrict__ out, int hidden, float eps) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.y;
+    float s = 0.f;
+    for (int p = threadIdx.x; p < parts; p += blockDim.x) s += sumsq[static_cast<size_t>(row) * parts + p];
+    const float inv = 1.0f / sqrtf(block_sum(s, scratch) / static_cast<float>(hidden) + eps);
+    const int h = blockIdx.x * blockDim.x + threadIdx.x;
+    if (h < hidden)
+        out[static_cast<size_t>(row) * hidden + h] =
+            from_float<T>((residual[static_cast<size_t>(row) * hidden + h] * inv) * to_float(weight[h]));
+}
+
+CIE_API int cie_rmsnorm_from_sumsq(void* stream, int wdtype, const float* residual, const float* sumsq, int parts,
+                                   const void* weight, void* out, int rows, int hidden, float eps) {
+    if (rows < 0 || rows > 65535 || hidden <= 0 || parts < 1 || !(eps > 0.f)) return CIE_BAD_ARGUMENT;
+    if (rows == 0) return CIE_OK;
+    dim3 grid((hidden + 255) / 256, rows);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (wdtype == CIE_BF16)
+        rmsnorm_from_sumsq_kernel<bf16_t, bf16_t><<<grid, 256, 0, s>>>(
+            residual, sumsq, parts, static_cast<const bf16_t*>(weight), static_cast<bf16_t*>(out), hidden, eps);
+    else if (wdtype == CIE_F32)
+        rmsnorm_from_sumsq_kernel<bf16_t, float><<<grid, 256, 0, s>>>(
+            residual, sumsq, parts, static_cast<const float*>(weight), static_cast<bf16_t*>(out), hidden, eps);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
 // dtype: activation type of branch/out; wdtype: storage type of the weight.
 CIE_API int cie_add_rmsnorm(void* stream, int dtype, int wdtype, float* residual, const void* branch,
                             const void* weight, void* out, const int* rows, int n_out, int hidden,

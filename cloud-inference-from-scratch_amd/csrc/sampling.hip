@@ -95,7 +95,73 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     out[r] = pick;
 }
 
+// Greedy over a large vocabulary, stage 1: each workgroup scans one chunk of one row and leaves its
+// best (value, first index); stage 2 (one workgroup per row) picks among the chunks.
+__global__ void __launch_bounds__(kThreads)
+argmax_chunks_kernel(const float* __restrict__ logits, float* __restrict__ chunk_val, int* __restrict__ chunk_idx,
+                     int vocab, int ld, int chunk) {
+    __shared__ float s_val[kThreads];
+    __shared__ int s_idx[kThreads];
+    const int r = blockIdx.y;
+    const int begin = blockIdx.x * chunk;
+    const int count = min(chunk, vocab - begin);
+    float best;
+    int best_idx;
+    argmax_block(logits + static_cast<size_t>(r) * ld + begin, count, s_val, s_idx, best, best_idx);
+    if (threadIdx.x == 0) {
+        chunk_val[r * gridDim.x + blockIdx.x] = best;
+        chunk_idx[r * gridDim.x + blockIdx.x] = begin + best_idx;
+    }
+}
+
+__global__ void __launch_bounds__(kThreads)
+argmax_final_kernel(const float* __restrict__ chunk_val, const int* __restrict__ chunk_idx, int* __restrict__ out,
+                    int chunks) {
+    __shared__ float s_val[kThreads];
+    __shared__ int s_idx[kThreads];
+    const int r = blockIdx.x;
+    float best = -INFINITY;
+    int best_idx = 0x7fffffff;
+    for (int c = threadIdx.x; c < chunks; c += kThreads) {  // chunks are in index order: ties keep the lower index
+        const float v = chunk_val[r * chunks + c];
+        const int i = chunk_idx[r * chunks + c];
+        if (v > best || (v == best && i < best_idx)) {
+            best = v;
+            best_idx = i;
+        }
+    }
+    s_val[threadIdx.x] = best;
+    s_idx[threadIdx.x] = best_idx;
+    __syncthreads();
+    for (int stride = kThreads / 2; stride > 0; stride >>= 1) {
+        if (threadIdx.x < stride) {
+            const float v = s_val[threadIdx.x + stride];
+            const int i = s_idx[threadIdx.x + stride];
+            if (v > s_val[threadIdx.x] || (v == s_val[threadIdx.x] && i < s_idx[threadIdx.x])) {
+                s_val[threadIdx.x] = v;
+                s_idx[threadIdx.x] = i;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[r] = s_idx[0] == 0x7fffffff ? 0 : s_idx[0];
+}
+
 }  // namespace
+
+// Greedy for every row in two stages; chunk_val / chunk_idx hold rows * chunks entries, chunks = ceil(vocab / chunk).
+CIE_API int cie_argmax(void* stream, const float* logits, float* chunk_val, int* chunk_idx, int* out, int rows,
+                       int vocab, int ld, int chunk) {
+    if (rows < 0 || vocab <= 0 || ld < vocab || chunk <= 0 || rows > 65535 || !chunk_val || !chunk_idx)
+        return CIE_BAD_ARGUMENT;
+    if (rows == 0) return CIE_OK;
+    const int chunks = (vocab + chunk - 1) / chunk;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    argmax_chunks_kernel<<<dim3(chunks, rows), kThreads, 0, s>>>(logits, chunk_val, chunk_idx, vocab, ld, chunk);
+    if (cie_after_launch() != CIE_OK) return CIE_LAUNCH_FAILED;
+    argmax_final_kernel<<<rows, kThreads, 0, s>>>(chunk_val, chunk_idx, out, chunks);
+    return cie_after_launch();
+}
 
 CIE_API int cie_sample(void* stream, const float* logits, const float* temperature,
                        const float* uniform, int* out, int rows, int vocab, int ld) {

@@ -128,6 +128,22 @@ def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: 
     return out
 
 
+def rmsnorm_from_sumsq(residual: torch.Tensor, sumsq: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """bf16 RMSNorm of float32 rows whose partial sums of squares ``sumsq`` [rows, parts] are known."""
+    _gpu("residual", residual, torch.float32, 2)
+    rows, hidden = residual.shape
+    _gpu("sumsq", sumsq, torch.float32, 2)
+    _require(sumsq.shape[0] >= rows, f"sumsq has {sumsq.shape[0]} rows for {rows}")
+    _gpu("weight", weight, dims=1)
+    _require(weight.shape[0] == hidden and weight.dtype in (torch.bfloat16, torch.float32), "norm weight does not fit")
+    _require(eps > 0, f"eps must be positive, is {eps}")
+    out = torch.empty((rows, hidden), dtype=torch.bfloat16, device=residual.device)
+    _run("cie_rmsnorm_from_sumsq", load_library().cie_rmsnorm_from_sumsq(
+        _stream(), _i(_code(weight.dtype)), _ptr(residual), _ptr(sumsq), _i(sumsq.shape[1]), _ptr(weight), _ptr(out),
+        _i(rows), _i(hidden), _f(eps)))
+    return out
+
+
 def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
                   seq_of_token: torch.Tensor, seq_slot: torch.Tensor, block_table: torch.Tensor,
                   k_pool: torch.Tensor, v_pool: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int,
@@ -310,12 +326,119 @@ def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
     return out
 
 
+EPI_BF16, EPI_F32, EPI_SILU, EPI_RESID = 0, 1, 2, 3
+FUSED_TARGET_WAVES = 2048
+
+
+FUSED_HALF_BELOW = 256  # fewer 16-column workgroups than this: use 8-column workgroups
+
+
+def plan_fused(rows: int, column_tiles: int, k: int, may_halve: bool = True) -> tuple[int, int, int]:
+    """(row_tiles, waves per workgroup, half_tiles) for ``rows`` rows,
+    ``column_tiles`` 16-column tiles and inner size ``k``: enough waves to fill
+    the GPU, at least one 128-wide slice of k per wave, waves * row_tiles <= 16;
+    workgroups of 8 columns where 16-column ones would leave compute units idle."""
+    row_tiles = 1 if rows <= 16 else 2 if rows <= 32 else 4
+    half = 1 if may_halve and row_tiles == 1 and column_tiles < FUSED_HALF_BELOW else 0
+    blocks = column_tiles * (2 if half else 1) * -(-rows // (16 * row_tiles))
+    waves = 1
+    while (waves < 16 // row_tiles and blocks * waves < FUSED_TARGET_WAVES and waves * 2 * 128 <= k):
+        waves *= 2
+    return row_tiles, waves, half
+
+
+def gemm_fused(weight: torch.Tensor, epilogue: int, a: Optional[torch.Tensor] = None,
+               residual_in: Optional[torch.Tensor] = None, sumsq_in: Optional[torch.Tensor] = None,
+               norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+               bias: Optional[torch.Tensor] = None, residual_out: Optional[torch.Tensor] = None,
+               sumsq_out: Optional[torch.Tensor] = None, plan: Optional[tuple[int, int, int]] = None
+               ) -> Optional[torch.Tensor]:
+    """Few-row matrix product ``A @ weight.T`` fused with its neighbours.
+
+    A is either ``a`` (bf16 [M, K]) or made on the fly as the RMS-normalised
+    ``residual_in`` (float32 [M, K]) from the partial row sums of squares
+    ``sumsq_in`` [M, parts] and ``norm_weight``.  ``epilogue``: ``EPI_BF16`` /
+    ``EPI_F32`` return ``A W^T + bias``; ``EPI_SILU`` (weight = gate rows over up
+    rows) returns ``silu(gate) * up`` [M, N/2]; ``EPI_RESID`` adds the product
+    into ``residual_out`` (float32 [M, N]) and writes the partial sums of squares
+    of its new rows to ``sumsq_out`` [M, N/16], returning nothing."""
+    _gpu("weight", weight, torch.bfloat16, 2)
+    n, k = weight.shape
+    _require(k % 8 == 0 and n % 16 == 0, f"gemm_fused needs K % 8 == 0 and N % 16 == 0, got N={n}, K={k}")
+    device = weight.device
+    rows = (residual_in if residual_in is not None else a).shape[0]
+    row_tiles, waves, half = plan or plan_fused(rows, (n // 2 if epilogue == EPI_SILU else n) // 16, k,
+                                                may_halve=epilogue != EPI_SILU)
+    _require(waves in (1, 2, 4, 8, 16) and waves * row_tiles <= 16, f"plan {(row_tiles, waves, half)} is not built")
+    _require(not half or (row_tiles == 1 and epilogue != EPI_SILU), "8-column workgroups need one row tile and no SiLU")
+    if residual_in is not None:
+        _gpu("residual_in", residual_in, torch.float32, 2)
+        m = residual_in.shape[0]
+        _require(residual_in.shape[1] == k, f"residual_in {tuple(residual_in.shape)} vs K={k}")
+        _require(sumsq_in is not None and norm_weight is not None and eps > 0, "the norm prologue needs sumsq, weight and eps")
+        _gpu("sumsq_in", sumsq_in, torch.float32, 2)
+        _require(sumsq_in.shape[0] >= m, f"sumsq_in has {sumsq_in.shape[0]} rows for {m}")
+        _gpu("norm_weight", norm_weight, dims=1)
+        _require(norm_weight.shape[0] == k and norm_weight.dtype in (torch.bfloat16, torch.float32), "norm weight does not fit")
+        lda = 0
+    else:
+        _require(a is not None and a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1,
+                 "a must be a bf16 GPU matrix with unit inner stride")
+        m = a.shape[0]
+        _require(a.shape[1] == k, f"a {tuple(a.shape)} vs K={k}")
+        lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+        _require(lda % 8 == 0 and a.data_ptr() % 16 == 0, "a must be 16-byte aligned with a row stride that is a multiple of 8")
+    _require(m >= 1, "gemm_fused needs at least one row")
+    if bias is not None:
+        _gpu("bias", bias, torch.bfloat16, 1)
+        _require(bias.shape[0] == n and epilogue != EPI_SILU, "bias does not fit")
+    out = None
+    if epilogue == EPI_BF16:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    elif epilogue == EPI_F32:
+        out = torch.empty((m, n), dtype=torch.float32, device=device)
+    elif epilogue == EPI_SILU:
+        _require(n % 32 == 0, f"the SiLU epilogue needs N % 32 == 0, got {n}")
+        out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=device)
+    elif epilogue == EPI_RESID:
+        _require(residual_out is not None, "the residual epilogue needs the residual to add into")
+        _gpu("residual_out", residual_out, torch.float32, 2)
+        _require(residual_out.shape == (m, n), f"residual_out {tuple(residual_out.shape)} vs {(m, n)}")
+        parts = n // (8 if half else 16)
+        if sumsq_out is None:
+            sumsq_out = torch.empty((m, parts), dtype=torch.float32, device=device)
+        out = sumsq_out
+        _gpu("sumsq_out", sumsq_out, torch.float32, 2)
+        _require(sumsq_out.shape[0] >= m and sumsq_out.shape[1] == parts, f"sumsq_out {tuple(sumsq_out.shape)} must be [>= {m}, {parts}]")
+    else:
+        raise ValueError(f"unknown epilogue {epilogue}")
+    _run("cie_gemm_fused", load_library().cie_gemm_fused(
+        _stream(), _ptr(a), _i(lda), _ptr(residual_in), _ptr(sumsq_in),
+        _i(sumsq_in.shape[1] if sumsq_in is not None else 0), _ptr(norm_weight),
+        _i(1 if norm_weight is not None and norm_weight.dtype == torch.float32 else 0), _f(eps), _ptr(weight),
+        _ptr(bias), _ptr(None if epilogue == EPI_RESID else out), _ptr(residual_out), _ptr(sumsq_out), _i(m), _i(n), _i(k), _i(epilogue),
+        _i(row_tiles), _i(waves), _i(half)))
+    return out
+
+
+ARGMAX_CHUNK = 2048
+
+
 def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
            uniform: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One token per row of float32 logits: argmax where the row's temperature
     is 0 (or none is given), else a draw with the row's uniform number."""
     _gpu("logits", logits, torch.float32, 2)
     rows, vocab = logits.shape
+    if temperature is None and vocab >= 4 * ARGMAX_CHUNK:
+        if out is None:
+            out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+        chunks = -(-vocab // ARGMAX_CHUNK)
+        chunk_val = torch.empty(rows * chunks, dtype=torch.float32, device=logits.device)
+        chunk_idx = torch.empty(rows * chunks, dtype=torch.int32, device=logits.device)
+        _run("cie_argmax", load_library().cie_argmax(_stream(), _ptr(logits), _ptr(chunk_val), _ptr(chunk_idx),
+                                                     _ptr(out), _i(rows), _i(vocab), _i(vocab), _i(ARGMAX_CHUNK)))
+        return out
     if temperature is not None:
         _gpu("temperature", temperature, torch.float32, 1)
         _require(uniform is not None, "temperature sampling needs the uniform numbers")

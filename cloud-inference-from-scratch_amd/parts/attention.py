@@ -26,6 +26,8 @@ from .linear import linear
 
 class Attention(Part):
     graph_safe = True
+    takes_lazy_norm = True
+    adds_to_residual = True
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool, out_bias: bool, position: PartSpec, window: Optional[int] = None,
                  scale: Optional[float] = None) -> None:
@@ -77,7 +79,7 @@ class Attention(Part):
         self.b_o = tensors[prefix + "o_proj.bias"].contiguous() if self.out_bias else None
         self.cos, self.sin = self.position.tables(device)
 
-    def forward(self, x: torch.Tensor, batch, view, writes: bool = True) -> torch.Tensor:
+    def forward(self, x, batch, view, writes: bool = True, residual: Optional[torch.Tensor] = None):
         if batch.max_context > self.position.max_position and self.position.rotates:
             raise ValueError(
                 f"position {batch.max_context - 1} is beyond the rotary table of {self.position.max_position}"
@@ -88,7 +90,7 @@ class Attention(Part):
                           self.head_dim, rotate=self.position.rotates, write_kv=writes)
         context = attend(qkv, batch, view, self.num_heads, self.num_kv_heads, self.head_dim,
                          self.window, self.scale)
-        return linear(context, self.w_o, self.b_o)
+        return linear(context, self.w_o, self.b_o, into=residual)
 
 
 def plan_splits(units: int, max_keys: int, target_waves: int = 1024, min_keys: int = 128) -> tuple[int, int]:

@@ -10,9 +10,10 @@ Interfaces (``x`` is ``[tokens, hidden]`` in the engine's activation dtype,
 ``residual`` the float32 residual stream, ``batch`` a
 :class:`~cie_amd.engine.batch.StepBatch`):
 
-``Norm``        ``forward(residual, branch, out_dtype, rows=None) -> x``
+``Norm``        ``forward(residual, branch, out_dtype, rows=None, lazy=False) -> x``
                 adds ``branch`` into ``residual`` (in place, float32) and returns
-                the normalised rows.
+                the normalised rows (``branch`` may also be a ``RowSumsq``, see
+                ``parts/linear.py``; with ``lazy`` a ``LazyNorm`` may come back).
 ``Position``    ``tables(device) -> (cos, sin)`` or whatever its mixer asks of it.
 ``Mixer``       ``cache_need() -> PagedKV | FixedState | None`` and
                 ``forward(x, batch, view, writes) -> y``; ``view`` is the cache
@@ -69,6 +70,10 @@ class Part:
     size: only then may a decode step that contains it be captured in a graph."""
 
     graph_safe = False
+    # ``takes_lazy_norm``: ``forward`` accepts a ``LazyNorm`` in place of ``x``.  ``adds_to_residual``:
+    # ``forward`` takes ``residual=`` and may add its output there itself, returning a ``RowSumsq``.
+    takes_lazy_norm = False
+    adds_to_residual = False
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
         return {}

@@ -3,7 +3,10 @@
 ``PreNormBlock``: the reference's decoder layer (src/cloud_engine/model.py:211-220)
 ``h += mixer(norm1(h)); h += feed_forward(norm2(h))``.  The residual stream is
 float32; a branch's output is added inside the next norm kernel, so the block
-returns the feed-forward output as ``pending`` instead of adding it.
+returns the feed-forward output as ``pending`` instead of adding it.  A part
+that can add its output into the residual itself (the fused decode products do)
+returns a ``RowSumsq`` instead, and the next norm may then stay lazy and be
+folded into its consumer's product (``parts/linear.py``).
 """
 
 from __future__ import annotations
@@ -15,6 +18,7 @@ import torch
 from ..config.specs import LayerSpec
 from ..weights.tensors import TensorSpec
 from .base import build_part, register_part
+from .linear import RowSumsq
 
 
 class PreNormBlock:
@@ -49,10 +53,26 @@ class PreNormBlock:
 
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], batch, view,
                 writes: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
-        x = self.norm1.forward(residual, pending, self.dtype)
-        mixed = self.mixer.forward(x, batch, view, writes)
-        x = self.norm2.forward(residual, mixed, self.dtype)
-        return residual, self.feed_forward.forward(x)
+        x = normalise(self.norm1, residual, pending, self.dtype, self.mixer)
+        extra = {"residual": residual} if getattr(self.mixer, "adds_to_residual", False) else {}
+        mixed = self.mixer.forward(x, batch, view, writes, **extra)
+        x = normalise(self.norm2, residual, mixed, self.dtype, self.feed_forward)
+        extra = {"residual": residual} if getattr(self.feed_forward, "adds_to_residual", False) else {}
+        return residual, self.feed_forward.forward(x, **extra)
+
+
+def normalise(norm, residual: torch.Tensor, pending, dtype: torch.dtype, consumer=None, rows=None):
+    """Run ``norm`` on the residual stream plus what is pending.  Only a norm that
+    says so is shown a ``RowSumsq`` or asked to stay lazy; any other gets ``None``
+    for a branch that was already added."""
+    if isinstance(pending, RowSumsq):
+        if not getattr(norm, "takes_row_sumsq", False):
+            pending = None
+        elif rows is None and getattr(consumer, "takes_lazy_norm", False):
+            return norm.forward(residual, pending, dtype, lazy=True)
+    if rows is not None:
+        return norm.forward(residual, pending, dtype, rows=rows)
+    return norm.forward(residual, pending, dtype)
 
 
 register_part("block", "pre_norm", PreNormBlock)

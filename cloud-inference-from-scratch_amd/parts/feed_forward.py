@@ -6,9 +6,10 @@ one fused product here, the activation and the multiply one kernel.
 
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 
-from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, register_part
 from .linear import linear
@@ -16,6 +17,8 @@ from .linear import linear
 
 class GatedMLP(Part):
     graph_safe = True
+    takes_lazy_norm = True
+    adds_to_residual = True
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
         if activation != "silu":
             raise ValueError(f"gated feed-forward runs silu only, got {activation!r}")
@@ -36,9 +39,8 @@ class GatedMLP(Part):
         ).contiguous()
         self.w_down = tensors[prefix + "down_proj.weight"].contiguous()
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        gate_up = linear(x, self.w_gate_up)
-        return linear(ops.silu_mul(gate_up), self.w_down)
+    def forward(self, x, residual: Optional[torch.Tensor] = None):
+        return linear(linear(x, self.w_gate_up, epilogue="silu"), self.w_down, into=residual)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

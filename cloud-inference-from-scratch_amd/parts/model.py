@@ -15,6 +15,7 @@ from ..kernels import ops
 from ..weights.loader import torch_dtype
 from ..weights.tensors import TensorSpec
 from .base import BLOCKS, build_part
+from .block import normalise
 from .linear import linear
 
 
@@ -99,5 +100,5 @@ class DecoderModel:
         for call in self.spec.order:
             residual, pending = self.blocks[call.layer].forward(
                 residual, pending, batch, cache.view(call.cache), call.writes)
-        selected = self.final_norm.forward(residual, pending, self.dtype, rows=batch.logit_rows)
+        selected = normalise(self.final_norm, residual, pending, self.dtype, rows=batch.logit_rows)
         return linear(selected, self.head, None, out_dtype=torch.float32)

@@ -15,10 +15,12 @@ import torch
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, register_part
+from .linear import LazyNorm, RowSumsq
 
 
 class RMSNorm(Part):
     graph_safe = True
+    takes_row_sumsq = True
     def __init__(self, size: int, eps: float) -> None:
         if size <= 0 or not eps > 0:
             raise ValueError(f"RMSNorm needs a positive size and eps, got {size}, {eps}")
@@ -33,8 +35,16 @@ class RMSNorm(Part):
         super().bind(tensors, prefix, dtype, device)
         self.weight = tensors[prefix + "weight"].contiguous()
 
-    def forward(self, residual: torch.Tensor, branch: Optional[torch.Tensor], out_dtype: torch.dtype,
-                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, residual: torch.Tensor, branch, out_dtype: torch.dtype,
+                rows: Optional[torch.Tensor] = None, lazy: bool = False):
+        """``branch`` is a tensor still to be added into ``residual``, ``None``, or a
+        ``RowSumsq`` (already added; the rows' sums of squares are known).  With
+        ``lazy`` and a ``RowSumsq`` nothing runs here: the consumer's product
+        normalises its operand itself."""
+        if isinstance(branch, RowSumsq):
+            if lazy and rows is None:
+                return LazyNorm(residual, branch.sumsq, self.weight, self.eps, out_dtype)
+            branch = None
         return ops.add_rmsnorm(residual, branch, self.weight, self.eps, out_dtype, rows=rows)
 
 

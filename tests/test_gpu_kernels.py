@@ -425,3 +425,89 @@ def test_sample_frequencies(ops):
     freq = torch.bincount(got.long().cpu(), minlength=4).double() / 4000
     expect = torch.softmax(torch.tensor([0.0, 1.0, 2.0, -1.0]).double() / 0.8, dim=0)
     assert (freq - expect).abs().max() < 0.03
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 128), (8, 2560, 2048), (16, 96, 328), (17, 208, 1032), (40, 64, 264),
+                                   (64, 2048, 1408), (70, 48, 96)])
+@pytest.mark.parametrize("plan", [None, "one", "many", "half"])
+def test_gemm_fused_epilogues(ops, shape, plan):
+    """The fused few-row product: plain (bf16 / float32, with bias), SiLU-gate
+    and residual-accumulate epilogues, with one wave per workgroup and with as
+    many as are built (their partial tiles summed through LDS), against float64 products."""
+    m, n, k = shape
+    row_tiles = 1 if m <= 16 else 2 if m <= 32 else 4
+    if plan == "half" and row_tiles != 1:
+        pytest.skip("8-column workgroups exist for one row tile only")
+    chosen = {None: None, "one": (row_tiles, 1, 0), "many": (row_tiles, 16 // row_tiles, 0), "half": (1, 4, 1)}[plan]
+    halved = chosen[2] if chosen else ops.plan_fused(m, n // 16, k)[2]
+    cols = 8 if halved else 16
+    a, w, b = rand((m, k), torch.bfloat16, 80), rand((n, k), torch.bfloat16, 81, 0.3), rand((n,), torch.bfloat16, 82)
+    exact = a.double() @ w.double().t()
+    atol = 2e-4 * math.sqrt(k)
+    out = ops.gemm_fused(w, ops.EPI_F32, a=a, bias=b, plan=chosen)
+    torch.testing.assert_close(out.double(), exact + b.double(), rtol=1e-4, atol=atol)
+    out = ops.gemm_fused(w, ops.EPI_BF16, a=a, plan=chosen)
+    torch.testing.assert_close(out.double(), exact, rtol=1e-2, atol=1e-2 * math.sqrt(k) * 0.3)
+    if n % 32 == 0:
+        gate, up = exact[:, : n // 2], exact[:, n // 2:]
+        out = ops.gemm_fused(w, ops.EPI_SILU, a=a, plan=None if plan == "half" else chosen)
+        assert out.shape == (m, n // 2)
+        want = torch.nn.functional.silu(gate) * up
+        torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()))
+    residual = rand((m, n), torch.float32, 83, 2.0)
+    before = residual.clone()
+    sumsq = torch.full((m + 2, n // cols), float("nan")).cuda()
+    assert ops.gemm_fused(w, ops.EPI_RESID, a=a, residual_out=residual, sumsq_out=sumsq, plan=chosen) is sumsq
+    want = before.double() + exact
+    torch.testing.assert_close(residual.double(), want, rtol=1e-4, atol=atol)
+    torch.testing.assert_close(sumsq[:m].double(), want.pow(2).view(m, n // cols, cols).sum(-1), rtol=1e-4, atol=1e-3)
+    assert torch.isnan(sumsq[m:]).all()
+
+
+@pytest.mark.parametrize("norm_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 64, 128), (8, 320, 2048), (16, 96, 328), (33, 64, 264), (64, 128, 1408)])
+def test_gemm_fused_norm_prologue(ops, shape, norm_dtype):
+    """RMSNorm folded into the product's A operand: equals norm kernel followed by the plain product."""
+    m, n, k = shape
+    residual = rand((m, k), torch.float32, 84, 3.0)
+    norm_w = (rand((k,), torch.float32, 85) + 1).to(norm_dtype)
+    w = rand((n, k), torch.bfloat16, 86, 0.2)
+    eps = 1e-5
+    parts = 7
+    # any split of the row's sum of squares into parts must give the same norm
+    full = residual.pow(2).sum(-1, keepdim=True)
+    shares = torch.softmax(rand((m, parts), torch.float32, 87), dim=-1)
+    sumsq = (full * shares).contiguous()
+    normed = ops.add_rmsnorm(residual.clone(), None, norm_w, eps, torch.bfloat16)
+    want = ops.gemm_fused(w, ops.EPI_F32, a=normed)
+    for plan in (None, (1 if m <= 16 else 2 if m <= 32 else 4, 4, 0)):
+        got = ops.gemm_fused(w, ops.EPI_F32, residual_in=residual, sumsq_in=sumsq, norm_weight=norm_w, eps=eps, plan=plan)
+        # the normalised operand is rounded to bf16 in both; the inverse RMS may differ in its last bit
+        torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
+    exact = (plain_qwen2.rms_norm(residual.cpu(), norm_w.float().cpu(), eps).double() @ w.double().cpu().t())
+    torch.testing.assert_close(got.double().cpu(), exact, rtol=2e-2, atol=2e-2 * float(exact.abs().max()))
+
+
+@pytest.mark.parametrize("norm_dtype", [torch.bfloat16, torch.float32])
+def test_rmsnorm_from_sumsq(ops, norm_dtype):
+    residual = rand((5, 1000), torch.float32, 90, 2.0)
+    weight = (rand((1000,), torch.float32, 91) + 1).to(norm_dtype)
+    full = residual.pow(2).sum(-1, keepdim=True)
+    sumsq = (full * torch.softmax(rand((5, 13), torch.float32, 92), dim=-1)).contiguous()
+    out = ops.rmsnorm_from_sumsq(residual, sumsq, weight, 1e-5)
+    want = plain_qwen2.rms_norm(residual.cpu(), weight.float().cpu(), 1e-5)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(torch.bfloat16))
+
+
+def test_argmax_over_a_large_vocabulary(ops):
+    """Two-stage greedy: chunk edges, ties across chunks (the lower index wins), a vocabulary that is no multiple of the chunk."""
+    vocab = 151936 + 5
+    g = torch.Generator().manual_seed(93)
+    logits = torch.randn((9, vocab), generator=g).cuda()
+    logits[1, vocab - 1] = 50.0
+    logits[2, 0] = 50.0
+    logits[3, 2047] = logits[3, 2048] = 50.0
+    logits[4, 100000] = logits[4, 4096] = 50.0
+    out = ops.sample(logits).tolist()
+    assert out == torch.argmax(logits, dim=-1).tolist()
+    assert out[1:5] == [vocab - 1, 0, 2047, 4096]
