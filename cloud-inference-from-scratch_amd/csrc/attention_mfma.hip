@@ -20,7 +20,9 @@
 //   O[row, d] += P[row, key] * V[key, d]       A = P (bf16), B = V^T rows
 //   The spread of a block's keys (and of a head's dimensions) over the lanes is
 //   the same for both operands of a product, which is all a dot product needs.
-// Scores, running maximum, sums and the output accumulator are float32.
+// Scores, running maximum, sums and the output accumulator are float32.  The softmax runs in base 2:
+// scores are scaled by scale * log2(e) once, so that each probability is one v_exp_f32; the
+// accumulator is rescaled only in blocks where some row's running maximum moved.
 #include "common.h"
 
 namespace {
@@ -29,10 +31,6 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kKeysPerBlock = 32;
-
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    return static_cast<uint32_t>(bf16_bits_from_float(lo)) | (static_cast<uint32_t>(bf16_bits_from_float(hi)) << 16);
-}
 
 struct AttentionArgs {
     const bf16_t* q;
@@ -83,6 +81,7 @@ __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs 
     const int page_size = 1 << a.page_shift;
     const int page_mask = page_size - 1;
     const int* table = a.block_table + static_cast<size_t>(a.seq_slot[seq]) * a.table_width;
+    const float scale_log2 = a.scale * 1.44269504088896341f;
 
     // keys this tile can see at all, and this split's share of them
     const int hi = start + q0 + n_tok;
@@ -174,7 +173,7 @@ __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs 
                 for (int i = 0; i < 4; ++i) {
                     const int key = kb + kt * 16 + g * 4 + i;
                     const bool seen = key <= pos && key >= row_lo && key < range_end;
-                    const float v = seen ? s[rt][kt][i] * a.scale : -INFINITY;
+                    const float v = seen ? s[rt][kt][i] * scale_log2 : -INFINITY;
                     s[rt][kt][i] = v;
                     block_max = fmaxf(block_max, v);
                 }
@@ -183,33 +182,38 @@ __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs 
             block_max = fmaxf(block_max, __shfl_xor(block_max, 32, kWave));
             const float m_new = fmaxf(m_run[rt], block_max);
             const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = __expf(m_run[rt] - m_safe);  // m_run = -inf: 0, and l, O are 0 anyway
+            const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_safe);  // m_run = -inf: 0, and l, O are 0 anyway
+            const bool moved = m_new != m_run[rt];
             m_run[rt] = m_new;
             float p_sum = 0.f;
             uint32_t pw[4];
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
-                const float p0 = __expf(s[rt][kt][0] - m_safe);
-                const float p1 = __expf(s[rt][kt][1] - m_safe);
-                const float p2 = __expf(s[rt][kt][2] - m_safe);
-                const float p3 = __expf(s[rt][kt][3] - m_safe);
+                const float p0 = __builtin_amdgcn_exp2f(s[rt][kt][0] - m_safe);
+                const float p1 = __builtin_amdgcn_exp2f(s[rt][kt][1] - m_safe);
+                const float p2 = __builtin_amdgcn_exp2f(s[rt][kt][2] - m_safe);
+                const float p3 = __builtin_amdgcn_exp2f(s[rt][kt][3] - m_safe);
                 p_sum += (p0 + p1) + (p2 + p3);
                 pw[kt * 2] = pack_bf16(p0, p1);
                 pw[kt * 2 + 1] = pack_bf16(p2, p3);
             }
             l_run[rt] = l_run[rt] * alpha + p_sum;
-            // the accumulator's rows are g*4+i, the statistics' row is r: fetch alpha of those rows
-            float alpha_o[4];
+            // with one row tile (decode) the straight-line form schedules better than the branch
+            if (RT == 1 || __any(moved)) {
+                // the accumulator's rows are g*4+i, the statistics' row is r: fetch alpha of those rows
+                float alpha_o[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha, g * 4 + i, kWave);
+                for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha, g * 4 + i, kWave);
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) o[rt][dt][i] *= alpha_o[i];
+            }
             const bf16x8 p_frag = __builtin_bit_cast(bf16x8, (uint4{pw[0], pw[1], pw[2], pw[3]}));
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) {
-                floatx4 acc = o[rt][dt];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] *= alpha_o[i];
                 const uint4 v = uint4{vf[dt][0].x, vf[dt][0].y, vf[dt][1].x, vf[dt][1].y};
-                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_frag, __builtin_bit_cast(bf16x8, v), acc, 0, 0, 0);
+                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_frag, __builtin_bit_cast(bf16x8, v), o[rt][dt], 0, 0, 0);
             }
         }
     }
@@ -278,7 +282,7 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
     float den_local = 0.f;
     for (int s = threadIdx.x; s < a.n_splits; s += blockDim.x) {
         const float* ml = a.part_ml + ((unit0 + s) * rows_per_tile + row) * 2;
-        const float w = (ml[0] == -INFINITY) ? 0.f : __expf(ml[0] - m_all);
+        const float w = (ml[0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m_all);  // maxima are kept in base 2
         weight[s] = w;
         den_local += ml[1] * w;
     }

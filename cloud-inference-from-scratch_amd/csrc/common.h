@@ -37,6 +37,15 @@ __device__ __forceinline__ uint16_t bf16_bits_from_float(float x) {
     return static_cast<uint16_t>(u >> 16);
 }
 
+// Two floats to two bfloat16 in one word (low half first), round to nearest even: on gfx950 this is
+// the v_cvt_pk_bf16_f32 instruction.
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float floatx2_t __attribute__((ext_vector_type(2)));
+    const floatx2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 template <typename T>
 __device__ __forceinline__ T from_float(float x);
 template <>
@@ -46,7 +55,7 @@ __device__ __forceinline__ float from_float<float>(float x) {
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float x) {
     bf16_t r;
-    r.bits = bf16_bits_from_float(x);
+    r.bits = static_cast<uint16_t>(pack_bf16(x, 0.f) & 0xffffu);
     return r;
 }
 

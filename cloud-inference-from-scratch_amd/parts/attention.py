@@ -144,7 +144,14 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
                                  n_tiles, *common, tokens_per_tile=1, row_tiles=1, n_splits=n_splits,
                                  keys_per_split=per_split, part_o=part_o, part_ml=part_ml)
-    row_tiles = 2 if head_dim > 128 else 4  # 64 rows per wave; 32 where the accumulators would spill
+    # rows per wave: 64 share each key load best; fewer where that would leave SIMDs without a wave
+    # (about a thousand waves fill the GPU) or where the accumulators of a wide head would spill
+    row_tiles = 2 if head_dim > 128 else 4
+    prompt_tokens = sum(n for n in batch.host_q_lens if n > 1)
+    while row_tiles > 1 and (prompt_tokens * group // (16 * row_tiles)) * num_kv_heads < 1024:
+        row_tiles //= 2
+    while 16 * row_tiles < group:
+        row_tiles *= 2
     per_tile = (16 * row_tiles) // group
     tile_seq, tile_q0, n_tiles = batch.tiles(per_tile, decode=False)
     if n_tiles:
