@@ -14,6 +14,10 @@
 //             SILU   W stacks gate rows over up rows: C[m,n] = silu(acc_gate) * acc_up, bf16
 //             RESID  residual[m,n] += acc (float32, in place) and the partial sums of
 //                    squares of the new residual rows are written for the next NORM.
+//             PARTIAL  K is cut into grid.z parts, each workgroup writes its float32 partial
+//                    product to C[part, m, n]; the consumer (the add + norm kernel) sums the
+//                    parts.  For products with few columns and a long K, where one
+//                    workgroup per column tile cannot pull the weight fast enough.
 //
 // Work split: one workgroup owns NT tiles of 16 columns (NT = 2 only for SILU:
 // a gate tile and its up tile) and all rows; its WAVES waves cut K into slices of
@@ -31,7 +35,7 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-enum { EPI_PLAIN_BF16 = 0, EPI_PLAIN_F32 = 1, EPI_SILU = 2, EPI_RESID = 3 };
+enum { EPI_PLAIN_BF16 = 0, EPI_PLAIN_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4 };
 
 struct FusedArgs {
     // A: either a bf16 matrix, or residual + norm
@@ -50,6 +54,7 @@ struct FusedArgs {
     float* sumsq_out;           // RESID: [M, N/16]
     int M, N, K;
     int second_tile_offset;     // rows of W between a workgroup's first and second tile (NT == 2)
+    int k_per_part;             // PARTIAL: k values per grid.z part (a multiple of 128); otherwise K
 };
 
 template <int WAVES, int MT, int NT, int EPI, bool NORM, bool HALF>
@@ -93,7 +98,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_fused_kernel(FusedArgs a) {
     // U slices of 128 k values are in flight per wave: the loads of all of them are issued before the
     // first matrix product, which is what keeps enough bytes in flight to cover the memory latency
     constexpr int U = (MT == 1) ? (NT == 1 ? 4 : 2) : 1;
-    for (int kbase = wave * 128; kbase < a.K; kbase += U * WAVES * 128) {
+    const int k_begin = blockIdx.z * a.k_per_part;
+    const int k_end = min(a.K, k_begin + a.k_per_part);
+    for (int kbase = k_begin + wave * 128; kbase < k_end; kbase += U * WAVES * 128) {
         uint4 b[U][NT][4];
 #pragma unroll
         for (int u = 0; u < U; ++u)
@@ -104,7 +111,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_fused_kernel(FusedArgs a) {
                     const int k0 = kbase + u * WAVES * 128;
                     // the four lane groups read one contiguous 64-byte piece of each row per load
                     const int k = k0 + j * 32 + g * 8;
-                    b[u][t][j] = (k < a.K) ? *reinterpret_cast<const uint4*>(w_row[t] + k0 + j * 32) : uint4{0, 0, 0, 0};
+                    b[u][t][j] = (k < k_end) ? *reinterpret_cast<const uint4*>(w_row[t] + k0 + j * 32) : uint4{0, 0, 0, 0};
                 }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -117,7 +124,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_fused_kernel(FusedArgs a) {
                 for (int j = 0; j < 4; ++j) {
                     const int k = k0 + j * 32 + g * 8;
                     av[j] = uint4{0, 0, 0, 0};
-                    if (m < a.M && k < a.K) {
+                    if (m < a.M && k < k_end) {
                         if (NORM) {
                             const float* src = a.residual_in + static_cast<size_t>(m) * a.K + k;
                             const float4 x0 = *reinterpret_cast<const float4*>(src);
@@ -205,7 +212,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_fused_kernel(FusedArgs a) {
             }
         } else {
             const int n = n_first + r;
-            const float add = a.bias ? to_float(a.bias[n]) : 0.f;
+            const float add = (a.bias && blockIdx.z == 0) ? to_float(a.bias[n]) : 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int m = m0 + mt * 16 + g * 4 + i;
@@ -227,7 +234,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_fused_kernel(FusedArgs a) {
                     if (!HALF) sq += __shfl_xor(sq, 8, kWave);
                     if (r == 0 && ok) a.sumsq_out[static_cast<size_t>(m) * (a.N / TILE_N) + blockIdx.x] = sq;
                 } else if (ok) {
-                    if (EPI == EPI_PLAIN_F32)
+                    if (EPI == EPI_PARTIAL)
+                        static_cast<float*>(a.c)[(static_cast<size_t>(blockIdx.z) * a.M + m) * a.N + n] = v;
+                    else if (EPI == EPI_PLAIN_F32)
                         static_cast<float*>(a.c)[static_cast<size_t>(m) * a.N + n] = v;
                     else
                         static_cast<bf16_t*>(a.c)[static_cast<size_t>(m) * a.N + n] = from_float<bf16_t>(v);
@@ -281,13 +290,15 @@ int launch_rows(hipStream_t s, int mt, int waves, dim3 grid, const FusedArgs& a,
 
 }  // namespace
 
-// epilogue: 0 bf16 out, 1 float32 out, 2 SiLU-gate (W = [gate rows; up rows], N = 2 * outputs), 3 residual accumulate.
+// epilogue: 0 bf16 out, 1 float32 out, 2 SiLU-gate (W = [gate rows; up rows], N = 2 * outputs), 3 residual accumulate,
+// 4 partial products of k_parts parts of K to c[k_parts, M, N] (float32).
 // row_tiles: 16-row tiles per workgroup (1, 2 or 4); waves: waves per workgroup that share K (1, 2, 4, 8, 16).
 // half_tiles: workgroups of 8 columns instead of 16 (row_tiles 1, not SiLU); sumsq_out is then [M, N/8].
 CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const float* residual_in,
                            const float* sumsq_in, int parts_in, const void* norm_w, int norm_w_f32, float eps,
                            const void* w, const void* bias, void* c, float* residual_out, float* sumsq_out,
-                           int M, int N, int K, int epilogue, int row_tiles, int waves, int half_tiles) {
+                           int M, int N, int K, int epilogue, int row_tiles, int waves, int half_tiles,
+                           int k_parts) {
     const bool norm = residual_in != nullptr;
     if (M <= 0 || N <= 0 || K <= 0 || K % 8 || N % 16) return CIE_BAD_ARGUMENT;
     if (!norm && (!a || lda < K || lda % 8)) return CIE_BAD_ARGUMENT;
@@ -295,7 +306,9 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const float* re
     if (row_tiles != 1 && row_tiles != 2 && row_tiles != 4) return CIE_BAD_ARGUMENT;
     if (epilogue == EPI_SILU && (N % 32 || bias)) return CIE_BAD_ARGUMENT;
     if (epilogue == EPI_RESID && (!residual_out || !sumsq_out)) return CIE_BAD_ARGUMENT;
-    if ((epilogue == EPI_PLAIN_BF16 || epilogue == EPI_PLAIN_F32 || epilogue == EPI_SILU) && !c) return CIE_BAD_ARGUMENT;
+    if ((epilogue == EPI_PLAIN_BF16 || epilogue == EPI_PLAIN_F32 || epilogue == EPI_SILU || epilogue == EPI_PARTIAL) && !c)
+        return CIE_BAD_ARGUMENT;
+    if (k_parts < 1 || k_parts > 64 || (k_parts > 1 && epilogue != EPI_PARTIAL)) return CIE_BAD_ARGUMENT;
     const int m_blocks = (M + 16 * row_tiles - 1) / (16 * row_tiles);
     if (m_blocks > 65535) return CIE_BAD_ARGUMENT;
     FusedArgs f;
@@ -315,6 +328,7 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const float* re
     f.M = M;
     f.N = N;
     f.K = K;
+    f.k_per_part = ((K + k_parts - 1) / k_parts + 127) / 128 * 128;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (epilogue == EPI_SILU) {
         f.second_tile_offset = N / 2;
@@ -322,11 +336,12 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const float* re
     }
     f.second_tile_offset = 0;
     const bool half = half_tiles != 0;
-    dim3 grid(N / (half ? 8 : 16), m_blocks);
+    dim3 grid(N / (half ? 8 : 16), m_blocks, k_parts);
     switch (epilogue) {
         case EPI_PLAIN_BF16: return launch_rows<1, EPI_PLAIN_BF16>(s, row_tiles, waves, grid, f, norm, half);
         case EPI_PLAIN_F32: return launch_rows<1, EPI_PLAIN_F32>(s, row_tiles, waves, grid, f, norm, half);
         case EPI_RESID: return launch_rows<1, EPI_RESID>(s, row_tiles, waves, grid, f, norm, half);
+        case EPI_PARTIAL: return launch_rows<1, EPI_PARTIAL>(s, row_tiles, waves, grid, f, norm, half);
     }
     return CIE_BAD_ARGUMENT;
 }

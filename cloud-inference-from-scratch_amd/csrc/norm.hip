@@ -38,11 +38,61 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __rest
         dst[h] = from_float<T>((staged[h] * inv) * to_float(weight[h]));
 }
 
+// The same, with the branch given as `n_parts` float32 partial products [n_parts, rows_total, hidden]
+// (left by a product whose K was cut into parts): residual += sum of the parts, then the norm.
+template <typename W>
+__global__ void add_parts_rmsnorm_kernel(float* __restrict__ residual, const float* __restrict__ parts,
+                                         int n_parts, int rows_total, const W* __restrict__ weight,
+                                         bf16_t* __restrict__ out, const int* __restrict__ rows, int hidden,
+                                         float eps, int write_residual) {
+    extern __shared__ float staged[];
+    __shared__ float scratch[16];
+    const int out_row = blockIdx.x;
+    const int row = rows ? rows[out_row] : out_row;
+    float* res = residual + static_cast<size_t>(row) * hidden;
+    float sum_sq = 0.f;
+    for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
+        float x = res[h];
+        for (int p = 0; p < n_parts; ++p) x += parts[(static_cast<size_t>(p) * rows_total + row) * hidden + h];
+        if (write_residual) res[h] = x;
+        staged[h] = x;
+        sum_sq += x * x;
+    }
+    const float total = block_sum(sum_sq, scratch);
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    bf16_t* dst = out + static_cast<size_t>(out_row) * hidden;
+    for (int h = threadIdx.x; h < hidden; h += blockDim.x)
+        dst[h] = from_float<bf16_t>((staged[h] * inv) * to_float(weight[h]));
+}
+
+CIE_API int cie_add_parts_rmsnorm(void* stream, int wdtype, float* residual, const float* parts, int n_parts,
+                                  int rows_total, const void* weight, void* out, const int* rows, int n_out,
+                                  int hidden, float eps, int write_residual) {
+    if (n_out < 0 || hidden <= 0 || hidden * sizeof(float) > 64 * 1024 || !(eps > 0.f) || n_parts < 1 || rows_total < 1)
+        return CIE_BAD_ARGUMENT;
+    if (rows && write_residual) return CIE_BAD_ARGUMENT;
+    if (n_out == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // few rows (a decode step): a row's loads are spread over 1024 threads so that they all travel at once
+    const int threads = n_out <= 64 ? 1024 : 256;
+    if (wdtype == CIE_BF16)
+        add_parts_rmsnorm_kernel<bf16_t><<<n_out, threads, hidden * sizeof(float), s>>>(
+            residual, parts, n_parts, rows_total, static_cast<const bf16_t*>(weight), static_cast<bf16_t*>(out), rows,
+            hidden, eps, write_residual);
+    else if (wdtype == CIE_F32)
+        add_parts_rmsnorm_kernel<float><<<n_out, threads, hidden * sizeof(float), s>>>(
+            residual, parts, n_parts, rows_total, static_cast<const float*>(weight), static_cast<bf16_t*>(out), rows,
+            hidden, eps, write_residual);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
 template <typename T, typename W>
 static int launch_norm(hipStream_t s, float* residual, const void* branch, const void* weight,
                        void* out, const int* rows, int n_out, int hidden, float eps,
                        int write_residual) {
-    add_rmsnorm_kernel<T, W><<<n_out, 256, hidden * sizeof(float), s>>>(
+    add_rmsnorm_kernel<T, W><<<n_out, n_out <= 64 ? 1024 : 256, hidden * sizeof(float), s>>>(
         residual, static_cast<const T*>(branch), static_cast<const W*>(weight), static_cast<T*>(out),
         rows, hidden, eps, write_residual);
     return cie_after_launch();

@@ -128,6 +128,26 @@ def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: 
     return out
 
 
+def add_parts_rmsnorm(residual: torch.Tensor, parts: torch.Tensor, weight: torch.Tensor, eps: float,
+                      rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``residual += parts.sum(0)`` (written back unless ``rows``), then bf16 RMSNorm; parts float32 [P, T, H]."""
+    _gpu("residual", residual, torch.float32, 2)
+    tokens, hidden = residual.shape
+    _gpu("parts", parts, torch.float32, 3)
+    _require(parts.shape[1:] == residual.shape, f"parts {tuple(parts.shape)} vs residual {tuple(residual.shape)}")
+    _gpu("weight", weight, dims=1)
+    _require(weight.shape[0] == hidden and weight.dtype in (torch.bfloat16, torch.float32), "norm weight does not fit")
+    _require(hidden * 4 <= 64 * 1024 and eps > 0, f"hidden {hidden} or eps {eps} out of range")
+    if rows is not None:
+        _gpu("rows", rows, torch.int32, 1)
+    n_out = rows.shape[0] if rows is not None else tokens
+    out = torch.empty((n_out, hidden), dtype=torch.bfloat16, device=residual.device)
+    _run("cie_add_parts_rmsnorm", load_library().cie_add_parts_rmsnorm(
+        _stream(), _i(_code(weight.dtype)), _ptr(residual), _ptr(parts), _i(parts.shape[0]), _i(tokens), _ptr(weight),
+        _ptr(out), _ptr(rows), _i(n_out), _i(hidden), _f(eps), _i(0 if rows is not None else 1)))
+    return out
+
+
 def rmsnorm_from_sumsq(residual: torch.Tensor, sumsq: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """bf16 RMSNorm of float32 rows whose partial sums of squares ``sumsq`` [rows, parts] are known."""
     _gpu("residual", residual, torch.float32, 2)
@@ -326,11 +346,11 @@ def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor
     return out
 
 
-EPI_BF16, EPI_F32, EPI_SILU, EPI_RESID = 0, 1, 2, 3
+EPI_BF16, EPI_F32, EPI_SILU, EPI_RESID, EPI_PARTIAL = 0, 1, 2, 3, 4
 FUSED_TARGET_WAVES = 2048
 
 
-FUSED_HALF_BELOW = 256  # fewer 16-column workgroups than this: use 8-column workgroups
+FUSED_HALF_BELOW = 0  # fewer 16-column workgroups than this: use 8-column workgroups (measured: no gain on MI355X)
 
 
 def plan_fused(rows: int, column_tiles: int, k: int, may_halve: bool = True) -> tuple[int, int, int]:
@@ -351,7 +371,8 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: Optional[torch.Tensor] = 
                residual_in: Optional[torch.Tensor] = None, sumsq_in: Optional[torch.Tensor] = None,
                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
                bias: Optional[torch.Tensor] = None, residual_out: Optional[torch.Tensor] = None,
-               sumsq_out: Optional[torch.Tensor] = None, plan: Optional[tuple[int, int, int]] = None
+               sumsq_out: Optional[torch.Tensor] = None, plan: Optional[tuple[int, int, int]] = None,
+               k_parts: int = 1
                ) -> Optional[torch.Tensor]:
     """Few-row matrix product ``A @ weight.T`` fused with its neighbours.
 
@@ -367,8 +388,9 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: Optional[torch.Tensor] = 
     _require(k % 8 == 0 and n % 16 == 0, f"gemm_fused needs K % 8 == 0 and N % 16 == 0, got N={n}, K={k}")
     device = weight.device
     rows = (residual_in if residual_in is not None else a).shape[0]
-    row_tiles, waves, half = plan or plan_fused(rows, (n // 2 if epilogue == EPI_SILU else n) // 16, k,
-                                                may_halve=epilogue != EPI_SILU)
+    _require(1 <= k_parts <= 64 and (k_parts == 1 or epilogue == EPI_PARTIAL), f"k_parts {k_parts} does not fit the epilogue")
+    row_tiles, waves, half = plan or plan_fused(rows, (n // 2 if epilogue == EPI_SILU else n) // 16 * k_parts,
+                                                -(-k // k_parts), may_halve=epilogue != EPI_SILU and k_parts == 1)
     _require(waves in (1, 2, 4, 8, 16) and waves * row_tiles <= 16, f"plan {(row_tiles, waves, half)} is not built")
     _require(not half or (row_tiles == 1 and epilogue != EPI_SILU), "8-column workgroups need one row tile and no SiLU")
     if residual_in is not None:
@@ -397,6 +419,8 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: Optional[torch.Tensor] = 
         out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
     elif epilogue == EPI_F32:
         out = torch.empty((m, n), dtype=torch.float32, device=device)
+    elif epilogue == EPI_PARTIAL:
+        out = torch.empty((k_parts, m, n), dtype=torch.float32, device=device)
     elif epilogue == EPI_SILU:
         _require(n % 32 == 0, f"the SiLU epilogue needs N % 32 == 0, got {n}")
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=device)
@@ -417,7 +441,7 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: Optional[torch.Tensor] = 
         _i(sumsq_in.shape[1] if sumsq_in is not None else 0), _ptr(norm_weight),
         _i(1 if norm_weight is not None and norm_weight.dtype == torch.float32 else 0), _f(eps), _ptr(weight),
         _ptr(bias), _ptr(None if epilogue == EPI_RESID else out), _ptr(residual_out), _ptr(sumsq_out), _i(m), _i(n), _i(k), _i(epilogue),
-        _i(row_tiles), _i(waves), _i(half)))
+        _i(row_tiles), _i(waves), _i(half), _i(k_parts)))
     return out
 
 

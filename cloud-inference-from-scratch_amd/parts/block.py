@@ -18,7 +18,7 @@ import torch
 from ..config.specs import LayerSpec
 from ..weights.tensors import TensorSpec
 from .base import build_part, register_part
-from .linear import RowSumsq
+from .linear import PartialSum, RowSumsq
 
 
 class PreNormBlock:
@@ -65,6 +65,9 @@ def normalise(norm, residual: torch.Tensor, pending, dtype: torch.dtype, consume
     """Run ``norm`` on the residual stream plus what is pending.  Only a norm that
     says so is shown a ``RowSumsq`` or asked to stay lazy; any other gets ``None``
     for a branch that was already added."""
+    if isinstance(pending, PartialSum) and not getattr(norm, "takes_row_sumsq", False):
+        residual.add_(pending.parts.sum(0))
+        pending = None
     if isinstance(pending, RowSumsq):
         if not getattr(norm, "takes_row_sumsq", False):
             pending = None

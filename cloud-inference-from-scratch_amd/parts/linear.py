@@ -20,6 +20,10 @@ from ..kernels import ops
 
 # Rows up to which the hand-written fused bf16 kernel replaces the library product.
 FUSED_ROWS = 16
+# An ``into=`` product with fewer than this many 16-column tiles and K of at least 2 * PART_K cuts K
+# into parts of about PART_K for more workgroups (partial products, summed by the next norm kernel).
+PART_BELOW_TILES = 512
+PART_K = 2752
 # Fold a pending RMSNorm into the product's operand.  Measured on MI355X it loses: every workgroup
 # re-reads and re-normalises the same few rows, and those reads pile up on a few cache channels; a
 # separate small norm kernel from the known sums of squares is faster.  Kept for experiments.
@@ -33,6 +37,14 @@ class RowSumsq:
     the residual's rows (what an RMSNorm needs of them)."""
 
     sumsq: torch.Tensor
+
+
+@dataclass
+class PartialSum:
+    """Stands where a branch output would: float32 partial products ``parts``
+    [P, rows, hidden] whose sum is the branch (a product whose K was cut)."""
+
+    parts: torch.Tensor
 
 
 @dataclass
@@ -64,14 +76,15 @@ def _fusable(rows: int, weight: torch.Tensor, silu: bool) -> bool:
 
 def linear(x: Union[torch.Tensor, LazyNorm], weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None, epilogue: Optional[str] = None,
-           into: Optional[torch.Tensor] = None) -> Union[torch.Tensor, RowSumsq]:
+           into: Optional[torch.Tensor] = None) -> Union[torch.Tensor, RowSumsq, PartialSum]:
     """``x @ weight.T + bias``.
 
     ``epilogue="silu"``: weight stacks gate rows over up rows; returns
     ``silu(gate) * up``.  ``into=residual``: the caller wants the result added to
     the float32 residual stream; if the fused kernel runs it adds it in place and
-    a :class:`RowSumsq` comes back, otherwise the plain result comes back and the
-    caller adds it (the next norm kernel does)."""
+    a :class:`RowSumsq` comes back (or a :class:`PartialSum` of partial products
+    that the next norm kernel adds), otherwise the plain result comes back and
+    the caller adds it (the next norm kernel does)."""
     rows = x.shape[0]
     silu = epilogue == "silu"
     if _fusable(rows, weight, silu):
@@ -80,6 +93,9 @@ def linear(x: Union[torch.Tensor, LazyNorm], weight: torch.Tensor, bias: Optiona
         source = (dict(residual_in=x.residual, sumsq_in=x.sumsq, norm_weight=x.weight, eps=x.eps)
                   if isinstance(x, LazyNorm) else dict(a=x))
         if into is not None:
+            n, k = weight.shape
+            if n // 16 < PART_BELOW_TILES and k >= 2 * PART_K:
+                return PartialSum(ops.gemm_fused(weight, ops.EPI_PARTIAL, bias=bias, k_parts=-(-k // PART_K), **source))
             return RowSumsq(ops.gemm_fused(weight, ops.EPI_RESID, bias=bias, residual_out=into, **source))
         kind = ops.EPI_SILU if silu else ops.EPI_F32 if out_dtype == torch.float32 else ops.EPI_BF16
         return ops.gemm_fused(weight, kind, bias=bias, **source)

@@ -488,6 +488,31 @@ def test_gemm_fused_norm_prologue(ops, shape, norm_dtype):
     torch.testing.assert_close(got.double().cpu(), exact, rtol=2e-2, atol=2e-2 * float(exact.abs().max()))
 
 
+@pytest.mark.parametrize("shape", [(1, 64, 256), (8, 2048, 11008), (13, 96, 328), (16, 48, 1032)])
+@pytest.mark.parametrize("k_parts", [1, 3, 4])
+def test_gemm_fused_partial_products_and_their_norm(ops, shape, k_parts):
+    """K cut into parts: the float32 partial products sum to the product (bias once), and the
+    add-parts norm kernel equals adding that product into the residual and normalising."""
+    m, n, k = shape
+    a, w, b = rand((m, k), torch.bfloat16, 94), rand((n, k), torch.bfloat16, 95, 0.3), rand((n,), torch.bfloat16, 96)
+    parts = ops.gemm_fused(w, ops.EPI_PARTIAL, a=a, bias=b, k_parts=k_parts)
+    assert parts.shape == (k_parts, m, n) and parts.dtype == torch.float32
+    exact = a.double() @ w.double().t() + b.double()
+    torch.testing.assert_close(parts.double().sum(0), exact, rtol=1e-4, atol=2e-4 * math.sqrt(k))
+    residual = rand((m, n), torch.float32, 97, 2.0)
+    weight = rand((n,), torch.bfloat16, 98) + 1
+    want_residual = residual.double() + parts.double().sum(0)
+    want = plain_qwen2.rms_norm(want_residual.float().cpu(), weight.float().cpu(), 1e-6)
+    rows = torch.tensor([m - 1, 0], dtype=torch.int32).cuda()
+    before = residual.clone()
+    picked = ops.add_parts_rmsnorm(residual, parts, weight, 1e-6, rows=rows)
+    assert torch.equal(residual, before)
+    torch.testing.assert_close(picked.float().cpu(), want[rows.long().cpu()], **tol(torch.bfloat16))
+    out = ops.add_parts_rmsnorm(residual, parts, weight, 1e-6)
+    torch.testing.assert_close(residual.double(), want_residual, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("norm_dtype", [torch.bfloat16, torch.float32])
 def test_rmsnorm_from_sumsq(ops, norm_dtype):
     residual = rand((5, 1000), torch.float32, 90, 2.0)

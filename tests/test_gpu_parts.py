@@ -157,10 +157,16 @@ def test_attention_part_whole_and_in_portions(dtype, rotary):
     check(torch.cat([first, second, third, fourth]).float().cpu(), expected[1], dtype)
 
 
+@pytest.mark.parametrize("part_k", [None, 32])
 @pytest.mark.parametrize("rows", [13, 40])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_block_part(dtype, rows):
-    """norm -> mixer -> add -> norm -> feed-forward, the add of the second branch left pending."""
+def test_block_part(dtype, rows, part_k, monkeypatch):
+    """norm -> mixer -> add -> norm -> feed-forward, the add of the second branch left pending
+    (as a tensor, as partial products, or already done, depending on rows and dtype)."""
+    if part_k is not None:
+        from cie_amd.parts import linear
+
+        monkeypatch.setattr(linear, "PART_K", part_k)
     from cie_amd.config import Qwen2Config
     from cie_amd.parts.block import PreNormBlock
 
@@ -180,9 +186,12 @@ def test_block_part(dtype, rows):
     mid = h + plain.attention_layer(a, w, p + "self_attn.", raw, cos, sin, torch.arange(rows))
     m = plain.rms_norm(mid, w[p + "post_attention_layernorm.weight"], 1e-5)
     branch = plain.swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
-    from cie_amd.parts.linear import RowSumsq
+    from cie_amd.parts.linear import PartialSum, RowSumsq
 
-    if isinstance(pending, RowSumsq):  # few rows in bfloat16: the fused products added both branches themselves
+    if isinstance(pending, PartialSum):  # the last product left its K in parts for the next norm to add
+        check(out_residual.cpu(), mid, dtype)
+        check(pending.parts.sum(0).cpu(), branch, dtype)
+    elif isinstance(pending, RowSumsq):  # few rows in bfloat16: the fused products added both branches themselves
         check(out_residual.cpu(), mid + branch, dtype)
         check(pending.sumsq.sum(-1).cpu(), (mid + branch).pow(2).sum(-1), dtype)
     else:

@@ -108,6 +108,21 @@ def test_captured_decode_steps_match_plain(tiny_folders, plain, name, dtype):
         print(f"{name} {schedule} {dtype}: {runner.graph_captures} captures, {runner.graph_replays} replays", flush=True)
 
 
+@pytest.mark.parametrize("graph", [False, True])
+def test_products_cut_along_k_match_plain(tiny_folders, plain, monkeypatch, graph):
+    """The decode products that cut a long K into parts (summed by the next norm
+    kernel) only engage at sizes the tiny models do not have; force them."""
+    from cie_amd.parts import linear
+
+    monkeypatch.setattr(linear, "PART_K", 128)  # Tiny-B's down product has K = 328: three parts
+    folder, raw, _ = tiny_folders["B"]
+    requests, expected = plain["B"]
+    steps = replay_util.mixed(requests, live=4, decode_tail=30, seed=6)
+    runner = make_runner(folder, "bfloat16", replay_util.max_live_tokens(steps, page=8), 8, graph_decode=graph)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    replay_util.compare(rows, expected, **TOL["bfloat16"])
+
+
 def test_mixed_reuses_pages(tiny_folders, plain):
     """The mixed schedule runs in a pool smaller than the sum of all requests."""
     _, raw, _ = tiny_folders["B"]
