@@ -1,33 +1,31 @@
-// Decode-step matrix products on the matrix cores, fused with what surrounds them.
+// Matrix products for steps with few rows (decode steps, the output head), on the
+// matrix cores, fused with the small operations around them.
 //
-//   C = A * W^T     A [M, K] with few rows (M <= 64 per workgroup row), W [N, K] bf16
+//   C = A * W^T     A [M, K] bf16 with few rows, W [N, K] bf16 (a Linear's weight), float32 sums
 //
-// A step with few tokens is bound by streaming W once and by the number of
-// kernel launches, so this kernel takes over its neighbours' work:
+// Such a product is bound by streaming W once and by the number of kernel launches
+// (no kernel on this GPU finishes in under about 5 microseconds), so the epilogue
+// takes over the neighbour's work:
+//   BF16 / F32  C[m,n] = acc + bias[n]
+//   SILU        W stacks gate rows over up rows: C[m,n] = silu(acc_gate) * acc_up, bf16
+//   RESID       residual[m,n] += acc + bias[n] (float32, in place), and the partial sums of
+//               squares of the new residual row (one per 16 columns) are written, so that the
+//               RMSNorm that follows needs no reduction over the row
+//   PARTIAL     K is cut into grid.z parts; part p writes acc to C[p, m, n] (float32, bias in
+//               part 0).  The add + norm kernel sums the parts.  For few columns and long K.
 //
-//   prologue  NORM   A is not given; it is made on the fly from the float32
-//                    residual stream: A[m,k] = bf16(residual[m,k] * inv_rms[m] * norm_w[k]),
-//                    inv_rms[m] = 1/sqrt(sum_p sumsq[m,p] / K + eps), where sumsq holds
-//                    partial sums of squares of the row that the producer of the
-//                    residual left (one per 16 columns).
-//   epilogue  PLAIN  C[m,n] = acc + bias[n], bf16 or float32
-//             SILU   W stacks gate rows over up rows: C[m,n] = silu(acc_gate) * acc_up, bf16
-//             RESID  residual[m,n] += acc (float32, in place) and the partial sums of
-//                    squares of the new residual rows are written for the next NORM.
-//             PARTIAL  K is cut into grid.z parts, each workgroup writes its float32 partial
-//                    product to C[part, m, n]; the consumer (the add + norm kernel) sums the
-//                    parts.  For products with few columns and a long K, where one
-//                    workgroup per column tile cannot pull the weight fast enough.
-//
-// Work split: one workgroup owns NT tiles of 16 columns (NT = 2 only for SILU:
-// a gate tile and its up tile) and all rows; its WAVES waves cut K into slices of
-// 128 and take them round-robin.  Every lane streams its W row(s) with 16-byte
-// loads straight into B operands of v_mfma_f32_16x16x32_bf16 and loads (or
-// makes) its own row of A for the same k values; nothing is shared until the
-// end, when the waves' partial tiles are summed through LDS in wave order and
-// wave 0 runs the epilogue.  No workgroup ever waits for another one: on this
-// GPU a device-wide fence between workgroups costs more than the whole product.
-// Sums are float32 throughout.
+// Two kernels:
+//   rows16  M <= 16.  One workgroup per tile of 16 columns (SILU: a gate tile and its up tile);
+//           its WAVES waves cut K into slices of 128 and take them round-robin; every lane
+//           loads its own row of A and of W for the same k values straight into MFMA
+//           operands; the waves' partial tiles are summed through LDS in wave order.
+//   rows64  M <= 64 per workgroup.  Four waves own four column tiles and share the slice of A
+//           that all threads stage in LDS; every lane streams its row of W.
+// Both use v_mfma_f32_16x16x32_bf16 with A = activations (16 rows), B = weight rows; the four
+// lane groups of a wave read one contiguous 64-byte piece of each weight row per load, and the
+// same k values of A (the order of k inside a product is free as long as both operands agree).
+// No workgroup ever waits for another: a device-wide fence between workgroups costs more on
+// this GPU than the whole product.
 #include "common.h"
 
 namespace {
@@ -35,69 +33,91 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-enum { EPI_PLAIN_BF16 = 0, EPI_PLAIN_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4 };
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4 };
 
 struct FusedArgs {
-    // A: either a bf16 matrix, or residual + norm
-    const bf16_t* a;
+    const bf16_t* a;       // [M, K], row stride lda
     int lda;
-    const float* residual_in;   // [M, K] float32 (NORM)
-    const float* sumsq_in;      // [M, parts_in]
-    int parts_in;
-    const void* norm_w;         // [K] bf16 or float32
-    int norm_w_f32;
-    float eps;
-    const bf16_t* w;            // [N, K]
-    const bf16_t* bias;         // [N] or null
-    void* c;                    // PLAIN: [M, N]; SILU: [M, N/2]
-    float* residual_out;        // RESID: [M, N] float32, accumulated in place
-    float* sumsq_out;           // RESID: [M, N/16]
+    const bf16_t* w;       // [N, K]
+    const bf16_t* bias;    // [N] or null
+    void* c;               // BF16/F32: [M, N]; SILU: [M, N/2]; PARTIAL: [parts, M, N] float32
+    float* residual;       // RESID: [M, N] float32, accumulated in place
+    float* sumsq;          // RESID: [M, ceil(N/16)]
     int M, N, K;
-    int second_tile_offset;     // rows of W between a workgroup's first and second tile (NT == 2)
-    int k_per_part;             // PARTIAL: k values per grid.z part (a multiple of 128); otherwise K
+    int up_offset;         // SILU: rows of W between a gate row and its up row (N/2)
+    int k_per_part;        // k values per grid.z part (a multiple of 128); K with one part
 };
 
-template <int WAVES, int MT, int NT, int EPI, bool NORM, bool HALF>
-__global__ void __launch_bounds__(WAVES * 64) gemm_fused_kernel(FusedArgs a) {
-    // HALF: the workgroup owns 8 columns only (lanes r and r + 8 read the same row of W and compute the
-    // same column; the upper copies are dropped).  Twice as many workgroups for products with few columns.
-    constexpr int TILE_N = HALF ? 8 : 16;
-    constexpr int ROWS = 16 * MT;
-    __shared__ float reduce[WAVES > 1 ? (WAVES - 1) * MT * NT * 64 * 4 : 1];
-    __shared__ float inv_rms[ROWS];
+// One 16x16 tile of results in its MFMA layout: lane (r, g) holds rows g*4+i of column r.
+// `n` is the lane's column (of C, or of the SILU output), `m_base` the tile's first row.
+template <int EPI>
+__device__ __forceinline__ void store_tile(const FusedArgs& a, const floatx4& acc, const floatx4& acc_up,
+                                           int m_base, int n, int n_tile, int lane) {
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
+    const bool col_ok = n < cols;
+    const float add = (EPI != EPI_SILU && col_ok && a.bias && blockIdx.z == 0) ? to_float(a.bias[n]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m_base + g * 4 + i;
+        const bool ok = col_ok && m < a.M;
+        if (EPI == EPI_SILU) {
+            if (ok) {
+                const float gate = acc[i];
+                static_cast<bf16_t*>(a.c)[static_cast<size_t>(m) * cols + n] =
+                    from_float<bf16_t>((gate / (1.0f + __expf(-gate))) * acc_up[i]);
+            }
+        } else if (EPI == EPI_RESID) {
+            float v = 0.f;
+            if (ok) {
+                float* dst = a.residual + static_cast<size_t>(m) * a.N + n;
+                v = *dst + acc[i] + add;
+                *dst = v;
+            }
+            float sq = v * v;  // sum over the tile's 16 columns: the lanes that share g
+            sq += __shfl_xor(sq, 1, kWave);
+            sq += __shfl_xor(sq, 2, kWave);
+            sq += __shfl_xor(sq, 4, kWave);
+            sq += __shfl_xor(sq, 8, kWave);
+            if (r == 0 && m < a.M) a.sumsq[static_cast<size_t>(m) * ((a.N + 15) / 16) + n_tile] = sq;
+        } else if (ok) {
+            const float v = acc[i] + add;
+            if (EPI == EPI_PARTIAL)
+                static_cast<float*>(a.c)[(static_cast<size_t>(blockIdx.z) * a.M + m) * a.N + n] = v;
+            else if (EPI == EPI_F32)
+                static_cast<float*>(a.c)[static_cast<size_t>(m) * a.N + n] = v;
+            else
+                static_cast<bf16_t*>(a.c)[static_cast<size_t>(m) * a.N + n] = from_float<bf16_t>(v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <int WAVES, int EPI>
+__global__ void __launch_bounds__(WAVES * 64) gemm_rows16_kernel(FusedArgs a) {
+    constexpr int NT = (EPI == EPI_SILU) ? 2 : 1;
+    constexpr int U = (NT == 1) ? 4 : 2;  // slices of 128 k values whose loads are in flight together
+    __shared__ float reduce[WAVES > 1 ? (WAVES - 1) * NT * 64 * 4 : 1];
 
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int r = lane & 15;
     const int g = lane >> 4;
-    const int m0 = blockIdx.y * ROWS;
-    const int n_first = blockIdx.x * TILE_N;
-    const int col = HALF ? (r & 7) : r;  // column of this lane within the tile
-
-    if (NORM) {
-        for (int m = wave; m < ROWS; m += WAVES) {
-            float s = 0.f;
-            if (m0 + m < a.M)
-                for (int p = lane; p < a.parts_in; p += kWave) s += a.sumsq_in[static_cast<size_t>(m0 + m) * a.parts_in + p];
-            s = wave_sum(s);
-            if (lane == 0) inv_rms[m] = 1.0f / sqrtf(s / static_cast<float>(a.K) + a.eps);
-        }
-        __syncthreads();
-    }
+    const int n_first = blockIdx.x * 16;
+    const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
+    const int n_row = min(n_first + r, cols - 1);  // a column past the end computes a copy that is not stored
 
     const bf16_t* w_row[NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) w_row[t] = a.w + static_cast<size_t>(n_first + t * a.second_tile_offset + col) * a.K + g * 8;
+    for (int t = 0; t < NT; ++t) w_row[t] = a.w + static_cast<size_t>(n_row + t * a.up_offset) * a.K + g * 8;
+    const bf16_t* a_row = a.a + static_cast<size_t>(min(r, a.M - 1)) * a.lda + g * 8;
+    const bool row_ok = r < a.M;
 
-    floatx4 acc[MT][NT];
+    floatx4 acc[NT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // U slices of 128 k values are in flight per wave: the loads of all of them are issued before the
-    // first matrix product, which is what keeps enough bytes in flight to cover the memory latency
-    constexpr int U = (MT == 1) ? (NT == 1 ? 4 : 2) : 1;
     const int k_begin = blockIdx.z * a.k_per_part;
     const int k_end = min(a.K, k_begin + a.k_per_part);
     for (int kbase = k_begin + wave * 128; kbase < k_end; kbase += U * WAVES * 128) {
@@ -105,243 +125,186 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
+            for (int j = 0; j < 4; ++j) {
+                const int k0 = kbase + u * WAVES * 128 + j * 32;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int k0 = kbase + u * WAVES * 128;
-                    // the four lane groups read one contiguous 64-byte piece of each row per load
-                    const int k = k0 + j * 32 + g * 8;
-                    b[u][t][j] = (k < k_end) ? *reinterpret_cast<const uint4*>(w_row[t] + k0 + j * 32) : uint4{0, 0, 0, 0};
-                }
+                for (int t = 0; t < NT; ++t)
+                    b[u][t][j] = (k0 + g * 8 < k_end) ? *reinterpret_cast<const uint4*>(w_row[t] + k0) : uint4{0, 0, 0, 0};
+            }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int k0 = kbase + u * WAVES * 128;
+            uint4 av[4];  // the few rows of A come from the cache; their loads are issued slice by slice
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int m = m0 + mt * 16 + r;
-                uint4 av[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int k = k0 + j * 32 + g * 8;
-                    av[j] = uint4{0, 0, 0, 0};
-                    if (m < a.M && k < k_end) {
-                        if (NORM) {
-                            const float* src = a.residual_in + static_cast<size_t>(m) * a.K + k;
-                            const float4 x0 = *reinterpret_cast<const float4*>(src);
-                            const float4 x1 = *reinterpret_cast<const float4*>(src + 4);
-                            float wv[8];
-                            if (a.norm_w_f32) {
-                                const float* wp = static_cast<const float*>(a.norm_w) + k;
-                                const float4 w0 = *reinterpret_cast<const float4*>(wp);
-                                const float4 w1 = *reinterpret_cast<const float4*>(wp + 4);
-                                wv[0] = w0.x; wv[1] = w0.y; wv[2] = w0.z; wv[3] = w0.w;
-                                wv[4] = w1.x; wv[5] = w1.y; wv[6] = w1.z; wv[7] = w1.w;
-                            } else {
-                                const uint4 raw = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(a.norm_w) + k);
-                                const uint32_t ww[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-                                for (int q = 0; q < 4; ++q) {
-                                    wv[2 * q] = __uint_as_float(ww[q] << 16);
-                                    wv[2 * q + 1] = __uint_as_float(ww[q] & 0xffff0000u);
-                                }
-                            }
-                            const float inv = inv_rms[mt * 16 + r];
-                            const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-                            uint32_t packed[4];
-#pragma unroll
-                            for (int q = 0; q < 4; ++q) {
-                                const uint32_t lo = bf16_bits_from_float((x[2 * q] * inv) * wv[2 * q]);
-                                const uint32_t hi = bf16_bits_from_float((x[2 * q + 1] * inv) * wv[2 * q + 1]);
-                                packed[q] = lo | (hi << 16);
-                            }
-                            av[j] = uint4{packed[0], packed[1], packed[2], packed[3]};
-                        } else {
-                            av[j] = *reinterpret_cast<const uint4*>(a.a + static_cast<size_t>(m) * a.lda + k);
-                        }
-                    }
-                }
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int t = 0; t < NT; ++t)
-                        acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            __builtin_bit_cast(bf16x8, av[j]), __builtin_bit_cast(bf16x8, b[u][t][j]), acc[mt][t], 0, 0, 0);
+            for (int j = 0; j < 4; ++j) {
+                const int k0 = kbase + u * WAVES * 128 + j * 32;
+                av[j] = (row_ok && k0 + g * 8 < k_end) ? *reinterpret_cast<const uint4*>(a_row + k0) : uint4{0, 0, 0, 0};
             }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, av[j]), __builtin_bit_cast(bf16x8, b[u][t][j]), acc[t], 0, 0, 0);
         }
     }
 
-    // ---- sum the waves' partial tiles in wave order; wave 0 keeps the result
-    if (WAVES > 1) {
+    if (WAVES > 1) {  // sum the waves' partial tiles in wave order; wave 0 keeps the result
         if (wave > 0) {
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
+            for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int t = 0; t < NT; ++t)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        reduce[((((wave - 1) * MT + mt) * NT + t) * 4 + i) * 64 + lane] = acc[mt][t][i];
+                for (int i = 0; i < 4; ++i) reduce[(((wave - 1) * NT + t) * 4 + i) * 64 + lane] = acc[t][i];
         }
         __syncthreads();
         if (wave > 0) return;
         for (int w = 1; w < WAVES; ++w)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
+            for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int t = 0; t < NT; ++t)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        acc[mt][t][i] += reduce[((((w - 1) * MT + mt) * NT + t) * 4 + i) * 64 + lane];
+                for (int i = 0; i < 4; ++i) acc[t][i] += reduce[(((w - 1) * NT + t) * 4 + i) * 64 + lane];
     }
-
-    // ---- epilogue (wave 0): lane (r, g) holds rows g*4+i of column r of each tile
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        if (HALF && r >= 8) continue;
-        if (EPI == EPI_SILU) {
-            const int n = n_first + r;  // column of the gate tile = column of the output
-            const int out_cols = a.second_tile_offset;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int m = m0 + mt * 16 + g * 4 + i;
-                if (m < a.M) {
-                    const float gate = acc[mt][0][i];
-                    const float up = acc[mt][NT - 1][i];
-                    static_cast<bf16_t*>(a.c)[static_cast<size_t>(m) * out_cols + n] =
-                        from_float<bf16_t>((gate / (1.0f + __expf(-gate))) * up);
-                }
-            }
-        } else {
-            const int n = n_first + r;
-            const float add = (a.bias && blockIdx.z == 0) ? to_float(a.bias[n]) : 0.f;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int m = m0 + mt * 16 + g * 4 + i;
-                const bool ok = m < a.M;
-                float v = acc[mt][0][i] + add;
-                if (EPI == EPI_RESID) {
-                    float* dst = a.residual_out + static_cast<size_t>(m) * a.N + n;
-                    if (ok) {
-                        v += *dst;
-                        *dst = v;
-                    } else {
-                        v = 0.f;
-                    }
-                    // sum of squares over the tile's 16 columns (the lanes that share g)
-                    float sq = v * v;
-                    sq += __shfl_xor(sq, 1, kWave);
-                    sq += __shfl_xor(sq, 2, kWave);
-                    sq += __shfl_xor(sq, 4, kWave);
-                    if (!HALF) sq += __shfl_xor(sq, 8, kWave);
-                    if (r == 0 && ok) a.sumsq_out[static_cast<size_t>(m) * (a.N / TILE_N) + blockIdx.x] = sq;
-                } else if (ok) {
-                    if (EPI == EPI_PARTIAL)
-                        static_cast<float*>(a.c)[(static_cast<size_t>(blockIdx.z) * a.M + m) * a.N + n] = v;
-                    else if (EPI == EPI_PLAIN_F32)
-                        static_cast<float*>(a.c)[static_cast<size_t>(m) * a.N + n] = v;
-                    else
-                        static_cast<bf16_t*>(a.c)[static_cast<size_t>(m) * a.N + n] = from_float<bf16_t>(v);
-                }
-            }
-        }
-    }
+    store_tile<EPI>(a, acc[0], acc[NT - 1], 0, n_first + r, blockIdx.x, lane);
 }
 
-template <int WAVES, int MT, int NT, int EPI>
-int launch_norm(hipStream_t s, dim3 grid, const FusedArgs& a, bool norm, bool half) {
-    if constexpr (NT == 1 && MT == 1) {
-        if (half) {
-            if (norm)
-                gemm_fused_kernel<WAVES, MT, NT, EPI, true, true><<<grid, WAVES * 64, 0, s>>>(a);
-            else
-                gemm_fused_kernel<WAVES, MT, NT, EPI, false, true><<<grid, WAVES * 64, 0, s>>>(a);
-            return cie_after_launch();
+// ---------------------------------------------------------------------------------------------
+template <int MT, int EPI>
+__global__ void __launch_bounds__(256) gemm_rows64_kernel(FusedArgs a) {
+    constexpr int NT = (EPI == EPI_SILU) ? 2 : 1;
+    constexpr int STRIDE = 128 + 8;  // staged row stride in bf16 elements (padding against bank conflicts)
+    __shared__ __attribute__((aligned(16))) uint16_t a_lds[MT * 16 * STRIDE];
+
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int m0 = blockIdx.y * (MT * 16);
+    const int n_first = (blockIdx.x * 4 + wave) * 16;
+    const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
+    const int n_row = min(n_first + r, cols - 1);
+
+    const bf16_t* w_row[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) w_row[t] = a.w + static_cast<size_t>(n_row + t * a.up_offset) * a.K + g * 8;
+
+    floatx4 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const int k_begin = blockIdx.z * a.k_per_part;
+    const int k_end = min(a.K, k_begin + a.k_per_part);
+    for (int k0 = k_begin; k0 < k_end; k0 += 128) {
+        uint4 b[NT][4];  // requested before the barrier so that they travel while A is staged
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                b[t][j] = (k0 + j * 32 + g * 8 < k_end) ? *reinterpret_cast<const uint4*>(w_row[t] + k0 + j * 32)
+                                                         : uint4{0, 0, 0, 0};
+        __syncthreads();  // the previous slice's readers are done with a_lds
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const int piece = threadIdx.x + 256 * i;  // 16 pieces of 8 k values per row
+            const int row = piece / 16;
+            const int col = (piece % 16) * 8;
+            const int m = m0 + row;
+            const int k = k0 + col;
+            const uint4 v = (m < a.M && k < k_end) ? *reinterpret_cast<const uint4*>(a.a + static_cast<size_t>(m) * a.lda + k)
+                                                   : uint4{0, 0, 0, 0};
+            *reinterpret_cast<uint4*>(&a_lds[row * STRIDE + col]) = v;
         }
+        __syncthreads();
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint4 av = *reinterpret_cast<const uint4*>(&a_lds[(mt * 16 + r) * STRIDE + j * 32 + g * 8]);
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, b[t][j]), acc[mt][t], 0, 0, 0);
+            }
     }
-    if (half) return CIE_BAD_ARGUMENT;
-    if (norm)
-        gemm_fused_kernel<WAVES, MT, NT, EPI, true, false><<<grid, WAVES * 64, 0, s>>>(a);
-    else
-        gemm_fused_kernel<WAVES, MT, NT, EPI, false, false><<<grid, WAVES * 64, 0, s>>>(a);
+    if (n_first >= cols) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+        store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, n_first + r, n_first / 16, lane);
+}
+
+template <int EPI>
+int launch_rows16(hipStream_t s, int waves, dim3 grid, const FusedArgs& a) {
+    switch (waves) {
+        case 1: gemm_rows16_kernel<1, EPI><<<grid, 64, 0, s>>>(a); break;
+        case 2: gemm_rows16_kernel<2, EPI><<<grid, 128, 0, s>>>(a); break;
+        case 4: gemm_rows16_kernel<4, EPI><<<grid, 256, 0, s>>>(a); break;
+        case 8: gemm_rows16_kernel<8, EPI><<<grid, 512, 0, s>>>(a); break;
+        default: return CIE_BAD_ARGUMENT;
+    }
     return cie_after_launch();
 }
 
-// waves * row tiles <= 16 keeps the LDS of the final sum within bounds
-template <int MT, int NT, int EPI>
-int launch_waves(hipStream_t s, int waves, dim3 grid, const FusedArgs& a, bool norm, bool half) {
-    if (waves == 1) return launch_norm<1, MT, NT, EPI>(s, grid, a, norm, half);
-    if (waves == 2) return launch_norm<2, MT, NT, EPI>(s, grid, a, norm, half);
-    if (waves == 4) return launch_norm<4, MT, NT, EPI>(s, grid, a, norm, half);
-    if constexpr (MT <= 2)
-        if (waves == 8) return launch_norm<8, MT, NT, EPI>(s, grid, a, norm, half);
-    if constexpr (MT == 1)
-        if (waves == 16) return launch_norm<16, MT, NT, EPI>(s, grid, a, norm, half);
-    return CIE_BAD_ARGUMENT;
+template <int EPI>
+int launch_rows64(hipStream_t s, int row_tiles, dim3 grid, const FusedArgs& a) {
+    if constexpr (EPI == EPI_RESID) {
+        return CIE_BAD_ARGUMENT;  // the sums of squares of a row need one workgroup per row block and tile: rows16 only
+    } else {
+        switch (row_tiles) {
+            case 2: gemm_rows64_kernel<2, EPI><<<grid, 256, 0, s>>>(a); break;
+            case 4: gemm_rows64_kernel<4, EPI><<<grid, 256, 0, s>>>(a); break;
+            default: return CIE_BAD_ARGUMENT;
+        }
+        return cie_after_launch();
+    }
 }
 
-template <int NT, int EPI>
-int launch_rows(hipStream_t s, int mt, int waves, dim3 grid, const FusedArgs& a, bool norm, bool half) {
-    switch (mt) {
-        case 1: return launch_waves<1, NT, EPI>(s, waves, grid, a, norm, half);
-        case 2: return launch_waves<2, NT, EPI>(s, waves, grid, a, norm, half);
-        case 4: return launch_waves<4, NT, EPI>(s, waves, grid, a, norm, half);
-    }
-    return CIE_BAD_ARGUMENT;
+template <int EPI>
+int launch(hipStream_t s, int row_tiles, int waves, int k_parts, const FusedArgs& a) {
+    const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
+    const int tiles = (cols + 15) / 16;
+    if (row_tiles == 1) return launch_rows16<EPI>(s, waves, dim3(tiles, 1, k_parts), a);
+    const int m_blocks = (a.M + 16 * row_tiles - 1) / (16 * row_tiles);
+    if (m_blocks > 65535) return CIE_BAD_ARGUMENT;
+    return launch_rows64<EPI>(s, row_tiles, dim3((tiles + 3) / 4, m_blocks, k_parts), a);
 }
 
 }  // namespace
 
-// epilogue: 0 bf16 out, 1 float32 out, 2 SiLU-gate (W = [gate rows; up rows], N = 2 * outputs), 3 residual accumulate,
-// 4 partial products of k_parts parts of K to c[k_parts, M, N] (float32).
-// row_tiles: 16-row tiles per workgroup (1, 2 or 4); waves: waves per workgroup that share K (1, 2, 4, 8, 16).
-// half_tiles: workgroups of 8 columns instead of 16 (row_tiles 1, not SiLU); sumsq_out is then [M, N/8].
-CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const float* residual_in,
-                           const float* sumsq_in, int parts_in, const void* norm_w, int norm_w_f32, float eps,
-                           const void* w, const void* bias, void* c, float* residual_out, float* sumsq_out,
-                           int M, int N, int K, int epilogue, int row_tiles, int waves, int half_tiles,
-                           int k_parts) {
-    const bool norm = residual_in != nullptr;
-    if (M <= 0 || N <= 0 || K <= 0 || K % 8 || N % 16) return CIE_BAD_ARGUMENT;
-    if (!norm && (!a || lda < K || lda % 8)) return CIE_BAD_ARGUMENT;
-    if (norm && (!sumsq_in || parts_in < 1 || !norm_w || !(eps > 0.f))) return CIE_BAD_ARGUMENT;
+// epilogue: 0 bf16, 1 float32, 2 SiLU-gate (W = [gate rows; up rows], N = 2 * outputs), 3 residual
+// accumulate (+ sums of squares), 4 partial products of k_parts parts of K to c[k_parts, M, N].
+// row_tiles 1: M <= 16, `waves` waves per workgroup share K (1, 2, 4, 8).
+// row_tiles 2 or 4: up to 32 or 64 rows per workgroup (more rows: more workgroups), A staged in LDS.
+// K and lda must be multiples of 8 (16-byte loads); N is free.
+CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
+                           float* residual, float* sumsq, int M, int N, int K, int epilogue, int row_tiles,
+                           int waves, int k_parts) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % 8 || !a || !w || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
     if (row_tiles != 1 && row_tiles != 2 && row_tiles != 4) return CIE_BAD_ARGUMENT;
-    if (epilogue == EPI_SILU && (N % 32 || bias)) return CIE_BAD_ARGUMENT;
-    if (epilogue == EPI_RESID && (!residual_out || !sumsq_out)) return CIE_BAD_ARGUMENT;
-    if ((epilogue == EPI_PLAIN_BF16 || epilogue == EPI_PLAIN_F32 || epilogue == EPI_SILU || epilogue == EPI_PARTIAL) && !c)
-        return CIE_BAD_ARGUMENT;
+    if (row_tiles == 1 && M > 16) return CIE_BAD_ARGUMENT;
+    if (epilogue == EPI_SILU && (N % 2 || bias)) return CIE_BAD_ARGUMENT;
+    if (epilogue == EPI_RESID && (!residual || !sumsq || row_tiles != 1)) return CIE_BAD_ARGUMENT;
+    if (epilogue != EPI_RESID && !c) return CIE_BAD_ARGUMENT;
     if (k_parts < 1 || k_parts > 64 || (k_parts > 1 && epilogue != EPI_PARTIAL)) return CIE_BAD_ARGUMENT;
-    const int m_blocks = (M + 16 * row_tiles - 1) / (16 * row_tiles);
-    if (m_blocks > 65535) return CIE_BAD_ARGUMENT;
     FusedArgs f;
     f.a = static_cast<const bf16_t*>(a);
     f.lda = lda;
-    f.residual_in = residual_in;
-    f.sumsq_in = sumsq_in;
-    f.parts_in = parts_in;
-    f.norm_w = norm_w;
-    f.norm_w_f32 = norm_w_f32;
-    f.eps = eps;
     f.w = static_cast<const bf16_t*>(w);
     f.bias = static_cast<const bf16_t*>(bias);
     f.c = c;
-    f.residual_out = residual_out;
-    f.sumsq_out = sumsq_out;
+    f.residual = residual;
+    f.sumsq = sumsq;
     f.M = M;
     f.N = N;
     f.K = K;
+    f.up_offset = (epilogue == EPI_SILU) ? N / 2 : 0;
     f.k_per_part = ((K + k_parts - 1) / k_parts + 127) / 128 * 128;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (epilogue == EPI_SILU) {
-        f.second_tile_offset = N / 2;
-        return launch_rows<2, EPI_SILU>(s, row_tiles, waves, dim3((N / 2) / 16, m_blocks), f, norm, half_tiles != 0);
-    }
-    f.second_tile_offset = 0;
-    const bool half = half_tiles != 0;
-    dim3 grid(N / (half ? 8 : 16), m_blocks, k_parts);
     switch (epilogue) {
-        case EPI_PLAIN_BF16: return launch_rows<1, EPI_PLAIN_BF16>(s, row_tiles, waves, grid, f, norm, half);
-        case EPI_PLAIN_F32: return launch_rows<1, EPI_PLAIN_F32>(s, row_tiles, waves, grid, f, norm, half);
-        case EPI_RESID: return launch_rows<1, EPI_RESID>(s, row_tiles, waves, grid, f, norm, half);
-        case EPI_PARTIAL: return launch_rows<1, EPI_PARTIAL>(s, row_tiles, waves, grid, f, norm, half);
+        case EPI_BF16: return launch<EPI_BF16>(s, row_tiles, waves, k_parts, f);
+        case EPI_F32: return launch<EPI_F32>(s, row_tiles, waves, k_parts, f);
+        case EPI_SILU: return launch<EPI_SILU>(s, row_tiles, waves, k_parts, f);
+        case EPI_RESID: return launch<EPI_RESID>(s, row_tiles, waves, k_parts, f);
+        case EPI_PARTIAL: return launch<EPI_PARTIAL>(s, row_tiles, waves, k_parts, f);
     }
     return CIE_BAD_ARGUMENT;
 }

@@ -321,100 +321,55 @@ def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]
     return out
 
 
-def gemm_bf16(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-              out_dtype: torch.dtype = torch.bfloat16, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Matrix-core ``a @ weight.T + bias`` for few rows: bf16 operands, float32
-    accumulation, float32 or bf16 result.  K must be a multiple of 8."""
-    _require(a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1,
-             "a must be a bfloat16 GPU matrix with unit inner stride")
+EPI_BF16, EPI_F32, EPI_SILU, EPI_RESID, EPI_PARTIAL = 0, 1, 2, 3, 4
+FUSED_TARGET_WAVES = 2048
+FUSED_MAX_ROWS = 64  # rows one workgroup of ``gemm_fused`` takes; more rows run as more workgroup rows
+
+
+def plan_fused(rows: int, column_tiles: int, k: int) -> tuple[int, int]:
+    """(row_tiles, waves per workgroup) of ``gemm_fused`` for ``rows`` rows,
+    ``column_tiles`` tiles of 16 columns (times the parts of K) and inner size
+    ``k`` per part.  Up to 16 rows: as many waves share K as it takes to fill the
+    GPU, each with at least one 128-wide slice.  More rows: four waves side by
+    side that share the staged activations."""
+    if rows > 16:
+        return (2 if rows <= 32 else 4), 4
+    waves = 1
+    while waves < 8 and column_tiles * waves < FUSED_TARGET_WAVES and waves * 2 * 128 <= k:
+        waves *= 2
+    return 1, waves
+
+
+def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               residual_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None,
+               plan: Optional[tuple[int, int]] = None, k_parts: int = 1) -> torch.Tensor:
+    """Few-row matrix product ``a @ weight.T`` (bf16 operands, float32 sums) fused
+    with its neighbour.  ``epilogue``: ``EPI_BF16`` / ``EPI_F32`` return
+    ``a W^T + bias``; ``EPI_SILU`` (weight = gate rows over up rows) returns
+    ``silu(gate) * up`` [M, N/2]; ``EPI_RESID`` (up to 16 rows) adds the product
+    into ``residual_out`` (float32 [M, N]) and returns the partial sums of
+    squares of its new rows [M, ceil(N/16)]; ``EPI_PARTIAL`` cuts K into
+    ``k_parts`` parts and returns their float32 partial products
+    [k_parts, M, N] (bias in part 0), to be summed by ``add_parts_rmsnorm``."""
     _gpu("weight", weight, torch.bfloat16, 2)
-    m, k = a.shape
-    n = weight.shape[0]
-    _require(weight.shape[1] == k, f"a is [{m},{k}] but weight is {tuple(weight.shape)}")
+    n, k = weight.shape
+    _require(a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1,
+             "a must be a bf16 GPU matrix with unit inner stride")
+    m = a.shape[0]
+    _require(m >= 1 and a.shape[1] == k, f"a {tuple(a.shape)} vs K={k}")
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
     _require(k % 8 == 0 and lda % 8 == 0, f"K and the row stride must be multiples of 8, are {k} and {lda}")
     _require(a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
-    if bias is not None:
-        _gpu("bias", bias, torch.bfloat16, 1)
-        _require(bias.shape[0] == n, f"bias must be [{n}]")
-    if out is None:
-        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
-    _gpu("out", out, out_dtype, 2)
-    _require(out.shape == (m, n), f"out must be {(m, n)}")
-    _run("cie_gemm_bf16", load_library().cie_gemm_bf16(_stream(), _ptr(a), _ptr(weight), _ptr(bias), _ptr(out),
-                                                       _i(_code(out_dtype)), _i(m), _i(n), _i(k), _i(lda), _i(n)))
-    return out
-
-
-EPI_BF16, EPI_F32, EPI_SILU, EPI_RESID, EPI_PARTIAL = 0, 1, 2, 3, 4
-FUSED_TARGET_WAVES = 2048
-
-
-FUSED_HALF_BELOW = 0  # fewer 16-column workgroups than this: use 8-column workgroups (measured: no gain on MI355X)
-
-
-def plan_fused(rows: int, column_tiles: int, k: int, may_halve: bool = True) -> tuple[int, int, int]:
-    """(row_tiles, waves per workgroup, half_tiles) for ``rows`` rows,
-    ``column_tiles`` 16-column tiles and inner size ``k``: enough waves to fill
-    the GPU, at least one 128-wide slice of k per wave, waves * row_tiles <= 16;
-    workgroups of 8 columns where 16-column ones would leave compute units idle."""
-    row_tiles = 1 if rows <= 16 else 2 if rows <= 32 else 4
-    half = 1 if may_halve and row_tiles == 1 and column_tiles < FUSED_HALF_BELOW else 0
-    blocks = column_tiles * (2 if half else 1) * -(-rows // (16 * row_tiles))
-    waves = 1
-    while (waves < 16 // row_tiles and blocks * waves < FUSED_TARGET_WAVES and waves * 2 * 128 <= k):
-        waves *= 2
-    return row_tiles, waves, half
-
-
-def gemm_fused(weight: torch.Tensor, epilogue: int, a: Optional[torch.Tensor] = None,
-               residual_in: Optional[torch.Tensor] = None, sumsq_in: Optional[torch.Tensor] = None,
-               norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
-               bias: Optional[torch.Tensor] = None, residual_out: Optional[torch.Tensor] = None,
-               sumsq_out: Optional[torch.Tensor] = None, plan: Optional[tuple[int, int, int]] = None,
-               k_parts: int = 1
-               ) -> Optional[torch.Tensor]:
-    """Few-row matrix product ``A @ weight.T`` fused with its neighbours.
-
-    A is either ``a`` (bf16 [M, K]) or made on the fly as the RMS-normalised
-    ``residual_in`` (float32 [M, K]) from the partial row sums of squares
-    ``sumsq_in`` [M, parts] and ``norm_weight``.  ``epilogue``: ``EPI_BF16`` /
-    ``EPI_F32`` return ``A W^T + bias``; ``EPI_SILU`` (weight = gate rows over up
-    rows) returns ``silu(gate) * up`` [M, N/2]; ``EPI_RESID`` adds the product
-    into ``residual_out`` (float32 [M, N]) and writes the partial sums of squares
-    of its new rows to ``sumsq_out`` [M, N/16], returning nothing."""
-    _gpu("weight", weight, torch.bfloat16, 2)
-    n, k = weight.shape
-    _require(k % 8 == 0 and n % 16 == 0, f"gemm_fused needs K % 8 == 0 and N % 16 == 0, got N={n}, K={k}")
-    device = weight.device
-    rows = (residual_in if residual_in is not None else a).shape[0]
     _require(1 <= k_parts <= 64 and (k_parts == 1 or epilogue == EPI_PARTIAL), f"k_parts {k_parts} does not fit the epilogue")
-    row_tiles, waves, half = plan or plan_fused(rows, (n // 2 if epilogue == EPI_SILU else n) // 16 * k_parts,
-                                                -(-k // k_parts), may_halve=epilogue != EPI_SILU and k_parts == 1)
-    _require(waves in (1, 2, 4, 8, 16) and waves * row_tiles <= 16, f"plan {(row_tiles, waves, half)} is not built")
-    _require(not half or (row_tiles == 1 and epilogue != EPI_SILU), "8-column workgroups need one row tile and no SiLU")
-    if residual_in is not None:
-        _gpu("residual_in", residual_in, torch.float32, 2)
-        m = residual_in.shape[0]
-        _require(residual_in.shape[1] == k, f"residual_in {tuple(residual_in.shape)} vs K={k}")
-        _require(sumsq_in is not None and norm_weight is not None and eps > 0, "the norm prologue needs sumsq, weight and eps")
-        _gpu("sumsq_in", sumsq_in, torch.float32, 2)
-        _require(sumsq_in.shape[0] >= m, f"sumsq_in has {sumsq_in.shape[0]} rows for {m}")
-        _gpu("norm_weight", norm_weight, dims=1)
-        _require(norm_weight.shape[0] == k and norm_weight.dtype in (torch.bfloat16, torch.float32), "norm weight does not fit")
-        lda = 0
-    else:
-        _require(a is not None and a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1,
-                 "a must be a bf16 GPU matrix with unit inner stride")
-        m = a.shape[0]
-        _require(a.shape[1] == k, f"a {tuple(a.shape)} vs K={k}")
-        lda = a.stride(0) if m > 1 else max(a.stride(0), k)
-        _require(lda % 8 == 0 and a.data_ptr() % 16 == 0, "a must be 16-byte aligned with a row stride that is a multiple of 8")
-    _require(m >= 1, "gemm_fused needs at least one row")
+    device = weight.device
     if bias is not None:
         _gpu("bias", bias, torch.bfloat16, 1)
         _require(bias.shape[0] == n and epilogue != EPI_SILU, "bias does not fit")
-    out = None
+    columns = n // 2 if epilogue == EPI_SILU else n
+    row_tiles, waves = plan or plan_fused(m, -(-columns // 16) * k_parts, -(-k // k_parts))
+    _require(row_tiles in (1, 2, 4) and (row_tiles > 1 or (m <= 16 and waves in (1, 2, 4, 8))),
+             f"plan {(row_tiles, waves)} does not fit {m} rows")
+    residual = sumsq = None
     if epilogue == EPI_BF16:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
     elif epilogue == EPI_F32:
@@ -422,26 +377,24 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: Optional[torch.Tensor] = 
     elif epilogue == EPI_PARTIAL:
         out = torch.empty((k_parts, m, n), dtype=torch.float32, device=device)
     elif epilogue == EPI_SILU:
-        _require(n % 32 == 0, f"the SiLU epilogue needs N % 32 == 0, got {n}")
+        _require(n % 2 == 0, f"the SiLU epilogue needs an even N, got {n}")
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=device)
     elif epilogue == EPI_RESID:
+        _require(row_tiles == 1, "the residual epilogue takes up to 16 rows")
         _require(residual_out is not None, "the residual epilogue needs the residual to add into")
         _gpu("residual_out", residual_out, torch.float32, 2)
         _require(residual_out.shape == (m, n), f"residual_out {tuple(residual_out.shape)} vs {(m, n)}")
-        parts = n // (8 if half else 16)
+        parts = -(-n // 16)
         if sumsq_out is None:
             sumsq_out = torch.empty((m, parts), dtype=torch.float32, device=device)
-        out = sumsq_out
         _gpu("sumsq_out", sumsq_out, torch.float32, 2)
         _require(sumsq_out.shape[0] >= m and sumsq_out.shape[1] == parts, f"sumsq_out {tuple(sumsq_out.shape)} must be [>= {m}, {parts}]")
+        out, residual, sumsq = sumsq_out, residual_out, sumsq_out
     else:
         raise ValueError(f"unknown epilogue {epilogue}")
     _run("cie_gemm_fused", load_library().cie_gemm_fused(
-        _stream(), _ptr(a), _i(lda), _ptr(residual_in), _ptr(sumsq_in),
-        _i(sumsq_in.shape[1] if sumsq_in is not None else 0), _ptr(norm_weight),
-        _i(1 if norm_weight is not None and norm_weight.dtype == torch.float32 else 0), _f(eps), _ptr(weight),
-        _ptr(bias), _ptr(None if epilogue == EPI_RESID else out), _ptr(residual_out), _ptr(sumsq_out), _i(m), _i(n), _i(k), _i(epilogue),
-        _i(row_tiles), _i(waves), _i(half), _i(k_parts)))
+        _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(None if epilogue == EPI_RESID else out),
+        _ptr(residual), _ptr(sumsq), _i(m), _i(n), _i(k), _i(epilogue), _i(row_tiles), _i(waves), _i(k_parts)))
     return out
 
 

@@ -26,7 +26,6 @@ from .linear import linear
 
 class Attention(Part):
     graph_safe = True
-    takes_lazy_norm = True
     adds_to_residual = True
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool, out_bias: bool, position: PartSpec, window: Optional[int] = None,

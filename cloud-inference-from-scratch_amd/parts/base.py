@@ -10,10 +10,11 @@ Interfaces (``x`` is ``[tokens, hidden]`` in the engine's activation dtype,
 ``residual`` the float32 residual stream, ``batch`` a
 :class:`~cie_amd.engine.batch.StepBatch`):
 
-``Norm``        ``forward(residual, branch, out_dtype, rows=None, lazy=False) -> x``
+``Norm``        ``forward(residual, branch, out_dtype, rows=None) -> x``
                 adds ``branch`` into ``residual`` (in place, float32) and returns
-                the normalised rows (``branch`` may also be a ``RowSumsq``, see
-                ``parts/linear.py``; with ``lazy`` a ``LazyNorm`` may come back).
+                the normalised rows.  A norm that sets ``takes_row_sumsq`` is
+                also handed the ``RowSumsq`` / ``PartialSum`` forms of a branch
+                (``parts/linear.py``); any other gets a tensor or ``None``.
 ``Position``    ``tables(device) -> (cos, sin)`` or whatever its mixer asks of it.
 ``Mixer``       ``cache_need() -> PagedKV | FixedState | None`` and
                 ``forward(x, batch, view, writes) -> y``; ``view`` is the cache
@@ -70,9 +71,8 @@ class Part:
     size: only then may a decode step that contains it be captured in a graph."""
 
     graph_safe = False
-    # ``takes_lazy_norm``: ``forward`` accepts a ``LazyNorm`` in place of ``x``.  ``adds_to_residual``:
-    # ``forward`` takes ``residual=`` and may add its output there itself, returning a ``RowSumsq``.
-    takes_lazy_norm = False
+    # ``adds_to_residual``: ``forward`` takes ``residual=`` and may add its output there itself
+    # (returning a ``RowSumsq``) or leave partial products for the next norm (a ``PartialSum``).
     adds_to_residual = False
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:

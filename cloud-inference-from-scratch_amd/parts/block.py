@@ -5,8 +5,8 @@
 float32; a branch's output is added inside the next norm kernel, so the block
 returns the feed-forward output as ``pending`` instead of adding it.  A part
 that can add its output into the residual itself (the fused decode products do)
-returns a ``RowSumsq`` instead, and the next norm may then stay lazy and be
-folded into its consumer's product (``parts/linear.py``).
+returns a ``RowSumsq`` instead (or a ``PartialSum`` of partial products), and
+the next norm then runs its cheaper form (``parts/linear.py``).
 """
 
 from __future__ import annotations
@@ -53,26 +53,25 @@ class PreNormBlock:
 
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], batch, view,
                 writes: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
-        x = normalise(self.norm1, residual, pending, self.dtype, self.mixer)
+        x = normalise(self.norm1, residual, pending, self.dtype)
         extra = {"residual": residual} if getattr(self.mixer, "adds_to_residual", False) else {}
         mixed = self.mixer.forward(x, batch, view, writes, **extra)
-        x = normalise(self.norm2, residual, mixed, self.dtype, self.feed_forward)
+        x = normalise(self.norm2, residual, mixed, self.dtype)
         extra = {"residual": residual} if getattr(self.feed_forward, "adds_to_residual", False) else {}
         return residual, self.feed_forward.forward(x, **extra)
 
 
-def normalise(norm, residual: torch.Tensor, pending, dtype: torch.dtype, consumer=None, rows=None):
+def normalise(norm, residual: torch.Tensor, pending, dtype: torch.dtype, rows=None):
     """Run ``norm`` on the residual stream plus what is pending.  Only a norm that
-    says so is shown a ``RowSumsq`` or asked to stay lazy; any other gets ``None``
-    for a branch that was already added."""
-    if isinstance(pending, PartialSum) and not getattr(norm, "takes_row_sumsq", False):
-        residual.add_(pending.parts.sum(0))
-        pending = None
-    if isinstance(pending, RowSumsq):
-        if not getattr(norm, "takes_row_sumsq", False):
+    says so (``takes_row_sumsq``) is shown the fused forms of a branch; for any
+    other the partial products are added here and an already added branch
+    becomes ``None``."""
+    if not getattr(norm, "takes_row_sumsq", False):
+        if isinstance(pending, PartialSum):
+            residual.add_(pending.parts.sum(0))
             pending = None
-        elif rows is None and getattr(consumer, "takes_lazy_norm", False):
-            return norm.forward(residual, pending, dtype, lazy=True)
+        elif isinstance(pending, RowSumsq):
+            pending = None
     if rows is not None:
         return norm.forward(residual, pending, dtype, rows=rows)
     return norm.forward(residual, pending, dtype)

@@ -17,7 +17,6 @@ from .linear import linear
 
 class GatedMLP(Part):
     graph_safe = True
-    takes_lazy_norm = True
     adds_to_residual = True
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
         if activation != "silu":

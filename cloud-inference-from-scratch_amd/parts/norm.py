@@ -15,7 +15,7 @@ import torch
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, register_part
-from .linear import LazyNorm, PartialSum, RowSumsq
+from .linear import PartialSum, RowSumsq
 
 
 class RMSNorm(Part):
@@ -36,17 +36,16 @@ class RMSNorm(Part):
         self.weight = tensors[prefix + "weight"].contiguous()
 
     def forward(self, residual: torch.Tensor, branch, out_dtype: torch.dtype,
-                rows: Optional[torch.Tensor] = None, lazy: bool = False):
-        """``branch`` is a tensor still to be added into ``residual``, ``None``, or a
-        ``RowSumsq`` (already added; the rows' sums of squares are known) or a
-        ``PartialSum`` (float32 partial products still to be added).  With
-        ``lazy`` and a ``RowSumsq`` nothing runs here: the consumer's product
-        normalises its operand itself."""
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``branch`` is a tensor still to be added into ``residual``, ``None``, a
+        ``PartialSum`` (float32 partial products still to be added) or a
+        ``RowSumsq`` (already added; the rows' sums of squares are known, so the
+        norm needs no reduction)."""
         if isinstance(branch, PartialSum):
             return ops.add_parts_rmsnorm(residual, branch.parts, self.weight, self.eps, rows=rows)
         if isinstance(branch, RowSumsq):
-            if lazy and rows is None:
-                return LazyNorm(residual, branch.sumsq, self.weight, self.eps, out_dtype)
+            if rows is None and out_dtype == torch.bfloat16:
+                return ops.rmsnorm_from_sumsq(residual, branch.sumsq, self.weight, self.eps)
             branch = None
         return ops.add_rmsnorm(residual, branch, self.weight, self.eps, out_dtype, rows=rows)
 

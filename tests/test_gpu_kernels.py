@@ -95,18 +95,25 @@ def test_gemm_f32(ops, shape):
 @pytest.mark.parametrize("shape", [(1, 40, 24), (5, 515, 96), (16, 64, 128), (17, 130, 200), (33, 70, 1032),
                                    (64, 256, 264), (150, 99, 72)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-def test_gemm_bf16(ops, shape, out_dtype):
+def test_gemm_fused_plain_any_size(ops, shape, out_dtype):
+    """Plain product with bias: rows from 1 to more than a workgroup takes, column counts
+    that are no multiple of 16, inner sizes that are no multiple of 128."""
     m, n, k = shape
     a, w, b = rand((m, k), torch.bfloat16, 10), rand((n, k), torch.bfloat16, 11), rand((n,), torch.bfloat16, 12)
     expect = a.double() @ w.double().t()
-    out = ops.gemm_bf16(a, w, None, out_dtype)
-    assert out.dtype == out_dtype
+    epilogue = ops.EPI_F32 if out_dtype == torch.float32 else ops.EPI_BF16
+    out = ops.gemm_fused(w, epilogue, a)
+    assert out.dtype == out_dtype and out.shape == (m, n)
     if out_dtype == torch.float32:
         torch.testing.assert_close(out.double(), expect, rtol=1e-4, atol=1e-4 * math.sqrt(k))
     else:
         torch.testing.assert_close(out.double(), expect, rtol=1e-2, atol=1e-2 * math.sqrt(k))
-    out = ops.gemm_bf16(a, w, b, torch.float32)
+    out = ops.gemm_fused(w, ops.EPI_F32, a, bias=b)
     torch.testing.assert_close(out.double(), expect + b.double(), rtol=1e-4, atol=1e-4 * math.sqrt(k))
+    # rows given as a strided view (a slice of a wider buffer)
+    wide = torch.zeros((m, k + 64), dtype=torch.bfloat16).cuda()
+    wide[:, :k] = a
+    torch.testing.assert_close(ops.gemm_fused(w, ops.EPI_F32, wide[:, :k]), ops.gemm_fused(w, ops.EPI_F32, a), rtol=0, atol=0)
 
 
 def build_cache(dtype, lengths, kv_heads, head_dim, page_size, seed, shuffle=True):
@@ -209,7 +216,9 @@ def run_mfma(ops, q_all, contexts, q_lens, k_pool, v_pool, table, slots, q_heads
     return out.float().cpu()
 
 
-MFMA_GEOMETRY = [(16, 2, 128, 16), (4, 2, 32, 8), (3, 1, 32, 8), (6, 6, 64, 4), (16, 1, 96, 32), (12, 4, 256, 16)]
+# (query heads, KV heads, head size, page size); 28/4 and 40/8 are the head counts of the 7B and 14B shapes
+MFMA_GEOMETRY = [(16, 2, 128, 16), (4, 2, 32, 8), (3, 1, 32, 8), (6, 6, 64, 4), (16, 1, 96, 32), (12, 4, 256, 16),
+                 (28, 4, 128, 16), (40, 8, 128, 64)]
 
 
 @pytest.mark.parametrize("geometry", MFMA_GEOMETRY)
@@ -427,75 +436,50 @@ def test_sample_frequencies(ops):
     assert (freq - expect).abs().max() < 0.03
 
 
-@pytest.mark.parametrize("shape", [(1, 64, 128), (8, 2560, 2048), (16, 96, 328), (17, 208, 1032), (40, 64, 264),
+@pytest.mark.parametrize("shape", [(1, 64, 128), (8, 2560, 2048), (16, 96, 328), (17, 208, 1032), (40, 66, 264),
                                    (64, 2048, 1408), (70, 48, 96)])
-@pytest.mark.parametrize("plan", [None, "one", "many", "half"])
+@pytest.mark.parametrize("plan", [None, "one", "many"])
 def test_gemm_fused_epilogues(ops, shape, plan):
-    """The fused few-row product: plain (bf16 / float32, with bias), SiLU-gate
-    and residual-accumulate epilogues, with one wave per workgroup and with as
-    many as are built (their partial tiles summed through LDS), against float64 products."""
+    """The fused few-row product: SiLU-gate and residual-accumulate epilogues, with one wave per
+    workgroup and with eight (partial tiles summed through LDS), against float64 products."""
     m, n, k = shape
-    row_tiles = 1 if m <= 16 else 2 if m <= 32 else 4
-    if plan == "half" and row_tiles != 1:
-        pytest.skip("8-column workgroups exist for one row tile only")
-    chosen = {None: None, "one": (row_tiles, 1, 0), "many": (row_tiles, 16 // row_tiles, 0), "half": (1, 4, 1)}[plan]
-    halved = chosen[2] if chosen else ops.plan_fused(m, n // 16, k)[2]
-    cols = 8 if halved else 16
-    a, w, b = rand((m, k), torch.bfloat16, 80), rand((n, k), torch.bfloat16, 81, 0.3), rand((n,), torch.bfloat16, 82)
+    if m > 16 and plan is not None:
+        pytest.skip("the waves-share-K form takes up to 16 rows")
+    chosen = {None: None, "one": (1, 1), "many": (1, 8)}[plan]
+    a, w = rand((m, k), torch.bfloat16, 80), rand((n, k), torch.bfloat16, 81, 0.3)
+    b = rand((n,), torch.bfloat16, 82)
     exact = a.double() @ w.double().t()
-    atol = 2e-4 * math.sqrt(k)
-    out = ops.gemm_fused(w, ops.EPI_F32, a=a, bias=b, plan=chosen)
-    torch.testing.assert_close(out.double(), exact + b.double(), rtol=1e-4, atol=atol)
-    out = ops.gemm_fused(w, ops.EPI_BF16, a=a, plan=chosen)
-    torch.testing.assert_close(out.double(), exact, rtol=1e-2, atol=1e-2 * math.sqrt(k) * 0.3)
-    if n % 32 == 0:
-        gate, up = exact[:, : n // 2], exact[:, n // 2:]
-        out = ops.gemm_fused(w, ops.EPI_SILU, a=a, plan=None if plan == "half" else chosen)
-        assert out.shape == (m, n // 2)
-        want = torch.nn.functional.silu(gate) * up
-        torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()))
+    gate, up = exact[:, : n // 2], exact[:, n // 2:]
+    out = ops.gemm_fused(w, ops.EPI_SILU, a, plan=chosen)
+    assert out.shape == (m, n // 2) and out.dtype == torch.bfloat16
+    want = torch.nn.functional.silu(gate) * up
+    torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()))
+    if m > 16:
+        with pytest.raises(ValueError, match="16 rows"):
+            ops.gemm_fused(w, ops.EPI_RESID, a, residual_out=rand((m, n), torch.float32, 83))
+        return
     residual = rand((m, n), torch.float32, 83, 2.0)
     before = residual.clone()
-    sumsq = torch.full((m + 2, n // cols), float("nan")).cuda()
-    assert ops.gemm_fused(w, ops.EPI_RESID, a=a, residual_out=residual, sumsq_out=sumsq, plan=chosen) is sumsq
-    want = before.double() + exact
-    torch.testing.assert_close(residual.double(), want, rtol=1e-4, atol=atol)
-    torch.testing.assert_close(sumsq[:m].double(), want.pow(2).view(m, n // cols, cols).sum(-1), rtol=1e-4, atol=1e-3)
+    parts = -(-n // 16)
+    sumsq = torch.full((m + 2, parts), float("nan")).cuda()
+    assert ops.gemm_fused(w, ops.EPI_RESID, a, bias=b, residual_out=residual, sumsq_out=sumsq, plan=chosen) is sumsq
+    want = before.double() + exact + b.double()
+    torch.testing.assert_close(residual.double(), want, rtol=1e-4, atol=2e-4 * math.sqrt(k))
+    padded = torch.zeros((m, parts * 16), dtype=torch.float64).cuda()
+    padded[:, :n] = want
+    torch.testing.assert_close(sumsq[:m].double(), padded.pow(2).view(m, parts, 16).sum(-1), rtol=1e-4, atol=1e-3)
     assert torch.isnan(sumsq[m:]).all()
 
 
-@pytest.mark.parametrize("norm_dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("shape", [(1, 64, 128), (8, 320, 2048), (16, 96, 328), (33, 64, 264), (64, 128, 1408)])
-def test_gemm_fused_norm_prologue(ops, shape, norm_dtype):
-    """RMSNorm folded into the product's A operand: equals norm kernel followed by the plain product."""
-    m, n, k = shape
-    residual = rand((m, k), torch.float32, 84, 3.0)
-    norm_w = (rand((k,), torch.float32, 85) + 1).to(norm_dtype)
-    w = rand((n, k), torch.bfloat16, 86, 0.2)
-    eps = 1e-5
-    parts = 7
-    # any split of the row's sum of squares into parts must give the same norm
-    full = residual.pow(2).sum(-1, keepdim=True)
-    shares = torch.softmax(rand((m, parts), torch.float32, 87), dim=-1)
-    sumsq = (full * shares).contiguous()
-    normed = ops.add_rmsnorm(residual.clone(), None, norm_w, eps, torch.bfloat16)
-    want = ops.gemm_fused(w, ops.EPI_F32, a=normed)
-    for plan in (None, (1 if m <= 16 else 2 if m <= 32 else 4, 4, 0)):
-        got = ops.gemm_fused(w, ops.EPI_F32, residual_in=residual, sumsq_in=sumsq, norm_weight=norm_w, eps=eps, plan=plan)
-        # the normalised operand is rounded to bf16 in both; the inverse RMS may differ in its last bit
-        torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
-    exact = (plain_qwen2.rms_norm(residual.cpu(), norm_w.float().cpu(), eps).double() @ w.double().cpu().t())
-    torch.testing.assert_close(got.double().cpu(), exact, rtol=2e-2, atol=2e-2 * float(exact.abs().max()))
-
-
-@pytest.mark.parametrize("shape", [(1, 64, 256), (8, 2048, 11008), (13, 96, 328), (16, 48, 1032)])
+@pytest.mark.parametrize("shape", [(1, 64, 256), (8, 2048, 11008), (13, 96, 328), (16, 48, 1032), (40, 200, 1032),
+                                   (64, 2048, 2752)])
 @pytest.mark.parametrize("k_parts", [1, 3, 4])
 def test_gemm_fused_partial_products_and_their_norm(ops, shape, k_parts):
     """K cut into parts: the float32 partial products sum to the product (bias once), and the
     add-parts norm kernel equals adding that product into the residual and normalising."""
     m, n, k = shape
     a, w, b = rand((m, k), torch.bfloat16, 94), rand((n, k), torch.bfloat16, 95, 0.3), rand((n,), torch.bfloat16, 96)
-    parts = ops.gemm_fused(w, ops.EPI_PARTIAL, a=a, bias=b, k_parts=k_parts)
+    parts = ops.gemm_fused(w, ops.EPI_PARTIAL, a, bias=b, k_parts=k_parts)
     assert parts.shape == (k_parts, m, n) and parts.dtype == torch.float32
     exact = a.double() @ w.double().t() + b.double()
     torch.testing.assert_close(parts.double().sum(0), exact, rtol=1e-4, atol=2e-4 * math.sqrt(k))
