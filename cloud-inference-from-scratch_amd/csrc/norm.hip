@@ -88,6 +88,49 @@ CIE_API int cie_add_parts_rmsnorm(void* stream, int wdtype, float* residual, con
     return cie_after_launch();
 }
 
+// bf16 activations and weight, hidden a multiple of 8: eight elements per thread, 16-byte accesses.
+__global__ void add_rmsnorm_vec8_kernel(float* __restrict__ residual, const bf16_t* __restrict__ branch,
+                                        const bf16_t* __restrict__ weight, bf16_t* __restrict__ out,
+                                        int hidden, float eps) {
+    extern __shared__ float staged[];
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    float* res = residual + static_cast<size_t>(row) * hidden;
+    const bf16_t* add = branch ? branch + static_cast<size_t>(row) * hidden : nullptr;
+    float sum_sq = 0.f;
+    for (int h = threadIdx.x * 8; h < hidden; h += blockDim.x * 8) {
+        float4 x0 = *reinterpret_cast<const float4*>(res + h);
+        float4 x1 = *reinterpret_cast<const float4*>(res + h + 4);
+        if (add) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(add + h);
+            x0.x += __uint_as_float(raw.x << 16); x0.y += __uint_as_float(raw.x & 0xffff0000u);
+            x0.z += __uint_as_float(raw.y << 16); x0.w += __uint_as_float(raw.y & 0xffff0000u);
+            x1.x += __uint_as_float(raw.z << 16); x1.y += __uint_as_float(raw.z & 0xffff0000u);
+            x1.z += __uint_as_float(raw.w << 16); x1.w += __uint_as_float(raw.w & 0xffff0000u);
+            *reinterpret_cast<float4*>(res + h) = x0;
+            *reinterpret_cast<float4*>(res + h + 4) = x1;
+        }
+        *reinterpret_cast<float4*>(staged + h) = x0;
+        *reinterpret_cast<float4*>(staged + h + 4) = x1;
+        sum_sq += (x0.x * x0.x + x0.y * x0.y) + (x0.z * x0.z + x0.w * x0.w) + (x1.x * x1.x + x1.y * x1.y) +
+                  (x1.z * x1.z + x1.w * x1.w);
+    }
+    const float total = block_sum(sum_sq, scratch);
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    bf16_t* dst = out + static_cast<size_t>(row) * hidden;
+    for (int h = threadIdx.x * 8; h < hidden; h += blockDim.x * 8) {
+        const float4 x0 = *reinterpret_cast<const float4*>(staged + h);
+        const float4 x1 = *reinterpret_cast<const float4*>(staged + h + 4);
+        const uint4 raw = *reinterpret_cast<const uint4*>(weight + h);
+        uint4 packed;
+        packed.x = pack_bf16((x0.x * inv) * __uint_as_float(raw.x << 16), (x0.y * inv) * __uint_as_float(raw.x & 0xffff0000u));
+        packed.y = pack_bf16((x0.z * inv) * __uint_as_float(raw.y << 16), (x0.w * inv) * __uint_as_float(raw.y & 0xffff0000u));
+        packed.z = pack_bf16((x1.x * inv) * __uint_as_float(raw.z << 16), (x1.y * inv) * __uint_as_float(raw.z & 0xffff0000u));
+        packed.w = pack_bf16((x1.z * inv) * __uint_as_float(raw.w << 16), (x1.w * inv) * __uint_as_float(raw.w & 0xffff0000u));
+        *reinterpret_cast<uint4*>(dst + h) = packed;
+    }
+}
+
 template <typename T, typename W>
 static int launch_norm(hipStream_t s, float* residual, const void* branch, const void* weight,
                        void* out, const int* rows, int n_out, int hidden, float eps,
@@ -143,6 +186,12 @@ CIE_API int cie_add_rmsnorm(void* stream, int dtype, int wdtype, float* residual
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == CIE_F32 && wdtype == CIE_F32)
         return launch_norm<float, float>(s, residual, branch, weight, out, rows, n_out, hidden, eps, write_residual);
+    if (dtype == CIE_BF16 && wdtype == CIE_BF16 && !rows && write_residual && hidden % 8 == 0) {
+        add_rmsnorm_vec8_kernel<<<n_out, n_out <= 64 ? 1024 : 256, hidden * sizeof(float), s>>>(
+            residual, static_cast<const bf16_t*>(branch), static_cast<const bf16_t*>(weight), static_cast<bf16_t*>(out),
+            hidden, eps);
+        return cie_after_launch();
+    }
     if (dtype == CIE_BF16 && wdtype == CIE_BF16)
         return launch_norm<bf16_t, bf16_t>(s, residual, branch, weight, out, rows, n_out, hidden, eps, write_residual);
     if (dtype == CIE_BF16 && wdtype == CIE_F32)
