@@ -31,6 +31,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kKeysPerBlock = 32;
+constexpr int kTileWaves = 4;  // waves of a workgroup in the prompt form
+constexpr float kLazyRescale = 8.f;  // base-2 units a score may pass a row's reference before it moves
 
 struct AttentionArgs {
     const bf16_t* q;
@@ -56,6 +58,8 @@ struct AttentionArgs {
     int n_splits;
     int tokens_per_tile;
     int keys_per_split;  // multiple of kKeysPerBlock; 0 with one split
+    int n_tiles;
+    int xcds_per_head;  // prompt form: > 0 if every kv head has that many of the 8 XCDs (and their L2) to itself
     const int* max_context_dev;  // if set (a captured graph replays with other lengths): keys per split are
                                  // derived from this device value, the longest context of the step
 };
@@ -257,6 +261,323 @@ __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs 
     }
 }
 
+template <int D>
+struct KeyBlock {
+    uint4 k[2][D / 32];   // A operand of K.Q^T: key kt*16 + r, dimensions (j*4 + g)*8 .. +7
+    uint2 v[D / 16][2];   // B operand of P.V: dimension dt*16 + r, keys kt*16 + g*4 .. +3
+};
+
+// The prompt form: a workgroup of WAVES waves per (tile, kv head).  Every wave holds all rows of the tile
+// and takes every WAVES-th block of 32 keys, so each key and value is read once per workgroup, straight
+// from memory into the operand registers; the waves' partial results meet in LDS at the end.
+//  * Pages hold at least 16 keys here, so the 16 keys of a product lie in one page: page numbers and
+//    base addresses are wave-uniform (scalar loads and scalar arithmetic), and a lane's part of every
+//    address is the same for all blocks.
+//  * Loads run one block ahead of the products that use them (the key registers are free once the scores
+//    are made, the value registers once the output is updated), page numbers two blocks ahead.
+//  * Masks are applied only in blocks that reach the causal edge or the window's edge of some row.
+//  * The output accumulators stay in the accumulation registers for the whole loop; the vector ALU
+//    cannot multiply there, so the rescaling after a moved maximum (rare once the first blocks have set
+//    every row's scale) goes through a temporary, register by register.
+//  * Tiles are taken from the last to the first: in a prompt the last tiles see the most keys, and
+//    starting them first evens out the finish.
+__device__ __forceinline__ void scale_accumulator(float& acc, float factor) {
+    float t;
+    asm volatile(
+        "v_accvgpr_read_b32 %1, %0\n\t"
+        "v_mul_f32 %1, %1, %2\n\t"
+        "v_accvgpr_write_b32 %0, %1"
+        : "+a"(acc), "=&v"(t)
+        : "v"(factor));
+}
+
+template <int D, int RT, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(AttentionArgs a) {
+    constexpr int NK = D / 32;
+    constexpr int ND = D / 16;
+    constexpr int ROWS = 16 * RT;
+    constexpr int STEP = kKeysPerBlock * WAVES;
+    __shared__ float lds_ml[WAVES][ROWS][2];
+    __shared__ float lds_o[(WAVES > 1 ? WAVES - 1 : 1) * ND * 4 * kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    // Workgroups go to the 8 XCDs in turn (workgroup b to XCD b % 8), and each XCD has an L2 of its own.
+    // All tiles of a kv head read the same keys and values, so where the heads divide the XCDs a head's
+    // tiles are given to its own XCDs: that L2 then holds one head's cache instead of every head's.
+    int tile_index, kv_head;
+    if (a.xcds_per_head > 0) {
+        const int xcd = blockIdx.x & 7;
+        kv_head = xcd % a.kv_heads;
+        tile_index = (blockIdx.x >> 3) * a.xcds_per_head + xcd / a.kv_heads;
+    } else {
+        kv_head = blockIdx.x % a.kv_heads;
+        tile_index = blockIdx.x / a.kv_heads;
+    }
+    if (tile_index >= a.n_tiles) return;  // padding of the grid; the whole workgroup leaves
+    const int tile = a.n_tiles - 1 - tile_index;
+    const int group = a.q_heads / a.kv_heads;
+    const int seq = a.tile_seq[tile];
+    const int q0 = a.tile_q0[tile];
+    const int start = a.seq_start[seq];
+    const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
+    const int n_rows = n_tok * group;
+    const int first_row_token = a.q_start_loc[seq] + q0;
+    const int page_mask = (1 << a.page_shift) - 1;
+    const int* table = a.block_table + static_cast<size_t>(a.seq_slot[seq]) * a.table_width;
+    const float scale_log2 = a.scale * 1.44269504088896341f;
+    const int hi = start + q0 + n_tok;
+    const int lo = (a.window > 0) ? max(0, start + q0 + 1 - a.window) : 0;
+    const int range_begin = lo & ~(kKeysPerBlock - 1);
+    const int range_end = hi;
+    const int first_pos = start + q0;              // position of the tile's first token
+    const int last_pos = start + q0 + n_tok - 1;   // and of its last
+    const int last_group = (hi - 1) & ~15;         // the last 16 keys that have a page
+
+    uint4 qf[RT][NK];
+    int row_pos[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = rt * 16 + r;
+        const bool valid = row < n_rows;
+        const int tok = row / group;
+        const int head = row - tok * group;
+        row_pos[rt] = valid ? start + q0 + tok : -1;
+        const bf16_t* q_row = a.q + static_cast<size_t>(first_row_token + tok) * a.q_row_stride +
+                              static_cast<size_t>(kv_head * group + head) * D + g * 8;
+#pragma unroll
+        for (int j = 0; j < NK; ++j)  // product j takes dimensions (j*4 + g)*8 .. +7 of both operands
+            qf[rt][j] = valid ? *reinterpret_cast<const uint4*>(q_row + j * 32) : uint4{0, 0, 0, 0};
+    }
+    float m_run[RT], l_run[RT];
+    float o[RT][ND][4];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        m_run[rt] = -INFINITY;
+        l_run[rt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[rt][dt][i] = 0.f;
+    }
+
+    // a lane's share of the addresses, in bytes from the start of a (page, kv head)'s keys or values
+    const uint32_t k_lane = static_cast<uint32_t>(r * D + g * 8) * 2u;
+    uint32_t v_lane[ND];
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt) v_lane[dt] = static_cast<uint32_t>(((dt * 16 + r) << a.page_shift) + g * 4) * 2u;
+
+    // the wave-uniform rest: the 16 keys from `first` on (clamped to keys that have a page; what lies past
+    // the end is masked where it is used)
+    auto group_of = [&](int first) { return min(first, last_group); };
+    // block tables do not change while a kernel runs: read them through the constant address space, with a
+    // wave-uniform index, so that they come through the scalar cache and do not queue behind the key loads
+    typedef const __attribute__((address_space(4))) int* const_int_ptr;
+    const const_int_ptr table_c = (const_int_ptr)(uintptr_t)table;
+    auto page_of = [&](int first) {
+        return table_c[__builtin_amdgcn_readfirstlane(group_of(first) >> a.page_shift)];
+    };
+    auto load_keys = [&](int kb, const int (&page)[2], KeyBlock<D>& b) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            const int in_page = group_of(kb + kt * 16) & page_mask;
+            const char* base = reinterpret_cast<const char*>(
+                a.k_pool + (((static_cast<size_t>(page[kt]) * a.kv_heads + kv_head) << a.page_shift) + in_page) * D);
+#pragma unroll
+            for (int j = 0; j < NK; ++j) b.k[kt][j] = *reinterpret_cast<const uint4*>(base + k_lane + j * 64);
+        }
+    };
+    auto load_values = [&](int kb, const int (&page)[2], KeyBlock<D>& b) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            const int in_page = group_of(kb + kt * 16) & page_mask;
+            const char* base = reinterpret_cast<const char*>(
+                a.v_pool + ((static_cast<size_t>(page[kt]) * a.kv_heads + kv_head) * D << a.page_shift) + in_page);
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) b.v[dt][kt] = *reinterpret_cast<const uint2*>(base + v_lane[dt]);
+        }
+    };
+
+    KeyBlock<D> blk;
+    int page[2], page_next[2];
+    int kb = range_begin + wave * kKeysPerBlock;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+        page[kt] = page_of(kb + kt * 16);
+        page_next[kt] = page_of(kb + STEP + kt * 16);
+    }
+    load_keys(kb, page, blk);
+    load_values(kb, page, blk);
+    for (; kb < range_end; kb += STEP) {
+        floatx4 s[RT][2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < NK; ++j)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, blk.k[kt][j]),
+                                                                  __builtin_bit_cast(bf16x8, qf[rt][j]), acc, 0, 0, 0);
+                s[rt][kt] = acc;
+            }
+        load_keys(kb + STEP, page_next, blk);  // the next block's keys travel while this block's softmax runs
+        int page_after[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) page_after[kt] = page_of(kb + 2 * STEP + kt * 16);
+
+        // ---- running maxima of all row tiles first; masks only in blocks that reach a row's edge
+        const bool edge = kb + kKeysPerBlock - 1 > first_pos || (a.window > 0 && kb < last_pos + 1 - a.window);
+        float m_use[RT], alpha[RT];
+        bool moved = false;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            if (edge) {
+                const int pos = row_pos[rt];
+                const int row_lo = (a.window > 0) ? pos + 1 - a.window : 0;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = kb + kt * 16 + g * 4 + i;
+                        if (!(key <= pos && key >= row_lo)) s[rt][kt][i] = -INFINITY;
+                    }
+            }
+            float block_max = fmaxf(fmaxf(fmaxf(s[rt][0][0], s[rt][0][1]), fmaxf(s[rt][0][2], s[rt][0][3])),
+                                    fmaxf(fmaxf(s[rt][1][0], s[rt][1][1]), fmaxf(s[rt][1][2], s[rt][1][3])));
+            block_max = rows_max(block_max) * scale_log2;  // maxima are kept in scaled base-2 units
+            // the reference of a row moves only when a score passes it by more than kLazyRescale: until then
+            // probabilities may reach 2^kLazyRescale, which float32 sums and bfloat16 products hold as well
+            const float m_new = (block_max > m_run[rt] + kLazyRescale) ? block_max : m_run[rt];
+            m_use[rt] = (m_new == -INFINITY) ? 0.f : m_new;
+            alpha[rt] = __builtin_amdgcn_exp2f(m_run[rt] - m_use[rt]);  // m_run = -inf: 0, and l, O are 0 anyway
+            moved = moved || (m_new != m_run[rt]);
+            m_run[rt] = m_new;
+            l_run[rt] *= alpha[rt];
+        }
+        if (__any(moved)) {
+            // the products that wrote these accumulators were issued a whole score phase ago
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                float alpha_o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha[rt], g * 4 + i, kWave);
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) scale_accumulator(o[rt][dt][i], alpha_o[i]);
+            }
+            asm volatile("s_nop 7");  // before a product reads what was just written
+        }
+        // ---- probabilities (one fused multiply-add and one exp2 each) and O += P . V, row tile by row tile
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            float p_sum = 0.f;
+            uint32_t pw[4];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rt][kt][0], scale_log2, -m_use[rt]));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rt][kt][1], scale_log2, -m_use[rt]));
+                const float p2 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rt][kt][2], scale_log2, -m_use[rt]));
+                const float p3 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rt][kt][3], scale_log2, -m_use[rt]));
+                p_sum += (p0 + p1) + (p2 + p3);
+                pw[kt * 2] = pack_bf16(p0, p1);
+                pw[kt * 2 + 1] = pack_bf16(p2, p3);
+            }
+            l_run[rt] += p_sum;
+            const bf16x8 p_frag = __builtin_bit_cast(bf16x8, (uint4{pw[0], pw[1], pw[2], pw[3]}));
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                const uint4 v = uint4{blk.v[dt][0].x, blk.v[dt][0].y, blk.v[dt][1].x, blk.v[dt][1].y};
+                floatx4 acc = {o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]};
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_frag, __builtin_bit_cast(bf16x8, v), acc, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[rt][dt][i] = acc[i];
+            }
+        }
+        load_values(kb + STEP, page_next, blk);  // and its values while the next scores are made
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) page_next[kt] = page_after[kt];
+    }
+
+    // ---- the waves' partial results meet: statistics first, then one row tile at a time through LDS
+    float l_all[RT], own_weight[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const float l = rows_sum(l_run[rt]);
+        l_all[rt] = l;
+        own_weight[rt] = 1.f;
+        if (WAVES > 1 && g == 0) {
+            lds_ml[wave][rt * 16 + r][0] = m_run[rt];
+            lds_ml[wave][rt * 16 + r][1] = l;
+        }
+    }
+    if (WAVES > 1) {
+        __syncthreads();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            float m_all = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) m_all = fmaxf(m_all, lds_ml[w][rt * 16 + r][0]);
+            const float m_safe = (m_all == -INFINITY) ? 0.f : m_all;
+            float l = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w)
+                l += lds_ml[w][rt * 16 + r][1] * __builtin_amdgcn_exp2f(lds_ml[w][rt * 16 + r][0] - m_safe);
+            l_all[rt] = l;
+            own_weight[rt] = __builtin_amdgcn_exp2f(m_run[rt] - m_safe);
+        }
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int owner = rt % WAVES;
+        if (WAVES > 1) {
+            float w_o[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w_o[i] = __shfl(own_weight[rt], g * 4 + i, kWave);
+            if (rt > 0) __syncthreads();  // the tile before has been read
+            if (wave != owner) {
+                float* slot = lds_o + (wave < owner ? wave : wave - 1) * (ND * 4 * kWave);
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) slot[(dt * 4 + i) * kWave + lane] = o[rt][dt][i] * w_o[i];
+            } else {
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) o[rt][dt][i] *= w_o[i];
+            }
+            __syncthreads();
+            if (wave == owner) {
+#pragma unroll
+                for (int w = 0; w < WAVES - 1; ++w)
+#pragma unroll
+                    for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) o[rt][dt][i] += lds_o[w * (ND * 4 * kWave) + (dt * 4 + i) * kWave + lane];
+            }
+        }
+        if (wave == owner) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = rt * 16 + g * 4 + i;
+                const float l_row = __shfl(l_all[rt], g * 4 + i, kWave);
+                if (row < n_rows) {
+                    const int tok = row / group;
+                    const int head = row - tok * group;
+                    bf16_t* dst = a.out + static_cast<size_t>(first_row_token + tok) * a.q_heads * D +
+                                  static_cast<size_t>(kv_head * group + head) * D;
+                    const float inv = 1.0f / l_row;
+#pragma unroll
+                    for (int dt = 0; dt < ND; ++dt) dst[dt * 16 + r] = from_float<bf16_t>(o[rt][dt][i] * inv);
+                }
+            }
+        }
+    }
+}
+
 // Merge the splits of every (tile, kv head): out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M).
 // One workgroup per (tile, kv head, row); the splits' weights are made once in LDS, then every thread
 // sums its head dimensions over the splits with independent loads.
@@ -302,8 +623,24 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
 }
 
 template <int D>
-int launch_for_dim(hipStream_t s, const AttentionArgs& a, int n_tiles, int row_tiles) {
+int launch_for_dim(hipStream_t s, const AttentionArgs& a, int n_tiles, int row_tiles, int tile_waves) {
     dim3 grid(n_tiles, a.kv_heads, a.n_splits);
+    if (tile_waves == kTileWaves) {
+        grid = a.xcds_per_head > 0 ? dim3(8 * ((n_tiles + a.xcds_per_head - 1) / a.xcds_per_head))
+                                   : dim3(static_cast<unsigned>(n_tiles) * a.kv_heads);
+        if (row_tiles == 1)
+            paged_attention_tile_kernel<D, 1, kTileWaves><<<grid, 64 * kTileWaves, 0, s>>>(a);
+        else if constexpr (D <= 128) {  // wider heads hold one row tile of accumulators without spilling
+            if (row_tiles == 2)
+                paged_attention_tile_kernel<D, 2, kTileWaves><<<grid, 64 * kTileWaves, 0, s>>>(a);
+            else if (row_tiles == 4)
+                paged_attention_tile_kernel<D, 4, kTileWaves><<<grid, 64 * kTileWaves, 0, s>>>(a);
+            else
+                return CIE_BAD_ARGUMENT;
+        } else
+            return CIE_BAD_ARGUMENT;
+        return cie_after_launch();
+    }
     if (row_tiles == 1)
         paged_attention_mfma_kernel<D, 1><<<grid, 64, 0, s>>>(a);
     else if (row_tiles == 2)
@@ -327,7 +664,7 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
                                      void* out, float* part_o, float* part_ml, int n_tiles, int q_heads,
                                      int kv_heads, int head_dim, int page_size, int window, float scale,
                                      int n_splits, int tokens_per_tile, int row_tiles, int keys_per_split,
-                                     const int* max_context_dev) {
+                                     const int* max_context_dev, int tile_waves) {
     if (n_tiles < 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || page_size < 4 ||
         (page_size & (page_size - 1)) || table_width <= 0 || n_splits < 1 || n_splits > 65535 ||
         kv_heads > 65535 || tokens_per_tile < 1 || q_row_stride % 8)
@@ -335,6 +672,10 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     const int group = q_heads / kv_heads;
     if (tokens_per_tile * group > 16 * row_tiles) return CIE_BAD_ARGUMENT;
     if (n_splits > kMergeMaxSplits) return CIE_BAD_ARGUMENT;
+    // the prompt form takes maxima before scaling, which needs a positive scale, and keeps the 16 keys of a
+    // product in one page
+    if (tile_waves != 1 && (tile_waves != kTileWaves || n_splits != 1 || !(scale > 0.f) || page_size < 16))
+        return CIE_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml ||
                          (!max_context_dev && (keys_per_split <= 0 || keys_per_split % kKeysPerBlock))))
         return CIE_BAD_ARGUMENT;
@@ -366,14 +707,16 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     a.tokens_per_tile = tokens_per_tile;
     a.keys_per_split = n_splits > 1 ? keys_per_split : 0;
     a.max_context_dev = n_splits > 1 ? max_context_dev : nullptr;
+    a.n_tiles = n_tiles;
+    a.xcds_per_head = (kv_heads <= 8 && 8 % kv_heads == 0) ? 8 / kv_heads : 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;
     switch (head_dim) {
-        case 32: rc = launch_for_dim<32>(s, a, n_tiles, row_tiles); break;
-        case 64: rc = launch_for_dim<64>(s, a, n_tiles, row_tiles); break;
-        case 96: rc = launch_for_dim<96>(s, a, n_tiles, row_tiles); break;
-        case 128: rc = launch_for_dim<128>(s, a, n_tiles, row_tiles); break;
-        case 256: rc = launch_for_dim<256>(s, a, n_tiles, row_tiles); break;
+        case 32: rc = launch_for_dim<32>(s, a, n_tiles, row_tiles, tile_waves); break;
+        case 64: rc = launch_for_dim<64>(s, a, n_tiles, row_tiles, tile_waves); break;
+        case 96: rc = launch_for_dim<96>(s, a, n_tiles, row_tiles, tile_waves); break;
+        case 128: rc = launch_for_dim<128>(s, a, n_tiles, row_tiles, tile_waves); break;
+        case 256: rc = launch_for_dim<256>(s, a, n_tiles, row_tiles, tile_waves); break;
         default: return CIE_BAD_ARGUMENT;
     }
     if (rc != CIE_OK || n_splits == 1) return rc;

@@ -71,6 +71,27 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Reductions over the four 16-lane rows of a wave (lanes r, r+16, r+32, r+48; every lane gets the
+// result) with gfx950's row-swap instructions, which stay in the vector ALU: no round trip through LDS.
+// v_permlane16_swap(a, b) exchanges the odd rows of a with the even rows of b; v_permlane32_swap(a, b)
+// the upper half of a with the lower half of b.  Fed the same value twice, the two results hold, in
+// every lane, the lane's own value and its partner's.
+typedef unsigned swap_pair_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float rows_max(float v) {
+    swap_pair_t a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    swap_pair_t b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+__device__ __forceinline__ float rows_sum(float v) {
+    swap_pair_t a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    swap_pair_t b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Sum over a workgroup of up to 16 waves; every thread gets the result.
 // `scratch` is at least 16 floats of LDS; the call contains barriers.
 __device__ __forceinline__ float block_sum(float v, float* scratch) {

@@ -243,6 +243,7 @@ def paged_attention_generic(q: torch.Tensor, q_row_stride: int, k_pool: torch.Te
 
 
 MFMA_HEAD_DIMS = (32, 64, 96, 128, 256)
+TILE_WAVES = 4  # waves per workgroup of the prompt form of the matrix-core attention
 
 
 def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
@@ -252,13 +253,16 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
                          window: Optional[int], scale: float, tokens_per_tile: int, row_tiles: int,
                          n_splits: int = 1, keys_per_split: int = 0,
                          max_context_dev: Optional[torch.Tensor] = None,
-                         part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None) -> None:
+                         part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
+                         tile_waves: int = 1) -> None:
     """Matrix-core attention (bf16) for the tiles ``(tile_seq[i], tile_q0[i])``: tile i
     holds up to ``tokens_per_tile`` tokens of sequence ``tile_seq[i]`` from its
     ``tile_q0[i]``-th token of this step on.  Rows of other tokens of ``out`` are left alone.
     With ``n_splits > 1`` every tile's keys are cut into parts of ``keys_per_split``
     (a multiple of 32; or, with ``max_context_dev``, derived on the device from the
-    step's longest context) and merged through the workspaces."""
+    step's longest context) and merged through the workspaces.  ``tile_waves=4`` (the
+    prompt form, unsplit only) gives every tile a workgroup of four waves that share
+    the tile's keys among them."""
     _require(q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 2 and q.stride(1) == 1
              and q.stride(0) == q_row_stride, "q must be a bf16 GPU matrix with unit inner stride")
     _require(q.shape[1] >= q_heads * head_dim and q_row_stride % 8 == 0, f"q {tuple(q.shape)} does not fit")
@@ -279,6 +283,9 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
     _gpu("out", out, torch.bfloat16, 2)
     _require(out.shape[1] == q_heads * head_dim and out.shape[0] <= q.shape[0], f"out is {tuple(out.shape)}")
     _require(1 <= n_splits <= 65535, f"n_splits {n_splits} out of range")
+    _require(tile_waves == 1 or (tile_waves == TILE_WAVES and n_splits == 1 and scale > 0 and page_size >= 16
+                                 and (row_tiles == 1 or head_dim <= 128)),
+             f"tile_waves {tile_waves} with {n_splits} splits, {row_tiles} row tiles, head size {head_dim}, pages of {page_size}")
     if n_splits > 1:
         rows = 16 * row_tiles
         _require(part_o is not None and part_ml is not None, "split attention needs its workspaces")
@@ -296,7 +303,7 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
         _i(block_table.shape[1]), _ptr(tile_seq), _ptr(tile_q0), _ptr(seq_slot), _ptr(seq_start), _ptr(seq_q_len),
         _ptr(q_start_loc), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_tiles), _i(q_heads), _i(kv_heads),
         _i(head_dim), _i(page_size), _i(window or 0), _f(scale), _i(n_splits), _i(tokens_per_tile), _i(row_tiles),
-        _i(keys_per_split), _ptr(max_context_dev)))
+        _i(keys_per_split), _ptr(max_context_dev), _i(tile_waves)))
 
 
 def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,

@@ -109,7 +109,8 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
 
     bfloat16 with a head size the matrix-core kernel takes: sequences that bring
     one token go to the split-context decode form, prompt portions to the tiled
-    form with up to 64 rows per wave.  Everything else (float32, other head
+    form with up to 64 rows per tile (four waves per tile where pages hold at
+    least 16 keys, one wave otherwise).  Everything else (float32, other head
     sizes, groups of more than 16 heads, pages of fewer than 4 tokens): the
     generic kernel."""
     group = num_heads // num_kv_heads
@@ -143,19 +144,29 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
                                  n_tiles, *common, tokens_per_tile=1, row_tiles=1, n_splits=n_splits,
                                  keys_per_split=per_split, part_o=part_o, part_ml=part_ml)
-    # rows per wave: 64 share each key load best; fewer where that would leave SIMDs without a wave
-    # (about a thousand waves fill the GPU) or where the accumulators of a wide head would spill
-    row_tiles = 2 if head_dim > 128 else 4
     prompt_tokens = sum(n for n in batch.host_q_lens if n > 1)
-    while row_tiles > 1 and (prompt_tokens * group // (16 * row_tiles)) * num_kv_heads < 1024:
-        row_tiles //= 2
+    if page_size >= 16 and scale > 0:
+        # the prompt form: four waves share a tile's keys.  More rows per tile re-use each key more often,
+        # fewer tiles leave compute units idle: the most rows that still give most units a workgroup
+        tile_waves = ops.TILE_WAVES
+        row_tiles = 4 if head_dim <= 128 else 1
+        while row_tiles > 1 and -(-prompt_tokens * group // (16 * row_tiles)) * num_kv_heads < 192:
+            row_tiles //= 2
+    else:
+        # one wave per tile; fewer rows where that would leave SIMDs without a wave (about a thousand
+        # waves fill the GPU) or where the accumulators of a wide head would spill
+        tile_waves = 1
+        row_tiles = 2 if head_dim > 128 else 4
+        while row_tiles > 1 and (prompt_tokens * group // (16 * row_tiles)) * num_kv_heads < 1024:
+            row_tiles //= 2
     while 16 * row_tiles < group:
         row_tiles *= 2
     per_tile = (16 * row_tiles) // group
     tile_seq, tile_q0, n_tiles = batch.tiles(per_tile, decode=False)
     if n_tiles:
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
-                                 n_tiles, *common, tokens_per_tile=per_tile, row_tiles=row_tiles)
+                                 n_tiles, *common, tokens_per_tile=per_tile, row_tiles=row_tiles,
+                                 tile_waves=tile_waves)
     return out
 
 

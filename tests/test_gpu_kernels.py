@@ -183,7 +183,7 @@ def test_paged_attention_generic(ops, dtype, geometry):
 
 
 def run_mfma(ops, q_all, contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim, window,
-             scale, per_tile, row_tiles, n_splits=1, keys_per_split=0, decode_only=None):
+             scale, per_tile, row_tiles, n_splits=1, keys_per_split=0, decode_only=None, tile_waves=1):
     """Drive the matrix-core kernel the way the attention part does: tiles of
     ``per_tile`` tokens for the chosen sequences; returns [tokens, Hq*D] (rows of
     sequences that were not chosen stay zero)."""
@@ -212,7 +212,7 @@ def run_mfma(ops, q_all, contexts, q_lens, k_pool, v_pool, table, slots, q_heads
     ops.paged_attention_mfma(buffer, stride, k_pool, v_pool, table, as_dev(tile_seq), as_dev(tile_q0), len(tile_seq),
                              as_dev(slots), as_dev(contexts), as_dev(q_lens), as_dev(loc), out, q_heads, kv_heads,
                              head_dim, window, scale, per_tile, row_tiles, n_splits=n_splits,
-                             keys_per_split=keys_per_split, part_o=part_o, part_ml=part_ml)
+                             keys_per_split=keys_per_split, part_o=part_o, part_ml=part_ml, tile_waves=tile_waves)
     return out.float().cpu()
 
 
@@ -223,14 +223,18 @@ MFMA_GEOMETRY = [(16, 2, 128, 16), (4, 2, 32, 8), (3, 1, 32, 8), (6, 6, 64, 4), 
 
 @pytest.mark.parametrize("geometry", MFMA_GEOMETRY)
 @pytest.mark.parametrize("row_tiles", [1, 2, 4])
-def test_paged_attention_mfma_ragged(ops, geometry, row_tiles):
-    """The tiled form on a ragged batch (reference matrix of contexts and query
-    lengths, tests/remote_ragged_gpu_tests.py:118-121): portions with and without
-    context, lengths that do not fill a tile, single tokens at page edges."""
+@pytest.mark.parametrize("tile_waves", [1, 4])
+def test_paged_attention_mfma_ragged(ops, geometry, row_tiles, tile_waves):
+    """The tiled forms (one wave per tile; four waves that share a tile's keys) on
+    a ragged batch (reference matrix of contexts and query lengths,
+    tests/remote_ragged_gpu_tests.py:118-121): portions with and without context,
+    lengths that do not fill a tile, single tokens at page edges."""
     q_heads, kv_heads, head_dim, page_size = geometry
     group = q_heads // kv_heads
-    if group > 16 * row_tiles or (head_dim == 256 and row_tiles == 4):
-        pytest.skip("more heads per group than rows, or a variant the dispatcher never picks")
+    if group > 16 * row_tiles or (head_dim == 256 and row_tiles > (2 if tile_waves == 1 else 1)):
+        pytest.skip("more heads per group than rows, or a variant the kernel refuses")
+    if tile_waves == 4:
+        page_size = max(page_size, 16)  # the four-wave form keeps the 16 keys of a product in one page
     contexts = [0, 15, 16, 17, 127, 511, 1, 40]
     q_lens = [7, 1, 2, 16, 1, 33, 64, 5]
     lengths = [c + q for c, q in zip(contexts, q_lens)]
@@ -244,7 +248,7 @@ def test_paged_attention_mfma_ragged(ops, geometry, row_tiles):
         expected.append(plain_qwen2.causal_attention(q, *dense[s], scale, past_len=c))
     per_tile = (16 * row_tiles) // group
     out = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
-                   None, scale, per_tile, row_tiles)
+                   None, scale, per_tile, row_tiles, tile_waves=tile_waves)
     torch.testing.assert_close(out, torch.cat(expected), **tol(torch.bfloat16))
 
 
@@ -274,26 +278,28 @@ def test_paged_attention_mfma_decode_splits(ops, geometry, splits):
 
 @pytest.mark.parametrize("window", [5, 32, 100])
 def test_paged_attention_mfma_window(ops, window):
-    q_heads, kv_heads, head_dim, page_size = 4, 2, 64, 8
+    q_heads, kv_heads, head_dim = 4, 2, 64
     contexts = [0, 90, 300, 33]
     q_lens = [40, 1, 17, 1]
     lengths = [c + q for c, q in zip(contexts, q_lens)]
-    k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=74)
     scale = 1.0 / math.sqrt(head_dim)
-    g = torch.Generator().manual_seed(75)
-    qs, expected = [], []
-    for s, (c, n) in enumerate(zip(contexts, q_lens)):
-        q = (torch.randn((n, q_heads, head_dim), generator=g) * 2).to(torch.bfloat16).float()
-        qs.append(q.reshape(n, -1))
-        expected.append(plain_qwen2.causal_attention(q, *dense[s], scale, past_len=c, window=window))
-    want = torch.cat(expected)
-    tiled = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
-                     window, scale, 8, 1)
-    torch.testing.assert_close(tiled, want, **tol(torch.bfloat16))
-    split = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
-                     window, scale, 1, 1, n_splits=4, keys_per_split=32, decode_only=True)
-    rows = [40, 58]  # the two single-token sequences
-    torch.testing.assert_close(split[rows], want[rows], **tol(torch.bfloat16))
+    for page_size, variants in ((8, ((1, 1),)), (16, ((4, 1), (4, 2))), (64, ((4, 4),))):
+        k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=74)
+        g = torch.Generator().manual_seed(75)
+        qs, expected = [], []
+        for s, (c, n) in enumerate(zip(contexts, q_lens)):
+            q = (torch.randn((n, q_heads, head_dim), generator=g) * 2).to(torch.bfloat16).float()
+            qs.append(q.reshape(n, -1))
+            expected.append(plain_qwen2.causal_attention(q, *dense[s], scale, past_len=c, window=window))
+        want = torch.cat(expected)
+        for tile_waves, row_tiles in variants:
+            tiled = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads,
+                             head_dim, window, scale, 8 * row_tiles, row_tiles, tile_waves=tile_waves)
+            torch.testing.assert_close(tiled, want, **tol(torch.bfloat16))
+        split = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads,
+                         head_dim, window, scale, 1, 1, n_splits=4, keys_per_split=32, decode_only=True)
+        rows = [40, 58]  # the two single-token sequences
+        torch.testing.assert_close(split[rows], want[rows], **tol(torch.bfloat16))
 
 
 def test_paged_attention_mfma_far_key(ops):
@@ -311,6 +317,16 @@ def test_paged_attention_mfma_far_key(ops):
                        head_dim, None, scale, 1, 1, n_splits=n_splits, keys_per_split=per_split)
         torch.testing.assert_close(out, expect, **tol(torch.bfloat16))
         torch.testing.assert_close(out.view(q_heads, head_dim), v[far].repeat_interleave(8, dim=0), rtol=0.05, atol=0.05)
+    # the prompt form: the last of 40 tokens asks for the far key; the four waves of its tile each see a
+    # quarter of the keys and only one of them holds the key that counts
+    q_many = torch.cat([torch.randn((39, q_heads, head_dim), generator=torch.Generator().manual_seed(77)), q])
+    q_many = q_many.to(torch.bfloat16).float()
+    expect = plain_qwen2.causal_attention(q_many, k, v, scale, past_len=length - 40)
+    for row_tiles in (1, 2, 4):
+        out = run_mfma(ops, q_many.reshape(40, -1), [length - 40], [40], k_pool, v_pool, table, slots, q_heads,
+                       kv_heads, head_dim, None, scale, 2 * row_tiles, row_tiles, tile_waves=4)
+        torch.testing.assert_close(out, expect, **tol(torch.bfloat16))
+        torch.testing.assert_close(out[-1].view(q_heads, head_dim), v[far].repeat_interleave(8, dim=0), rtol=0.05, atol=0.05)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

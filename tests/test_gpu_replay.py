@@ -86,6 +86,32 @@ def test_replay_matches_plain(tiny_folders, plain, name, schedule, dtype):
     assert runner.cache.stats().pages_used == 0
 
 
+@pytest.mark.parametrize("schedule", ["whole", "portions", "mixed"])
+@pytest.mark.parametrize("page", [16, 64])
+def test_replay_with_the_four_wave_prompt_attention(tiny_folders, plain, monkeypatch, schedule, page):
+    """Pages of 16 keys and more send prompt portions to the attention form in which
+    four waves share a tile's keys (Tiny-B: head size 32, three heads per group)."""
+    from cie_amd.kernels import ops
+
+    seen = []
+    real = ops.paged_attention_mfma
+
+    def spy(*args, **kwargs):
+        seen.append(kwargs.get("tile_waves", 1))
+        return real(*args, **kwargs)
+
+    monkeypatch.setattr(ops, "paged_attention_mfma", spy)
+    folder, raw, _ = tiny_folders["B"]
+    requests, expected = plain["B"]
+    steps = SCHEDULES[schedule](requests)
+    pool = replay_util.max_live_tokens(steps, page=page)
+    runner = make_runner(folder, "bfloat16", pool, page)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    replay_util.compare(rows, expected, **TOL["bfloat16"])
+    assert ops.TILE_WAVES in seen
+    assert runner.cache.stats().pages_used == 0
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_captured_decode_steps_match_plain(tiny_folders, plain, name, dtype):
