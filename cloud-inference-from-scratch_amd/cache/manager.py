@@ -270,6 +270,13 @@ class CacheManager:
         self._free_slots.append(slot)
 
     # -- prefix index -----------------------------------------------------------
+    def publish_prefix(self, request_id: str, prompt_tokens: Sequence[int]) -> int:
+        """Offer the full prompt pages a live request has committed to the prefix index; the request
+        keeps them (a page then has two holders and is read-only for both).  Returns the tokens indexed."""
+        if request_id not in self._slots or not self.prefix_cache_pages:
+            return 0
+        return self._store_prefix(request_id, prompt_tokens)
+
     def _restore_prefix(self, request_id: str, tokens: Sequence[int]) -> int:
         group = self.groups[0]
         candidate_pages = (len(tokens) - 1) // self.page_size

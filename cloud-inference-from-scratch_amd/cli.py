@@ -64,6 +64,8 @@ def parser() -> argparse.ArgumentParser:
     replay.add_argument("rest", nargs=argparse.REMAINDER)
     bench = commands.add_parser("bench", help="the serving benchmark (bench.py)", add_help=False)
     bench.add_argument("rest", nargs=argparse.REMAINDER)
+    workload = commands.add_parser("workload", help="an offline serving workload with random weights", add_help=False)
+    workload.add_argument("rest", nargs=argparse.REMAINDER)
     return cli
 
 
@@ -100,7 +102,12 @@ def _run_script(path: Path, rest: list[str]) -> int:
 
 
 def main(argv: list[str] | None = None) -> int:
-    args = parser().parse_args(argv)
+    argv = list(sys.argv[1:] if argv is None else argv)
+    if argv and argv[0] in ("replay", "bench", "workload"):
+        # these hand all their options on; argparse would claim the ones that start with a dash
+        args = argparse.Namespace(command=argv[0], rest=argv[1:])
+    else:
+        args = parser().parse_args(argv)
     if args.command == "models":
         from .config import ARCHITECTURES
 
@@ -118,6 +125,10 @@ def main(argv: list[str] | None = None) -> int:
         return _run_script(ROOT / "bin" / "trace_run", args.rest)
     if args.command == "bench":
         return _run_script(ROOT / "bench.py", args.rest)
+    if args.command == "workload":
+        from .workloads import main as workload_main
+
+        return workload_main([r for r in args.rest if r != "--"])
 
     from .engine import GenerationConfig
 

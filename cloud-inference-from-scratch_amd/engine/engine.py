@@ -114,6 +114,12 @@ class Engine:
     def step(self) -> bool:
         return self.scheduler.step()
 
+    def warm_up(self) -> int:
+        """Capture the decode graphs of all bucket sizes before the first request (a serving process
+        does this at start; otherwise each bucket is captured by the first step that needs it)."""
+        warm = getattr(self.runner, "warm_up", None)
+        return warm() if warm is not None else 0
+
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 

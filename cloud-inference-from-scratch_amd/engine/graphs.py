@@ -125,6 +125,18 @@ class DecodeGraphs:
         self.captures += 1
         return bucket
 
+    def capture_all(self) -> int:
+        """Capture every bucket that is not captured yet (rows of padding only), so that no later step
+        pays for a capture; returns how many were made."""
+        made = 0
+        size = 1
+        while size <= self.largest:
+            if size not in self.buckets:
+                self._capture(size)
+                made += 1
+            size *= 2
+        return made
+
     def run(self, entries: Sequence[Any]) -> torch.Tensor:
         """Replay the bucket's graph for single-token entries; logits [wanted, vocab]."""
         runner = self.runner

@@ -84,6 +84,16 @@ class Runner:
     def release(self, request: Any, preempted: bool = False) -> None:
         self.cache.release(request.request_id, None if preempted else request.prompt_token_ids)
 
+    def warm_up(self) -> int:
+        """Do now what the first steps would otherwise do on the clock: capture the decode graphs of
+        all bucket sizes.  Returns the number of graphs captured."""
+        return self.graphs.capture_all() if self.graphs is not None else 0
+
+    def publish_prefix(self, request: Any) -> None:
+        """The request's prompt is in the cache: offer its full pages to the prefix index now, not only
+        when it ends (the reference stores at release, src/cloud_engine/engine.py:224-226)."""
+        self.cache.publish_prefix(request.request_id, request.prompt_token_ids)
+
     def allocated_tokens(self, request: Any) -> int:
         return self.cache.allocated_tokens(request.request_id)
 

@@ -192,6 +192,7 @@ class Scheduler:
         self.finished: deque[Request] = deque(maxlen=4096)
         self._counter = 0
         self._release_takes_flag = "preempted" in inspect.signature(runner.release).parameters
+        self._publish_prefix = getattr(runner, "publish_prefix", None)
 
     # -- public ------------------------------------------------------------------
     def submit(self, prompt_token_ids: Sequence[int], gen_config: GenerationConfig, label: str = "",
@@ -369,6 +370,7 @@ class Scheduler:
             self.runner.release(request)
 
     def _after_token(self, request: Request, token_id: int, now: int) -> None:
+        finished_prompt = request.state is RequestState.PREFILL
         request.generated_token_ids.append(token_id)
         if request.first_token_ns is None:
             request.first_token_ns = now
@@ -390,6 +392,10 @@ class Scheduler:
             self._finalize(request)
         else:
             request.state = RequestState.DECODING
+            if finished_prompt and self._publish_prefix is not None:
+                # the prompt's full pages are final from here on: requests that arrive while this one
+                # still decodes can already share them
+                self._publish_prefix(request)
 
     def _fail(self, request: Request, detail: str, rejected: bool = False) -> None:
         if request.is_terminal:

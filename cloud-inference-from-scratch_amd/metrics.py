@@ -23,6 +23,12 @@ def percentile(values: list[float], pct: float) -> float:
 
 class Metrics:
     def __init__(self, latency_capacity: int = 4096) -> None:
+        self._latency_capacity = latency_capacity
+        self.reset()
+
+    def reset(self) -> None:
+        """Forget everything recorded so far (after a warm-up, before a measured run)."""
+        latency_capacity = self._latency_capacity
         self._ttft: deque[float] = deque(maxlen=latency_capacity)
         self._itl: deque[float] = deque(maxlen=latency_capacity)
         self._e2e: deque[float] = deque(maxlen=latency_capacity)

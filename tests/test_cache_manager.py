@@ -293,6 +293,31 @@ def test_prefix_not_stored_on_preemption_nor_beyond_committed_length():
     assert m.stats().prefix_pages_used == 1
 
 
+def test_prefix_published_by_a_live_request_is_shared_and_outlives_it():
+    m = manager(prefix_cache_pages=8)
+    prompt = list(range(10))
+    m.admit("a", prompt)
+    m.ensure_capacity_batch({"a": 10})
+    m.commit_lengths({"a": 6})
+    assert m.publish_prefix("a", prompt) == 4  # only what is committed
+    m.commit_lengths({"a": 10})
+    assert m.publish_prefix("a", prompt) == 8  # full pages before the last prompt token
+    assert m.publish_prefix("a", prompt) == 8 and m.stats().prefix_pages_used == 2  # again: nothing new
+    pages = m.block_table(0, "a")
+    # a second request arrives while the first is still alive: same pages, three holders in all
+    assert m.admit("b", prompt[:8] + [50, 51]) == 8 and m.block_table(0, "b") == pages[:2]
+    assert set(m.groups[0].allocator.holders_of(pages[0])) == {"a", "b", PREFIX_HOLDER}
+    m.ensure_capacity_batch({"a": 14, "b": 12})  # both go on writing behind the shared pages
+    assert m.block_table(0, "a")[:2] == m.block_table(0, "b")[:2] and m.block_table(0, "a")[2] != m.block_table(0, "b")[2]
+    m.assert_invariants()
+    m.release("a")  # preempted or ended without storing: the index and b keep the pages
+    assert m.groups[0].allocator.holders_of(pages[0]) == ("b", PREFIX_HOLDER) or \
+        set(m.groups[0].allocator.holders_of(pages[0])) == {"b", PREFIX_HOLDER}
+    m.release("b", prompt[:8] + [50, 51])
+    assert m.stats().pages_used == 2 and m.publish_prefix("gone", prompt) == 0
+    m.assert_invariants()
+
+
 def test_prefix_entries_are_bounded_and_evicted_before_a_request_starves():
     m = manager(kv_tokens=32, prefix_cache_pages=3)  # 8 pages
     for i in range(3):

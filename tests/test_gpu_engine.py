@@ -152,6 +152,53 @@ def test_prefix_reuse_keeps_tokens_and_saves_work(tiny_folders):
     engine.runner.cache.assert_invariants()
 
 
+def test_prefix_is_shared_with_a_request_that_arrives_while_the_first_still_decodes(tiny_folders):
+    """The first request's prompt pages are offered to the index when its prompt is
+    done, not when it ends: a sibling submitted during its decoding takes them over,
+    both go on writing behind the shared pages, and both match the plain model."""
+    from cie_amd import GenerationConfig
+    from cie_amd.engine import RequestState
+
+    folder, raw, tensors = tiny_folders["A"]
+    prompt = random_tokens(45, raw["vocab_size"], 610)
+    sibling = prompt[:32] + random_tokens(9, raw["vocab_size"], 611)
+    gen = GenerationConfig(max_output_tokens=12, eos_token_id=None)
+    engine = make_engine(folder, page_size=16, prefix_cache_pages=8)
+    first = engine.submit(prompt, gen)
+    while first.generated_count < 3:
+        engine.step()
+    assert first.state is RequestState.DECODING
+    second = engine.submit(sibling, gen)
+    while engine.has_work():
+        engine.step()
+    weights = float_weights(tensors)
+    assert engine.result_of(first).token_ids == plain.generate_greedy(raw, weights, prompt, 12)
+    assert engine.result_of(second).token_ids == plain.generate_greedy(raw, weights, sibling, 12)
+    cache = engine.snapshot_metrics()["kv_cache"]
+    assert cache["prefix_cache_hits"] == 1 and cache["request_pages_used"] == 0
+    # tokens run through the model: both prompts less the 32 shared tokens, plus the decoded tokens fed back
+    assert engine.snapshot_metrics()["tokens"]["input_total"] <= len(prompt) + len(sibling) - 32 + 2 * 12
+    engine.runner.cache.assert_invariants()
+
+
+def test_warm_up_captures_every_decode_bucket_once(tiny_folders):
+    from cie_amd import GenerationConfig
+
+    folder, raw, tensors = tiny_folders["B"]
+    engine = make_engine(folder, dtype="bfloat16", max_running=6, graph_decode=True)
+    assert engine.warm_up() == 4  # buckets of 1, 2, 4 and 8 rows for up to 6 requests
+    assert engine.warm_up() == 0
+    prompts = [random_tokens(n, raw["vocab_size"], 700 + n) for n in (3, 9, 20, 33, 40)]
+    results = engine.generate(prompts, GenerationConfig(max_output_tokens=10, eos_token_id=None))
+    runner = engine.snapshot_metrics()["runner"]
+    assert runner["graph_captures"] == 4 and runner["graph_replays"] >= 9
+    weights = float_weights(tensors)
+    for prompt, result in zip(prompts, results):
+        # bfloat16 may flip a near-tie: the first token at least is the plain model's, and all are valid ids
+        assert result.token_ids[0] == plain.generate_greedy(raw, weights, prompt, 1)[0]
+        assert len(result.token_ids) == 10
+
+
 def test_step_refuses_what_it_cannot_run(tiny_folders):
     from cie_amd.cache import CacheCapacityFull
     from cie_amd.engine.runner import StepEntry

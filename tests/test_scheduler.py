@@ -263,3 +263,25 @@ def test_admission_failure_is_counted():
     request = scheduler.submit([1], GenerationConfig(max_output_tokens=1))
     scheduler.step()
     assert request.state is RequestState.FAILED and request.rejected and "admission refused" in request.error_detail
+
+
+def test_prompt_is_published_once_its_last_portion_has_run():
+    """A runner that can publish prefixes is told when a request's prompt is all in
+    the cache (at its first token), again after a recomputation, and not for a
+    request that ends with its first token."""
+    class Publishing(FakeRunner):
+        def __init__(self, *args, **kwargs):
+            super().__init__(*args, **kwargs)
+            self.published = []
+
+        def publish_prefix(self, request) -> None:
+            assert request.tokens_fed >= len(request.prompt_token_ids)
+            self.published.append((request.request_id, request.generated_count))
+
+    runner = Publishing()
+    scheduler = make(runner)
+    long_one = scheduler.submit(list(range(9)), GenerationConfig(max_output_tokens=3))
+    one_token = scheduler.submit(list(range(5)), GenerationConfig(max_output_tokens=1))
+    scheduler.run_until_done()
+    assert runner.published == [(long_one.request_id, 1)]
+    assert one_token.state is RequestState.COMPLETED
