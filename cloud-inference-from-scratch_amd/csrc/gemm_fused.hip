@@ -14,16 +14,14 @@
 //   PARTIAL     K is cut into grid.z parts; part p writes acc to C[p, m, n] (float32, bias in
 //               part 0).  The add + norm kernel sums the parts.  For few columns and long K.
 //
-// Two kernels:
-//   rows16  M <= 16.  One workgroup per tile of 16 columns (SILU: a gate tile and its up tile);
-//           its WAVES waves cut K into slices of 128 and take them round-robin; every lane
-//           loads its own row of A and of W for the same k values straight into MFMA
-//           operands; the waves' partial tiles are summed through LDS in wave order.
-//   rows64  M <= 64 per workgroup.  Four waves own four column tiles and share the slice of A
-//           that all threads stage in LDS; every lane streams its row of W.
-// Both use v_mfma_f32_16x16x32_bf16 with A = activations (16 rows), B = weight rows; the four
-// lane groups of a wave read one contiguous 64-byte piece of each weight row per load, and the
-// same k values of A (the order of k inside a product is free as long as both operands agree).
+// One kernel: a workgroup owns one or two tiles of 16 columns (SILU: a gate tile and its up tile)
+// and 16, 32 or 64 rows; its WAVES waves cut K into slices of 128 and take them round-robin;
+// every lane loads its own rows of A and of W for the same k values straight into MFMA operands
+// (W from memory, once; the few rows of A from the cache); the waves' partial tiles are summed
+// through LDS in wave order.  v_mfma_f32_16x16x32_bf16 with A = activations (16 rows), B = weight
+// rows; the four lane groups of a wave read one contiguous 64-byte piece of each weight row per
+// load, and the same k values of A (the order of k inside a product is free as long as both
+// operands agree).
 // No workgroup ever waits for another: a device-wide fence between workgroups costs more on
 // this GPU than the whole product.
 #include "common.h"
@@ -94,32 +92,50 @@ __device__ __forceinline__ void store_tile(const FusedArgs& a, const floatx4& ac
 }
 
 // ---------------------------------------------------------------------------------------------
-template <int WAVES, int EPI>
-__global__ void __launch_bounds__(WAVES * 64) gemm_rows16_kernel(FusedArgs a) {
-    constexpr int NT = (EPI == EPI_SILU) ? 2 : 1;
-    constexpr int U = (NT == 1) ? 4 : 2;  // slices of 128 k values whose loads are in flight together
-    __shared__ float reduce[WAVES > 1 ? (WAVES - 1) * NT * 64 * 4 : 1];
+// MT row tiles (M <= 16*MT per workgroup row; more rows: more workgroup rows) and NT column tiles
+// per workgroup: with SILU the gate tile and its up tile, else NT adjacent tiles.  Every weight
+// value a wave loads meets all MT row tiles; every activation value meets the NT column tiles.
+template <int WAVES, int EPI, int MT, int NT>
+__global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
+    static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
+    // slices of 128 k values whose weight loads are in flight together
+    constexpr int U = (MT == 1 && NT == 1) ? 4 : (MT == 4) ? 1 : 2;
+    __shared__ float reduce[WAVES > 1 ? (WAVES - 1) * MT * NT * 64 * 4 : 1];
 
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int r = lane & 15;
     const int g = lane >> 4;
-    const int n_first = blockIdx.x * 16;
+    const int m0 = blockIdx.y * (16 * MT);
     const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
-    const int n_row = min(n_first + r, cols - 1);  // a column past the end computes a copy that is not stored
+    const int tile_first = (EPI == EPI_SILU) ? blockIdx.x : blockIdx.x * NT;
 
+    // a column past the end computes a copy that is not stored
     const bf16_t* w_row[NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) w_row[t] = a.w + static_cast<size_t>(n_row + t * a.up_offset) * a.K + g * 8;
-    const bf16_t* a_row = a.a + static_cast<size_t>(min(r, a.M - 1)) * a.lda + g * 8;
-    const bool row_ok = r < a.M;
-
-    floatx4 acc[NT];
+    for (int t = 0; t < NT; ++t) {
+        const int n = (EPI == EPI_SILU) ? min(tile_first * 16 + r, cols - 1) + t * a.up_offset
+                                        : min((tile_first + t) * 16 + r, cols - 1);
+        w_row[t] = a.w + static_cast<size_t>(n) * a.K + g * 8;
+    }
+    const bf16_t* a_row[MT];
+    bool row_ok[MT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = m0 + mt * 16 + r;
+        row_ok[mt] = m < a.M;
+        a_row[mt] = a.a + static_cast<size_t>(min(m, a.M - 1)) * a.lda + g * 8;
+    }
+
+    floatx4 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     const int k_begin = blockIdx.z * a.k_per_part;
     const int k_end = min(a.K, k_begin + a.k_per_part);
+#pragma unroll 1
     for (int kbase = k_begin + wave * 128; kbase < k_end; kbase += U * WAVES * 128) {
         uint4 b[U][NT][4];
 #pragma unroll
@@ -133,156 +149,123 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows16_kernel(FusedArgs a) {
             }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            uint4 av[4];  // the few rows of A come from the cache; their loads are issued slice by slice
+            // the few rows of A come from the cache; their loads are issued slice by slice
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int k0 = kbase + u * WAVES * 128 + j * 32;
-                av[j] = (row_ok && k0 + g * 8 < k_end) ? *reinterpret_cast<const uint4*>(a_row + k0) : uint4{0, 0, 0, 0};
+            for (int mt = 0; mt < MT; ++mt) {
+                uint4 av[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int k0 = kbase + u * WAVES * 128 + j * 32;
+                    av[j] = (row_ok[mt] && k0 + g * 8 < k_end) ? *reinterpret_cast<const uint4*>(a_row[mt] + k0)
+                                                               : uint4{0, 0, 0, 0};
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int t = 0; t < NT; ++t)
+                        acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8, av[j]), __builtin_bit_cast(bf16x8, b[u][t][j]), acc[mt][t], 0, 0, 0);
             }
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int t = 0; t < NT; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        __builtin_bit_cast(bf16x8, av[j]), __builtin_bit_cast(bf16x8, b[u][t][j]), acc[t], 0, 0, 0);
         }
     }
 
     if (WAVES > 1) {  // sum the waves' partial tiles in wave order; wave 0 keeps the result
         if (wave > 0) {
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
+            for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) reduce[(((wave - 1) * NT + t) * 4 + i) * 64 + lane] = acc[t][i];
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        reduce[((((wave - 1) * MT + mt) * NT + t) * 4 + i) * 64 + lane] = acc[mt][t][i];
         }
         __syncthreads();
         if (wave > 0) return;
+        // many tiles: one wave's partial tiles at a time, or the loads of all of them would not fit the registers
+        constexpr int kWavesAtOnce = (MT * NT > 2) ? 1 : WAVES;
+#pragma unroll kWavesAtOnce
         for (int w = 1; w < WAVES; ++w)
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[t][i] += reduce[(((w - 1) * NT + t) * 4 + i) * 64 + lane];
-    }
-    store_tile<EPI>(a, acc[0], acc[NT - 1], 0, n_first + r, blockIdx.x, lane);
-}
-
-// ---------------------------------------------------------------------------------------------
-template <int MT, int EPI>
-__global__ void __launch_bounds__(256) gemm_rows64_kernel(FusedArgs a) {
-    constexpr int NT = (EPI == EPI_SILU) ? 2 : 1;
-    constexpr int STRIDE = 128 + 8;  // staged row stride in bf16 elements (padding against bank conflicts)
-    __shared__ __attribute__((aligned(16))) uint16_t a_lds[MT * 16 * STRIDE];
-
-    const int lane = threadIdx.x % kWave;
-    const int wave = threadIdx.x / kWave;
-    const int r = lane & 15;
-    const int g = lane >> 4;
-    const int m0 = blockIdx.y * (MT * 16);
-    const int n_first = (blockIdx.x * 4 + wave) * 16;
-    const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
-    const int n_row = min(n_first + r, cols - 1);
-
-    const bf16_t* w_row[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) w_row[t] = a.w + static_cast<size_t>(n_row + t * a.up_offset) * a.K + g * 8;
-
-    floatx4 acc[MT][NT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    const int k_begin = blockIdx.z * a.k_per_part;
-    const int k_end = min(a.K, k_begin + a.k_per_part);
-    for (int k0 = k_begin; k0 < k_end; k0 += 128) {
-        uint4 b[NT][4];  // requested before the barrier so that they travel while A is staged
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                b[t][j] = (k0 + j * 32 + g * 8 < k_end) ? *reinterpret_cast<const uint4*>(w_row[t] + k0 + j * 32)
-                                                         : uint4{0, 0, 0, 0};
-        __syncthreads();  // the previous slice's readers are done with a_lds
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const int piece = threadIdx.x + 256 * i;  // 16 pieces of 8 k values per row
-            const int row = piece / 16;
-            const int col = (piece % 16) * 8;
-            const int m = m0 + row;
-            const int k = k0 + col;
-            const uint4 v = (m < a.M && k < k_end) ? *reinterpret_cast<const uint4*>(a.a + static_cast<size_t>(m) * a.lda + k)
-                                                   : uint4{0, 0, 0, 0};
-            *reinterpret_cast<uint4*>(&a_lds[row * STRIDE + col]) = v;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint4 av = *reinterpret_cast<const uint4*>(&a_lds[(mt * 16 + r) * STRIDE + j * 32 + g * 8]);
+            for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int t = 0; t < NT; ++t)
-                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                        __builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, b[t][j]), acc[mt][t], 0, 0, 0);
-            }
-    }
-    if (n_first >= cols) return;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-        store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, n_first + r, n_first / 16, lane);
+                    for (int i = 0; i < 4; ++i)
+                        acc[mt][t][i] += reduce[((((w - 1) * MT + mt) * NT + t) * 4 + i) * 64 + lane];
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        if (EPI == EPI_SILU) {
+            store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, tile_first * 16 + r, tile_first, lane);
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                if ((tile_first + t) * 16 < cols)  // wave-uniform
+                    store_tile<EPI>(a, acc[mt][t], acc[mt][t], m0 + mt * 16, (tile_first + t) * 16 + r, tile_first + t, lane);
+        }
+    }
 }
 
-template <int EPI>
-int launch_rows16(hipStream_t s, int waves, dim3 grid, const FusedArgs& a) {
-    switch (waves) {
-        case 1: gemm_rows16_kernel<1, EPI><<<grid, 64, 0, s>>>(a); break;
-        case 2: gemm_rows16_kernel<2, EPI><<<grid, 128, 0, s>>>(a); break;
-        case 4: gemm_rows16_kernel<4, EPI><<<grid, 256, 0, s>>>(a); break;
-        case 8: gemm_rows16_kernel<8, EPI><<<grid, 512, 0, s>>>(a); break;
-        default: return CIE_BAD_ARGUMENT;
+template <int EPI, int MT, int NT>
+int launch_waves(hipStream_t s, int waves, dim3 grid, const FusedArgs& a) {
+    if constexpr (MT == 1) {
+        switch (waves) {
+            case 1: gemm_rows_kernel<1, EPI, MT, NT><<<grid, 64, 0, s>>>(a); break;
+            case 2: gemm_rows_kernel<2, EPI, MT, NT><<<grid, 128, 0, s>>>(a); break;
+            case 4: gemm_rows_kernel<4, EPI, MT, NT><<<grid, 256, 0, s>>>(a); break;
+            case 8: gemm_rows_kernel<8, EPI, MT, NT><<<grid, 512, 0, s>>>(a); break;
+            default: return CIE_BAD_ARGUMENT;
+        }
+    } else {  // more row tiles: four or eight waves (waves that find no slice of K add zeros)
+        switch (waves) {
+            case 4: gemm_rows_kernel<4, EPI, MT, NT><<<grid, 256, 0, s>>>(a); break;
+            case 8: gemm_rows_kernel<8, EPI, MT, NT><<<grid, 512, 0, s>>>(a); break;
+            default: return CIE_BAD_ARGUMENT;
+        }
     }
     return cie_after_launch();
 }
 
 template <int EPI>
-int launch_rows64(hipStream_t s, int row_tiles, dim3 grid, const FusedArgs& a) {
-    if constexpr (EPI == EPI_RESID) {
-        return CIE_BAD_ARGUMENT;  // the sums of squares of a row need one workgroup per row block and tile: rows16 only
-    } else {
-        switch (row_tiles) {
-            case 2: gemm_rows64_kernel<2, EPI><<<grid, 256, 0, s>>>(a); break;
-            case 4: gemm_rows64_kernel<4, EPI><<<grid, 256, 0, s>>>(a); break;
-            default: return CIE_BAD_ARGUMENT;
-        }
-        return cie_after_launch();
-    }
-}
-
-template <int EPI>
-int launch(hipStream_t s, int row_tiles, int waves, int k_parts, const FusedArgs& a) {
+int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, int k_parts, const FusedArgs& a) {
     const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
     const int tiles = (cols + 15) / 16;
-    if (row_tiles == 1) return launch_rows16<EPI>(s, waves, dim3(tiles, 1, k_parts), a);
     const int m_blocks = (a.M + 16 * row_tiles - 1) / (16 * row_tiles);
     if (m_blocks > 65535) return CIE_BAD_ARGUMENT;
-    return launch_rows64<EPI>(s, row_tiles, dim3((tiles + 3) / 4, m_blocks, k_parts), a);
+    constexpr int NT1 = (EPI == EPI_SILU) ? 2 : 1;  // the SiLU epilogue always pairs a gate tile with its up tile
+    if (row_tiles == 1) {
+        if (column_tiles != 1) return CIE_BAD_ARGUMENT;
+        return launch_waves<EPI, 1, NT1>(s, waves, dim3(tiles, m_blocks, k_parts), a);
+    }
+    if (EPI == EPI_SILU || column_tiles == 2) {
+        const int groups = (EPI == EPI_SILU) ? tiles : (tiles + 1) / 2;
+        if (row_tiles == 2) return launch_waves<EPI, 2, 2>(s, waves, dim3(groups, m_blocks, k_parts), a);
+        if (row_tiles == 4) return launch_waves<EPI, 4, 2>(s, waves, dim3(groups, m_blocks, k_parts), a);
+    } else if constexpr (EPI != EPI_SILU) {
+        if (column_tiles != 1) return CIE_BAD_ARGUMENT;
+        if (row_tiles == 2) return launch_waves<EPI, 2, 1>(s, waves, dim3(tiles, m_blocks, k_parts), a);
+        if (row_tiles == 4) return launch_waves<EPI, 4, 1>(s, waves, dim3(tiles, m_blocks, k_parts), a);
+    }
+    return CIE_BAD_ARGUMENT;
 }
 
 }  // namespace
 
 // epilogue: 0 bf16, 1 float32, 2 SiLU-gate (W = [gate rows; up rows], N = 2 * outputs), 3 residual
 // accumulate (+ sums of squares), 4 partial products of k_parts parts of K to c[k_parts, M, N].
-// row_tiles 1: M <= 16, `waves` waves per workgroup share K (1, 2, 4, 8).
-// row_tiles 2 or 4: up to 32 or 64 rows per workgroup (more rows: more workgroups), A staged in LDS.
+// row_tiles 1, 2, 4: 16, 32, 64 rows per workgroup (more rows: more workgroups, each streaming W again);
+// `waves` waves per workgroup share K (1, 2, 4, 8; with more than one row tile 4 or 8);
+// column_tiles 1 or 2 tiles of 16 columns per workgroup (2 only with more than one row tile: the rows of
+// A that a wave loads then meet two tiles of W; the SiLU epilogue always takes a gate tile and its up tile).
 // K and lda must be multiples of 8 (16-byte loads); N is free.
 CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
                            float* residual, float* sumsq, int M, int N, int K, int epilogue, int row_tiles,
-                           int waves, int k_parts) {
+                           int waves, int column_tiles, int k_parts) {
     if (M <= 0 || N <= 0 || K <= 0 || K % 8 || !a || !w || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
     if (row_tiles != 1 && row_tiles != 2 && row_tiles != 4) return CIE_BAD_ARGUMENT;
-    if (row_tiles == 1 && M > 16) return CIE_BAD_ARGUMENT;
+    if (waves != 1 && waves != 2 && waves != 4 && waves != 8) return CIE_BAD_ARGUMENT;
     if (epilogue == EPI_SILU && (N % 2 || bias)) return CIE_BAD_ARGUMENT;
-    if (epilogue == EPI_RESID && (!residual || !sumsq || row_tiles != 1)) return CIE_BAD_ARGUMENT;
+    if (epilogue == EPI_RESID && (!residual || !sumsq)) return CIE_BAD_ARGUMENT;
     if (epilogue != EPI_RESID && !c) return CIE_BAD_ARGUMENT;
     if (k_parts < 1 || k_parts > 64 || (k_parts > 1 && epilogue != EPI_PARTIAL)) return CIE_BAD_ARGUMENT;
     FusedArgs f;
@@ -300,11 +283,11 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     f.k_per_part = ((K + k_parts - 1) / k_parts + 127) / 128 * 128;
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (epilogue) {
-        case EPI_BF16: return launch<EPI_BF16>(s, row_tiles, waves, k_parts, f);
-        case EPI_F32: return launch<EPI_F32>(s, row_tiles, waves, k_parts, f);
-        case EPI_SILU: return launch<EPI_SILU>(s, row_tiles, waves, k_parts, f);
-        case EPI_RESID: return launch<EPI_RESID>(s, row_tiles, waves, k_parts, f);
-        case EPI_PARTIAL: return launch<EPI_PARTIAL>(s, row_tiles, waves, k_parts, f);
+        case EPI_BF16: return launch<EPI_BF16>(s, row_tiles, waves, column_tiles, k_parts, f);
+        case EPI_F32: return launch<EPI_F32>(s, row_tiles, waves, column_tiles, k_parts, f);
+        case EPI_SILU: return launch<EPI_SILU>(s, row_tiles, waves, column_tiles, k_parts, f);
+        case EPI_RESID: return launch<EPI_RESID>(s, row_tiles, waves, column_tiles, k_parts, f);
+        case EPI_PARTIAL: return launch<EPI_PARTIAL>(s, row_tiles, waves, column_tiles, k_parts, f);
     }
     return CIE_BAD_ARGUMENT;
 }

@@ -331,29 +331,33 @@ def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]
 EPI_BF16, EPI_F32, EPI_SILU, EPI_RESID, EPI_PARTIAL = 0, 1, 2, 3, 4
 FUSED_TARGET_WAVES = 2048
 FUSED_MAX_ROWS = 64  # rows one workgroup of ``gemm_fused`` takes; more rows run as more workgroup rows
+FUSED_PAIR_WORKGROUPS = 256  # workgroups that must remain when workgroups of many rows take two column tiles
 
 
-def plan_fused(rows: int, column_tiles: int, k: int) -> tuple[int, int]:
-    """(row_tiles, waves per workgroup) of ``gemm_fused`` for ``rows`` rows,
-    ``column_tiles`` tiles of 16 columns (times the parts of K) and inner size
-    ``k`` per part.  Up to 16 rows: as many waves share K as it takes to fill the
-    GPU, each with at least one 128-wide slice.  More rows: four waves side by
-    side that share the staged activations."""
-    if rows > 16:
-        return (2 if rows <= 32 else 4), 4
-    waves = 1
-    while waves < 8 and column_tiles * waves < FUSED_TARGET_WAVES and waves * 2 * 128 <= k:
+def plan_fused(rows: int, column_tiles: int, k: int, k_parts: int = 1) -> tuple[int, int, int]:
+    """(row tiles, waves per workgroup, column tiles per workgroup) of ``gemm_fused``
+    for ``rows`` rows, ``column_tiles`` tiles of 16 columns, ``k_parts`` parts of
+    K of ``k`` each.  16, 32 or 64 rows per workgroup (more rows: more workgroups,
+    each streaming the weight again).  With more than 16 rows a workgroup takes
+    two column tiles if that still leaves enough workgroups (each activation
+    value a wave loads then meets two weight tiles).  As many waves share K as it
+    takes to fill the GPU, each with at least one 128-wide slice."""
+    row_tiles = 1 if rows <= 16 else 2 if rows <= 32 else 4
+    pair = row_tiles > 1 and column_tiles * k_parts >= 2 * FUSED_PAIR_WORKGROUPS
+    groups = (-(-column_tiles // 2) if pair else column_tiles) * k_parts
+    waves = 1 if row_tiles == 1 else 4
+    while waves < 8 and groups * waves < FUSED_TARGET_WAVES and waves * 2 * 128 <= k:
         waves *= 2
-    return 1, waves
+    return row_tiles, waves, 2 if pair else 1
 
 
 def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optional[torch.Tensor] = None,
                residual_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None,
-               plan: Optional[tuple[int, int]] = None, k_parts: int = 1) -> torch.Tensor:
+               plan: Optional[tuple[int, int, int]] = None, k_parts: int = 1) -> torch.Tensor:
     """Few-row matrix product ``a @ weight.T`` (bf16 operands, float32 sums) fused
     with its neighbour.  ``epilogue``: ``EPI_BF16`` / ``EPI_F32`` return
     ``a W^T + bias``; ``EPI_SILU`` (weight = gate rows over up rows) returns
-    ``silu(gate) * up`` [M, N/2]; ``EPI_RESID`` (up to 16 rows) adds the product
+    ``silu(gate) * up`` [M, N/2]; ``EPI_RESID`` adds the product
     into ``residual_out`` (float32 [M, N]) and returns the partial sums of
     squares of its new rows [M, ceil(N/16)]; ``EPI_PARTIAL`` cuts K into
     ``k_parts`` parts and returns their float32 partial products
@@ -373,9 +377,12 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
         _gpu("bias", bias, torch.bfloat16, 1)
         _require(bias.shape[0] == n and epilogue != EPI_SILU, "bias does not fit")
     columns = n // 2 if epilogue == EPI_SILU else n
-    row_tiles, waves = plan or plan_fused(m, -(-columns // 16) * k_parts, -(-k // k_parts))
-    _require(row_tiles in (1, 2, 4) and (row_tiles > 1 or (m <= 16 and waves in (1, 2, 4, 8))),
-             f"plan {(row_tiles, waves)} does not fit {m} rows")
+    row_tiles, waves, column_tiles = plan or plan_fused(m, -(-columns // 16), -(-k // k_parts), k_parts)
+    if epilogue == EPI_SILU:
+        column_tiles = 1 if row_tiles == 1 else 2  # always a gate tile with its up tile
+    _require(row_tiles in (1, 2, 4) and waves in ((1, 2, 4, 8) if row_tiles == 1 else (4, 8))
+             and column_tiles in ((1,) if row_tiles == 1 else (1, 2)),
+             f"plan {(row_tiles, waves, column_tiles)} is not one the kernel has")
     residual = sumsq = None
     if epilogue == EPI_BF16:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
@@ -387,7 +394,6 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
         _require(n % 2 == 0, f"the SiLU epilogue needs an even N, got {n}")
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=device)
     elif epilogue == EPI_RESID:
-        _require(row_tiles == 1, "the residual epilogue takes up to 16 rows")
         _require(residual_out is not None, "the residual epilogue needs the residual to add into")
         _gpu("residual_out", residual_out, torch.float32, 2)
         _require(residual_out.shape == (m, n), f"residual_out {tuple(residual_out.shape)} vs {(m, n)}")
@@ -401,7 +407,7 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
         raise ValueError(f"unknown epilogue {epilogue}")
     _run("cie_gemm_fused", load_library().cie_gemm_fused(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(None if epilogue == EPI_RESID else out),
-        _ptr(residual), _ptr(sumsq), _i(m), _i(n), _i(k), _i(epilogue), _i(row_tiles), _i(waves), _i(k_parts)))
+        _ptr(residual), _ptr(sumsq), _i(m), _i(n), _i(k), _i(epilogue), _i(row_tiles), _i(waves), _i(column_tiles), _i(k_parts)))
     return out
 
 

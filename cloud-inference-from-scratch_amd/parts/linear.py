@@ -20,8 +20,11 @@ import torch
 from ..kernels import ops
 
 # Rows up to which the hand-written fused bf16 kernel replaces the library product.  Measured on
-# MI355X: up to 16 rows it beats the library by 1.5-2x; at 64 rows its LDS-staged form loses.
+# MI355X (3B shapes): up to 16 rows it beats the library by 1.5-2x; with 17 to 64 rows it only wins where K
+# is long and is cut into parts (the down product: 18-23 us against the library's 27-32 us); its gate/up
+# product loses from 24 rows on (41 us against 25 us at 64 rows: every workgroup re-reads the rows of A).
 FUSED_ROWS = 16
+FUSED_PARTS_ROWS = 64
 # An ``into=`` product with fewer than this many 16-column tiles and K of at least 2 * PART_K cuts K
 # into parts of about PART_K for more workgroups (partial products, summed by the next norm kernel).
 PART_BELOW_TILES = 512
@@ -64,10 +67,12 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     n = weight.shape[0]
     silu = epilogue == "silu"
     wants_f32 = out_dtype == torch.float32
-    if _fusable(rows, k, x.stride(0) if rows > 1 else k, weight) and (rows <= FUSED_ROWS or wants_f32):
+    fusable = _fusable(rows, k, x.stride(0) if rows > 1 else k, weight)
+    cut_k = into is not None and -(-n // 16) < PART_BELOW_TILES and k >= 2 * PART_K
+    if fusable and cut_k and rows <= FUSED_PARTS_ROWS:
+        return PartialSum(ops.gemm_fused(weight, ops.EPI_PARTIAL, x, bias=bias, k_parts=-(-k // PART_K)))
+    if fusable and (rows <= FUSED_ROWS or wants_f32):
         if into is not None:
-            if -(-n // 16) < PART_BELOW_TILES and k >= 2 * PART_K:
-                return PartialSum(ops.gemm_fused(weight, ops.EPI_PARTIAL, x, bias=bias, k_parts=-(-k // PART_K)))
             return RowSumsq(ops.gemm_fused(weight, ops.EPI_RESID, x, bias=bias, residual_out=into))
         elif silu and n % 2 == 0:
             return ops.gemm_fused(weight, ops.EPI_SILU, x)

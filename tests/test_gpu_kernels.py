@@ -454,14 +454,18 @@ def test_sample_frequencies(ops):
 
 @pytest.mark.parametrize("shape", [(1, 64, 128), (8, 2560, 2048), (16, 96, 328), (17, 208, 1032), (40, 66, 264),
                                    (64, 2048, 1408), (70, 48, 96)])
-@pytest.mark.parametrize("plan", [None, "one", "many"])
+@pytest.mark.parametrize("plan", [None, "few", "many", "paired"])
 def test_gemm_fused_epilogues(ops, shape, plan):
-    """The fused few-row product: SiLU-gate and residual-accumulate epilogues, with one wave per
-    workgroup and with eight (partial tiles summed through LDS), against float64 products."""
+    """The fused few-row product: SiLU-gate and residual-accumulate epilogues, for every plan the
+    kernel has (the fewest and the most waves per workgroup, partial tiles summed through LDS;
+    one or two column tiles per workgroup with more than 16 rows; more than 64 rows as several
+    rows of workgroups), against float64 products."""
     m, n, k = shape
-    if m > 16 and plan is not None:
-        pytest.skip("the waves-share-K form takes up to 16 rows")
-    chosen = {None: None, "one": (1, 1), "many": (1, 8)}[plan]
+    row_tiles = 1 if m <= 16 else 2 if m <= 32 else 4
+    if plan == "paired" and row_tiles == 1:
+        pytest.skip("workgroups of 16 rows take one column tile")
+    chosen = {None: None, "few": (row_tiles, 1 if row_tiles == 1 else 4, 1), "many": (row_tiles, 8, 1),
+              "paired": (row_tiles, 8, 2)}[plan]
     a, w = rand((m, k), torch.bfloat16, 80), rand((n, k), torch.bfloat16, 81, 0.3)
     b = rand((n,), torch.bfloat16, 82)
     exact = a.double() @ w.double().t()
@@ -470,10 +474,8 @@ def test_gemm_fused_epilogues(ops, shape, plan):
     assert out.shape == (m, n // 2) and out.dtype == torch.bfloat16
     want = torch.nn.functional.silu(gate) * up
     torch.testing.assert_close(out.double(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()))
-    if m > 16:
-        with pytest.raises(ValueError, match="16 rows"):
-            ops.gemm_fused(w, ops.EPI_RESID, a, residual_out=rand((m, n), torch.float32, 83))
-        return
+    plain_out = ops.gemm_fused(w, ops.EPI_F32, a, bias=b, plan=chosen)
+    torch.testing.assert_close(plain_out.double(), exact + b.double(), rtol=1e-4, atol=2e-4 * math.sqrt(k))
     residual = rand((m, n), torch.float32, 83, 2.0)
     before = residual.clone()
     parts = -(-n // 16)
