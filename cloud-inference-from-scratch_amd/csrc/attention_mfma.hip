@@ -329,8 +329,18 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
     const float scale_log2 = a.scale * 1.44269504088896341f;
     const int hi = start + q0 + n_tok;
     const int lo = (a.window > 0) ? max(0, start + q0 + 1 - a.window) : 0;
-    const int range_begin = lo & ~(kKeysPerBlock - 1);
-    const int range_end = hi;
+    int range_begin = lo & ~(kKeysPerBlock - 1);
+    int range_end = hi;
+    if (a.n_splits > 1) {  // this workgroup's share of the keys (blockIdx.y); the merge kernel joins the shares
+        int per_split = a.keys_per_split;
+        if (a.max_context_dev) {
+            int most = *a.max_context_dev;
+            if (a.window > 0) most = min(most, a.window + 2 * kKeysPerBlock);
+            per_split = ((most + a.n_splits - 1) / a.n_splits + kKeysPerBlock - 1) & ~(kKeysPerBlock - 1);
+        }
+        range_begin += blockIdx.y * per_split;
+        range_end = min(hi, range_begin + per_split);
+    }
     const int first_pos = start + q0;              // position of the tile's first token
     const int last_pos = start + q0 + n_tok - 1;   // and of its last
     const int last_group = (hi - 1) & ~15;         // the last 16 keys that have a page
@@ -502,11 +512,12 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
     }
 
     // ---- the waves' partial results meet: statistics first, then one row tile at a time through LDS
-    float l_all[RT], own_weight[RT];
+    float l_all[RT], m_all[RT], own_weight[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         const float l = rows_sum(l_run[rt]);
         l_all[rt] = l;
+        m_all[rt] = m_run[rt];
         own_weight[rt] = 1.f;
         if (WAVES > 1 && g == 0) {
             lds_ml[wave][rt * 16 + r][0] = m_run[rt];
@@ -517,10 +528,11 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
         __syncthreads();
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-            float m_all = -INFINITY;
+            float m_max = -INFINITY;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) m_all = fmaxf(m_all, lds_ml[w][rt * 16 + r][0]);
-            const float m_safe = (m_all == -INFINITY) ? 0.f : m_all;
+            for (int w = 0; w < WAVES; ++w) m_max = fmaxf(m_max, lds_ml[w][rt * 16 + r][0]);
+            m_all[rt] = m_max;
+            const float m_safe = (m_max == -INFINITY) ? 0.f : m_max;
             float l = 0.f;
 #pragma unroll
             for (int w = 0; w < WAVES; ++w)
@@ -559,20 +571,35 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
                         for (int i = 0; i < 4; ++i) o[rt][dt][i] += lds_o[w * (ND * 4 * kWave) + (dt * 4 + i) * kWave + lane];
             }
         }
-        if (wave == owner) {
+        if (wave != owner) continue;
+        if (a.n_splits > 1) {  // this share's sums and statistics for the merge kernel
+            const size_t unit = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + blockIdx.y;
+            float* po = a.part_o + unit * ROWS * D;
+            float* pml = a.part_ml + unit * ROWS * 2;
+            if (g == 0) {
+                pml[(rt * 16 + r) * 2] = m_all[rt];
+                pml[(rt * 16 + r) * 2 + 1] = l_all[rt];
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int row = rt * 16 + g * 4 + i;
-                const float l_row = __shfl(l_all[rt], g * 4 + i, kWave);
-                if (row < n_rows) {
-                    const int tok = row / group;
-                    const int head = row - tok * group;
-                    bf16_t* dst = a.out + static_cast<size_t>(first_row_token + tok) * a.q_heads * D +
-                                  static_cast<size_t>(kv_head * group + head) * D;
-                    const float inv = 1.0f / l_row;
 #pragma unroll
-                    for (int dt = 0; dt < ND; ++dt) dst[dt * 16 + r] = from_float<bf16_t>(o[rt][dt][i] * inv);
-                }
+                for (int dt = 0; dt < ND; ++dt) po[static_cast<size_t>(row) * D + dt * 16 + r] = o[rt][dt][i];
+            }
+            continue;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = rt * 16 + g * 4 + i;
+            const float l_row = __shfl(l_all[rt], g * 4 + i, kWave);
+            if (row < n_rows) {
+                const int tok = row / group;
+                const int head = row - tok * group;
+                bf16_t* dst = a.out + static_cast<size_t>(first_row_token + tok) * a.q_heads * D +
+                              static_cast<size_t>(kv_head * group + head) * D;
+                const float inv = 1.0f / l_row;
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt) dst[dt * 16 + r] = from_float<bf16_t>(o[rt][dt][i] * inv);
             }
         }
     }
@@ -626,8 +653,8 @@ template <int D>
 int launch_for_dim(hipStream_t s, const AttentionArgs& a, int n_tiles, int row_tiles, int tile_waves) {
     dim3 grid(n_tiles, a.kv_heads, a.n_splits);
     if (tile_waves == kTileWaves) {
-        grid = a.xcds_per_head > 0 ? dim3(8 * ((n_tiles + a.xcds_per_head - 1) / a.xcds_per_head))
-                                   : dim3(static_cast<unsigned>(n_tiles) * a.kv_heads);
+        grid = a.xcds_per_head > 0 ? dim3(8 * ((n_tiles + a.xcds_per_head - 1) / a.xcds_per_head), a.n_splits)
+                                   : dim3(static_cast<unsigned>(n_tiles) * a.kv_heads, a.n_splits);
         if (row_tiles == 1)
             paged_attention_tile_kernel<D, 1, kTileWaves><<<grid, 64 * kTileWaves, 0, s>>>(a);
         else if constexpr (D <= 128) {  // wider heads hold one row tile of accumulators without spilling
@@ -674,7 +701,7 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     if (n_splits > kMergeMaxSplits) return CIE_BAD_ARGUMENT;
     // the prompt form takes maxima before scaling, which needs a positive scale, and keeps the 16 keys of a
     // product in one page
-    if (tile_waves != 1 && (tile_waves != kTileWaves || n_splits != 1 || !(scale > 0.f) || page_size < 16))
+    if (tile_waves != 1 && (tile_waves != kTileWaves || !(scale > 0.f) || page_size < 16))
         return CIE_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml ||
                          (!max_context_dev && (keys_per_split <= 0 || keys_per_split % kKeysPerBlock))))

@@ -260,9 +260,9 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
     ``tile_q0[i]``-th token of this step on.  Rows of other tokens of ``out`` are left alone.
     With ``n_splits > 1`` every tile's keys are cut into parts of ``keys_per_split``
     (a multiple of 32; or, with ``max_context_dev``, derived on the device from the
-    step's longest context) and merged through the workspaces.  ``tile_waves=4`` (the
-    prompt form, unsplit only) gives every tile a workgroup of four waves that share
-    the tile's keys among them."""
+    step's longest context) and merged through the workspaces.  ``tile_waves=4`` gives
+    every tile (and every part of its keys) a workgroup of four waves that take the
+    blocks of 32 keys in turn; it needs pages of at least 16 keys."""
     _require(q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 2 and q.stride(1) == 1
              and q.stride(0) == q_row_stride, "q must be a bf16 GPU matrix with unit inner stride")
     _require(q.shape[1] >= q_heads * head_dim and q_row_stride % 8 == 0, f"q {tuple(q.shape)} does not fit")
@@ -283,7 +283,7 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
     _gpu("out", out, torch.bfloat16, 2)
     _require(out.shape[1] == q_heads * head_dim and out.shape[0] <= q.shape[0], f"out is {tuple(out.shape)}")
     _require(1 <= n_splits <= 65535, f"n_splits {n_splits} out of range")
-    _require(tile_waves == 1 or (tile_waves == TILE_WAVES and n_splits == 1 and scale > 0 and page_size >= 16
+    _require(tile_waves == 1 or (tile_waves == TILE_WAVES and scale > 0 and page_size >= 16
                                  and (row_tiles == 1 or head_dim <= 128)),
              f"tile_waves {tile_waves} with {n_splits} splits, {row_tiles} row tiles, head size {head_dim}, pages of {page_size}")
     if n_splits > 1:

@@ -92,6 +92,9 @@ class Attention(Part):
         return linear(context, self.w_o, self.b_o, into=residual)
 
 
+WIDE_DECODE_KEYS = 2048  # contexts from which decode rows go to the four-wave form
+
+
 def plan_splits(units: int, max_keys: int, target_waves: int = 1024, min_keys: int = 128) -> tuple[int, int]:
     """How many parts to cut a decode tile's keys into so that the GPU is filled:
     (number of splits, keys per split as a multiple of 32)."""
@@ -124,28 +127,40 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     common = (batch.seq_slot, batch.seq_start, batch.seq_q_len, batch.q_start_loc, out, num_heads, num_kv_heads,
               head_dim, window, scale)
     max_keys = batch.max_context if window is None else min(batch.max_context, window + 64)
+    wide = page_size >= 16 and scale > 0
+
+    def decode_form(bound: int) -> tuple[int, dict]:
+        # Decode rows.  Long contexts: four waves per (sequence, kv head, part of the keys) take the part's
+        # blocks in turn with their loads running ahead (15.8 against 18.1 us for 8 x 4,096 keys); short
+        # ones: one wave per part (9.1 against 10.9 us for 8 x 1,024 keys).
+        waves = ops.TILE_WAVES if wide and bound >= WIDE_DECODE_KEYS else 1
+        return waves, dict(target_waves=1024 // waves, min_keys=32 * waves if waves > 1 else 128)
+
     if batch.static_plan is not None:  # a captured decode step: the grid is fixed, lengths live on the device
         plan = batch.static_plan
         bound = plan.max_keys if window is None else min(plan.max_keys, window + 64)
-        n_splits, _ = plan_splits(batch.sequences * num_kv_heads, bound)
+        decode_waves, split_options = decode_form(bound)
+        n_splits, _ = plan_splits(batch.sequences * num_kv_heads, bound, **split_options)
         part_o = part_ml = None
         if n_splits > 1:
             part_o, part_ml = _workspaces(qkv.device, batch.sequences * num_kv_heads * n_splits, 16, head_dim)
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, plan.tile_seq,
                                  plan.tile_q0, batch.sequences, *common, tokens_per_tile=1, row_tiles=1,
-                                 n_splits=n_splits, max_context_dev=plan.max_context, part_o=part_o, part_ml=part_ml)
+                                 n_splits=n_splits, max_context_dev=plan.max_context, part_o=part_o, part_ml=part_ml,
+                                 tile_waves=decode_waves)
         return out
     tile_seq, tile_q0, n_tiles = batch.tiles(1, decode=True)
     if n_tiles:
-        n_splits, per_split = plan_splits(n_tiles * num_kv_heads, max_keys)
+        decode_waves, split_options = decode_form(max_keys)
+        n_splits, per_split = plan_splits(n_tiles * num_kv_heads, max_keys, **split_options)
         part_o = part_ml = None
         if n_splits > 1:
             part_o, part_ml = _workspaces(qkv.device, n_tiles * num_kv_heads * n_splits, 16, head_dim)
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
                                  n_tiles, *common, tokens_per_tile=1, row_tiles=1, n_splits=n_splits,
-                                 keys_per_split=per_split, part_o=part_o, part_ml=part_ml)
+                                 keys_per_split=per_split, part_o=part_o, part_ml=part_ml, tile_waves=decode_waves)
     prompt_tokens = sum(n for n in batch.host_q_lens if n > 1)
-    if page_size >= 16 and scale > 0:
+    if wide:
         # the prompt form: four waves share a tile's keys.  More rows per tile re-use each key more often,
         # fewer tiles leave compute units idle: the most rows that still give most units a workgroup
         tile_waves = ops.TILE_WAVES

@@ -183,7 +183,8 @@ def test_paged_attention_generic(ops, dtype, geometry):
 
 
 def run_mfma(ops, q_all, contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim, window,
-             scale, per_tile, row_tiles, n_splits=1, keys_per_split=0, decode_only=None, tile_waves=1):
+             scale, per_tile, row_tiles, n_splits=1, keys_per_split=0, decode_only=None, tile_waves=1,
+             max_context_dev=None):
     """Drive the matrix-core kernel the way the attention part does: tiles of
     ``per_tile`` tokens for the chosen sequences; returns [tokens, Hq*D] (rows of
     sequences that were not chosen stay zero)."""
@@ -212,7 +213,8 @@ def run_mfma(ops, q_all, contexts, q_lens, k_pool, v_pool, table, slots, q_heads
     ops.paged_attention_mfma(buffer, stride, k_pool, v_pool, table, as_dev(tile_seq), as_dev(tile_q0), len(tile_seq),
                              as_dev(slots), as_dev(contexts), as_dev(q_lens), as_dev(loc), out, q_heads, kv_heads,
                              head_dim, window, scale, per_tile, row_tiles, n_splits=n_splits,
-                             keys_per_split=keys_per_split, part_o=part_o, part_ml=part_ml, tile_waves=tile_waves)
+                             keys_per_split=keys_per_split, part_o=part_o, part_ml=part_ml, tile_waves=tile_waves,
+                             max_context_dev=max_context_dev)
     return out.float().cpu()
 
 
@@ -254,11 +256,15 @@ def test_paged_attention_mfma_ragged(ops, geometry, row_tiles, tile_waves):
 
 @pytest.mark.parametrize("geometry", MFMA_GEOMETRY)
 @pytest.mark.parametrize("splits", [(1, 0), (3, 704), (16, 128), (64, 32)])
-def test_paged_attention_mfma_decode_splits(ops, geometry, splits):
+@pytest.mark.parametrize("tile_waves", [1, 4])
+def test_paged_attention_mfma_decode_splits(ops, geometry, splits, tile_waves):
     """Single tokens over contexts up to 2047 (boundary lengths of
     tests/remote_gpu_tests.py:204), the keys cut into parts that are merged;
-    parts beyond a short context are empty."""
+    parts beyond a short context are empty.  With one wave per part and with four
+    (a part of 32 keys then leaves three of them without a key)."""
     q_heads, kv_heads, head_dim, page_size = geometry
+    if tile_waves == 4:
+        page_size = max(page_size, 16)
     n_splits, per_split = splits
     contexts = [0, 1, 15, 16, 17, 127, 128, 129, 1000, 2047]
     q_lens = [1] * len(contexts)
@@ -272,8 +278,16 @@ def test_paged_attention_mfma_decode_splits(ops, geometry, splits):
         qs.append(q.reshape(1, -1))
         expected.append(plain_qwen2.causal_attention(q, *dense[s], scale, past_len=c))
     out = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
-                   None, scale, 1, 1, n_splits=n_splits, keys_per_split=per_split)
+                   None, scale, 1, 1, n_splits=n_splits, keys_per_split=per_split, tile_waves=tile_waves)
     torch.testing.assert_close(out, torch.cat(expected), **tol(torch.bfloat16))
+    if n_splits > 1:
+        # as in a captured step: the size of a part is derived on the device from the longest context,
+        # here once the true one and once a loose bound
+        for longest in (max(lengths), 3000):
+            out = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads,
+                           head_dim, None, scale, 1, 1, n_splits=n_splits, tile_waves=tile_waves,
+                           max_context_dev=torch.tensor([longest], dtype=torch.int32).cuda())
+            torch.testing.assert_close(out, torch.cat(expected), **tol(torch.bfloat16))
 
 
 @pytest.mark.parametrize("window", [5, 32, 100])
@@ -296,10 +310,12 @@ def test_paged_attention_mfma_window(ops, window):
             tiled = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads,
                              head_dim, window, scale, 8 * row_tiles, row_tiles, tile_waves=tile_waves)
             torch.testing.assert_close(tiled, want, **tol(torch.bfloat16))
-        split = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads,
-                         head_dim, window, scale, 1, 1, n_splits=4, keys_per_split=32, decode_only=True)
         rows = [40, 58]  # the two single-token sequences
-        torch.testing.assert_close(split[rows], want[rows], **tol(torch.bfloat16))
+        for tile_waves in ((1,) if page_size < 16 else (1, 4)):
+            split = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads,
+                             head_dim, window, scale, 1, 1, n_splits=4, keys_per_split=32, decode_only=True,
+                             tile_waves=tile_waves)
+            torch.testing.assert_close(split[rows], want[rows], **tol(torch.bfloat16))
 
 
 def test_paged_attention_mfma_far_key(ops):
@@ -312,11 +328,13 @@ def test_paged_attention_mfma_far_key(ops):
     q = torch.stack([k[far, h // 8] * 2.0 for h in range(q_heads)])[None].to(torch.bfloat16).float()
     scale = 1.0 / math.sqrt(head_dim)
     expect = plain_qwen2.causal_attention(q, k, v, scale, past_len=length - 1)
-    for n_splits, per_split in [(1, 0), (7, 288), (63, 32)]:
-        out = run_mfma(ops, q.reshape(1, -1), [length - 1], [1], k_pool, v_pool, table, slots, q_heads, kv_heads,
-                       head_dim, None, scale, 1, 1, n_splits=n_splits, keys_per_split=per_split)
-        torch.testing.assert_close(out, expect, **tol(torch.bfloat16))
-        torch.testing.assert_close(out.view(q_heads, head_dim), v[far].repeat_interleave(8, dim=0), rtol=0.05, atol=0.05)
+    for tile_waves in (1, 4):
+        for n_splits, per_split in [(1, 0), (7, 288), (63, 32)]:
+            out = run_mfma(ops, q.reshape(1, -1), [length - 1], [1], k_pool, v_pool, table, slots, q_heads, kv_heads,
+                           head_dim, None, scale, 1, 1, n_splits=n_splits, keys_per_split=per_split,
+                           tile_waves=tile_waves)
+            torch.testing.assert_close(out, expect, **tol(torch.bfloat16))
+            torch.testing.assert_close(out.view(q_heads, head_dim), v[far].repeat_interleave(8, dim=0), rtol=0.05, atol=0.05)
     # the prompt form: the last of 40 tokens asks for the far key; the four waves of its tile each see a
     # quarter of the keys and only one of them holds the key that counts
     q_many = torch.cat([torch.randn((39, q_heads, head_dim), generator=torch.Generator().manual_seed(77)), q])

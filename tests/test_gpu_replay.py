@@ -112,6 +112,34 @@ def test_replay_with_the_four_wave_prompt_attention(tiny_folders, plain, monkeyp
     assert runner.cache.stats().pages_used == 0
 
 
+@pytest.mark.parametrize("graph", [False, True])
+def test_replay_with_the_four_wave_decode_attention(tiny_folders, plain, monkeypatch, graph):
+    """Decode rows go to the four-wave attention form only for long contexts; make
+    every context long enough, eagerly and in captured steps."""
+    from cie_amd.kernels import ops
+    from cie_amd.parts import attention
+
+    monkeypatch.setattr(attention, "WIDE_DECODE_KEYS", 0)
+    seen = []
+    real = ops.paged_attention_mfma
+
+    def spy(*args, **kwargs):
+        seen.append((kwargs["tokens_per_tile"], kwargs.get("tile_waves", 1), kwargs.get("n_splits", 1)))
+        return real(*args, **kwargs)
+
+    monkeypatch.setattr(ops, "paged_attention_mfma", spy)
+    folder, raw, _ = tiny_folders["B"]
+    requests, expected = plain["B"]
+    steps = replay_util.mixed(requests, live=4, decode_tail=30, seed=8)
+    runner = make_runner(folder, "bfloat16", replay_util.max_live_tokens(steps, page=16), 16, graph_decode=graph)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    replay_util.compare(rows, expected, **TOL["bfloat16"])
+    assert any(per_tile == 1 and waves == ops.TILE_WAVES for per_tile, waves, _ in seen), seen[:8]
+    if graph:  # captured steps size their parts for the longest request the engine takes: more than one part
+        assert any(per_tile == 1 and waves == ops.TILE_WAVES and splits > 1 for per_tile, waves, splits in seen), seen[:8]
+        assert runner.graph_replays >= 20
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_captured_decode_steps_match_plain(tiny_folders, plain, name, dtype):
