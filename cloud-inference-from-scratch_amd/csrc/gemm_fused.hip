@@ -13,6 +13,10 @@
 //               RMSNorm that follows needs no reduction over the row
 //   PARTIAL     K is cut into grid.z parts; part p writes acc to C[p, m, n] (float32, bias in
 //               part 0).  The add + norm kernel sums the parts.  For few columns and long K.
+//   ROPE        W stacks the rows of q, k and v heads: a workgroup takes 16 dimensions of a head's
+//               first half and the 16 they rotate with (half-split pairing), adds the bias, rounds
+//               to bf16 as the plain epilogue would, rotates q and k by the row's position and
+//               writes q to C[m, n], k and v into the paged cache (v transposed).
 //
 // One kernel: a workgroup owns one or two tiles of 16 columns (SILU: a gate tile and its up tile)
 // and 16, 32 or 64 rows; its WAVES waves cut K into slices of 128 and take them round-robin;
@@ -31,7 +35,22 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4 };
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4, EPI_ROPE = 5 };
+
+// What the ROPE epilogue needs beside the product: where each row's token sits, and the cache.
+struct RopeArgs {
+    const float* cos_table;  // [max_position, D/2]
+    const float* sin_table;
+    const int* positions;     // [M]
+    const int* seq_of_token;  // [M]
+    const int* seq_slot;      // [sequences]
+    const int* block_table;   // [slots, table_width]
+    int table_width;
+    bf16_t* k_pool;           // [pages, Hkv, page_size, D]
+    bf16_t* v_pool;           // [pages, Hkv, D, page_size]
+    int q_heads, kv_heads, head_dim, page_size;
+    int rotate, write_kv;
+};
 
 struct FusedArgs {
     const bf16_t* a;       // [M, K], row stride lda
@@ -44,6 +63,7 @@ struct FusedArgs {
     int M, N, K;
     int up_offset;         // SILU: rows of W between a gate row and its up row (N/2)
     int k_per_part;        // k values per grid.z part (a multiple of 128); K with one part
+    RopeArgs rope;         // ROPE only
 };
 
 // One 16x16 tile of results in its MFMA layout: lane (r, g) holds rows g*4+i of column r.
@@ -91,6 +111,93 @@ __device__ __forceinline__ void store_tile(const FusedArgs& a, const floatx4& ac
     }
 }
 
+// The ROPE epilogue for one pair of tiles: `lo` holds dimensions j*16 + r of head `head`, `hi` those
+// plus D/2.  Values are rounded to bf16 before the rotation, so that the results equal those of the
+// plain epilogue followed by the rotation kernel.  What the epilogue needs of each of the lane's four
+// rows (position, angle, cache page) is fetched before the product starts, so that these dependent
+// loads travel while the weights stream.
+struct RopeRows {
+    int pos[4];
+    int page[4];    // -1: nothing to write for this row
+    float c[4], s[4];
+    float bias_lo, bias_hi;
+};
+
+__device__ __forceinline__ RopeRows rope_prefetch(const FusedArgs& a, int head, int j, int lane) {
+    const RopeArgs& p = a.rope;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int half = p.head_dim / 2;
+    const int d = j * 16 + r;
+    const bool is_query = head < p.q_heads;
+    const bool is_value = head >= p.q_heads + p.kv_heads;
+    RopeRows rows;
+    rows.bias_lo = a.bias ? to_float(a.bias[head * p.head_dim + d]) : 0.f;
+    rows.bias_hi = a.bias ? to_float(a.bias[head * p.head_dim + d + half]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = g * 4 + i;
+        rows.pos[i] = 0;
+        rows.page[i] = -1;
+        rows.c[i] = 1.f;
+        rows.s[i] = 0.f;
+        if (m >= a.M) continue;
+        const int pos = p.positions[m];
+        rows.pos[i] = pos;
+        if (!is_value && p.rotate) {
+            rows.c[i] = p.cos_table[static_cast<size_t>(pos) * half + d];
+            rows.s[i] = p.sin_table[static_cast<size_t>(pos) * half + d];
+        }
+        if (!is_query && p.write_kv) {
+            const int slot = p.seq_slot[p.seq_of_token[m]];
+            rows.page[i] = p.block_table[static_cast<size_t>(slot) * p.table_width + pos / p.page_size];
+        }
+    }
+    return rows;
+}
+
+__device__ __forceinline__ void store_rope(const FusedArgs& a, const floatx4& lo, const floatx4& hi, int head,
+                                           int j, int lane, const RopeRows& rows) {
+    const RopeArgs& p = a.rope;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int D = p.head_dim;
+    const int half = D / 2;
+    const int d = j * 16 + r;
+    const bool is_query = head < p.q_heads;
+    const bool is_value = head >= p.q_heads + p.kv_heads;
+    const int kv_head = is_query ? 0 : (head - p.q_heads) % p.kv_heads;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = g * 4 + i;
+        if (m >= a.M) continue;
+        const float x_lo = to_float(from_float<bf16_t>(lo[i] + rows.bias_lo));
+        const float x_hi = to_float(from_float<bf16_t>(hi[i] + rows.bias_hi));
+        // values and unrotated heads have c = 1, s = 0: the products are exact and the sums unchanged
+        const bf16_t y_lo = from_float<bf16_t>(x_lo * rows.c[i] - x_hi * rows.s[i]);
+        const bf16_t y_hi = from_float<bf16_t>(x_hi * rows.c[i] + x_lo * rows.s[i]);
+        if (is_query) {
+            bf16_t* dst = static_cast<bf16_t*>(a.c) + static_cast<size_t>(m) * a.N + head * D + d;
+            dst[0] = y_lo;
+            dst[half] = y_hi;
+            continue;
+        }
+        const int page = rows.page[i];
+        if (page < 0) continue;  // no cache write wanted (the host never schedules a token without a page)
+        const int in_page = rows.pos[i] % p.page_size;
+        const size_t head_base = (static_cast<size_t>(page) * p.kv_heads + kv_head) * p.page_size * D;
+        if (is_value) {  // element d of the token goes to [d, in_page] of the transposed page
+            bf16_t* column = p.v_pool + head_base + in_page;
+            column[static_cast<size_t>(d) * p.page_size] = y_lo;
+            column[static_cast<size_t>(d + half) * p.page_size] = y_hi;
+        } else {
+            bf16_t* dst = p.k_pool + head_base + static_cast<size_t>(in_page) * D + d;
+            dst[0] = y_lo;
+            dst[half] = y_hi;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // MT row tiles (M <= 16*MT per workgroup row; more rows: more workgroup rows) and NT column tiles
 // per workgroup: with SILU the gate tile and its up tile, else NT adjacent tiles.  Every weight
@@ -98,6 +205,7 @@ __device__ __forceinline__ void store_tile(const FusedArgs& a, const floatx4& ac
 template <int WAVES, int EPI, int MT, int NT>
 __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
+    static_assert(EPI != EPI_ROPE || (NT == 2 && MT == 1), "the ROPE epilogue pairs the two halves of a head");
     // slices of 128 k values whose weight loads are in flight together
     constexpr int U = (MT == 1 && NT == 1) ? 4 : (MT == 4) ? 1 : 2;
     __shared__ float reduce[WAVES > 1 ? (WAVES - 1) * MT * NT * 64 * 4 : 1];
@@ -108,14 +216,23 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     const int g = lane >> 4;
     const int m0 = blockIdx.y * (16 * MT);
     const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
-    const int tile_first = (EPI == EPI_SILU) ? blockIdx.x : blockIdx.x * NT;
+    const int tile_first = (EPI == EPI_SILU || EPI == EPI_ROPE) ? blockIdx.x : blockIdx.x * NT;
+    // ROPE: workgroup b takes tile b % (D/32) of the first half of head b / (D/32), and its partner
+    const int rope_tiles = (EPI == EPI_ROPE) ? a.rope.head_dim / 32 : 1;
+    const int rope_head = blockIdx.x / rope_tiles;
+    const int rope_tile = blockIdx.x - rope_head * rope_tiles;
 
     // a column past the end computes a copy that is not stored
     const bf16_t* w_row[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        const int n = (EPI == EPI_SILU) ? min(tile_first * 16 + r, cols - 1) + t * a.up_offset
-                                        : min((tile_first + t) * 16 + r, cols - 1);
+        int n;
+        if (EPI == EPI_ROPE)
+            n = rope_head * a.rope.head_dim + rope_tile * 16 + r + t * (a.rope.head_dim / 2);
+        else if (EPI == EPI_SILU)
+            n = min(tile_first * 16 + r, cols - 1) + t * a.up_offset;
+        else
+            n = min((tile_first + t) * 16 + r, cols - 1);
         w_row[t] = a.w + static_cast<size_t>(n) * a.K + g * 8;
     }
     const bf16_t* a_row[MT];
@@ -132,6 +249,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    RopeRows rope_rows;
+    if (EPI == EPI_ROPE && wave == 0) rope_rows = rope_prefetch(a, rope_head, rope_tile, lane);
 
     const int k_begin = blockIdx.z * a.k_per_part;
     const int k_end = min(a.K, k_begin + a.k_per_part);
@@ -195,7 +314,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        if (EPI == EPI_SILU) {
+        if (EPI == EPI_ROPE) {
+            store_rope(a, acc[mt][0], acc[mt][NT - 1], rope_head, rope_tile, lane, rope_rows);
+        } else if (EPI == EPI_SILU) {
             store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, tile_first * 16 + r, tile_first, lane);
         } else {
 #pragma unroll
@@ -281,6 +402,7 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     f.K = K;
     f.up_offset = (epilogue == EPI_SILU) ? N / 2 : 0;
     f.k_per_part = ((K + k_parts - 1) / k_parts + 127) / 128 * 128;
+    f.rope = RopeArgs{};
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (epilogue) {
         case EPI_BF16: return launch<EPI_BF16>(s, row_tiles, waves, column_tiles, k_parts, f);
@@ -290,4 +412,40 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
         case EPI_PARTIAL: return launch<EPI_PARTIAL>(s, row_tiles, waves, column_tiles, k_parts, f);
     }
     return CIE_BAD_ARGUMENT;
+}
+
+// q/k/v product of up to 16 rows with the ROPE epilogue: `w` [N, K] stacks the rows of q_heads query
+// heads, kv_heads key heads and kv_heads value heads of head_dim dimensions each (a multiple of 32);
+// `c` [M, N] receives the rotated queries (its key and value columns are left alone); rotated keys and
+// values go to the cache page of each row's position.  `waves` waves per workgroup share K (1, 2, 4, 8).
+CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
+                              int M, int N, int K, int waves, const float* cos_table, const float* sin_table,
+                              const int* positions, const int* seq_of_token, const int* seq_slot,
+                              const int* block_table, int table_width, void* k_pool, void* v_pool, int q_heads,
+                              int kv_heads, int head_dim, int page_size, int rotate, int write_kv) {
+    if (M <= 0 || M > 16 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
+    if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 32 || page_size <= 0 || table_width <= 0 ||
+        N != (q_heads + 2 * kv_heads) * head_dim)
+        return CIE_BAD_ARGUMENT;
+    if (!positions || (rotate && (!cos_table || !sin_table)) ||
+        (write_kv && (!seq_of_token || !seq_slot || !block_table || !k_pool || !v_pool)))
+        return CIE_BAD_ARGUMENT;
+    FusedArgs f;
+    f.a = static_cast<const bf16_t*>(a);
+    f.lda = lda;
+    f.w = static_cast<const bf16_t*>(w);
+    f.bias = static_cast<const bf16_t*>(bias);
+    f.c = c;
+    f.residual = nullptr;
+    f.sumsq = nullptr;
+    f.M = M;
+    f.N = N;
+    f.K = K;
+    f.up_offset = 0;
+    f.k_per_part = (K + 127) / 128 * 128;
+    f.rope = RopeArgs{cos_table, sin_table, positions, seq_of_token, seq_slot, block_table, table_width,
+                      static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads, head_dim,
+                      page_size, rotate, write_kv};
+    const dim3 grid((q_heads + 2 * kv_heads) * (head_dim / 32), 1, 1);
+    return launch_waves<EPI_ROPE, 1, 2>(static_cast<hipStream_t>(stream), waves, grid, f);
 }

@@ -411,6 +411,53 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
     return out
 
 
+def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Tensor], cos: torch.Tensor,
+                  sin: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, seq_slot: torch.Tensor,
+                  block_table: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, q_heads: int,
+                  kv_heads: int, head_dim: int, rotate: bool = True, write_kv: bool = True,
+                  waves: Optional[int] = None) -> torch.Tensor:
+    """The q/k/v product of up to 16 rows fused with what ``rope_kv_write`` does:
+    ``a @ weight.T + bias`` for weight [(Hq+2Hkv)*D, K], queries and keys rotated
+    by each row's position, keys and values written into the cache.  Returns the
+    buffer [M, (Hq+2Hkv)*D] whose query columns hold the rotated queries (its key
+    and value columns are not written).  Same results as ``gemm_fused`` followed
+    by ``rope_kv_write``.  Head sizes in steps of 32."""
+    _gpu("weight", weight, torch.bfloat16, 2)
+    n, k = weight.shape
+    _require(a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1,
+             "a must be a bf16 GPU matrix with unit inner stride")
+    m = a.shape[0]
+    _require(1 <= m <= 16 and a.shape[1] == k, f"a {tuple(a.shape)}: up to 16 rows of K={k}")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    _require(k % 8 == 0 and lda % 8 == 0, f"K and the row stride must be multiples of 8, are {k} and {lda}")
+    _require(a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
+    _require(head_dim % 32 == 0, f"the fused rotation takes head sizes in steps of 32, not {head_dim}")
+    _require(n == (q_heads + 2 * kv_heads) * head_dim, f"weight has {n} rows, heads say {(q_heads + 2 * kv_heads) * head_dim}")
+    if bias is not None:
+        _gpu("bias", bias, torch.bfloat16, 1)
+        _require(bias.shape[0] == n, "bias does not fit")
+    for name, table in (("cos", cos), ("sin", sin)):
+        _gpu(name, table, torch.float32, 2)
+        _require(table.shape[1] == head_dim // 2, f"{name} must be [max_position, {head_dim // 2}]")
+    _require(cos.shape == sin.shape, "cos and sin tables differ in shape")
+    for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
+        _gpu(name, meta, torch.int32, 1)
+        _require(meta.shape[0] >= m, f"{name} has {meta.shape[0]} entries for {m} rows")
+    _gpu("seq_slot", seq_slot, torch.int32, 1)
+    _gpu("block_table", block_table, torch.int32, 2)
+    page_size = _check_pools(k_pool, v_pool, torch.bfloat16, kv_heads, head_dim)
+    if waves is None:
+        _, waves, _ = plan_fused(m, n // 32, k)
+    _require(waves in (1, 2, 4, 8), f"{waves} waves per workgroup is not a form the kernel has")
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=weight.device)
+    _run("cie_gemm_qkv_rope", load_library().cie_gemm_qkv_rope(
+        _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k), _i(waves), _ptr(cos),
+        _ptr(sin), _ptr(positions), _ptr(seq_of_token), _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]),
+        _ptr(k_pool), _ptr(v_pool), _i(q_heads), _i(kv_heads), _i(head_dim), _i(page_size),
+        _i(1 if rotate else 0), _i(1 if write_kv else 0)))
+    return out
+
+
 ARGMAX_CHUNK = 2048
 
 

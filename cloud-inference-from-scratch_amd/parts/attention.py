@@ -21,7 +21,7 @@ from ..config.specs import PartSpec
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, build_part, register_part
-from .linear import linear
+from .linear import FUSED_ROWS, linear
 
 
 class Attention(Part):
@@ -83,10 +83,19 @@ class Attention(Part):
             raise ValueError(
                 f"position {batch.max_context - 1} is beyond the rotary table of {self.position.max_position}"
             )
-        qkv = linear(x, self.w_qkv, self.b_qkv)
-        ops.rope_kv_write(qkv, self.cos, self.sin, batch.positions, batch.seq_of_token, batch.seq_slot,
-                          view.block_table, view.k_pool, view.v_pool, self.num_heads, self.num_kv_heads,
-                          self.head_dim, rotate=self.position.rotates, write_kv=writes)
+        rows = x.shape[0]
+        if (x.dtype == torch.bfloat16 and rows <= FUSED_ROWS and self.head_dim % 32 == 0
+                and x.shape[1] % 8 == 0 and (rows == 1 or x.stride(0) % 8 == 0)):
+            # few rows: the product's epilogue rotates and writes the cache itself
+            qkv = ops.gemm_qkv_rope(self.w_qkv, x, self.b_qkv, self.cos, self.sin, batch.positions,
+                                    batch.seq_of_token, batch.seq_slot, view.block_table, view.k_pool, view.v_pool,
+                                    self.num_heads, self.num_kv_heads, self.head_dim,
+                                    rotate=self.position.rotates, write_kv=writes)
+        else:
+            qkv = linear(x, self.w_qkv, self.b_qkv)
+            ops.rope_kv_write(qkv, self.cos, self.sin, batch.positions, batch.seq_of_token, batch.seq_slot,
+                              view.block_table, view.k_pool, view.v_pool, self.num_heads, self.num_kv_heads,
+                              self.head_dim, rotate=self.position.rotates, write_kv=writes)
         context = attend(qkv, batch, view, self.num_heads, self.num_kv_heads, self.head_dim,
                          self.window, self.scale)
         return linear(context, self.w_o, self.b_o, into=residual)

@@ -420,6 +420,55 @@ def test_rope_kv_write(ops, dtype, geometry):
     assert torch.equal(v_pool.transpose(2, 3)[untouched], v_before.transpose(2, 3)[untouched])
 
 
+@pytest.mark.parametrize("geometry", [(16, 2, 128, 16, 2048), (4, 2, 32, 8, 96), (3, 1, 64, 4, 328), (5, 5, 96, 32, 200)])
+@pytest.mark.parametrize("rows", [1, 7, 16])
+@pytest.mark.parametrize("waves", [None, 1, 8])
+def test_gemm_qkv_rope_equals_product_then_rotation(ops, geometry, rows, waves):
+    """The q/k/v product whose epilogue rotates and writes the cache, against the plain
+    product followed by the rotation kernel (themselves checked against the plain
+    implementation above): rotated queries, touched cache rows and untouched ones."""
+    q_heads, kv_heads, head_dim, page_size, hidden = geometry
+    n = (q_heads + 2 * kv_heads) * head_dim
+    lengths = [40, 5, 100, 17][: max(1, min(4, rows))]  # every sequence has at least rows / 4 tokens
+    k_pool, v_pool, table, slots, _ = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=44)
+    k_two, v_two = k_pool.clone(), v_pool.clone()
+    # the rows: the last tokens of the sequences in turn (decode rows), several per sequence when rows > sequences
+    positions, seq_of_token = [], []
+    for i in range(rows):
+        s = i % len(lengths)
+        positions.append(lengths[s] - 1 - i // len(lengths))
+        seq_of_token.append(s)
+    assert min(positions) >= 0
+    a = rand((rows, hidden), torch.bfloat16, 45)
+    w, b = rand((n, hidden), torch.bfloat16, 46, 0.3), rand((n,), torch.bfloat16, 47)
+    cos, sin = plain_qwen2.rope_tables(head_dim, 512, 1e6)
+    half = head_dim // 2
+    cos, sin = cos[:, :half].contiguous().cuda(), sin[:, :half].contiguous().cuda()
+    meta = (torch.tensor(positions, dtype=torch.int32).cuda(), torch.tensor(seq_of_token, dtype=torch.int32).cuda(),
+            torch.tensor(slots, dtype=torch.int32).cuda(), table)
+    fused = ops.gemm_qkv_rope(w, a, b, cos, sin, *meta, k_pool, v_pool, q_heads, kv_heads, head_dim, waves=waves)
+    plain_qkv = ops.gemm_fused(w, ops.EPI_BF16, a, bias=b, plan=None if waves is None else (1, waves, 1))
+    ops.rope_kv_write(plain_qkv, cos, sin, *meta, k_two, v_two, q_heads, kv_heads, head_dim)
+    q_cols = q_heads * head_dim
+    # one bf16 step at most (the two kernels may round a fused multiply-add differently)
+    step = dict(rtol=2 ** -7, atol=1e-6)
+    torch.testing.assert_close(fused[:, :q_cols].float(), plain_qkv[:, :q_cols].float(), **step)
+    torch.testing.assert_close(k_pool.float(), k_two.float(), **step)
+    assert torch.equal(v_pool, v_two)
+    # without rotation and without cache writes
+    k_before, v_before = k_pool.clone(), v_pool.clone()
+    bare = ops.gemm_qkv_rope(w, a, b, cos, sin, *meta, k_pool, v_pool, q_heads, kv_heads, head_dim, rotate=False,
+                             write_kv=False, waves=waves)
+    if waves is None:  # the two plans may cut K differently: sums in another order
+        torch.testing.assert_close(bare[:, :q_cols].float(), ops.gemm_fused(w, ops.EPI_BF16, a, bias=b)[:, :q_cols].float(), **step)
+    else:
+        assert torch.equal(bare[:, :q_cols], ops.gemm_fused(w, ops.EPI_BF16, a, bias=b, plan=(1, waves, 1))[:, :q_cols])
+    assert torch.equal(k_pool, k_before) and torch.equal(v_pool, v_before)
+    with pytest.raises(ValueError, match="steps of 32"):
+        ops.gemm_qkv_rope(w[: 3 * 16], a, None, cos[:, :8].contiguous(), sin[:, :8].contiguous(), *meta,
+                          k_pool[..., :16].contiguous(), v_pool[:, :, :16].contiguous(), 1, 1, 16)
+
+
 def test_rope_shift_invariance():
     """Scores of rotated q and k depend on the distance of their positions only
     (pins sign and pairing of the rotation in the plain implementation)."""
