@@ -322,3 +322,191 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         replay_util.compare(rows, reference, rtol=1e-4, atol=2e-5)
     # a slot handed to a new request starts from a cleared state (slots were reused above)
     assert runner.cache.stats().slots_used == 0
+
+
+# ----------------------------------------------------------------------------------------------------
+# A second toy architecture, again defined here and registered from outside the package: a feed-forward
+# with a router and experts, a position encoding of its own, and a windowed attention layer beside a
+# full one (two cache groups with pages of their own).  It is no model of anyone's.
+def register_routed_toy():
+    from cie_amd.config import register_architecture
+    from cie_amd.config.qwen2 import Qwen2Config
+    from cie_amd.config.specs import LayerCall, LayerSpec, ModelSpec, PartSpec
+    from cie_amd.parts.base import Part, register_part
+    from cie_amd.parts.position import RotaryHalf
+    from cie_amd.weights.tensors import TensorSpec
+
+    class RoutedExperts(Part):
+        """Top-1 of E small gated experts per token; router logits and softmax in float32; the
+        chosen expert's output is scaled by its probability."""
+
+        def __init__(self, hidden_size: int, expert_size: int, experts: int) -> None:
+            self.hidden_size, self.expert_size, self.experts = hidden_size, expert_size, experts
+
+        def expected_tensors(self, prefix):
+            out = {prefix + "router.weight": TensorSpec((self.experts, self.hidden_size))}
+            for e in range(self.experts):
+                out[f"{prefix}experts.{e}.gate_up.weight"] = TensorSpec((2 * self.expert_size, self.hidden_size))
+                out[f"{prefix}experts.{e}.down.weight"] = TensorSpec((self.hidden_size, self.expert_size))
+            return out
+
+        def bind(self, tensors, prefix, dtype, device):
+            super().bind(tensors, prefix, dtype, device)
+            self.router = tensors[prefix + "router.weight"].float()
+            self.gate_up = [tensors[f"{prefix}experts.{e}.gate_up.weight"] for e in range(self.experts)]
+            self.down = [tensors[f"{prefix}experts.{e}.down.weight"] for e in range(self.experts)]
+
+        def forward(self, x, residual=None):
+            from cie_amd.parts.linear import linear
+
+            probabilities = torch.softmax(x.float() @ self.router.t(), dim=-1)
+            weight, chosen = probabilities.max(dim=-1)
+            out = torch.zeros((x.shape[0], self.hidden_size), dtype=torch.float32, device=x.device)
+            for e in range(self.experts):
+                rows = (chosen == e).nonzero().flatten()
+                if rows.numel():
+                    hidden = linear(x[rows].contiguous(), self.gate_up[e], epilogue="silu")
+                    out[rows] = linear(hidden, self.down[e]).float() * weight[rows, None]
+            return out.to(x.dtype)
+
+    class SlowRotary(RotaryHalf):
+        """Rotary encoding whose positions advance by 1/factor per token."""
+
+        def __init__(self, head_dim: int, theta: float, max_position: int, factor: float) -> None:
+            super().__init__(head_dim=head_dim, theta=theta, max_position=max_position)
+            self.factor = factor
+
+        def tables(self, device):
+            inv_freq = 1.0 / (self.theta ** (torch.arange(0, self.head_dim, 2, dtype=torch.float32) / self.head_dim))
+            angles = (torch.arange(self.max_position, dtype=torch.float32) / self.factor)[:, None] * inv_freq[None, :]
+            return angles.cos().to(device).contiguous(), angles.sin().to(device).contiguous()
+
+    class RoutedToyConfig(Qwen2Config):
+        architecture = "ToyRoutedWindowForCausalLM"
+        WINDOW, FACTOR, EXPERTS, EXPERT_SIZE = 20, 4.0, 3, 24
+
+        def model_spec(self) -> ModelSpec:
+            base = super().model_spec()
+            plain_layer = base.layers[0]
+            slow = PartSpec.of("slow_rotary", head_dim=self.head_dim, theta=self.rope_theta,
+                               max_position=self.max_position_embeddings, factor=self.FACTOR)
+            windowed = PartSpec.of("attention", **{**dict(plain_layer.mixer.params), "window": self.WINDOW})
+            slowed = PartSpec.of("attention", **{**dict(plain_layer.mixer.params), "position": slow})
+            routed = PartSpec.of("routed_experts", hidden_size=self.hidden_size, expert_size=self.EXPERT_SIZE,
+                                 experts=self.EXPERTS)
+            first = LayerSpec(mixer=windowed, feed_forward=routed, norm1=plain_layer.norm1, norm2=plain_layer.norm2,
+                              names=(("norm1", "input_layernorm"), ("mixer", "self_attn"),
+                                     ("norm2", "post_attention_layernorm"), ("feed_forward", "moe")))
+            second = LayerSpec(mixer=slowed, feed_forward=plain_layer.feed_forward, norm1=plain_layer.norm1,
+                               norm2=plain_layer.norm2, names=plain_layer.names)
+            return ModelSpec(
+                architecture=self.architecture, vocab_size=self.vocab_size, hidden_size=self.hidden_size,
+                layers=(first, second), order=(LayerCall(0, 0), LayerCall(1, 1)),
+                final_norm=base.final_norm, tie_word_embeddings=True, max_position=self.max_position_embeddings)
+
+    register_part("feed_forward", "routed_experts", RoutedExperts)
+    register_part("position", "slow_rotary", SlowRotary)
+    register_architecture("ToyRoutedWindowForCausalLM", RoutedToyConfig)
+    return RoutedToyConfig
+
+
+def routed_toy_plain(raw, weights, tokens, config_class):
+    """Whole-sequence reference of the second toy model, from the plain parts."""
+    eps, d = raw["rms_norm_eps"], plain.head_dim_of(raw)
+    t = len(tokens)
+    h = weights["model.embed_tokens.weight"][torch.tensor(tokens)]
+    positions = torch.arange(t)
+    cos, sin = plain.rope_tables(d, t, raw["rope_theta"])
+    inv_freq = 1.0 / (raw["rope_theta"] ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    slow_angles = (positions.float() / config_class.FACTOR)[:, None] * inv_freq[None, :]
+    slow_cos, slow_sin = torch.cat([slow_angles.cos()] * 2, dim=-1), torch.cat([slow_angles.sin()] * 2, dim=-1)
+
+    def attention(x, p, cos_t, sin_t, window):
+        def proj(name):
+            return plain.linear(x, weights[f"{p}{name}.weight"], weights[f"{p}{name}.bias"]).view(t, -1, d)
+        q, k, v = proj("q_proj"), proj("k_proj"), proj("v_proj")
+        q, k = plain.apply_rope(q, cos_t, sin_t, positions), plain.apply_rope(k, cos_t, sin_t, positions)
+        context = plain.causal_attention(q, k, v, 1.0 / math.sqrt(d), past_len=0, window=window)
+        return plain.linear(context, weights[p + "o_proj.weight"])
+
+    def routed(x, p):
+        probabilities = torch.softmax(x @ weights[p + "router.weight"].t(), dim=-1)
+        weight, chosen = probabilities.max(dim=-1)
+        out = torch.zeros_like(x)
+        for row in range(t):
+            e = int(chosen[row])
+            gate_up = weights[f"{p}experts.{e}.gate_up.weight"]
+            half = gate_up.shape[0] // 2
+            out[row] = plain.swiglu(x[row:row + 1], gate_up[:half], gate_up[half:], weights[f"{p}experts.{e}.down.weight"])[0] * weight[row]
+        return out
+
+    p = "model.layers.0."
+    h = h + attention(plain.rms_norm(h, weights[p + "input_layernorm.weight"], eps), p + "self_attn.", cos, sin,
+                      config_class.WINDOW)
+    h = h + routed(plain.rms_norm(h, weights[p + "post_attention_layernorm.weight"], eps), p + "moe.")
+    p = "model.layers.1."
+    h = h + attention(plain.rms_norm(h, weights[p + "input_layernorm.weight"], eps), p + "self_attn.", slow_cos[:, :d],
+                      slow_sin[:, :d], None)
+    h = h + plain.swiglu(plain.rms_norm(h, weights[p + "post_attention_layernorm.weight"], eps),
+                         weights[p + "mlp.gate_proj.weight"], weights[p + "mlp.up_proj.weight"],
+                         weights[p + "mlp.down_proj.weight"])
+    h = plain.rms_norm(h, weights["model.norm.weight"], eps)
+    return h @ weights["model.embed_tokens.weight"].t()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_own_position_encoding_and_window_layer(tmp_path, dtype):
+    """Registered from here: a feed-forward with a router, a position encoding of its own, and a layer
+    whose attention sees a window only.  The windowed layer's cache is a group of its own: its pages
+    come back as the window passes them, while the full layer keeps all of its pages."""
+    from cie_amd.config import build_engine_config, load_config
+    from cie_amd.engine import Runner, load_model
+    from cie_amd.parts.model import expected_tensors
+    from cie_amd.weights import RandomSource, write_tensors
+
+    config_class = register_routed_toy()
+    # bfloat16 could choose another expert than float32 where two router logits nearly tie, and everything
+    # after would differ: there the toy runs a single expert (probability 1: the router changes nothing)
+    config_class.EXPERTS = 3 if dtype == "float32" else 1
+    raw = dict(architectures=["ToyRoutedWindowForCausalLM"], model_type="qwen2", hidden_size=64, num_hidden_layers=2,
+               num_attention_heads=4, num_key_value_heads=2, head_dim=32, intermediate_size=72, vocab_size=80,
+               rms_norm_eps=1e-5, rope_theta=1e4, max_position_embeddings=160, tie_word_embeddings=True)
+    write_tensors(tmp_path, raw, {})
+    config = load_config(tmp_path)
+    expected = expected_tensors(config.model_spec())
+    last_expert = config_class.EXPERTS - 1
+    assert f"model.layers.0.moe.experts.{last_expert}.down.weight" in expected
+    assert "model.layers.1.mlp.down_proj.weight" in expected
+    tensors = RandomSource(9, std=0.15).load(expected, "float32", "cpu")
+    if dtype == "bfloat16":  # the plain model runs the weights the engine holds
+        tensors = {k: (v.to(torch.bfloat16).float() if v.is_floating_point() else v) for k, v in tensors.items()}
+    write_tensors(tmp_path, raw, tensors)
+    model, _ = load_model(tmp_path, dtype)
+    engine_config = build_engine_config(dtype=dtype, page_size=8, kv_tokens=512, max_running=4, max_model_len=160,
+                                        prefix_cache_pages=0, graph_decode=False)
+    runner = Runner(model, engine_config)
+    groups = runner.cache.groups
+    assert len(groups) == 2 and {g.spec.window for g in groups} == {config_class.WINDOW, None}
+    requests = {f"r{i}": random_tokens(n, 80, 90 + i) for i, n in enumerate([70, 33, 9, 120, 41])}
+    reference = {rid: routed_toy_plain(raw, tensors, tokens, config_class) for rid, tokens in requests.items()}
+    # bfloat16 rounds every activation to 8 bits of a row's magnitude: the absolute part of the tolerance is
+    # the replay tests' 2e-2 per unit of logit magnitude (these weights are larger than theirs: logits of +-3)
+    magnitude = max(1.0, max(float(r.abs().max()) for r in reference.values()))
+    tolerance = dict(rtol=1e-4, atol=2e-5) if dtype == "float32" else dict(rtol=2e-2, atol=2e-2 * magnitude)
+    for schedule in (replay_util.whole, replay_util.portions, lambda r: replay_util.mixed(r, live=3)):
+        steps = schedule(requests)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        replay_util.compare(rows, reference, **tolerance)
+        assert runner.cache.stats().pages_used == 0
+    # while a long request is alive, the windowed group holds a few pages, the full group all of them
+    runner.cache.admit("long")
+    from cie_amd.engine.runner import StepEntry
+    tokens = requests["r3"]
+    for start in range(0, 120, 24):
+        runner.run([StepEntry("long", tokens[start:start + 24], start, [])])
+    windowed = next(g for g in groups if g.spec.window is not None)
+    full = next(g for g in groups if g.spec.window is None)
+    held = lambda g: sum(1 for page in g.tables["long"] if page >= 0)  # noqa: E731
+    assert held(full) == 15 and held(windowed) <= -(-config_class.WINDOW // 8) + 1
+    runner.cache.release("long")
+    runner.cache.assert_invariants()
