@@ -1,0 +1,106 @@
+// Matrix products with many rows go to the vendor library (hipBLASLt), as the reference leaves its
+// products to a library.  This is the thin host side of that: one handle, and for every shape the
+// descriptors and the algorithm the library's heuristic picks, kept after the first call, so that a
+// step's few hundred products cost a table lookup and one launch each instead of a heuristic query.
+//
+//   C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]),  bf16 operands, bias and result, float32 sums
+//
+// In the library's column-major terms: D (N x M, ld N) = W^T (W stored K x N, ld K, transposed) *
+// A (K x M, ld lda); the bias is added along D's rows (the N dimension).
+#include <hipblaslt/hipblaslt.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "common.h"
+
+namespace {
+
+struct Plan {
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatrixLayout_t w = nullptr, a = nullptr, d = nullptr;
+    hipblasLtMatmulAlgo_t algo;
+    size_t workspace = 0;
+};
+
+using Key = std::tuple<int, int, int, int, int>;  // M, N, K, lda, has bias
+
+hipblasLtHandle_t g_handle = nullptr;
+std::map<Key, Plan> g_plans;
+std::mutex g_mutex;
+
+bool ok(hipblasStatus_t status) { return status == HIPBLAS_STATUS_SUCCESS; }
+
+void destroy(Plan& plan) {
+    if (plan.d) hipblasLtMatrixLayoutDestroy(plan.d);
+    if (plan.a) hipblasLtMatrixLayoutDestroy(plan.a);
+    if (plan.w) hipblasLtMatrixLayoutDestroy(plan.w);
+    if (plan.desc) hipblasLtMatmulDescDestroy(plan.desc);
+    plan = Plan{};
+}
+
+// Descriptors and the heuristic's first algorithm for a shape; false if the library has none.
+bool make_plan(Plan& plan, int M, int N, int K, int lda, bool has_bias, size_t workspace_limit) {
+    const hipblasOperation_t transposed = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
+    bool good = ok(hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F)) &&
+                ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed))) &&
+                ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain))) &&
+                ok(hipblasLtMatrixLayoutCreate(&plan.w, HIP_R_16BF, K, N, K)) &&
+                ok(hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, K, M, lda)) &&
+                ok(hipblasLtMatrixLayoutCreate(&plan.d, HIP_R_16BF, N, M, N));
+    if (good && has_bias) {
+        const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
+        const hipDataType bias_type = HIP_R_16BF;
+        good = ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue))) &&
+               ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)));
+    }
+    if (!good) return false;
+    hipblasLtMatmulPreference_t preference = nullptr;
+    if (!ok(hipblasLtMatmulPreferenceCreate(&preference))) return false;
+    const uint64_t limit = workspace_limit;
+    hipblasLtMatmulHeuristicResult_t found;
+    int count = 0;
+    good = ok(hipblasLtMatmulPreferenceSetAttribute(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit))) &&
+           ok(hipblasLtMatmulAlgoGetHeuristic(g_handle, plan.desc, plan.w, plan.a, plan.d, plan.d, preference, 1, &found, &count)) &&
+           count > 0 && ok(found.state);
+    hipblasLtMatmulPreferenceDestroy(preference);
+    if (!good) return false;
+    plan.algo = found.algo;
+    plan.workspace = found.workspaceSize;
+    return plan.workspace <= workspace_limit;
+}
+
+}  // namespace
+
+// Returns CIE_BAD_ARGUMENT for a shape the library has no algorithm for (the caller then takes another
+// route) and CIE_LAUNCH_FAILED if the library's call itself fails.  `workspace` is device memory of
+// `workspace_bytes` that stays valid while the product runs; calls on one stream may share it.
+CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w, const void* bias, void* c, int M,
+                             int N, int K, void* workspace, size_t workspace_bytes) {
+    if (M <= 0 || N <= 0 || K <= 0 || lda < K || !a || !w || !c) return CIE_BAD_ARGUMENT;
+    Plan* plan = nullptr;
+    {
+        std::lock_guard<std::mutex> guard(g_mutex);
+        if (!g_handle && !ok(hipblasLtCreate(&g_handle))) return CIE_LAUNCH_FAILED;
+        const Key key{M, N, K, lda, bias ? 1 : 0};
+        auto it = g_plans.find(key);
+        if (it == g_plans.end()) {
+            Plan fresh;
+            if (!make_plan(fresh, M, N, K, lda, bias != nullptr, workspace ? workspace_bytes : 0)) {
+                destroy(fresh);
+                return CIE_BAD_ARGUMENT;
+            }
+            it = g_plans.emplace(key, fresh).first;
+        }
+        plan = &it->second;
+    }
+    if (bias &&
+        !ok(hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias))))
+        return CIE_LAUNCH_FAILED;
+    const float one = 1.f, zero = 0.f;
+    const hipblasStatus_t status =
+        hipblasLtMatmul(g_handle, plan->desc, &one, w, plan->w, a, plan->a, &zero, c, plan->d, c, plan->d, &plan->algo,
+                        workspace, plan->workspace, static_cast<hipStream_t>(stream));
+    return ok(status) ? CIE_OK : CIE_LAUNCH_FAILED;
+}

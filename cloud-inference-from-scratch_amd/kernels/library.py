@@ -32,6 +32,9 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
+# The products with many rows go through the vendor's library (csrc/gemm_library.hip).
+LINK_LIBS = ["-lhipblaslt"]
+
 _lock = threading.Lock()
 _library: ctypes.CDLL | None = None
 
@@ -49,7 +52,7 @@ def source_hash() -> str:
     for path in sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h"))):
         digest.update(path.name.encode())
         digest.update(path.read_bytes())
-    digest.update(" ".join(HIPCC_FLAGS).encode())
+    digest.update(" ".join(HIPCC_FLAGS + LINK_LIBS).encode())
     return digest.hexdigest()
 
 
@@ -116,7 +119,7 @@ def build_library(force: bool = True) -> Path:
     with ThreadPoolExecutor(max_workers=workers) as pool:
         objects = list(pool.map(compile_one, files))
     scratch = folder / f"{LIB_NAME}.{os.getpid()}.tmp"
-    link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(scratch), *map(str, objects)]
+    link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(scratch), *map(str, objects), *LINK_LIBS]
     done = subprocess.run(link, env=env, capture_output=True, text=True)
     if done.returncode != 0:
         raise KernelLibraryError(f"linking {LIB_NAME} failed:\n{done.stderr[-4000:]}")

@@ -31,18 +31,17 @@ def _code(dtype: torch.dtype) -> int:
         raise ValueError(f"kernels take float32 or bfloat16, got {dtype}") from None
 
 
-def _require(condition: bool, message: str) -> None:
-    if not condition:
-        raise ValueError(message)
-
-
 def _gpu(name: str, tensor: torch.Tensor, dtype: Optional[torch.dtype] = None, dims: Optional[int] = None) -> None:
-    _require(tensor.is_cuda, f"{name} must live on the GPU, is on {tensor.device}")
-    _require(tensor.is_contiguous(), f"{name} must be contiguous")
+    if not tensor.is_cuda:
+        raise ValueError(f"{name} must live on the GPU, is on {tensor.device}")
+    if not tensor.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
     if dtype is not None:
-        _require(tensor.dtype == dtype, f"{name} must be {dtype}, is {tensor.dtype}")
+        if not (tensor.dtype == dtype):
+            raise ValueError(f"{name} must be {dtype}, is {tensor.dtype}")
     if dims is not None:
-        _require(tensor.dim() == dims, f"{name} must have {dims} dims, has shape {tuple(tensor.shape)}")
+        if not (tensor.dim() == dims):
+            raise ValueError(f"{name} must have {dims} dims, has shape {tuple(tensor.shape)}")
 
 
 def _ptr(tensor: Optional[torch.Tensor]) -> ctypes.c_void_p:
@@ -50,7 +49,8 @@ def _ptr(tensor: Optional[torch.Tensor]) -> ctypes.c_void_p:
 
 
 def _stream() -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the raw handle of torch's current stream (also the capturing one), without building a Stream object
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
 
 
 def _run(name: str, code: int) -> None:
@@ -72,10 +72,10 @@ def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, dtype: torch.dtype,
     _gpu("k_pool", k_pool, dtype, 4)
     _gpu("v_pool", v_pool, dtype, 4)
     pages, heads, page_size, dim = k_pool.shape
-    _require(heads == kv_heads and dim == head_dim,
-             f"k_pool {tuple(k_pool.shape)} does not match Hkv={kv_heads}, D={head_dim}")
-    _require(tuple(v_pool.shape) == (pages, kv_heads, head_dim, page_size),
-             f"v_pool {tuple(v_pool.shape)} must be {(pages, kv_heads, head_dim, page_size)}")
+    if not (heads == kv_heads and dim == head_dim):
+        raise ValueError(f"k_pool {tuple(k_pool.shape)} does not match Hkv={kv_heads}, D={head_dim}")
+    if not (tuple(v_pool.shape) == (pages, kv_heads, head_dim, page_size)):
+        raise ValueError(f"v_pool {tuple(v_pool.shape)} must be {(pages, kv_heads, head_dim, page_size)}")
     return page_size
 
 
@@ -89,7 +89,8 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = 
     if out is None:
         out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
     _gpu("out", out, torch.float32, 2)
-    _require(out.shape == (tokens, hidden), f"out must be {(tokens, hidden)}, is {tuple(out.shape)}")
+    if not (out.shape == (tokens, hidden)):
+        raise ValueError(f"out must be {(tokens, hidden)}, is {tuple(out.shape)}")
     _run("cie_embed", load_library().cie_embed(_stream(), _i(_code(table.dtype)), _ptr(table), _ptr(ids),
                                                _ptr(out), _i(tokens), _i(hidden), _i(vocab)))
     return out
@@ -106,13 +107,18 @@ def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: 
     _gpu("residual", residual, torch.float32, 2)
     tokens, hidden = residual.shape
     _gpu("weight", weight, dims=1)
-    _require(weight.shape[0] == hidden, f"weight must be [{hidden}], is {tuple(weight.shape)}")
-    _require(weight.dtype in (out_dtype, torch.float32), f"weight dtype {weight.dtype} does not fit {out_dtype}")
-    _require(hidden * 4 <= 64 * 1024, f"hidden size {hidden} exceeds the norm kernel's 16384")
-    _require(eps > 0, f"eps must be positive, is {eps}")
+    if not (weight.shape[0] == hidden):
+        raise ValueError(f"weight must be [{hidden}], is {tuple(weight.shape)}")
+    if not (weight.dtype in (out_dtype, torch.float32)):
+        raise ValueError(f"weight dtype {weight.dtype} does not fit {out_dtype}")
+    if not (hidden * 4 <= 64 * 1024):
+        raise ValueError(f"hidden size {hidden} exceeds the norm kernel's 16384")
+    if not (eps > 0):
+        raise ValueError(f"eps must be positive, is {eps}")
     if branch is not None:
         _gpu("branch", branch, out_dtype, 2)
-        _require(branch.shape == residual.shape, f"branch {tuple(branch.shape)} vs residual {tuple(residual.shape)}")
+        if not (branch.shape == residual.shape):
+            raise ValueError(f"branch {tuple(branch.shape)} vs residual {tuple(residual.shape)}")
     if rows is not None:
         _gpu("rows", rows, torch.int32, 1)
         n_out = rows.shape[0]
@@ -121,7 +127,8 @@ def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: 
     if out is None:
         out = torch.empty((n_out, hidden), dtype=out_dtype, device=residual.device)
     _gpu("out", out, out_dtype, 2)
-    _require(out.shape == (n_out, hidden), f"out must be {(n_out, hidden)}, is {tuple(out.shape)}")
+    if not (out.shape == (n_out, hidden)):
+        raise ValueError(f"out must be {(n_out, hidden)}, is {tuple(out.shape)}")
     _run("cie_add_rmsnorm", load_library().cie_add_rmsnorm(
         _stream(), _i(_code(out_dtype)), _i(_code(weight.dtype)), _ptr(residual), _ptr(branch), _ptr(weight),
         _ptr(out), _ptr(rows), _i(n_out), _i(hidden), _f(eps), _i(0 if rows is not None else 1)))
@@ -134,10 +141,13 @@ def add_parts_rmsnorm(residual: torch.Tensor, parts: torch.Tensor, weight: torch
     _gpu("residual", residual, torch.float32, 2)
     tokens, hidden = residual.shape
     _gpu("parts", parts, torch.float32, 3)
-    _require(parts.shape[1:] == residual.shape, f"parts {tuple(parts.shape)} vs residual {tuple(residual.shape)}")
+    if not (parts.shape[1:] == residual.shape):
+        raise ValueError(f"parts {tuple(parts.shape)} vs residual {tuple(residual.shape)}")
     _gpu("weight", weight, dims=1)
-    _require(weight.shape[0] == hidden and weight.dtype in (torch.bfloat16, torch.float32), "norm weight does not fit")
-    _require(hidden * 4 <= 64 * 1024 and eps > 0, f"hidden {hidden} or eps {eps} out of range")
+    if not (weight.shape[0] == hidden and weight.dtype in (torch.bfloat16, torch.float32)):
+        raise ValueError("norm weight does not fit")
+    if not (hidden * 4 <= 64 * 1024 and eps > 0):
+        raise ValueError(f"hidden {hidden} or eps {eps} out of range")
     if rows is not None:
         _gpu("rows", rows, torch.int32, 1)
     n_out = rows.shape[0] if rows is not None else tokens
@@ -153,10 +163,13 @@ def rmsnorm_from_sumsq(residual: torch.Tensor, sumsq: torch.Tensor, weight: torc
     _gpu("residual", residual, torch.float32, 2)
     rows, hidden = residual.shape
     _gpu("sumsq", sumsq, torch.float32, 2)
-    _require(sumsq.shape[0] >= rows, f"sumsq has {sumsq.shape[0]} rows for {rows}")
+    if not (sumsq.shape[0] >= rows):
+        raise ValueError(f"sumsq has {sumsq.shape[0]} rows for {rows}")
     _gpu("weight", weight, dims=1)
-    _require(weight.shape[0] == hidden and weight.dtype in (torch.bfloat16, torch.float32), "norm weight does not fit")
-    _require(eps > 0, f"eps must be positive, is {eps}")
+    if not (weight.shape[0] == hidden and weight.dtype in (torch.bfloat16, torch.float32)):
+        raise ValueError("norm weight does not fit")
+    if not (eps > 0):
+        raise ValueError(f"eps must be positive, is {eps}")
     out = torch.empty((rows, hidden), dtype=torch.bfloat16, device=residual.device)
     _run("cie_rmsnorm_from_sumsq", load_library().cie_rmsnorm_from_sumsq(
         _stream(), _i(_code(weight.dtype)), _ptr(residual), _ptr(sumsq), _i(sumsq.shape[1]), _ptr(weight), _ptr(out),
@@ -175,16 +188,20 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
     dtype; block_table int32 [slots, width]."""
     _gpu("qkv", qkv, dims=2)
     tokens = qkv.shape[0]
-    _require(qkv.shape[1] == (q_heads + 2 * kv_heads) * head_dim,
-             f"qkv row is {qkv.shape[1]}, heads say {(q_heads + 2 * kv_heads) * head_dim}")
-    _require(head_dim % 2 == 0, f"head_dim must be even, is {head_dim}")
+    if not (qkv.shape[1] == (q_heads + 2 * kv_heads) * head_dim):
+        raise ValueError(f"qkv row is {qkv.shape[1]}, heads say {(q_heads + 2 * kv_heads) * head_dim}")
+    if not (head_dim % 2 == 0):
+        raise ValueError(f"head_dim must be even, is {head_dim}")
     for name, table in (("cos", cos), ("sin", sin)):
         _gpu(name, table, torch.float32, 2)
-        _require(table.shape[1] == head_dim // 2, f"{name} must be [max_position, {head_dim // 2}]")
-    _require(cos.shape == sin.shape, "cos and sin tables differ in shape")
+        if not (table.shape[1] == head_dim // 2):
+            raise ValueError(f"{name} must be [max_position, {head_dim // 2}]")
+    if not (cos.shape == sin.shape):
+        raise ValueError("cos and sin tables differ in shape")
     for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
         _gpu(name, meta, torch.int32, 1)
-        _require(meta.shape[0] >= tokens, f"{name} has {meta.shape[0]} entries for {tokens} tokens")
+        if not (meta.shape[0] >= tokens):
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {tokens} tokens")
     _gpu("seq_slot", seq_slot, torch.int32, 1)
     _gpu("block_table", block_table, torch.int32, 2)
     page_size = _check_pools(k_pool, v_pool, qkv.dtype, kv_heads, head_dim)
@@ -198,12 +215,14 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for gate_up [T, 2I]."""
     _gpu("gate_up", gate_up, dims=2)
     tokens, twice = gate_up.shape
-    _require(twice % 2 == 0, f"gate_up row must be even, is {twice}")
+    if not (twice % 2 == 0):
+        raise ValueError(f"gate_up row must be even, is {twice}")
     inter = twice // 2
     if out is None:
         out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
     _gpu("out", out, gate_up.dtype, 2)
-    _require(out.shape == (tokens, inter), f"out must be {(tokens, inter)}, is {tuple(out.shape)}")
+    if not (out.shape == (tokens, inter)):
+        raise ValueError(f"out must be {(tokens, inter)}, is {tuple(out.shape)}")
     _run("cie_silu_mul", load_library().cie_silu_mul(_stream(), _i(_code(gate_up.dtype)), _ptr(gate_up),
                                                      _ptr(out), _i(tokens), _i(inter)))
     return out
@@ -219,22 +238,28 @@ def paged_attention_generic(q: torch.Tensor, q_row_stride: int, k_pool: torch.Te
     ``q`` is any tensor whose row ``t`` holds the token's q heads in its first
     ``q_heads*head_dim`` elements, rows ``q_row_stride`` elements apart (the
     fused qkv buffer qualifies).  Returns [tokens, q_heads*head_dim]."""
-    _require(q.is_cuda and q.dim() == 2 and q.stride(1) == 1 and q.stride(0) == q_row_stride,
-             f"q must be 2-d on the GPU with unit inner stride and row stride {q_row_stride}")
-    _require(q.shape[0] >= tokens and q.shape[1] >= q_heads * head_dim, f"q {tuple(q.shape)} too small")
-    _require(q_heads % kv_heads == 0, f"{q_heads} query heads are no multiple of {kv_heads} key heads")
-    _require(head_dim % 8 == 0 and head_dim <= 256, f"head_dim must be a multiple of 8 up to 256, is {head_dim}")
-    _require(q_row_stride % 8 == 0, f"q row stride must be a multiple of 8, is {q_row_stride}")
+    if not (q.is_cuda and q.dim() == 2 and q.stride(1) == 1 and q.stride(0) == q_row_stride):
+        raise ValueError(f"q must be 2-d on the GPU with unit inner stride and row stride {q_row_stride}")
+    if not (q.shape[0] >= tokens and q.shape[1] >= q_heads * head_dim):
+        raise ValueError(f"q {tuple(q.shape)} too small")
+    if not (q_heads % kv_heads == 0):
+        raise ValueError(f"{q_heads} query heads are no multiple of {kv_heads} key heads")
+    if not (head_dim % 8 == 0 and head_dim <= 256):
+        raise ValueError(f"head_dim must be a multiple of 8 up to 256, is {head_dim}")
+    if not (q_row_stride % 8 == 0):
+        raise ValueError(f"q row stride must be a multiple of 8, is {q_row_stride}")
     _check_pools(k_pool, v_pool, q.dtype, kv_heads, head_dim)
     _gpu("block_table", block_table, torch.int32, 2)
     for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
         _gpu(name, meta, torch.int32, 1)
-        _require(meta.shape[0] >= tokens, f"{name} has {meta.shape[0]} entries for {tokens} tokens")
+        if not (meta.shape[0] >= tokens):
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {tokens} tokens")
     _gpu("seq_slot", seq_slot, torch.int32, 1)
     if out is None:
         out = torch.empty((tokens, q_heads * head_dim), dtype=q.dtype, device=q.device)
     _gpu("out", out, q.dtype, 2)
-    _require(out.shape == (tokens, q_heads * head_dim), f"out is {tuple(out.shape)}")
+    if not (out.shape == (tokens, q_heads * head_dim)):
+        raise ValueError(f"out is {tuple(out.shape)}")
     _run("cie_paged_attention_generic", load_library().cie_paged_attention_generic(
         _stream(), _i(_code(q.dtype)), _ptr(q), _i(q_row_stride), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
         _i(block_table.shape[1]), _ptr(positions), _ptr(seq_of_token), _ptr(seq_slot), _ptr(out), _i(tokens),
@@ -263,41 +288,55 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
     step's longest context) and merged through the workspaces.  ``tile_waves=4`` gives
     every tile (and every part of its keys) a workgroup of four waves that take the
     blocks of 32 keys in turn; it needs pages of at least 16 keys."""
-    _require(q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 2 and q.stride(1) == 1
-             and q.stride(0) == q_row_stride, "q must be a bf16 GPU matrix with unit inner stride")
-    _require(q.shape[1] >= q_heads * head_dim and q_row_stride % 8 == 0, f"q {tuple(q.shape)} does not fit")
-    _require(head_dim in MFMA_HEAD_DIMS, f"head_dim must be one of {MFMA_HEAD_DIMS}, is {head_dim}")
-    _require(q_heads % kv_heads == 0, f"{q_heads} query heads are no multiple of {kv_heads} key heads")
+    if not (
+        q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 2 and q.stride(1) == 1 and q.stride(0) == q_row_stride
+    ):
+        raise ValueError("q must be a bf16 GPU matrix with unit inner stride")
+    if not (q.shape[1] >= q_heads * head_dim and q_row_stride % 8 == 0):
+        raise ValueError(f"q {tuple(q.shape)} does not fit")
+    if not (head_dim in MFMA_HEAD_DIMS):
+        raise ValueError(f"head_dim must be one of {MFMA_HEAD_DIMS}, is {head_dim}")
+    if not (q_heads % kv_heads == 0):
+        raise ValueError(f"{q_heads} query heads are no multiple of {kv_heads} key heads")
     group = q_heads // kv_heads
-    _require(row_tiles in (1, 2, 4) and 1 <= tokens_per_tile and tokens_per_tile * group <= 16 * row_tiles,
-             f"{tokens_per_tile} tokens of {group} heads do not fit {row_tiles} row tiles")
+    if not (row_tiles in (1, 2, 4) and 1 <= tokens_per_tile and tokens_per_tile * group <= 16 * row_tiles):
+        raise ValueError(f"{tokens_per_tile} tokens of {group} heads do not fit {row_tiles} row tiles")
     page_size = _check_pools(k_pool, v_pool, torch.bfloat16, kv_heads, head_dim)
-    _require(page_size >= 4 and page_size & (page_size - 1) == 0, f"page size must be a power of two >= 4, is {page_size}")
+    if not (page_size >= 4 and page_size & (page_size - 1) == 0):
+        raise ValueError(f"page size must be a power of two >= 4, is {page_size}")
     _gpu("block_table", block_table, torch.int32, 2)
     for name, meta in (("tile_seq", tile_seq), ("tile_q0", tile_q0)):
         _gpu(name, meta, torch.int32, 1)
-        _require(meta.shape[0] >= n_tiles, f"{name} has {meta.shape[0]} entries for {n_tiles} tiles")
+        if not (meta.shape[0] >= n_tiles):
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {n_tiles} tiles")
     for name, meta in (("seq_slot", seq_slot), ("seq_start", seq_start), ("seq_q_len", seq_q_len),
                        ("q_start_loc", q_start_loc)):
         _gpu(name, meta, torch.int32, 1)
     _gpu("out", out, torch.bfloat16, 2)
-    _require(out.shape[1] == q_heads * head_dim and out.shape[0] <= q.shape[0], f"out is {tuple(out.shape)}")
-    _require(1 <= n_splits <= 65535, f"n_splits {n_splits} out of range")
-    _require(tile_waves == 1 or (tile_waves == TILE_WAVES and scale > 0 and page_size >= 16
-                                 and (row_tiles == 1 or head_dim <= 128)),
-             f"tile_waves {tile_waves} with {n_splits} splits, {row_tiles} row tiles, head size {head_dim}, pages of {page_size}")
+    if not (out.shape[1] == q_heads * head_dim and out.shape[0] <= q.shape[0]):
+        raise ValueError(f"out is {tuple(out.shape)}")
+    if not (1 <= n_splits <= 65535):
+        raise ValueError(f"n_splits {n_splits} out of range")
+    if not (
+        tile_waves == 1
+        or (tile_waves == TILE_WAVES and scale > 0 and page_size >= 16 and (row_tiles == 1 or head_dim <= 128))
+    ):
+        raise ValueError(f"tile_waves {tile_waves} with {n_splits} splits, {row_tiles} row tiles, head size {head_dim}, "
+                         f"pages of {page_size}")
     if n_splits > 1:
         rows = 16 * row_tiles
-        _require(part_o is not None and part_ml is not None, "split attention needs its workspaces")
+        if not (part_o is not None and part_ml is not None):
+            raise ValueError("split attention needs its workspaces")
         _gpu("part_o", part_o, torch.float32)
         _gpu("part_ml", part_ml, torch.float32)
         units = n_tiles * kv_heads * n_splits
-        _require(part_o.numel() >= units * rows * head_dim and part_ml.numel() >= units * rows * 2,
-                 "attention workspaces are too small")
+        if not (part_o.numel() >= units * rows * head_dim and part_ml.numel() >= units * rows * 2):
+            raise ValueError("attention workspaces are too small")
         if max_context_dev is not None:
             _gpu("max_context_dev", max_context_dev, torch.int32)
         else:
-            _require(keys_per_split > 0 and keys_per_split % 32 == 0, f"keys_per_split {keys_per_split} must be a multiple of 32")
+            if not (keys_per_split > 0 and keys_per_split % 32 == 0):
+                raise ValueError(f"keys_per_split {keys_per_split} must be a multiple of 32")
     _run("cie_paged_attention_mfma", load_library().cie_paged_attention_mfma(
         _stream(), _ptr(q), _i(q_row_stride), _ptr(k_pool), _ptr(v_pool), _ptr(block_table),
         _i(block_table.shape[1]), _ptr(tile_seq), _ptr(tile_q0), _ptr(seq_slot), _ptr(seq_start), _ptr(seq_q_len),
@@ -309,19 +348,22 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
 def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
              out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """True float32 ``a @ weight.T + bias``; a [M, K] (rows may be strided), weight [N, K]."""
-    _require(a.is_cuda and a.dtype == torch.float32 and a.dim() == 2 and a.stride(1) == 1,
-             "a must be a float32 GPU matrix with unit inner stride")
+    if not (a.is_cuda and a.dtype == torch.float32 and a.dim() == 2 and a.stride(1) == 1):
+        raise ValueError("a must be a float32 GPU matrix with unit inner stride")
     _gpu("weight", weight, torch.float32, 2)
     m, k = a.shape
     n = weight.shape[0]
-    _require(weight.shape[1] == k, f"a is [{m},{k}] but weight is {tuple(weight.shape)}")
+    if not (weight.shape[1] == k):
+        raise ValueError(f"a is [{m},{k}] but weight is {tuple(weight.shape)}")
     if bias is not None:
         _gpu("bias", bias, torch.float32, 1)
-        _require(bias.shape[0] == n, f"bias must be [{n}]")
+        if not (bias.shape[0] == n):
+            raise ValueError(f"bias must be [{n}]")
     if out is None:
         out = torch.empty((m, n), dtype=torch.float32, device=a.device)
     _gpu("out", out, torch.float32, 2)
-    _require(out.shape == (m, n), f"out must be {(m, n)}")
+    if not (out.shape == (m, n)):
+        raise ValueError(f"out must be {(m, n)}")
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
     _run("cie_gemm_f32", load_library().cie_gemm_f32(_stream(), _ptr(a), _ptr(weight), _ptr(bias), _ptr(out),
                                                      _i(m), _i(n), _i(k), _i(lda), _i(n)))
@@ -364,25 +406,32 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
     [k_parts, M, N] (bias in part 0), to be summed by ``add_parts_rmsnorm``."""
     _gpu("weight", weight, torch.bfloat16, 2)
     n, k = weight.shape
-    _require(a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1,
-             "a must be a bf16 GPU matrix with unit inner stride")
+    if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
+        raise ValueError("a must be a bf16 GPU matrix with unit inner stride")
     m = a.shape[0]
-    _require(m >= 1 and a.shape[1] == k, f"a {tuple(a.shape)} vs K={k}")
+    if not (m >= 1 and a.shape[1] == k):
+        raise ValueError(f"a {tuple(a.shape)} vs K={k}")
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
-    _require(k % 8 == 0 and lda % 8 == 0, f"K and the row stride must be multiples of 8, are {k} and {lda}")
-    _require(a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
-    _require(1 <= k_parts <= 64 and (k_parts == 1 or epilogue == EPI_PARTIAL), f"k_parts {k_parts} does not fit the epilogue")
+    if not (k % 8 == 0 and lda % 8 == 0):
+        raise ValueError(f"K and the row stride must be multiples of 8, are {k} and {lda}")
+    if not (a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
+        raise ValueError("operands must be 16-byte aligned")
+    if not (1 <= k_parts <= 64 and (k_parts == 1 or epilogue == EPI_PARTIAL)):
+        raise ValueError(f"k_parts {k_parts} does not fit the epilogue")
     device = weight.device
     if bias is not None:
         _gpu("bias", bias, torch.bfloat16, 1)
-        _require(bias.shape[0] == n and epilogue != EPI_SILU, "bias does not fit")
+        if not (bias.shape[0] == n and epilogue != EPI_SILU):
+            raise ValueError("bias does not fit")
     columns = n // 2 if epilogue == EPI_SILU else n
     row_tiles, waves, column_tiles = plan or plan_fused(m, -(-columns // 16), -(-k // k_parts), k_parts)
     if epilogue == EPI_SILU:
         column_tiles = 1 if row_tiles == 1 else 2  # always a gate tile with its up tile
-    _require(row_tiles in (1, 2, 4) and waves in ((1, 2, 4, 8) if row_tiles == 1 else (4, 8))
-             and column_tiles in ((1,) if row_tiles == 1 else (1, 2)),
-             f"plan {(row_tiles, waves, column_tiles)} is not one the kernel has")
+    if not (
+        row_tiles in (1, 2, 4) and waves in ((1, 2, 4, 8) if row_tiles == 1 else (4, 8))
+        and column_tiles in ((1,) if row_tiles == 1 else (1, 2))
+    ):
+        raise ValueError(f"plan {(row_tiles, waves, column_tiles)} is not one the kernel has")
     residual = sumsq = None
     if epilogue == EPI_BF16:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
@@ -391,23 +440,61 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
     elif epilogue == EPI_PARTIAL:
         out = torch.empty((k_parts, m, n), dtype=torch.float32, device=device)
     elif epilogue == EPI_SILU:
-        _require(n % 2 == 0, f"the SiLU epilogue needs an even N, got {n}")
+        if not (n % 2 == 0):
+            raise ValueError(f"the SiLU epilogue needs an even N, got {n}")
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=device)
     elif epilogue == EPI_RESID:
-        _require(residual_out is not None, "the residual epilogue needs the residual to add into")
+        if not (residual_out is not None):
+            raise ValueError("the residual epilogue needs the residual to add into")
         _gpu("residual_out", residual_out, torch.float32, 2)
-        _require(residual_out.shape == (m, n), f"residual_out {tuple(residual_out.shape)} vs {(m, n)}")
+        if not (residual_out.shape == (m, n)):
+            raise ValueError(f"residual_out {tuple(residual_out.shape)} vs {(m, n)}")
         parts = -(-n // 16)
         if sumsq_out is None:
             sumsq_out = torch.empty((m, parts), dtype=torch.float32, device=device)
         _gpu("sumsq_out", sumsq_out, torch.float32, 2)
-        _require(sumsq_out.shape[0] >= m and sumsq_out.shape[1] == parts, f"sumsq_out {tuple(sumsq_out.shape)} must be [>= {m}, {parts}]")
+        if not (sumsq_out.shape[0] >= m and sumsq_out.shape[1] == parts):
+            raise ValueError(f"sumsq_out {tuple(sumsq_out.shape)} must be [>= {m}, {parts}]")
         out, residual, sumsq = sumsq_out, residual_out, sumsq_out
     else:
         raise ValueError(f"unknown epilogue {epilogue}")
     _run("cie_gemm_fused", load_library().cie_gemm_fused(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(None if epilogue == EPI_RESID else out),
         _ptr(residual), _ptr(sumsq), _i(m), _i(n), _i(k), _i(epilogue), _i(row_tiles), _i(waves), _i(column_tiles), _i(k_parts)))
+    return out
+
+
+_WORKSPACES: dict[torch.device, torch.Tensor] = {}
+LIBRARY_WORKSPACE_BYTES = 64 << 20
+
+
+def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``a @ weight.T + bias`` through the vendor library (hipBLASLt) with the
+    descriptors and the chosen algorithm of every shape kept after its first call:
+    bf16 operands, bias and result, float32 sums.  For products with many rows.  Returns ``None`` if the library has no algorithm for the shape."""
+    _gpu("weight", weight, torch.bfloat16, 2)
+    n, k = weight.shape
+    if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
+        raise ValueError("a must be a bf16 GPU matrix with unit inner stride")
+    m = a.shape[0]
+    if not (m >= 1 and a.shape[1] == k):
+        raise ValueError(f"a {tuple(a.shape)} vs K={k}")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    if bias is not None:
+        _gpu("bias", bias, torch.bfloat16, 1)
+        if bias.shape[0] != n:
+            raise ValueError(f"bias must be [{n}]")
+    device = weight.device
+    workspace = _WORKSPACES.get(device)
+    if workspace is None:
+        workspace = _WORKSPACES[device] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    code = load_library().cie_gemm_library(
+        _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k),
+        _ptr(workspace), ctypes.c_size_t(workspace.numel()))
+    if code == 1:
+        return None
+    _run("cie_gemm_library", code)
     return out
 
 
@@ -424,31 +511,41 @@ def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Te
     by ``rope_kv_write``.  Head sizes in steps of 32."""
     _gpu("weight", weight, torch.bfloat16, 2)
     n, k = weight.shape
-    _require(a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1,
-             "a must be a bf16 GPU matrix with unit inner stride")
+    if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
+        raise ValueError("a must be a bf16 GPU matrix with unit inner stride")
     m = a.shape[0]
-    _require(1 <= m <= 16 and a.shape[1] == k, f"a {tuple(a.shape)}: up to 16 rows of K={k}")
+    if not (1 <= m <= 16 and a.shape[1] == k):
+        raise ValueError(f"a {tuple(a.shape)}: up to 16 rows of K={k}")
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
-    _require(k % 8 == 0 and lda % 8 == 0, f"K and the row stride must be multiples of 8, are {k} and {lda}")
-    _require(a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
-    _require(head_dim % 32 == 0, f"the fused rotation takes head sizes in steps of 32, not {head_dim}")
-    _require(n == (q_heads + 2 * kv_heads) * head_dim, f"weight has {n} rows, heads say {(q_heads + 2 * kv_heads) * head_dim}")
+    if not (k % 8 == 0 and lda % 8 == 0):
+        raise ValueError(f"K and the row stride must be multiples of 8, are {k} and {lda}")
+    if not (a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
+        raise ValueError("operands must be 16-byte aligned")
+    if not (head_dim % 32 == 0):
+        raise ValueError(f"the fused rotation takes head sizes in steps of 32, not {head_dim}")
+    if not (n == (q_heads + 2 * kv_heads) * head_dim):
+        raise ValueError(f"weight has {n} rows, heads say {(q_heads + 2 * kv_heads) * head_dim}")
     if bias is not None:
         _gpu("bias", bias, torch.bfloat16, 1)
-        _require(bias.shape[0] == n, "bias does not fit")
+        if not (bias.shape[0] == n):
+            raise ValueError("bias does not fit")
     for name, table in (("cos", cos), ("sin", sin)):
         _gpu(name, table, torch.float32, 2)
-        _require(table.shape[1] == head_dim // 2, f"{name} must be [max_position, {head_dim // 2}]")
-    _require(cos.shape == sin.shape, "cos and sin tables differ in shape")
+        if not (table.shape[1] == head_dim // 2):
+            raise ValueError(f"{name} must be [max_position, {head_dim // 2}]")
+    if not (cos.shape == sin.shape):
+        raise ValueError("cos and sin tables differ in shape")
     for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
         _gpu(name, meta, torch.int32, 1)
-        _require(meta.shape[0] >= m, f"{name} has {meta.shape[0]} entries for {m} rows")
+        if not (meta.shape[0] >= m):
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {m} rows")
     _gpu("seq_slot", seq_slot, torch.int32, 1)
     _gpu("block_table", block_table, torch.int32, 2)
     page_size = _check_pools(k_pool, v_pool, torch.bfloat16, kv_heads, head_dim)
     if waves is None:
         _, waves, _ = plan_fused(m, n // 32, k)
-    _require(waves in (1, 2, 4, 8), f"{waves} waves per workgroup is not a form the kernel has")
+    if not (waves in (1, 2, 4, 8)):
+        raise ValueError(f"{waves} waves per workgroup is not a form the kernel has")
     out = torch.empty((m, n), dtype=torch.bfloat16, device=weight.device)
     _run("cie_gemm_qkv_rope", load_library().cie_gemm_qkv_rope(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k), _i(waves), _ptr(cos),
@@ -478,13 +575,16 @@ def sample(logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
         return out
     if temperature is not None:
         _gpu("temperature", temperature, torch.float32, 1)
-        _require(uniform is not None, "temperature sampling needs the uniform numbers")
+        if not (uniform is not None):
+            raise ValueError("temperature sampling needs the uniform numbers")
         _gpu("uniform", uniform, torch.float32, 1)
-        _require(temperature.shape[0] == rows and uniform.shape[0] == rows, "one temperature and one uniform per row")
+        if not (temperature.shape[0] == rows and uniform.shape[0] == rows):
+            raise ValueError("one temperature and one uniform per row")
     if out is None:
         out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     _gpu("out", out, torch.int32, 1)
-    _require(out.shape[0] == rows, f"out must be [{rows}]")
+    if not (out.shape[0] == rows):
+        raise ValueError(f"out must be [{rows}]")
     _run("cie_sample", load_library().cie_sample(_stream(), _ptr(logits), _ptr(temperature), _ptr(uniform),
                                                  _ptr(out), _i(rows), _i(vocab), _i(vocab)))
     return out

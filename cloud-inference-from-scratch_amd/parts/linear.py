@@ -5,9 +5,9 @@ float32: the hand-written true-float32 kernel, always.  bfloat16 with up to
 matrix-core kernel that streams the weight once and takes over its neighbours'
 work: a SiLU-gate behind (``epilogue="silu"``), the add into the float32
 residual stream (``into=residual``), or float32 results for the logits.
-bfloat16 with more rows: the library product, as the reference leaves its
-products to a library (src/cloud_engine/model.py:89-137), with the small
-kernels around it.
+bfloat16 with more rows: the vendor library's product (hipBLASLt through a
+thin cached interface of this package), as the reference leaves its products to
+a library (src/cloud_engine/model.py:89-137), with the small kernels around it.
 """
 
 from __future__ import annotations
@@ -85,5 +85,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         out = x.float() @ weight.float().t()
         out = out if bias is None else out + bias.float()
     else:
-        out = torch.nn.functional.linear(x, weight, bias)
+        out = ops.gemm_library(x, weight, bias) if x.is_cuda and x.stride(1) == 1 else None
+        if out is None:  # a shape the library's own interface has no algorithm for
+            out = torch.nn.functional.linear(x, weight, bias)
     return ops.silu_mul(out) if silu else out

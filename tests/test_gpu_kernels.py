@@ -605,3 +605,25 @@ def test_argmax_over_a_large_vocabulary(ops):
     out = ops.sample(logits).tolist()
     assert out == torch.argmax(logits, dim=-1).tolist()
     assert out[1:5] == [vocab - 1, 0, 2047, 4096]
+
+
+@pytest.mark.parametrize("shape", [(17, 40, 24), (64, 2560, 2048), (150, 99, 72), (300, 515, 328), (2048, 256, 2048)])
+def test_gemm_library_matches_float64(ops, shape):
+    """The cached interface to the vendor library: with and without bias, rows given as a strided view,
+    twice (the second call takes the kept plan)."""
+    m, n, k = shape
+    a, w, b = rand((m, k), torch.bfloat16, 20), rand((n, k), torch.bfloat16, 21), rand((n,), torch.bfloat16, 22)
+    expect = a.double() @ w.double().t()
+    for _ in range(2):
+        out = ops.gemm_library(a, w)
+        if out is None:
+            pytest.skip("the library has no algorithm for this shape")
+        assert out.dtype == torch.bfloat16 and out.shape == (m, n)
+        torch.testing.assert_close(out.double(), expect, rtol=1e-2, atol=1e-2 * math.sqrt(k))
+        out = ops.gemm_library(a, w, b)
+        torch.testing.assert_close(out.double(), expect + b.double(), rtol=1e-2, atol=1e-2 * math.sqrt(k))
+    if k % 8 == 0:
+        wide = torch.zeros((m, k + 64), dtype=torch.bfloat16).cuda()
+        wide[:, :k] = a
+        torch.testing.assert_close(ops.gemm_library(wide[:, :k], w, b).double(), expect + b.double(), rtol=1e-2,
+                                   atol=1e-2 * math.sqrt(k))
