@@ -135,6 +135,7 @@ class CacheManager:
         self._slots: dict[str, int] = {}
         self._length: dict[str, int] = {}
         self._dirty: set[tuple[int, int]] = set()  # (group, slot) rows the device copy lacks
+        self._slot_serial: dict[int, int] = {}
         self._fresh_slots: set[int] = set()  # slots whose fixed state must be cleared before use
         self.prefix_cache_pages = (
             prefix_cache_pages
@@ -174,6 +175,11 @@ class CacheManager:
         self._dirty.clear()
         return rows
 
+    def slot_serial(self, slot: int) -> int:
+        """How many requests have been given this slot so far: tells the device side whether a dirty
+        row still belongs to the request whose table it has already copied."""
+        return self._slot_serial.get(slot, 0)
+
     def take_fresh_slots(self) -> list[int]:
         fresh = sorted(self._fresh_slots)
         self._fresh_slots.clear()
@@ -191,6 +197,7 @@ class CacheManager:
             raise CacheCapacityFull(f"all {self.max_running} request slots are taken")
         slot = self._free_slots.pop()
         self._slots[request_id] = slot
+        self._slot_serial[slot] = self._slot_serial.get(slot, 0) + 1
         self._length[request_id] = 0
         self._fresh_slots.add(slot)
         for index, group in enumerate(self.groups):

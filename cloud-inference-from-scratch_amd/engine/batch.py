@@ -17,6 +17,20 @@ from typing import Any
 import torch
 
 
+def to_device_staging(values: Any, device: torch.device | str) -> torch.Tensor:
+    """int32 values (a list, or a CPU tensor) in host memory that an asynchronous copy to ``device`` may
+    read later: a fresh page-locked tensor from torch's caching host allocator, which hands a block out
+    again only after the copies that read it have run.  (A page-locked buffer of one's own that is
+    rewritten step after step would be overwritten under a copy that is still queued behind earlier
+    kernels, whenever the host runs ahead of the GPU.)"""
+    pinned = torch.device(device).type == "cuda"
+    if isinstance(values, torch.Tensor):
+        staged = torch.empty(values.shape, dtype=torch.int32, pin_memory=pinned)
+        staged.copy_(values)
+        return staged
+    return torch.tensor(values, dtype=torch.int32, pin_memory=pinned)
+
+
 @dataclass
 class StepBatch:
     tokens: int
@@ -61,7 +75,7 @@ class StepBatch:
                     seqs.append(index)
                     firsts.append(first)
             if seqs:
-                both = torch.tensor(seqs + firsts, dtype=torch.int32).to(self.token_ids.device, non_blocking=True)
+                both = to_device_staging(seqs + firsts, self.token_ids.device).to(self.token_ids.device, non_blocking=True)
                 self._tiles[key] = (both[: len(seqs)], both[len(seqs):], len(seqs))
             else:
                 self._tiles[key] = (self.seq_slot, self.seq_slot, 0)

@@ -5,8 +5,8 @@ For every group of the :class:`~cie_amd.cache.manager.CacheManager` one pool
 second axis as ``[page_size, head_dim]``, values at index 1 transposed as
 ``[head_dim, page_size]``, the layouts the matrix-core attention reads with plain
 vector loads; a page of one head is contiguous) and one int32 block
-table ``[max_running, width]`` whose row ``slot`` mirrors the request's host
-table.  The reference keeps ``[layers, pages, page_size, kv_heads, head_dim]``
+table ``[max_running, width]`` whose row ``slot`` holds the request's host
+table in its first entries.  The reference keeps ``[layers, pages, page_size, kv_heads, head_dim]``
 pools (src/cloud_engine/cache.py:266-274) and uploads padded tables every step
 (src/cloud_engine/engine.py:264-278); here only rows that changed are copied.
 
@@ -24,7 +24,7 @@ from typing import Any
 import torch
 
 from ..cache.manager import CacheManager, FixedState
-from .batch import PagedView, StateView
+from .batch import PagedView, StateView, to_device_staging
 
 _STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
 
@@ -36,8 +36,8 @@ class DeviceCache:
         self.device = device
         self.pools: list[torch.Tensor] = []
         self.tables: list[torch.Tensor] = []
-        self.host_tables: list[torch.Tensor] = []
         self.pad_slot = manager.max_running
+        self._row_seen: dict[tuple[int, int], tuple[int, int]] = {}  # (group, slot) -> (slot serial, entries copied)
         for group in manager.groups:
             spec = group.spec
             pad_page = group.allocator.total_pages
@@ -46,8 +46,6 @@ class DeviceCache:
             table = torch.zeros((manager.max_running + 1, manager.table_width), dtype=torch.int32, device=device)
             table[self.pad_slot] = pad_page
             self.tables.append(table)
-            self.host_tables.append(torch.zeros((manager.max_running, manager.table_width), dtype=torch.int32,
-                                                pin_memory=device.type == "cuda"))
         self.states: dict[int, torch.Tensor] = {}
         for unit, spec in manager.state_units.items():
             assert isinstance(spec, FixedState)
@@ -78,11 +76,17 @@ class DeviceCache:
         """Bring the device block tables up to the host's; clear the state of
         slots that were handed to a new request."""
         for group, slot, table in self.manager.take_dirty_rows():
-            host = self.host_tables[group]
-            row = host[slot]
-            if table:
-                row[: len(table)] = torch.tensor([max(p, 0) for p in table], dtype=torch.int32)
-            self.tables[group][slot].copy_(row, non_blocking=True)
+            # A request's table only grows at its end (pages a window has passed turn to -1 in place, and
+            # are never read again): copy what was appended since the last time, all of it once the slot
+            # has gone to another request.  Entries past the request's pages keep what they held; nothing
+            # reads them.
+            serial = self.manager.slot_serial(slot)
+            seen, synced = self._row_seen.get((group, slot), (-1, 0))
+            first = synced if seen == serial and synced <= len(table) else 0
+            if len(table) > first:
+                staged = to_device_staging([max(p, 0) for p in table[first:]], self.device)
+                self.tables[group][slot, first: len(table)].copy_(staged, non_blocking=True)
+            self._row_seen[(group, slot)] = (serial, len(table))
         fresh = self.manager.take_fresh_slots()
         if fresh and self.states:
             for state in self.states.values():

@@ -19,7 +19,7 @@ from typing import Any
 
 import torch
 
-from .batch import StepBatch
+from .batch import StepBatch, to_device_staging
 
 
 @dataclass
@@ -37,7 +37,7 @@ class _Bucket:
     def __init__(self, size: int, device: torch.device, pad_slot: int, max_keys: int) -> None:
         self.size = size
         count = 10 * size + 2
-        self.host = torch.zeros(count, dtype=torch.int32, pin_memory=True)
+        self.host = torch.zeros(count, dtype=torch.int32)  # the template; every replay stages a copy of it
         self.dev = torch.zeros(count, dtype=torch.int32, device=device)
         names = ["token_ids", "positions", "seq_of_token", "seq_slot", "seq_start", "seq_q_len"]
         self.offsets: dict[str, int] = {}
@@ -146,7 +146,7 @@ class DecodeGraphs:
         positions = [e.start_pos for e in entries]
         bucket.fill([e.tokens[0] for e in entries], positions, [cache.slot(e.request_id) for e in entries],
                     max(positions) + 1)
-        bucket.dev.copy_(bucket.host, non_blocking=True)
+        bucket.dev.copy_(to_device_staging(bucket.host, runner.device), non_blocking=True)
         bucket.graph.replay()
         self.replays += 1
         rows = [index for index, e in enumerate(entries) for _ in e.want]

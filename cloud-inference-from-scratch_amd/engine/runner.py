@@ -23,7 +23,7 @@ from ..cache.manager import CacheManager
 from ..config.engine_config import EngineConfig
 from ..profiling import trace_range
 from ..sampling.sampler import Sampler
-from .batch import StepBatch
+from .batch import StepBatch, to_device_staging
 from .device_cache import DeviceCache
 from .graphs import DecodeGraphs
 
@@ -132,16 +132,16 @@ class Runner:
         return {r.request_id: token for r, token in zip(sampled, tokens)}
 
     # -- packing -----------------------------------------------------------------
-    def _stage(self, count: int) -> tuple[torch.Tensor, torch.Tensor]:
+    def _stage(self, count: int) -> torch.Tensor:
+        """The device buffer a step's metadata is copied into.  Two take turns: the copy of the next step
+        is ordered on the stream behind the kernels that read the buffer two steps earlier."""
         turn = self._staging_turn
         self._staging_turn ^= 1
-        pair = self._staging[turn]
-        if pair is None or pair[0].numel() < count:
-            size = max(1024, 1 << (count - 1).bit_length())
-            pair = (torch.empty(size, dtype=torch.int32, pin_memory=True),
-                    torch.empty(size, dtype=torch.int32, device=self.device))
-            self._staging[turn] = pair
-        return pair
+        dev = self._staging[turn]
+        if dev is None or dev.numel() < count:
+            dev = torch.empty(max(1024, 1 << (count - 1).bit_length()), dtype=torch.int32, device=self.device)
+            self._staging[turn] = dev
+        return dev
 
     def check(self, entries: Sequence[StepEntry]) -> None:
         """Refuse a step the kernels were not written for, before anything changes."""
@@ -190,9 +190,8 @@ class Runner:
             logit_rows.extend(base + place for place in entry.want)
         parts = [ids, positions, seq_of_token, slots, starts, q_lens, q_start_loc, logit_rows]
         flat = [value for part in parts for value in part]
-        host, dev = self._stage(len(flat))
-        host[: len(flat)] = torch.tensor(flat, dtype=torch.int32)
-        dev[: len(flat)].copy_(host[: len(flat)], non_blocking=True)
+        dev = self._stage(len(flat))
+        dev[: len(flat)].copy_(to_device_staging(flat, self.device), non_blocking=True)
         views = []
         offset = 0
         for part in parts:

@@ -487,7 +487,8 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     device = weight.device
     workspace = _WORKSPACES.get(device)
     if workspace is None:
-        workspace = _WORKSPACES[device] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+        # cleared once: algorithms that meet through flags in the workspace leave them cleared after each call
+        workspace = _WORKSPACES[device] = torch.zeros(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
     out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
     code = load_library().cie_gemm_library(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k),

@@ -177,6 +177,49 @@ def test_products_cut_along_k_match_plain(tiny_folders, plain, monkeypatch, grap
     replay_util.compare(rows, expected, **TOL["bfloat16"])
 
 
+@pytest.mark.parametrize("graph", [False, True])
+def test_steps_queued_behind_a_busy_gpu_keep_their_own_metadata(tiny_folders, plain, graph):
+    """The host may run many steps ahead of the GPU (prompt portions of a large model want no logits,
+    so nothing makes the host wait).  Each step's token ids, positions and table rows must then still be
+    the step's own when its copy finally runs: here the GPU is kept busy while portions of different
+    sizes, decode steps and a slot that changes hands are queued, and only the end is checked."""
+    from cie_amd.engine.runner import StepEntry
+
+    folder, raw, _ = tiny_folders["B"]
+    requests, expected = plain["B"]
+    runner = make_runner(folder, "float32", 512, 8, graph_decode=graph)
+    if graph:
+        runner.warm_up()
+    long_one, short_one, other = requests["B5"], requests["B2"], requests["B3"]  # 131, 40 and 64 tokens
+    runner.cache.admit("x"), runner.cache.admit("y")
+    torch.cuda.synchronize()
+    torch.cuda._sleep(int(1.5e9))  # the GPU spins for most of a second: everything below queues up behind it
+    fed = {"x": 0, "y": 0}
+
+    def step(*portions):
+        entries = []
+        for rid, tokens, count in portions:
+            entries.append(StepEntry(rid, tokens[fed[rid]: fed[rid] + count], fed[rid], []))
+            fed[rid] += count
+        runner.run(entries)
+
+    step(("x", long_one, 7))
+    step(("x", long_one, 33), ("y", short_one, 20))
+    step(("x", long_one, 2))
+    step(("y", short_one, 19), ("x", long_one, 16))
+    for _ in range(6):  # single tokens: captured steps when graphs are on
+        step(("x", long_one, 1))
+    runner.cache.release("y")  # its slot goes to another request while the copies above are still queued
+    runner.cache.admit("z")
+    fed["z"] = 0
+    step(("z", other, 50), ("x", long_one, 40))
+    step(("x", long_one, 2))
+    last_x = runner.run([StepEntry("x", long_one[fed["x"]:], fed["x"], [len(long_one) - fed["x"] - 1])])
+    last_z = runner.run([StepEntry("z", other[50:], 50, [len(other) - 51])])
+    torch.testing.assert_close(last_x[0].cpu(), expected["B5"][-1], **F32_TOL)
+    torch.testing.assert_close(last_z[0].cpu(), expected["B3"][-1], **F32_TOL)
+
+
 def test_mixed_reuses_pages(tiny_folders, plain):
     """The mixed schedule runs in a pool smaller than the sum of all requests."""
     _, raw, _ = tiny_folders["B"]
