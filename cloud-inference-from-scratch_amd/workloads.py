@@ -83,7 +83,7 @@ def make_requests(profile: Profile, vocab_size: int, seed: int) -> list[tuple[li
 
 
 def run_profile(profile: Profile, *, layers: int | None = None, dtype: str = "bfloat16", seed: int = 0,
-                page_size: int = 16, shape: str | None = None) -> dict[str, Any]:
+                page_size: int = 16, shape: str | None = None, verify: int = 0) -> dict[str, Any]:
     """Run the profile on a fresh engine with random weights; returns the record that
     ``cie workload`` prints.  ``layers`` runs fewer layers than the shape has (the
     record names both numbers)."""
@@ -138,6 +138,18 @@ def run_profile(profile: Profile, *, layers: int | None = None, dtype: str = "bf
 
     results = [engine.result_of(h) for h in handles]
     snapshot = engine.snapshot_metrics()
+    verified = None
+    if verify:
+        # each of the first requests once more, alone: in float32 every kernel gives a row the same result
+        # whatever else is in the batch and however the prompt was cut, so the tokens must be the same
+        engine.runner.cache.clear_prefix_index()
+        same = 0
+        for (prompt, n), result in list(zip(requests, results))[:verify]:
+            alone = engine.generate([prompt], GenerationConfig(max_output_tokens=n, eos_token_id=None))[0]
+            same += alone.token_ids == result.token_ids
+        verified = {"requests": min(verify, len(requests)), "same_tokens_alone": same}
+        if dtype == "float32" and same != verified["requests"]:
+            raise AssertionError(f"float32 tokens depend on the batch: {verified}")
     output_tokens = sum(r.output_tokens for r in results)
     input_tokens = sum(r.input_tokens for r in results)
     assert all(r.output_tokens == n for r, (_, n) in zip(results, requests))
@@ -151,7 +163,7 @@ def run_profile(profile: Profile, *, layers: int | None = None, dtype: str = "bf
         "ttft_ms": snapshot["latency_ms"]["ttft"], "itl_ms": snapshot["latency_ms"]["itl"],
         "e2e_ms": snapshot["latency_ms"]["e2e"], "preempted": snapshot["requests"]["preempted_total"],
         "recomputed_tokens": snapshot["tokens"]["recomputed_total"], "scheduler": snapshot["scheduler"],
-        "kv_cache": snapshot.get("kv_cache"), "runner": snapshot.get("runner"),
+        "kv_cache": snapshot.get("kv_cache"), "runner": snapshot.get("runner"), "verified": verified,
         "data": "synthetic (seeded uniform-random token ids, random weights)",
     }
 
@@ -165,7 +177,11 @@ def main(argv: list[str] | None = None) -> int:
     parser.add_argument("--shape", choices=sorted(SHAPES), default=None, help="another model shape than the profile's")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--verify", type=int, default=0, metavar="N",
+                        help="afterwards run the first N requests alone and compare their tokens "
+                             "(float32: must be equal; bfloat16: reported)")
     args = parser.parse_args(argv)
-    record = run_profile(PROFILES[args.name], layers=args.layers, dtype=args.dtype, seed=args.seed, shape=args.shape)
+    record = run_profile(PROFILES[args.name], layers=args.layers, dtype=args.dtype, seed=args.seed, shape=args.shape,
+                         verify=args.verify)
     print(json.dumps(record))
     return 0
