@@ -163,6 +163,26 @@ def test_captured_decode_steps_match_plain(tiny_folders, plain, name, dtype):
 
 
 @pytest.mark.parametrize("graph", [False, True])
+def test_many_decoding_requests_run_the_library_products(tiny_folders, plain, graph):
+    """More than 16 rows in a step send the products to the vendor library (and, with
+    17 to 64 rows, the down product to the split-K kernel for 32 and 64 rows); with
+    graphs on, the library calls are inside the captured steps and every replay is
+    checked.  24 requests live at once, decoded side by side for 30 steps."""
+    folder, raw, tensors = tiny_folders["B"]
+    lengths = [40 + (7 * i) % 23 for i in range(24)]
+    requests = {f"m{i}": random_tokens(n, raw["vocab_size"], seed=300 + i) for i, n in enumerate(lengths)}
+    expected = plain_all(raw, tensors, requests)
+    steps = replay_util.mixed(requests, live=24, chunk_sizes=(9, 4, 13), decode_tail=30, seed=9)
+    assert max(len(step["entries"]) for step in steps) > 16
+    pool = replay_util.max_live_tokens(steps, page=8)
+    runner = make_runner(folder, "bfloat16", pool, 8, max_running=24, graph_decode=graph)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    replay_util.compare(rows, expected, **TOL["bfloat16"])
+    if graph:
+        assert runner.graph_replays >= 10 and max(runner.graphs.buckets) == 32
+
+
+@pytest.mark.parametrize("graph", [False, True])
 def test_products_cut_along_k_match_plain(tiny_folders, plain, monkeypatch, graph):
     """The decode products that cut a long K into parts (summed by the next norm
     kernel) only engage at sizes the tiny models do not have; force them."""
