@@ -1,6 +1,7 @@
 // Matrix products with many rows go to the vendor library (hipBLASLt), as the reference leaves its
 // products to a library.  This is the thin host side of that: one handle, and for every shape the
-// descriptors and the algorithm the library's heuristic picks, kept after the first call, so that a
+// descriptors and the algorithm (the library's heuristic pick, or the fastest of its candidates), kept
+// after the first call, so that a
 // step's few hundred products cost a table lookup and one launch each instead of a heuristic query.
 //
 //   C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]),  bf16 operands, bias and result, float32 sums
@@ -40,8 +41,12 @@ void destroy(Plan& plan) {
     plan = Plan{};
 }
 
-// Descriptors and the heuristic's first algorithm for a shape; false if the library has none.
-bool make_plan(Plan& plan, int M, int N, int K, int lda, bool has_bias, size_t workspace_limit) {
+constexpr int kCandidates = 16;
+
+// Descriptors for a shape and the algorithms the library's heuristic proposes, best guess first;
+// returns how many fit the workspace (0: the library has none).
+int make_plan(Plan& plan, hipblasLtMatmulHeuristicResult_t (&found)[kCandidates], int M, int N, int K, int lda,
+              bool has_bias, size_t workspace_limit) {
     const hipblasOperation_t transposed = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
     bool good = ok(hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F)) &&
                 ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed))) &&
@@ -55,29 +60,60 @@ bool make_plan(Plan& plan, int M, int N, int K, int lda, bool has_bias, size_t w
         good = ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue))) &&
                ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)));
     }
-    if (!good) return false;
+    if (!good) return 0;
     hipblasLtMatmulPreference_t preference = nullptr;
-    if (!ok(hipblasLtMatmulPreferenceCreate(&preference))) return false;
+    if (!ok(hipblasLtMatmulPreferenceCreate(&preference))) return 0;
     const uint64_t limit = workspace_limit;
-    hipblasLtMatmulHeuristicResult_t found;
     int count = 0;
     good = ok(hipblasLtMatmulPreferenceSetAttribute(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit))) &&
-           ok(hipblasLtMatmulAlgoGetHeuristic(g_handle, plan.desc, plan.w, plan.a, plan.d, plan.d, preference, 1, &found, &count)) &&
-           count > 0 && ok(found.state);
+           ok(hipblasLtMatmulAlgoGetHeuristic(g_handle, plan.desc, plan.w, plan.a, plan.d, plan.d, preference, kCandidates,
+                                              found, &count));
     hipblasLtMatmulPreferenceDestroy(preference);
-    if (!good) return false;
-    plan.algo = found.algo;
-    plan.workspace = found.workspaceSize;
-    return plan.workspace <= workspace_limit;
+    if (!good) return 0;
+    int kept = 0;
+    for (int i = 0; i < count; ++i)
+        if (ok(found[i].state) && found[i].workspaceSize <= workspace_limit) found[kept++] = found[i];
+    return kept;
+}
+
+// Time the candidates on the call's own operands (the result is overwritten by the real call that
+// follows) and return the index of the fastest; 0 if timing is not possible.
+int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int count, hipStream_t stream,
+            const void* a, const void* w, void* c, void* workspace) {
+    hipEvent_t begin = nullptr, end = nullptr;
+    if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) return 0;
+    const float one = 1.f, zero = 0.f;
+    int best = 0;
+    float best_ms = 0.f;
+    for (int i = 0; i < count; ++i) {
+        bool good = true;
+        for (int run = 0; run < 4 && good; ++run) {  // the first run is the warm-up
+            if (run == 1) good = hipEventRecord(begin, stream) == hipSuccess;
+            good = good && ok(hipblasLtMatmul(g_handle, plan.desc, &one, w, plan.w, a, plan.a, &zero, c, plan.d, c, plan.d,
+                                              &found[i].algo, workspace, found[i].workspaceSize, stream));
+        }
+        float ms = 0.f;
+        good = good && hipEventRecord(end, stream) == hipSuccess && hipEventSynchronize(end) == hipSuccess &&
+               hipEventElapsedTime(&ms, begin, end) == hipSuccess;
+        if (good && (best_ms == 0.f || ms < best_ms)) {
+            best_ms = ms;
+            best = i;
+        }
+    }
+    hipEventDestroy(begin);
+    hipEventDestroy(end);
+    return best;
 }
 
 }  // namespace
 
+// With `tune`, a shape's first call (outside graph capture) times the heuristic's candidates on the call's
+// own operands and keeps the fastest; otherwise the heuristic's first choice is kept.
 // Returns CIE_BAD_ARGUMENT for a shape the library has no algorithm for (the caller then takes another
 // route) and CIE_LAUNCH_FAILED if the library's call itself fails.  `workspace` is device memory of
 // `workspace_bytes` that stays valid while the product runs; calls on one stream may share it.
 CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w, const void* bias, void* c, int M,
-                             int N, int K, void* workspace, size_t workspace_bytes) {
+                             int N, int K, void* workspace, size_t workspace_bytes, int tune) {
     if (M <= 0 || N <= 0 || K <= 0 || lda < K || !a || !w || !c) return CIE_BAD_ARGUMENT;
     Plan* plan = nullptr;
     {
@@ -87,10 +123,21 @@ CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w
         auto it = g_plans.find(key);
         if (it == g_plans.end()) {
             Plan fresh;
-            if (!make_plan(fresh, M, N, K, lda, bias != nullptr, workspace ? workspace_bytes : 0)) {
+            hipblasLtMatmulHeuristicResult_t found[kCandidates];
+            const int count = make_plan(fresh, found, M, N, K, lda, bias != nullptr, workspace ? workspace_bytes : 0);
+            if (count == 0) {
                 destroy(fresh);
                 return CIE_BAD_ARGUMENT;
             }
+            int chosen = 0;
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            if (tune && count > 1 && hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) == hipSuccess &&
+                capturing == hipStreamCaptureStatusNone) {
+                if (bias) hipblasLtMatmulDescSetAttribute(fresh.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
+                chosen = fastest(fresh, found, count, static_cast<hipStream_t>(stream), a, w, c, workspace);
+            }
+            fresh.algo = found[chosen].algo;
+            fresh.workspace = found[chosen].workspaceSize;
             it = g_plans.emplace(key, fresh).first;
         }
         plan = &it->second;
