@@ -466,8 +466,9 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
 
 _WORKSPACES: dict[torch.device, torch.Tensor] = {}
 LIBRARY_WORKSPACE_BYTES = 64 << 20
-# Products of at least this many rows, in steps of 256 (full prompt portions: the shapes that recur), time the
-# library's candidate algorithms at their first call and keep the fastest; others take its first choice.
+# Products of at least this many rows, in steps of 256 (full prompt portions), and of a power of two of rows
+# from 32 on (the buckets of captured decode steps) are the shapes that recur: they time the library's
+# candidate algorithms at their first call and keep the fastest; others take its first choice.
 LIBRARY_TUNE_ROWS = 512
 
 
@@ -496,7 +497,7 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     code = load_library().cie_gemm_library(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k),
         _ptr(workspace), ctypes.c_size_t(workspace.numel()),
-        _i(1 if m >= LIBRARY_TUNE_ROWS and m % 256 == 0 else 0))
+        _i(1 if (m >= LIBRARY_TUNE_ROWS and m % 256 == 0) or (m >= 32 and m & (m - 1) == 0) else 0))
     if code == 1:
         return None
     _run("cie_gemm_library", code)
