@@ -4,7 +4,8 @@
 // after the first call, so that a
 // step's few hundred products cost a table lookup and one launch each instead of a heuristic query.
 //
-//   C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]),  bf16 operands, bias and result, float32 sums
+//   C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]),  bf16 operands and bias, float32 sums, bf16 result
+//   (or, without bias, a float32 result: the logits)
 //
 // In the library's column-major terms: D (N x M, ld N) = W^T (W stored K x N, ld K, transposed) *
 // A (K x M, ld lda); the bias is added along D's rows (the N dimension).
@@ -25,7 +26,7 @@ struct Plan {
     size_t workspace = 0;
 };
 
-using Key = std::tuple<int, int, int, int, int>;  // M, N, K, lda, has bias
+using Key = std::tuple<int, int, int, int, int, int>;  // M, N, K, lda, has bias, float32 result
 
 hipblasLtHandle_t g_handle = nullptr;
 std::map<Key, Plan> g_plans;
@@ -46,14 +47,14 @@ constexpr int kCandidates = 16;
 // Descriptors for a shape and the algorithms the library's heuristic proposes, best guess first;
 // returns how many fit the workspace (0: the library has none).
 int make_plan(Plan& plan, hipblasLtMatmulHeuristicResult_t (&found)[kCandidates], int M, int N, int K, int lda,
-              bool has_bias, size_t workspace_limit) {
+              bool has_bias, bool f32_out, size_t workspace_limit) {
     const hipblasOperation_t transposed = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
     bool good = ok(hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F)) &&
                 ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed))) &&
                 ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain))) &&
                 ok(hipblasLtMatrixLayoutCreate(&plan.w, HIP_R_16BF, K, N, K)) &&
                 ok(hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, K, M, lda)) &&
-                ok(hipblasLtMatrixLayoutCreate(&plan.d, HIP_R_16BF, N, M, N));
+                ok(hipblasLtMatrixLayoutCreate(&plan.d, f32_out ? HIP_R_32F : HIP_R_16BF, N, M, N));
     if (good && has_bias) {
         const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
         const hipDataType bias_type = HIP_R_16BF;
@@ -113,18 +114,18 @@ int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int
 // route) and CIE_LAUNCH_FAILED if the library's call itself fails.  `workspace` is device memory of
 // `workspace_bytes` that stays valid while the product runs; calls on one stream may share it.
 CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w, const void* bias, void* c, int M,
-                             int N, int K, void* workspace, size_t workspace_bytes, int tune) {
-    if (M <= 0 || N <= 0 || K <= 0 || lda < K || !a || !w || !c) return CIE_BAD_ARGUMENT;
+                             int N, int K, int f32_out, void* workspace, size_t workspace_bytes, int tune) {
+    if (M <= 0 || N <= 0 || K <= 0 || lda < K || !a || !w || !c || (f32_out && bias)) return CIE_BAD_ARGUMENT;
     Plan* plan = nullptr;
     {
         std::lock_guard<std::mutex> guard(g_mutex);
         if (!g_handle && !ok(hipblasLtCreate(&g_handle))) return CIE_LAUNCH_FAILED;
-        const Key key{M, N, K, lda, bias ? 1 : 0};
+        const Key key{M, N, K, lda, bias ? 1 : 0, f32_out ? 1 : 0};
         auto it = g_plans.find(key);
         if (it == g_plans.end()) {
             Plan fresh;
             hipblasLtMatmulHeuristicResult_t found[kCandidates];
-            const int count = make_plan(fresh, found, M, N, K, lda, bias != nullptr, workspace ? workspace_bytes : 0);
+            const int count = make_plan(fresh, found, M, N, K, lda, bias != nullptr, f32_out != 0, workspace ? workspace_bytes : 0);
             if (count == 0) {
                 destroy(fresh);
                 return CIE_BAD_ARGUMENT;

@@ -472,10 +472,12 @@ LIBRARY_WORKSPACE_BYTES = 64 << 20
 LIBRARY_TUNE_ROWS = 512
 
 
-def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                 out_dtype: torch.dtype = torch.bfloat16) -> Optional[torch.Tensor]:
     """``a @ weight.T + bias`` through the vendor library (hipBLASLt) with the
     descriptors and the chosen algorithm of every shape kept after its first call:
-    bf16 operands, bias and result, float32 sums.  For products with many rows.  Returns ``None`` if the library has no algorithm for the shape."""
+    bf16 operands and bias, float32 sums, bf16 result, or without bias a float32
+    result.  For products with many rows.  Returns ``None`` if the library has no algorithm for the shape."""
     _gpu("weight", weight, torch.bfloat16, 2)
     n, k = weight.shape
     if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
@@ -484,6 +486,8 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     if not (m >= 1 and a.shape[1] == k):
         raise ValueError(f"a {tuple(a.shape)} vs K={k}")
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    if out_dtype not in (torch.bfloat16, torch.float32) or (out_dtype == torch.float32 and bias is not None):
+        raise ValueError(f"the result is bf16, or float32 without bias; asked for {out_dtype} with{'' if bias is not None else 'out'} bias")
     if bias is not None:
         _gpu("bias", bias, torch.bfloat16, 1)
         if bias.shape[0] != n:
@@ -493,10 +497,10 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     if workspace is None:
         # cleared once: algorithms that meet through flags in the workspace leave them cleared after each call
         workspace = _WORKSPACES[device] = torch.zeros(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
-    out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    out = torch.empty((m, n), dtype=out_dtype, device=device)
     code = load_library().cie_gemm_library(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k),
-        _ptr(workspace), ctypes.c_size_t(workspace.numel()),
+        _i(1 if out_dtype == torch.float32 else 0), _ptr(workspace), ctypes.c_size_t(workspace.numel()),
         _i(1 if (m >= LIBRARY_TUNE_ROWS and m % 256 == 0) or (m >= 32 and m & (m - 1) == 0) else 0))
     if code == 1:
         return None

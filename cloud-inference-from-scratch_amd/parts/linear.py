@@ -25,6 +25,9 @@ from ..kernels import ops
 # product loses from 24 rows on (41 us against 25 us at 64 rows: every workgroup re-reads the rows of A).
 FUSED_ROWS = 16
 FUSED_PARTS_ROWS = 64
+# float32 logits of more rows than this go to the library (the hand-written kernel streams the weight once per
+# 64 rows; up to 64 rows it is one pass either way)
+FUSED_LOGIT_ROWS = 64
 # An ``into=`` product with fewer than this many 16-column tiles and K of at least 2 * PART_K cuts K
 # into parts of about PART_K for more workgroups (partial products, summed by the next norm kernel).
 PART_BELOW_TILES = 512
@@ -71,6 +74,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     cut_k = into is not None and -(-n // 16) < PART_BELOW_TILES and k >= 2 * PART_K
     if fusable and cut_k and rows <= FUSED_PARTS_ROWS:
         return PartialSum(ops.gemm_fused(weight, ops.EPI_PARTIAL, x, bias=bias, k_parts=-(-k // PART_K)))
+    if fusable and wants_f32 and rows > FUSED_LOGIT_ROWS and into is None and not silu and bias is None:
+        out = ops.gemm_library(x, weight, out_dtype=torch.float32)  # logits of many rows: one pass over the weight
+        if out is not None:
+            return out
     if fusable and (rows <= FUSED_ROWS or wants_f32):
         if into is not None:
             return RowSumsq(ops.gemm_fused(weight, ops.EPI_RESID, x, bias=bias, residual_out=into))

@@ -622,6 +622,10 @@ def test_gemm_library_matches_float64(ops, shape):
         torch.testing.assert_close(out.double(), expect, rtol=1e-2, atol=1e-2 * math.sqrt(k))
         out = ops.gemm_library(a, w, b)
         torch.testing.assert_close(out.double(), expect + b.double(), rtol=1e-2, atol=1e-2 * math.sqrt(k))
+        exact = ops.gemm_library(a, w, out_dtype=torch.float32)  # as for logits
+        if exact is not None:
+            assert exact.dtype == torch.float32
+            torch.testing.assert_close(exact.double(), expect, rtol=1e-4, atol=1e-4 * math.sqrt(k))
     if k % 8 == 0:
         wide = torch.zeros((m, k + 64), dtype=torch.bfloat16).cuda()
         wide[:, :k] = a
