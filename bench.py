@@ -100,7 +100,8 @@ def time_decode(engine, config, batch: int, context: int, steps: int, warmup: in
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - start
     for r in requests:
-        assert not r.is_terminal and r.generated_count >= warmup + steps, (r.state, r.generated_count)
+        # (with decode steps started ahead of their tokens, the last step's token is still on its way)
+        assert not r.is_terminal and r.generated_count >= warmup + steps - 1, (r.state, r.generated_count)
     mean_context = sum(r.tokens_fed for r in requests) / batch - steps / 2.0
     for r in requests:
         engine.scheduler.cancel(r)

@@ -35,6 +35,9 @@ class EngineConfig:
     kv_cache_bytes: int = 4 << 30
     prefix_cache_pages: int = 256  # reference: prefix_cache_max_blocks
     graph_decode: bool = True  # reference: cuda_graph_decode
+    # a captured decode step is started before the tokens of the step before it have reached the host (it takes
+    # them on the device); a request that ends on an end-of-sequence token then has run one step too many
+    async_decode: bool = True
     seed: int = 0
 
     def validated(self) -> "EngineConfig":

@@ -80,7 +80,7 @@ int make_plan(Plan& plan, hipblasLtMatmulHeuristicResult_t (&found)[kCandidates]
 // Time the candidates on the call's own operands (the result is overwritten by the real call that
 // follows) and return the index of the fastest; 0 if timing is not possible.
 int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int count, hipStream_t stream,
-            const void* a, const void* w, void* c, void* workspace) {
+            const void* a, const void* w, void* c, void* workspace, int timed_runs) {
     hipEvent_t begin = nullptr, end = nullptr;
     if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) return 0;
     const float one = 1.f, zero = 0.f;
@@ -88,7 +88,7 @@ int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int
     float best_ms = 0.f;
     for (int i = 0; i < count; ++i) {
         bool good = true;
-        for (int run = 0; run < 4 && good; ++run) {  // the first run is the warm-up
+        for (int run = 0; run <= timed_runs && good; ++run) {  // the first run is the warm-up
             if (run == 1) good = hipEventRecord(begin, stream) == hipSuccess;
             good = good && ok(hipblasLtMatmul(g_handle, plan.desc, &one, w, plan.w, a, plan.a, &zero, c, plan.d, c, plan.d,
                                               &found[i].algo, workspace, found[i].workspaceSize, stream));
@@ -135,7 +135,8 @@ CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w
             if (tune && count > 1 && hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) == hipSuccess &&
                 capturing == hipStreamCaptureStatusNone) {
                 if (bias) hipblasLtMatmulDescSetAttribute(fresh.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
-                chosen = fastest(fresh, found, count, static_cast<hipStream_t>(stream), a, w, c, workspace);
+                // short products are timed over more runs: their times scatter more
+                chosen = fastest(fresh, found, count, static_cast<hipStream_t>(stream), a, w, c, workspace, M >= 512 ? 3 : 12);
             }
             fresh.algo = found[chosen].algo;
             fresh.workspace = found[chosen].workspaceSize;

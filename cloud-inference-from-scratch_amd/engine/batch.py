@@ -49,6 +49,10 @@ class StepBatch:
     request_ids: tuple[str, ...] = ()
     # filled for a step that replays a captured graph: everything a kernel plan reads comes from the device
     static_plan: Any = None
+    # a decode step that follows one whose tokens the host has not seen yet: row t takes token_pool[token_feed[t]]
+    # where token_feed[t] >= 0 (both int32 on the device)
+    token_feed: Any = None
+    token_pool: Any = None
     _tiles: dict = field(default_factory=dict)
 
     @property

@@ -34,9 +34,10 @@ class StaticPlan:
 
 
 class _Bucket:
-    def __init__(self, size: int, device: torch.device, pad_slot: int, max_keys: int) -> None:
+    def __init__(self, size: int, device: torch.device, pad_slot: int, max_keys: int,
+                 token_pool: torch.Tensor | None = None) -> None:
         self.size = size
-        count = 10 * size + 2
+        count = 11 * size + 2
         self.host = torch.zeros(count, dtype=torch.int32)  # the template; every replay stages a copy of it
         self.dev = torch.zeros(count, dtype=torch.int32, device=device)
         names = ["token_ids", "positions", "seq_of_token", "seq_slot", "seq_start", "seq_q_len"]
@@ -47,7 +48,7 @@ class _Bucket:
             offset += size
         self.offsets["q_start_loc"] = offset
         offset += size + 1
-        for name in ("logit_rows", "tile_seq", "tile_q0"):
+        for name in ("logit_rows", "tile_seq", "tile_q0", "token_feed"):
             self.offsets[name] = offset
             offset += size
         self.offsets["max_context"] = offset
@@ -72,15 +73,20 @@ class _Bucket:
             seq_q_len=view("seq_q_len"), q_start_loc=view("q_start_loc", size + 1), logit_rows=view("logit_rows"),
             host_slots=[pad_slot] * size, host_starts=[0] * size, host_q_lens=[1] * size,
             static_plan=StaticPlan(view("tile_seq"), view("tile_q0"), view("max_context", 1), max_keys),
+            token_feed=view("token_feed") if token_pool is not None else None, token_pool=token_pool,
         )
         self.graph: Any = None
         self.logits: torch.Tensor | None = None
 
-    def fill(self, tokens: Sequence[int], positions: Sequence[int], slots: Sequence[int], max_context: int) -> None:
-        """Real rows first, the rest padding: token 0 at position 0 of the pad slot."""
+    def fill(self, tokens: Sequence[int], positions: Sequence[int], slots: Sequence[int], max_context: int,
+             feed: Sequence[int] | None = None) -> None:
+        """Real rows first, the rest padding: token 0 at position 0 of the pad slot.  ``feed[i] >= 0``:
+        row i takes the token at that place of the token pool on the device instead of ``tokens[i]``."""
         o, size, n = self.offsets, self.size, len(tokens)
         pad = size - n
         host = self.host
+        host[o["token_feed"]: o["token_feed"] + size] = torch.tensor(
+            (list(feed) if feed is not None else [-1] * n) + [-1] * pad, dtype=torch.int32)
         host[o["token_ids"]: o["token_ids"] + size] = torch.tensor(list(tokens) + [0] * pad, dtype=torch.int32)
         host[o["positions"]: o["positions"] + size] = torch.tensor(list(positions) + [0] * pad, dtype=torch.int32)
         host[o["seq_start"]: o["seq_start"] + size] = host[o["positions"]: o["positions"] + size]
@@ -94,6 +100,8 @@ class DecodeGraphs:
         self.runner = runner
         self.largest = largest or 1 << (max(runner.config.max_running, 1) - 1).bit_length()
         self.buckets: dict[int, _Bucket] = {}
+        # the tokens the last step sampled, on the device: a step may start from them before the host has them
+        self.token_pool = torch.zeros(self.largest, dtype=torch.int32, device=runner.device)
         self.pool: Any = None
         self.captures = 0
         self.replays = 0
@@ -107,7 +115,8 @@ class DecodeGraphs:
 
     def _capture(self, size: int) -> _Bucket:
         runner = self.runner
-        bucket = _Bucket(size, runner.device, runner.device_cache.pad_slot, runner.config.max_model_len)
+        bucket = _Bucket(size, runner.device, runner.device_cache.pad_slot, runner.config.max_model_len,
+                         self.token_pool)
         torch.cuda.synchronize()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -137,15 +146,16 @@ class DecodeGraphs:
             size *= 2
         return made
 
-    def run(self, entries: Sequence[Any]) -> torch.Tensor:
-        """Replay the bucket's graph for single-token entries; logits [wanted, vocab]."""
+    def run(self, entries: Sequence[Any], feed: Sequence[int] | None = None) -> torch.Tensor:
+        """Replay the bucket's graph for single-token entries; logits [wanted, vocab].  ``feed[i] >= 0``:
+        entry i's token is the one at that place of ``token_pool`` (its own ``tokens`` are ignored)."""
         runner = self.runner
         size = self.bucket_of(len(entries))
         bucket = self.buckets.get(size) or self._capture(size)
         cache = runner.cache
         positions = [e.start_pos for e in entries]
         bucket.fill([e.tokens[0] for e in entries], positions, [cache.slot(e.request_id) for e in entries],
-                    max(positions) + 1)
+                    max(positions) + 1, feed)
         bucket.dev.copy_(to_device_staging(bucket.host, runner.device), non_blocking=True)
         bucket.graph.replay()
         self.replays += 1

@@ -40,6 +40,19 @@ class StepEntry:
     want: Sequence[int] = field(default_factory=tuple)
 
 
+@dataclass
+class PendingTokens:
+    """The tokens a launched decode step samples, on their way to the host."""
+
+    request_ids: tuple[str, ...]
+    host: torch.Tensor          # page-locked int32 [n]; valid once ``ready`` has passed
+    ready: Any                  # torch.cuda.Event behind the copy
+
+    def tokens(self) -> dict[str, int]:
+        self.ready.synchronize()
+        return dict(zip(self.request_ids, self.host.tolist()))
+
+
 class Runner:
     def __init__(self, model: Any, config: EngineConfig, device: str | torch.device = "cuda:0") -> None:
         if not torch.cuda.is_available():
@@ -127,9 +140,42 @@ class Runner:
             tokens = self.sampler.sample(
                 logits,
                 [r.config.temperature for r in sampled],
-                [self.sampler.uniform(r.config.seed, r.serial, r.generated_count) for r in sampled],
+                [self.sampler.uniform(r.config.seed, r.serial, r.generated_count) if r.config.temperature > 0 else 0.0
+                 for r in sampled],
             )
         return {r.request_id: token for r, token in zip(sampled, tokens)}
+
+    # -- decode steps that do not wait for their tokens -----------------------------------
+    def can_launch_decode(self, requests: int) -> bool:
+        """Whether a step of that many single tokens can be started without waiting (a captured graph takes it)."""
+        return self.graphs is not None and self.graphs.takes(requests)
+
+    def launch_decode(self, plan: Any, feed: Sequence[int], token_indices: Sequence[int]) -> "PendingTokens":
+        """Start a step in which every request brings one token and samples, and return at once.
+
+        ``feed[i] >= 0``: item i's token is the one the launch before this sampled at that place (it is
+        still on the device; the item's own token id is a placeholder).  ``token_indices[i]`` is the index of
+        the token item i is about to generate (what its random draw depends on).  The sampled tokens stay
+        on the device for the next launch and travel to the host behind the step;
+        :meth:`PendingTokens.tokens` waits for them."""
+        assert self.graphs is not None and all(item.query_length == 1 and item.sample for item in plan.items)
+        entries = [StepEntry(item.request.request_id, item.token_ids, item.start_pos, (0,)) for item in plan.items]
+        logits = self.run(entries, feed=feed)
+        requests = [item.request for item in plan.items]
+        for item in plan.items:
+            item.request.tokens_fed = item.end_pos
+        with trace_range("ragged.sample"):
+            pool = self.graphs.token_pool[: len(requests)]
+            self.sampler.sample_on_device(
+                logits, [r.config.temperature for r in requests],
+                [self.sampler.uniform(r.config.seed, r.serial, index) if r.config.temperature > 0 else 0.0
+                 for r, index in zip(requests, token_indices)],
+                out=pool)
+            host = torch.empty(len(requests), dtype=torch.int32, pin_memory=True)
+            host.copy_(pool, non_blocking=True)
+            ready = torch.cuda.Event()
+            ready.record()
+        return PendingTokens(tuple(r.request_id for r in requests), host, ready)
 
     # -- packing -----------------------------------------------------------------
     def _stage(self, count: int) -> torch.Tensor:
@@ -205,10 +251,11 @@ class Runner:
         )
 
     # -- the step ------------------------------------------------------------------
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], feed: Sequence[int] | None = None) -> torch.Tensor:
         """One step.  Returns float32 logits ``[sum(len(e.want)), vocab]`` on the
         device, in the order of the entries and of their ``want``.  Raises
-        ``CacheCapacityFull`` before anything changes if pages run out."""
+        ``CacheCapacityFull`` before anything changes if pages run out.
+        ``feed`` (captured decode steps only): see :meth:`launch_decode`."""
         self.check(entries)
         required = {e.request_id: e.start_pos + len(e.tokens) for e in entries}
         with trace_range("ragged.kv.ensure_capacity"):
@@ -223,7 +270,9 @@ class Runner:
         tokens = sum(len(e.tokens) for e in entries)
         with trace_range(f"ragged.forward.{'decode' if decode else 'mixed'}.requests_{len(entries)}.tokens_{tokens}"):
             if decode and self.graphs is not None and self.graphs.takes(len(entries)):
-                logits = self.graphs.run(entries)
+                logits = self.graphs.run(entries, feed)
+            elif feed is not None:
+                raise ValueError("tokens can be fed on the device to captured decode steps only")
             else:
                 logits = self.model.forward(self.pack(entries), self.device_cache)
         with trace_range("ragged.kv.commit"):

@@ -193,6 +193,13 @@ class Scheduler:
         self._counter = 0
         self._release_takes_flag = "preempted" in inspect.signature(runner.release).parameters
         self._publish_prefix = getattr(runner, "publish_prefix", None)
+        # decode steps that are started before the tokens of the step before have arrived (see step())
+        self._launch_decode = getattr(runner, "launch_decode", None)
+        self._can_launch_decode = getattr(runner, "can_launch_decode", None)
+        self.async_decode = bool(getattr(config, "async_decode", False)) and self._launch_decode is not None \
+            and self._can_launch_decode is not None
+        self._in_flight: tuple[BatchPlan, Any] | None = None  # (plan, its pending tokens)
+        self._resolving = False
 
     # -- public ------------------------------------------------------------------
     def submit(self, prompt_token_ids: Sequence[int], gen_config: GenerationConfig, label: str = "",
@@ -220,12 +227,16 @@ class Scheduler:
         """Idempotent; the request's pages go back at once."""
         if request.is_terminal:
             return
+        if self._in_flight is not None and not self._resolving:
+            self._take_in_flight()  # what it has generated so far is kept
+            if request.is_terminal:
+                return
         request.state = RequestState.CANCELLED
         request.finish_reason = "cancelled"
         self._finalize(request)
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.active)
+        return bool(self.waiting or self.active or self._in_flight is not None)
 
     def run_until_done(self, max_iterations: int | None = None) -> None:
         iterations = 0
@@ -237,28 +248,53 @@ class Scheduler:
 
     def step(self) -> bool:
         """One iteration: admit, plan, run the plan, take the tokens.  Returns
-        whether anything progressed."""
+        whether anything progressed.
+
+        With ``async_decode`` a plan in which every request decodes one token is
+        only started; its tokens are taken by the next call, after that call has
+        started the step that follows (whose rows take their tokens on the device).
+        The GPU then never waits for the host between two decode steps.  What the
+        host cannot know in time is an end-of-sequence token: such a request runs
+        one step more than needed, and that step's token is dropped."""
+        if self._in_flight is not None:
+            return self._step_behind_in_flight()
         progressed = self._admit_waiting()
         with trace_range("scheduler.build_batch_plan"):
             plan = self._build_batch_plan()
         if not plan.items:
             return progressed
+        if self._may_launch(plan):
+            try:
+                with trace_range("scheduler.launch_decode"):
+                    pending = self._launch_decode(plan, [-1] * len(plan.items),
+                                                  [item.request.generated_count for item in plan.items])
+            except Exception as exc:
+                self._plan_failed(plan, exc)
+                return True
+            self._in_flight = (plan, pending)
+            return True
         try:
             with trace_range("scheduler.execute_batch"):
                 outputs = self.runner.execute_batch(plan)
         except Exception as exc:
-            if bool(getattr(exc, "is_capacity_error", False)):
-                if not self._preempt_for_capacity(plan):
-                    for item in plan.items:
-                        if not item.request.is_terminal:
-                            self._fail(item.request,
-                                       f"KV capacity cannot fit one runnable sequence: {exc}", rejected=True)
-                return True
-            for item in plan.items:
-                if not item.request.is_terminal:
-                    self._fail(item.request, f"packed forward failed: {exc}")
+            self._plan_failed(plan, exc)
             return True
+        self._take_outputs(plan, outputs)
+        return True
 
+    def _plan_failed(self, plan: BatchPlan, exc: Exception) -> None:
+        if bool(getattr(exc, "is_capacity_error", False)):
+            if not self._preempt_for_capacity(plan):
+                for item in plan.items:
+                    if not item.request.is_terminal:
+                        self._fail(item.request,
+                                   f"KV capacity cannot fit one runnable sequence: {exc}", rejected=True)
+            return
+        for item in plan.items:
+            if not item.request.is_terminal:
+                self._fail(item.request, f"packed forward failed: {exc}")
+
+    def _take_outputs(self, plan: BatchPlan, outputs: dict[str, int]) -> None:
         stamp = self.clock()
         self.metrics.record_input_tokens(plan.token_count)
         for item in plan.items:
@@ -278,6 +314,61 @@ class Scheduler:
             else:
                 request.state = RequestState.PREFILL
         self.metrics.record_iteration(len(plan.items))
+
+    # -- decode steps whose tokens are taken one call later ------------------------------
+    def _may_launch(self, plan: BatchPlan) -> bool:
+        return (self.async_decode and all(item.is_decode and item.sample for item in plan.items)
+                and self._can_launch_decode(len(plan.items)))
+
+    def _take_in_flight(self) -> None:
+        """Wait for the tokens of the step in flight and hand them to their requests."""
+        plan, pending = self._in_flight
+        self._in_flight = None
+        self._resolving = True
+        try:
+            self._take_outputs(plan, pending.tokens())
+        finally:
+            self._resolving = False
+
+    def _follow_up(self, plan: BatchPlan) -> tuple[BatchPlan, list[int], list[int]] | None:
+        """The step after the one in flight, if it can be planned without that step's tokens: the same
+        requests, less those that reach their token limit with the token in flight; each row takes its
+        token from the place of its request in the step in flight."""
+        if self.waiting and len(self.active) < self.config.max_running:
+            return None  # a request wants in: let the step in flight end, then admit
+        in_flight = {id(item.request) for item in plan.items}
+        if any(id(request) not in in_flight for request in self.active if not request.is_terminal):
+            return None  # someone still has a prompt to run: the next step is a mixed one
+        items, feed, indices = [], [], []
+        for place, item in enumerate(plan.items):
+            request = item.request
+            if request.is_terminal or request.generated_count + 1 >= request.config.max_output_tokens:
+                continue
+            items.append(BatchItem(request=request, token_ids=(0,), start_pos=request.tokens_fed, sample=True,
+                                   is_decode=True))
+            feed.append(place)
+            indices.append(request.generated_count + 1)
+        if not items or not self._can_launch_decode(len(items)):
+            return None
+        return BatchPlan(tuple(items)), feed, indices
+
+    def _step_behind_in_flight(self) -> bool:
+        plan, _ = self._in_flight
+        follow = self._follow_up(plan) if self.async_decode else None
+        launched = None
+        failure: Exception | None = None
+        if follow is not None:
+            try:
+                with trace_range("scheduler.launch_decode"):
+                    launched = self._launch_decode(*follow)
+            except Exception as exc:  # nothing was started; the tokens in flight are taken first
+                failure = exc
+        self._take_in_flight()
+        if launched is not None:
+            self._in_flight = (follow[0], launched)
+        elif failure is not None and not bool(getattr(failure, "is_capacity_error", False)):
+            self._plan_failed(follow[0], failure)
+        # (a shortage of pages shows again in the next call, which plans with the tokens in hand and preempts)
         return True
 
     # -- internals -----------------------------------------------------------------
@@ -326,18 +417,26 @@ class Scheduler:
         for candidate, request in sorted(candidates, key=lambda pair: self.scheduling_priority(pair[0])):
             if budget <= 0:
                 break
-            known_ids = request.prompt_token_ids + request.generated_token_ids
-            remaining = len(known_ids) - request.tokens_fed
+            prompt, generated = request.prompt_token_ids, request.generated_token_ids
+            known = len(prompt) + len(generated)
+            remaining = known - request.tokens_fed
             limit = 1 if candidate.phase == "decode" else self.config.prefill_chunk
             query_length = min(remaining, limit, budget)
             start = request.tokens_fed
             end = start + query_length
+            # the portion's tokens, without joining the two lists (a decode step would copy the whole context)
+            if start >= len(prompt):
+                token_ids = tuple(generated[start - len(prompt): end - len(prompt)])
+            elif end <= len(prompt):
+                token_ids = tuple(prompt[start:end])
+            else:
+                token_ids = tuple(prompt[start:]) + tuple(generated[: end - len(prompt)])
             items.append(BatchItem(
                 request=request,
-                token_ids=tuple(known_ids[start:end]),
+                token_ids=token_ids,
                 start_pos=start,
-                sample=end == len(known_ids),
-                is_decode=query_length == 1 and start >= len(request.prompt_token_ids),
+                sample=end == known,
+                is_decode=query_length == 1 and start >= len(prompt),
             ))
             budget -= query_length
         return BatchPlan(tuple(items))

@@ -80,19 +80,28 @@ def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, dtype: torch.dtype,
 
 
 # ---------------------------------------------------------------------------
-def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``out[t] = float32(table[ids[t]])``; ids int32 [T] (already checked against the vocabulary)."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None,
+          feed: Optional[torch.Tensor] = None, pool: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t] = float32(table[ids[t]])``; ids int32 [T] (already checked against the vocabulary).
+    With ``feed`` (int32 [T]) and ``pool`` (int32): row t takes ``pool[feed[t]]`` as its id where
+    ``feed[t] >= 0`` (tokens another kernel left on the device; ``feed[t]`` must index ``pool``)."""
     _gpu("table", table, dims=2)
     _gpu("ids", ids, torch.int32, 1)
     vocab, hidden = table.shape
     tokens = ids.shape[0]
+    if feed is not None:
+        _gpu("feed", feed, torch.int32, 1)
+        if pool is None or feed.shape[0] < tokens:
+            raise ValueError("feed needs a pool and one entry per token")
+        _gpu("pool", pool, torch.int32, 1)
     if out is None:
         out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
     _gpu("out", out, torch.float32, 2)
     if not (out.shape == (tokens, hidden)):
         raise ValueError(f"out must be {(tokens, hidden)}, is {tuple(out.shape)}")
-    _run("cie_embed", load_library().cie_embed(_stream(), _i(_code(table.dtype)), _ptr(table), _ptr(ids),
-                                               _ptr(out), _i(tokens), _i(hidden), _i(vocab)))
+    _run("cie_embed", load_library().cie_embed(_stream(), _i(_code(table.dtype)), _ptr(table), _ptr(ids), _ptr(feed),
+                                               _ptr(pool if feed is not None else None), _ptr(out), _i(tokens),
+                                               _i(hidden), _i(vocab)))
     return out
 
 

@@ -95,7 +95,7 @@ class DecoderModel:
 
     def forward(self, batch, cache) -> torch.Tensor:
         """Run the step's tokens; float32 logits ``[len(logit_rows), vocab]``."""
-        residual = ops.embed(self.embedding, batch.token_ids)
+        residual = ops.embed(self.embedding, batch.token_ids, feed=batch.token_feed, pool=batch.token_pool)
         pending = None
         for call in self.spec.order:
             residual, pending = self.blocks[call.layer].forward(

@@ -49,9 +49,14 @@ class Sampler:
         """One token per row of ``logits`` [n, vocab] (float32, on the GPU)."""
         if logits.shape[0] == 0:
             return []
+        return self.sample_on_device(logits, temperatures, uniforms).tolist()
+
+    def sample_on_device(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float],
+                         out: torch.Tensor | None = None) -> torch.Tensor:
+        """The same, left on the GPU (int32 [n], in ``out`` if given): nothing waits for the result."""
         if all(t == 0 for t in temperatures):
-            return ops.sample(logits).tolist()
+            return ops.sample(logits, out=out)
         device = logits.device
         temperature = torch.tensor(list(temperatures), dtype=torch.float32).to(device)
         uniform = torch.tensor(list(uniforms), dtype=torch.float32).to(device)
-        return ops.sample(logits, temperature, uniform).tolist()
+        return ops.sample(logits, temperature, uniform, out=out)

@@ -39,6 +39,12 @@ def test_embed(ops, dtype):
     out = ops.embed(table, ids)
     assert out.dtype == torch.float32
     torch.testing.assert_close(out, table.float()[ids.long()], rtol=0, atol=0)
+    # rows 1 and 3 take their tokens from a pool on the device instead
+    feed = torch.tensor([-1, 2, -1, 0, -1], dtype=torch.int32).cuda()
+    pool = torch.tensor([77, 500, 901], dtype=torch.int32).cuda()
+    fed = ops.embed(table, ids, feed=feed, pool=pool)
+    expect = torch.tensor([0, 901, 5, 77, 321]).cuda()
+    torch.testing.assert_close(fed, table.float()[expect], rtol=0, atol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -285,3 +285,132 @@ def test_prompt_is_published_once_its_last_portion_has_run():
     scheduler.run_until_done()
     assert runner.published == [(long_one.request_id, 1)]
     assert one_token.state is RequestState.COMPLETED
+
+
+# -- decode steps that are started before the tokens of the step before have arrived ----------------
+class AsyncFakeRunner(FakeRunner):
+    """A fake with ``launch_decode``: tokens come back through a pending object that counts how often it
+    was waited for; a fed row's token is what the launch before produced (kept "on the device")."""
+
+    def __init__(self, *args, eos_token_at=None, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.launches: list[tuple[tuple[str, ...], tuple[int, ...]]] = []
+        self.device_tokens: list[int] = []
+        self.eos_token_at = eos_token_at or {}  # request serial -> (token index, token id)
+
+    def can_launch_decode(self, requests: int) -> bool:
+        return requests <= 8
+
+    def _token(self, request, index: int) -> int:
+        at = self.eos_token_at.get(request.serial)
+        return at[1] if at is not None and at[0] == index else 100 + index
+
+    def execute_batch(self, plan):
+        outputs = super().execute_batch(plan)
+        return {item.request.request_id: self._token(item.request, item.request.generated_count)
+                for item in plan.items if item.request.request_id in outputs}
+
+    def launch_decode(self, plan, feed, token_indices):
+        required = dict(self.resident)
+        for item in plan.items:
+            required[item.request.request_id] = max(required[item.request.request_id], item.end_pos)
+        if sum(required.values()) > self.token_capacity:
+            error = RuntimeError("fake KV capacity exhausted")
+            error.is_capacity_error = True
+            raise error
+        self.resident = required
+        fed_tokens = []
+        for item, source in zip(plan.items, feed):
+            assert item.start_pos == item.request.tokens_fed and item.query_length == 1
+            fed_tokens.append(self.device_tokens[source] if source >= 0 else item.token_ids[0])
+            item.request.tokens_fed = item.end_pos
+        self.launches.append((plan.request_ids, tuple(fed_tokens)))
+        self.device_tokens = [self._token(item.request, index) for item, index in zip(plan.items, token_indices)]
+        produced = dict(zip(plan.request_ids, self.device_tokens))
+
+        class Pending:
+            def tokens(_self):
+                return produced
+
+        return Pending()
+
+
+def make_async(runner, **overrides):
+    return make(runner, async_decode=True, **overrides)
+
+
+def test_async_decode_gives_the_same_tokens_with_one_launch_per_token():
+    def run(scheduler_of):
+        runner = AsyncFakeRunner()
+        scheduler = scheduler_of(runner)
+        a = scheduler.submit(list(range(6)), GenerationConfig(max_output_tokens=5))
+        b = scheduler.submit(list(range(3)), GenerationConfig(max_output_tokens=3))
+        scheduler.run_until_done()
+        return runner, a, b
+
+    sync_runner, a0, b0 = run(lambda r: make(r, async_decode=False))
+    runner, a, b = run(make_async)
+    assert not sync_runner.launches and runner.launches
+    assert a.generated_token_ids == a0.generated_token_ids == [100, 101, 102, 103, 104]
+    assert b.generated_token_ids == b0.generated_token_ids == [100, 101, 102]
+    # the first token of each comes with its prompt; every further token is one row of one launch, no more:
+    # b leaves the launches when its limit is in sight, nothing runs for a token that is not wanted
+    launched_rows = sum(len(ids) for ids, _ in runner.launches)
+    sampled_with_prompts = sum(item.sample for plan in runner.plans for item in plan.items)
+    assert launched_rows + sampled_with_prompts == 5 + 3
+    # from the second launch on, rows are fed the token the launch before made, not a placeholder
+    assert runner.launches[1][1][0] == 101
+    assert a.state is RequestState.COMPLETED and b.state is RequestState.COMPLETED and not runner.resident
+
+
+def test_async_decode_tokens_arrive_one_call_late():
+    runner = AsyncFakeRunner()
+    scheduler = make_async(runner)
+    request = scheduler.submit(list(range(4)), GenerationConfig(max_output_tokens=6))
+    scheduler.step()                    # the prompt, with its first token
+    assert request.generated_count == 1
+    scheduler.step()                    # launches token 2; nothing has arrived
+    assert request.generated_count == 1 and scheduler.has_work()
+    scheduler.step()                    # launches token 3, takes token 2
+    assert request.generated_count == 2
+    scheduler.run_until_done()
+    assert request.generated_token_ids == [100, 101, 102, 103, 104, 105]
+
+
+def test_async_decode_end_of_sequence_costs_one_dropped_step():
+    runner = AsyncFakeRunner(eos_token_at={1: (2, 7)})  # the first request's third token is token 7
+    scheduler = make_async(runner)
+    stops = scheduler.submit(list(range(4)), GenerationConfig(max_output_tokens=10, eos_token_id=7))
+    goes_on = scheduler.submit(list(range(4)), GenerationConfig(max_output_tokens=6))
+    scheduler.run_until_done()
+    assert stops.generated_token_ids == [100, 101, 7] and stops.finish_reason == "eos_token_reached"
+    assert goes_on.generated_token_ids == [100, 101, 102, 103, 104, 105]
+    launched_for_stops = sum(stops.request_id in ids for ids, _ in runner.launches)
+    assert launched_for_stops == 3  # tokens 2 and 3, and one step more that was under way when token 7 arrived
+    assert not runner.resident and (stops.request_id, False) in runner.released
+
+
+def test_async_decode_lets_a_new_request_in_and_survives_a_shortage():
+    runner = AsyncFakeRunner(token_capacity=30)
+    scheduler = make_async(runner, max_running=3)
+    first = scheduler.submit(list(range(8)), GenerationConfig(max_output_tokens=12))
+    for _ in range(4):
+        scheduler.step()
+    late = scheduler.submit(list(range(8)), GenerationConfig(max_output_tokens=12))  # both need 20: one must wait
+    scheduler.run_until_done(max_iterations=200)
+    assert first.generated_token_ids == [100 + i for i in range(12)]
+    assert late.generated_token_ids == [100 + i for i in range(12)]
+    assert scheduler.metrics.snapshot()["requests"]["preempted_total"] >= 1
+    assert not runner.resident
+
+
+def test_async_decode_cancel_takes_what_is_in_flight_first():
+    runner = AsyncFakeRunner()
+    scheduler = make_async(runner)
+    request = scheduler.submit(list(range(4)), GenerationConfig(max_output_tokens=9))
+    for _ in range(3):
+        scheduler.step()
+    assert request.generated_count == 2
+    scheduler.cancel(request)
+    assert request.state is RequestState.CANCELLED and request.generated_count == 3 and not scheduler.has_work()
+    assert not runner.resident
