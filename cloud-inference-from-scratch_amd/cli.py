@@ -64,6 +64,7 @@ def parser() -> argparse.ArgumentParser:
     replay.add_argument("rest", nargs=argparse.REMAINDER)
     bench = commands.add_parser("bench", help="the serving benchmark (bench.py)", add_help=False)
     bench.add_argument("rest", nargs=argparse.REMAINDER)
+    commands.add_parser("ceilings", help="memory bandwidth and bf16 matrix throughput this GPU reaches")
     workload = commands.add_parser("workload", help="an offline serving workload with random weights", add_help=False)
     workload.add_argument("rest", nargs=argparse.REMAINDER)
     return cli
@@ -103,7 +104,7 @@ def _run_script(path: Path, rest: list[str]) -> int:
 
 def main(argv: list[str] | None = None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
-    if argv and argv[0] in ("replay", "bench", "workload"):
+    if argv and argv[0] in ("replay", "bench", "workload", "ceilings"):
         # these hand all their options on; argparse would claim the ones that start with a dash
         args = argparse.Namespace(command=argv[0], rest=argv[1:])
     else:
@@ -125,6 +126,10 @@ def main(argv: list[str] | None = None) -> int:
         return _run_script(ROOT / "bin" / "trace_run", args.rest)
     if args.command == "bench":
         return _run_script(ROOT / "bench.py", args.rest)
+    if args.command == "ceilings":
+        from .ceilings import main as ceilings_main
+
+        return ceilings_main(args.rest)
     if args.command == "workload":
         from .workloads import main as workload_main
 
