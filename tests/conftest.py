@@ -57,7 +57,28 @@ TINY_B = {
     "hidden_act": "silu",
 }
 
-TINY = {"A": TINY_A, "B": TINY_B}
+# Sizes the fast paths refuse: a width and an intermediate size that are no multiples of 8 (no 16-byte rows),
+# a head size given in the configuration that is not hidden / heads, five heads on one key head, no biases.
+TINY_C = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "model_type": "qwen2",
+    "hidden_size": 100,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 5,
+    "num_key_value_heads": 1,
+    "head_dim": 16,
+    "intermediate_size": 108,
+    "vocab_size": 211,
+    "rope_theta": 500000.0,
+    "rms_norm_eps": 1e-4,
+    "attention_bias": False,
+    "tie_word_embeddings": False,
+    "use_sliding_window": False,
+    "max_position_embeddings": 200,
+    "eos_token_id": 2,
+}
+
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 
 
 def pytest_configure(config):

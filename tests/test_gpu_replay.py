@@ -27,7 +27,7 @@ F32_TOL = dict(rtol=1e-4, atol=2e-5)
 BF16_TOL = dict(rtol=2e-2, atol=2e-2)
 TOL = {"float32": F32_TOL, "bfloat16": BF16_TOL}
 
-LENGTHS = {"A": [5, 17, 33, 70, 100], "B": [1, 9, 40, 64, 100, 131]}
+LENGTHS = {"A": [5, 17, 33, 70, 100], "B": [1, 9, 40, 64, 100, 131], "C": [3, 30, 77, 48]}
 
 
 def make_requests(name: str, raw: dict) -> dict[str, list[int]]:
@@ -69,7 +69,7 @@ SCHEDULES = {
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("schedule", list(SCHEDULES))
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_replay_matches_plain(tiny_folders, plain, name, schedule, dtype):
     folder, raw, _ = tiny_folders[name]
     requests, expected = plain[name]
