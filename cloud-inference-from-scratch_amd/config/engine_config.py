@@ -38,6 +38,10 @@ class EngineConfig:
     # a captured decode step is started before the tokens of the step before it have reached the host (it takes
     # them on the device); a request that ends on an end-of-sequence token then has run one step too many
     async_decode: bool = True
+    # a waiting request is admitted only while the pool has room for the tokens known of it and of every
+    # request admitted before it (the reference admits without a look at the pool, src/cloud_engine/scheduler.py:
+    # 438-458, and long prompts then evict each other and are computed twice); False: as the reference
+    admit_within_pool: bool = True
     seed: int = 0
 
     def validated(self) -> "EngineConfig":

@@ -379,12 +379,28 @@ class Scheduler:
         known = len(request.prompt_token_ids) + request.generated_count
         return free_tokens() >= known + 1
 
+    def _room_beside_admitted(self, request: Request) -> bool:
+        """Whether the pool holds what is known of ``request`` beside what is known
+        of the admitted requests (the part of it that they have not taken yet)."""
+        free_tokens = getattr(self.runner, "free_tokens", None)
+        if free_tokens is None:
+            return True
+        allocated_tokens = getattr(self.runner, "allocated_tokens", lambda _r: 0)
+        owed = 0
+        for admitted in self.active:
+            if not admitted.is_terminal:
+                known = len(admitted.prompt_token_ids) + admitted.generated_count + 1
+                owed += max(0, known - allocated_tokens(admitted))
+        return free_tokens() - owed >= len(request.prompt_token_ids) + request.generated_count + 1
+
     def _admit_waiting(self) -> bool:
         progressed = False
         while self.waiting and len(self.active) < self.config.max_running:
             candidate = self.waiting[0]
             if candidate.preemption_count and self.active and not self._room_for(candidate):
                 break  # wait for room instead of thrashing; keeps its place at the head
+            if self.config.admit_within_pool and self.active and not self._room_beside_admitted(candidate):
+                break  # admitted now it would push another request out, or be pushed out, and be computed twice
             self.waiting.popleft()
             try:
                 self.runner.admit(candidate)

@@ -9,8 +9,8 @@ reference builds prompts from a word bank through a tokenizer; here prompts are
 seeded uniform-random token ids of the stated lengths and weights are random,
 EOS is ignored.  Two larger profiles exercise what the small ones do not: many
 live requests with chunked prompts beside decoding ones, and long prompts with a
-common prefix in a pool too small for all of them (prefix reuse, preemption and
-recomputation).
+common prefix in a pool too small for all of them (prefix reuse; admission that
+waits for room, or preemption and recomputation where all are admitted at once).
 """
 
 from __future__ import annotations
@@ -65,8 +65,11 @@ PROFILES: dict[str, Profile] = {p.name: p for p in (
     Profile("mixed-7b", "7b", 64, (128, 4096), (256, 256), token_budget=2048,
             purpose="64 live requests: prompt portions under a 2,048-token budget beside decoding requests"),
     Profile("prefix-14b", "14b", 32, (8192, 8192), (128, 128), shared_prefix=2048, pool_fraction=0.6, lead_requests=1,
-            purpose="long prompts with a common 2,048-token prefix in a pool too small for all: prefix reuse, "
-                    "preemption and recomputation"),
+            purpose="long prompts with a common 2,048-token prefix in a pool too small for all: prefix reuse, and "
+                    "admission that waits for room"),
+    Profile("pressure-14b", "14b", 32, (8192, 8192), (128, 128), shared_prefix=2048, pool_fraction=0.6, lead_requests=1,
+            engine_options={"admit_within_pool": False},
+            purpose="the same, all admitted at once as the reference admits: preemption and recomputation"),
 )}
 
 

@@ -156,6 +156,37 @@ def test_preempted_request_keeps_generated_tokens_and_its_place():
     assert recompute and recompute[0].token_ids == (2, 2, 2, 2, 2, 100, 101) and recompute[0].sample
 
 
+def test_long_prompts_are_admitted_only_while_the_pool_holds_them():
+    """Three prompts of which the pool holds two: the third waits until one has
+    ended, nothing is preempted and nothing computed twice; admitted as the
+    reference admits (without a look at the pool) they push each other out."""
+    def run(admit_within_pool):
+        runner = FakeRunner(token_capacity=24)
+        scheduler = make(runner, token_budget=8, prefill_chunk=4, admit_within_pool=admit_within_pool)
+        requests = [scheduler.submit([i + 1] * 9, GenerationConfig(max_output_tokens=2)) for i in range(3)]
+        scheduler.step()
+        admitted = len(scheduler.active)
+        scheduler.run_until_done(200)
+        assert [r.generated_token_ids for r in requests] == [[100, 101]] * 3 and not runner.resident
+        return admitted, sum(r.preemption_count for r in requests), sum(r.recomputed_tokens for r in requests)
+
+    assert run(True) == (2, 0, 0)
+    admitted, preempted, recomputed = run(False)
+    assert admitted == 3 and preempted > 0 and recomputed > 0
+
+
+def test_a_request_larger_than_what_is_left_is_admitted_when_nothing_else_runs():
+    runner = FakeRunner(token_capacity=12)
+    scheduler = make(runner, token_budget=16, prefill_chunk=16)
+    first = scheduler.submit([1] * 8, GenerationConfig(max_output_tokens=2))
+    second = scheduler.submit([2] * 8, GenerationConfig(max_output_tokens=2))
+    scheduler.step()
+    assert [r.request_id for r in scheduler.active] == [first.request_id] and scheduler.waiting[0] is second
+    scheduler.run_until_done(100)
+    assert first.generated_token_ids == second.generated_token_ids == [100, 101]
+    assert first.preemption_count == second.preemption_count == 0
+
+
 def test_custom_preemption_policy_selects_victim():
     runner = FakeRunner(token_capacity=10)
     scheduler = make(runner, token_budget=8, prefill_chunk=4)
