@@ -77,21 +77,42 @@ int make_plan(Plan& plan, hipblasLtMatmulHeuristicResult_t (&found)[kCandidates]
     return kept;
 }
 
-// Time the candidates on the call's own operands (the result is overwritten by the real call that
-// follows) and return the index of the fastest; 0 if timing is not possible.
+// Candidates are timed with the weight coming from memory, as it does inside a model's step: over copies
+// of the weight that together exceed what the caches hold (the last-level cache is 256 MB), used in turn.
+// Timed over one copy that stays in the caches, a short product picks an algorithm of few workgroups that
+// is 2.5 times slower than another once its weight has to be streamed.
+constexpr size_t kColdBytes = size_t(640) << 20;
+
+// Time the candidates on the call's own rows (the result is overwritten by the real call that follows)
+// and return the index of the fastest; 0 if timing is not possible.
 int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int count, hipStream_t stream,
-            const void* a, const void* w, void* c, void* workspace, int timed_runs) {
+            const void* a, const void* w, size_t w_bytes, void* c, void* workspace, int timed_runs) {
     hipEvent_t begin = nullptr, end = nullptr;
     if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) return 0;
+    int copies = static_cast<int>((kColdBytes + w_bytes - 1) / w_bytes);
+    copies = copies < 2 ? 2 : copies > 64 ? 64 : copies;
+    char* cold = nullptr;
+    if (hipMalloc(reinterpret_cast<void**>(&cold), w_bytes * copies) != hipSuccess) {
+        (void)hipGetLastError();
+        cold = nullptr;
+    }
+    for (int i = 0; cold && i < copies; ++i)
+        if (hipMemcpyAsync(cold + w_bytes * i, w, w_bytes, hipMemcpyDeviceToDevice, stream) != hipSuccess) {
+            (void)hipGetLastError();
+            hipStreamSynchronize(stream);
+            hipFree(cold);
+            cold = nullptr;
+        }
     const float one = 1.f, zero = 0.f;
-    int best = 0;
+    int best = 0, turn = 0;
     float best_ms = 0.f;
     for (int i = 0; i < count; ++i) {
         bool good = true;
         for (int run = 0; run <= timed_runs && good; ++run) {  // the first run is the warm-up
             if (run == 1) good = hipEventRecord(begin, stream) == hipSuccess;
-            good = good && ok(hipblasLtMatmul(g_handle, plan.desc, &one, w, plan.w, a, plan.a, &zero, c, plan.d, c, plan.d,
-                                              &found[i].algo, workspace, found[i].workspaceSize, stream));
+            const void* weight = cold ? cold + w_bytes * (turn++ % copies) : w;
+            good = good && ok(hipblasLtMatmul(g_handle, plan.desc, &one, weight, plan.w, a, plan.a, &zero, c, plan.d, c,
+                                              plan.d, &found[i].algo, workspace, found[i].workspaceSize, stream));
         }
         float ms = 0.f;
         good = good && hipEventRecord(end, stream) == hipSuccess && hipEventSynchronize(end) == hipSuccess &&
@@ -103,13 +124,17 @@ int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int
     }
     hipEventDestroy(begin);
     hipEventDestroy(end);
+    if (cold) {
+        hipStreamSynchronize(stream);
+        hipFree(cold);
+    }
     return best;
 }
 
 }  // namespace
 
 // With `tune`, a shape's first call (outside graph capture) times the heuristic's candidates on the call's
-// own operands and keeps the fastest; otherwise the heuristic's first choice is kept.
+// own rows and on copies of its weight (device memory of its own, freed again) and keeps the fastest; otherwise the heuristic's first choice is kept.
 // Returns CIE_BAD_ARGUMENT for a shape the library has no algorithm for (the caller then takes another
 // route) and CIE_LAUNCH_FAILED if the library's call itself fails.  `workspace` is device memory of
 // `workspace_bytes` that stays valid while the product runs; calls on one stream may share it.
@@ -136,7 +161,8 @@ CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w
                 capturing == hipStreamCaptureStatusNone) {
                 if (bias) hipblasLtMatmulDescSetAttribute(fresh.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
                 // short products are timed over more runs: their times scatter more
-                chosen = fastest(fresh, found, count, static_cast<hipStream_t>(stream), a, w, c, workspace, M >= 512 ? 3 : 12);
+                chosen = fastest(fresh, found, count, static_cast<hipStream_t>(stream), a, w, size_t(N) * K * 2, c, workspace,
+                                 M >= 512 ? 3 : 12);
             }
             fresh.algo = found[chosen].algo;
             fresh.workspace = found[chosen].workspaceSize;
