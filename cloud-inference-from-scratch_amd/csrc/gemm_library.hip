@@ -84,9 +84,49 @@ int make_plan(Plan& plan, hipblasLtMatmulHeuristicResult_t (&found)[kCandidates]
 constexpr size_t kColdBytes = size_t(640) << 20;
 
 // Time the candidates on the call's own rows (the result is overwritten by the real call that follows)
-// and return the index of the fastest; 0 if timing is not possible.
+// and return the index of the fastest; 0 if timing is not possible.  A candidate's time is the shortest of
+// a few batches of runs; all candidates are timed once, then the four best again with more batches, so
+// that a candidate is not chosen or dropped for what else happened while it ran (clocks that had not come
+// up yet, a neighbour's work).
+struct Timing {
+    const Plan& plan;
+    const hipblasLtMatmulHeuristicResult_t* found;
+    hipStream_t stream;
+    const void* a;
+    const char* w;
+    const char* cold;  // copies of w, or null
+    size_t w_bytes;
+    int copies;
+    void* c;
+    void* workspace;
+    hipEvent_t begin, end;
+    int turn = 0;
+
+    bool run(int i) {
+        const float one = 1.f, zero = 0.f;
+        const void* weight = cold ? cold + w_bytes * (turn++ % copies) : w;
+        return ok(hipblasLtMatmul(g_handle, plan.desc, &one, weight, plan.w, a, plan.a, &zero, c, plan.d, c, plan.d,
+                                  &found[i].algo, workspace, found[i].workspaceSize, stream));
+    }
+    // milliseconds of the fastest batch; negative if a call failed
+    float time(int i, int batches, int runs) {
+        float best = -1.f;
+        if (!run(i)) return -1.f;  // warm-up
+        for (int b = 0; b < batches; ++b) {
+            bool good = hipEventRecord(begin, stream) == hipSuccess;
+            for (int r = 0; r < runs && good; ++r) good = run(i);
+            float ms = 0.f;
+            good = good && hipEventRecord(end, stream) == hipSuccess && hipEventSynchronize(end) == hipSuccess &&
+                   hipEventElapsedTime(&ms, begin, end) == hipSuccess;
+            if (!good) return -1.f;
+            if (best < 0.f || ms < best) best = ms;
+        }
+        return best;
+    }
+};
+
 int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int count, hipStream_t stream,
-            const void* a, const void* w, size_t w_bytes, void* c, void* workspace, int timed_runs) {
+            const void* a, const void* w, size_t w_bytes, void* c, void* workspace, bool many_rows) {
     hipEvent_t begin = nullptr, end = nullptr;
     if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) return 0;
     int copies = static_cast<int>((kColdBytes + w_bytes - 1) / w_bytes);
@@ -103,23 +143,32 @@ int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int
             hipFree(cold);
             cold = nullptr;
         }
-    const float one = 1.f, zero = 0.f;
-    int best = 0, turn = 0;
-    float best_ms = 0.f;
-    for (int i = 0; i < count; ++i) {
-        bool good = true;
-        for (int run = 0; run <= timed_runs && good; ++run) {  // the first run is the warm-up
-            if (run == 1) good = hipEventRecord(begin, stream) == hipSuccess;
-            const void* weight = cold ? cold + w_bytes * (turn++ % copies) : w;
-            good = good && ok(hipblasLtMatmul(g_handle, plan.desc, &one, weight, plan.w, a, plan.a, &zero, c, plan.d, c,
-                                              plan.d, &found[i].algo, workspace, found[i].workspaceSize, stream));
+    Timing timing{plan, found, stream, a, static_cast<const char*>(w), cold, w_bytes, copies, c, workspace, begin, end};
+    // short products scatter more: more runs in a batch
+    const int runs = many_rows ? 2 : 6;
+    constexpr int kFinalists = 4;
+    int finalist[kCandidates];
+    float finalist_ms[kCandidates];
+    int finalists = 0;
+    for (int i = 0; i < count && i < kCandidates; ++i) {
+        const float ms = timing.time(i, 2, runs);
+        if (ms < 0.f) continue;
+        int at = finalists++;
+        for (; at > 0 && finalist_ms[at - 1] > ms; --at) {  // kept in order of time
+            finalist[at] = finalist[at - 1];
+            finalist_ms[at] = finalist_ms[at - 1];
         }
-        float ms = 0.f;
-        good = good && hipEventRecord(end, stream) == hipSuccess && hipEventSynchronize(end) == hipSuccess &&
-               hipEventElapsedTime(&ms, begin, end) == hipSuccess;
-        if (good && (best_ms == 0.f || ms < best_ms)) {
+        finalist[at] = i;
+        finalist_ms[at] = ms;
+    }
+    if (finalists > kFinalists) finalists = kFinalists;
+    int best = finalists ? finalist[0] : 0;
+    float best_ms = -1.f;
+    for (int f = 0; f < finalists; ++f) {
+        const float ms = timing.time(finalist[f], 5, runs);
+        if (ms >= 0.f && (best_ms < 0.f || ms < best_ms)) {
             best_ms = ms;
-            best = i;
+            best = finalist[f];
         }
     }
     hipEventDestroy(begin);
@@ -134,7 +183,8 @@ int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int
 }  // namespace
 
 // With `tune`, a shape's first call (outside graph capture) times the heuristic's candidates on the call's
-// own rows and on copies of its weight (device memory of its own, freed again) and keeps the fastest; otherwise the heuristic's first choice is kept.
+// own rows and on copies of its weight (device memory of its own, freed again) and keeps the fastest;
+// otherwise the heuristic's first choice is kept.
 // Returns CIE_BAD_ARGUMENT for a shape the library has no algorithm for (the caller then takes another
 // route) and CIE_LAUNCH_FAILED if the library's call itself fails.  `workspace` is device memory of
 // `workspace_bytes` that stays valid while the product runs; calls on one stream may share it.
@@ -162,7 +212,7 @@ CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w
                 if (bias) hipblasLtMatmulDescSetAttribute(fresh.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
                 // short products are timed over more runs: their times scatter more
                 chosen = fastest(fresh, found, count, static_cast<hipStream_t>(stream), a, w, size_t(N) * K * 2, c, workspace,
-                                 M >= 512 ? 3 : 12);
+                                 M >= 512);
             }
             fresh.algo = found[chosen].algo;
             fresh.workspace = found[chosen].workspaceSize;
