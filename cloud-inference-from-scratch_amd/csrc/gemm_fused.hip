@@ -202,13 +202,22 @@ __device__ __forceinline__ void store_rope(const FusedArgs& a, const floatx4& lo
 // MT row tiles (M <= 16*MT per workgroup row; more rows: more workgroup rows) and NT column tiles
 // per workgroup: with SILU the gate tile and its up tile, else NT adjacent tiles.  Every weight
 // value a wave loads meets all MT row tiles; every activation value meets the NT column tiles.
+constexpr int kStageRow = 256 + 16;           // bytes of a row in a staging area: the padding spreads the rows over the banks
+constexpr int kStageTile = 16 * kStageRow;    // a wave's staging area
+
 template <int WAVES, int EPI, int MT, int NT>
 __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
     static_assert(EPI != EPI_ROPE || (NT == 2 && MT == 1), "the ROPE epilogue pairs the two halves of a head");
     // slices of 128 k values whose weight loads are in flight together
     constexpr int U = (MT == 1 && NT == 1) ? 4 : (MT == 4) ? 1 : 2;
-    __shared__ float reduce[WAVES > 1 ? (WAVES - 1) * MT * NT * 64 * 4 : 1];
+    // During the product every wave has a staging area of its own for one 16 x 128 piece of W (below);
+    // afterwards the same memory takes the waves' partial tiles.
+    constexpr int kReduceBytes = WAVES > 1 ? (WAVES - 1) * MT * NT * 64 * 4 * 4 : 16;
+    constexpr int kStageBytes = WAVES * kStageTile;
+    __shared__ __attribute__((aligned(16))) char shared[kReduceBytes > kStageBytes ? kReduceBytes : kStageBytes];
+    float* reduce = reinterpret_cast<float*>(shared);
+    char* stage = shared + (threadIdx.x / kWave) * kStageTile;
 
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
@@ -222,27 +231,43 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     const int rope_head = blockIdx.x / rope_tiles;
     const int rope_tile = blockIdx.x - rope_head * rope_tiles;
 
-    // a column past the end computes a copy that is not stored
-    const bf16_t* w_row[NT];
+    // A 16 x 128 piece of W (16 rows of 256 bytes) is fetched by four loads of four rows each: sixteen
+    // neighbouring lanes read one row's 256 bytes, which the memory pipeline takes as whole cache lines
+    // (a load in which every lane reads another row costs it four times the cycles, and with as many
+    // loads of A as of W that, not the memory, bounded the kernel).  The piece then passes through the
+    // wave's staging area in LDS into the MFMA layout: lane (r, g) gets row r, k values j*32 + g*8 .. +7.
+    // A column past the end computes a copy that is not stored.
+    const int load_row = lane >> 4;        // of the four rows of a load
+    const int load_col = (lane & 15) * 8;  // k offset inside the 128
+    const bf16_t* w_rows[NT][4];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        int n;
-        if (EPI == EPI_ROPE)
-            n = rope_head * a.rope.head_dim + rope_tile * 16 + r + t * (a.rope.head_dim / 2);
-        else if (EPI == EPI_SILU)
-            n = min(tile_first * 16 + r, cols - 1) + t * a.up_offset;
-        else
-            n = min((tile_first + t) * 16 + r, cols - 1);
-        w_row[t] = a.w + static_cast<size_t>(n) * a.K + g * 8;
-    }
-    const bf16_t* a_row[MT];
-    bool row_ok[MT];
+    for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = m0 + mt * 16 + r;
-        row_ok[mt] = m < a.M;
-        a_row[mt] = a.a + static_cast<size_t>(min(m, a.M - 1)) * a.lda + g * 8;
-    }
+        for (int i = 0; i < 4; ++i) {
+            const int row = i * 4 + load_row;
+            int n;
+            if (EPI == EPI_ROPE)
+                n = rope_head * a.rope.head_dim + rope_tile * 16 + row + t * (a.rope.head_dim / 2);
+            else if (EPI == EPI_SILU)
+                n = min(tile_first * 16 + row, cols - 1) + t * a.up_offset;
+            else
+                n = min((tile_first + t) * 16 + row, cols - 1);
+            w_rows[t][i] = a.w + static_cast<size_t>(n) * a.K + load_col;
+        }
+    // With more than 16 rows the rows of A travel the same way (they come from the cache, but cost the
+    // memory pipeline the same); with one row tile the extra step only adds to each slice's latency
+    // and the lanes load A as the MFMA wants it: lane (r, g) row r, k values j*32 + g*8 .. +7.
+    constexpr bool kStageA = MT > 1;
+    const bf16_t* a_rows[MT][4];
+    bool row_ok[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = m0 + mt * 16 + (kStageA ? i * 4 + load_row : r);
+            row_ok[mt][i] = m < a.M;
+            a_rows[mt][i] = a.a + static_cast<size_t>(min(m, a.M - 1)) * a.lda + (kStageA ? load_col : i * 32 + g * 8);
+        }
 
     floatx4 acc[MT][NT];
 #pragma unroll
@@ -258,37 +283,59 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     for (int kbase = k_begin + wave * 128; kbase < k_end; kbase += U * WAVES * 128) {
         uint4 b[U][NT][4];
 #pragma unroll
-        for (int u = 0; u < U; ++u)
+        for (int u = 0; u < U; ++u) {
+            const int k0 = kbase + u * WAVES * 128;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int k0 = kbase + u * WAVES * 128 + j * 32;
+            for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int t = 0; t < NT; ++t)
-                    b[u][t][j] = (k0 + g * 8 < k_end) ? *reinterpret_cast<const uint4*>(w_row[t] + k0) : uint4{0, 0, 0, 0};
-            }
+                for (int i = 0; i < 4; ++i)
+                    b[u][t][i] = (k0 + load_col < k_end) ? *reinterpret_cast<const uint4*>(w_rows[t][i] + k0) : uint4{0, 0, 0, 0};
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             // the few rows of A come from the cache; their loads are issued slice by slice
+            const int ka = kbase + u * WAVES * 128;
+            uint4 av[MT][4];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                uint4 av[4];
+            for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int k0 = kbase + u * WAVES * 128 + j * 32;
-                    av[j] = (row_ok[mt] && k0 + g * 8 < k_end) ? *reinterpret_cast<const uint4*>(a_row[mt] + k0)
-                                                               : uint4{0, 0, 0, 0};
+                for (int i = 0; i < 4; ++i) {
+                    const int k_lane = ka + (kStageA ? load_col : i * 32 + g * 8);
+                    av[mt][i] = (row_ok[mt][i] && k_lane < k_end) ? *reinterpret_cast<const uint4*>(a_rows[mt][i] + ka)
+                                                                  : uint4{0, 0, 0, 0};
                 }
+            if (kStageA) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-                    for (int t = 0; t < NT; ++t)
+                    for (int i = 0; i < 4; ++i)
+                        *reinterpret_cast<uint4*>(stage + (i * 4 + load_row) * kStageRow + load_col * 2) = av[mt][i];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        av[mt][j] = *reinterpret_cast<const uint4*>(stage + r * kStageRow + j * 64 + g * 16);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                // through the staging area (a wave's LDS operations keep their order: no barrier)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    *reinterpret_cast<uint4*>(stage + (i * 4 + load_row) * kStageRow + load_col * 2) = b[u][t][i];
+                uint4 bt[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) bt[j] = *reinterpret_cast<const uint4*>(stage + r * kStageRow + j * 64 + g * 16);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
                         acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            __builtin_bit_cast(bf16x8, av[j]), __builtin_bit_cast(bf16x8, b[u][t][j]), acc[mt][t], 0, 0, 0);
+                            __builtin_bit_cast(bf16x8, av[mt][j]), __builtin_bit_cast(bf16x8, bt[j]), acc[mt][t], 0, 0, 0);
             }
         }
     }
 
     if (WAVES > 1) {  // sum the waves' partial tiles in wave order; wave 0 keeps the result
+        __syncthreads();  // every wave is done with its staging area
         if (wave > 0) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)

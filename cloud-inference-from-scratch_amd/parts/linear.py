@@ -20,11 +20,16 @@ import torch
 from ..kernels import ops
 
 # Rows up to which the hand-written fused bf16 kernel replaces the library product.  Measured on
-# MI355X (3B shapes): up to 16 rows it beats the library by 1.5-2x; with 17 to 64 rows it only wins where K
-# is long and is cut into parts (the down product: 18-23 us against the library's 27-32 us); its gate/up
-# product loses from 24 rows on (41 us against 25 us at 64 rows: every workgroup re-reads the rows of A).
+# MI355X (3B shapes): up to 16 rows it beats the library by 1.5-2x; with 17 to 64 rows it wins where K
+# is long and is cut into parts (the down product: 17-20 us against the library's 27-32 us); its gate/up
+# product loses from 32 rows on (34 us against 26 + 5 us at 64 rows: every workgroup re-reads the rows of A).
 FUSED_ROWS = 16
 FUSED_PARTS_ROWS = 64
+# With 17 to 64 rows it also wins where the weight is small (q/k/v and o_proj of the 3B shape: 7-9 us against
+# the library's 12-18 us inside a step, and the residual add rides along); from about 6M weight values on the
+# library is faster (7B o_proj at 64 rows: 12.6 us against 11.1 us).
+FUSED_SMALL_ROWS = 64
+FUSED_SMALL_WEIGHT = 6 << 20
 # float32 logits of more rows than this go to the library (the hand-written kernel streams the weight once per
 # 64 rows; up to 64 rows it is one pass either way)
 FUSED_LOGIT_ROWS = 64
@@ -78,7 +83,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         out = ops.gemm_library(x, weight, out_dtype=torch.float32)  # logits of many rows: one pass over the weight
         if out is not None:
             return out
-    if fusable and (rows <= FUSED_ROWS or wants_f32):
+    small = rows <= FUSED_SMALL_ROWS and n * k <= FUSED_SMALL_WEIGHT and not silu
+    if fusable and (rows <= FUSED_ROWS or wants_f32 or small):
         if into is not None:
             return RowSumsq(ops.gemm_fused(weight, ops.EPI_RESID, x, bias=bias, residual_out=into))
         elif silu and n % 2 == 0:
