@@ -111,6 +111,41 @@ __device__ __forceinline__ void store_tile(const FusedArgs& a, const floatx4& ac
     }
 }
 
+// The RESID epilogue for the MT row tiles of one column tile: all old values of the residual are fetched
+// before the first new one is written (taken tile by tile, every load would wait behind the stores of
+// the tile before it, which the compiler must assume to alias: one round trip to memory per row).
+template <int MT>
+__device__ __forceinline__ void store_resid(const FusedArgs& a, const floatx4 (&acc)[MT], int m_base, int n, int n_tile,
+                                            int lane) {
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const bool col_ok = n < a.N;
+    const float add = (col_ok && a.bias) ? to_float(a.bias[n]) : 0.f;
+    float old[MT][4];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = m_base + mt * 16 + g * 4 + i;
+            old[mt][i] = (col_ok && m < a.M) ? a.residual[static_cast<size_t>(m) * a.N + n] : 0.f;
+        }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = m_base + mt * 16 + g * 4 + i;
+            const bool ok = col_ok && m < a.M;
+            const float v = ok ? old[mt][i] + acc[mt][i] + add : 0.f;
+            if (ok) a.residual[static_cast<size_t>(m) * a.N + n] = v;
+            float sq = v * v;  // sum over the tile's 16 columns: the lanes that share g
+            sq += __shfl_xor(sq, 1, kWave);
+            sq += __shfl_xor(sq, 2, kWave);
+            sq += __shfl_xor(sq, 4, kWave);
+            sq += __shfl_xor(sq, 8, kWave);
+            if (r == 0 && m < a.M) a.sumsq[static_cast<size_t>(m) * ((a.N + 15) / 16) + n_tile] = sq;
+        }
+}
+
 // The ROPE epilogue for one pair of tiles: `lo` holds dimensions j*16 + r of head `head`, `hi` those
 // plus D/2.  Values are rounded to bf16 before the rotation, so that the results equal those of the
 // plain epilogue followed by the rotation kernel.  What the epilogue needs of each of the lane's four
@@ -358,6 +393,17 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
                         acc[mt][t][i] += reduce[((((w - 1) * MT + mt) * NT + t) * 4 + i) * 64 + lane];
+    }
+    if constexpr (EPI == EPI_RESID) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            if ((tile_first + t) * 16 < cols) {  // wave-uniform
+                floatx4 column[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) column[mt] = acc[mt][t];
+                store_resid<MT>(a, column, m0, (tile_first + t) * 16 + r, tile_first + t, lane);
+            }
+        return;
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
