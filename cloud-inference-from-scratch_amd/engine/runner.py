@@ -99,8 +99,16 @@ class Runner:
 
     def warm_up(self) -> int:
         """Do now what the first steps would otherwise do on the clock: capture the decode graphs of
-        all bucket sizes.  Returns the number of graphs captured."""
-        return self.graphs.capture_all() if self.graphs is not None else 0
+        all bucket sizes, and let the products of full prompt portions (one request's portion, and the
+        sizes up to the token budget that time the library's candidates) set themselves up.  Returns
+        the number of graphs captured."""
+        captured = self.graphs.capture_all() if self.graphs is not None else 0
+        budget, chunk = self.config.token_budget, min(self.config.prefill_chunk, self.config.token_budget)
+        rows = {chunk} | {n for n in range(512, budget + 1, 256)}
+        warm = getattr(self.model, "warm_up", None)
+        if warm is not None:
+            warm(sorted(rows))
+        return captured
 
     def publish_prefix(self, request: Any) -> None:
         """The request's prompt is in the cache: offer its full pages to the prefix index now, not only

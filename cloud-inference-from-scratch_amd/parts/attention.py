@@ -78,6 +78,11 @@ class Attention(Part):
         self.b_o = tensors[prefix + "o_proj.bias"].contiguous() if self.out_bias else None
         self.cos, self.sin = self.position.tables(device)
 
+    def warm_up(self, rows: int) -> None:
+        blank = lambda width: torch.zeros((rows, width), dtype=self.w_qkv.dtype, device=self.w_qkv.device)
+        linear(blank(self.hidden_size), self.w_qkv, self.b_qkv)
+        linear(blank(self.num_heads * self.head_dim), self.w_o, self.b_o)
+
     def forward(self, x, batch, view, writes: bool = True, residual: Optional[torch.Tensor] = None):
         if batch.max_context > self.position.max_position and self.position.rotates:
             raise ValueError(

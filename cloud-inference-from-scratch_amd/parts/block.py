@@ -51,6 +51,12 @@ class PreNormBlock:
     def graph_safe(self) -> bool:
         return all(getattr(part, "graph_safe", False) for _, part in self._parts())
 
+    def warm_up(self, rows: int) -> None:
+        for _, part in self._parts():
+            warm = getattr(part, "warm_up", None)
+            if warm is not None:
+                warm(rows)
+
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], batch, view,
                 writes: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
         x = normalise(self.norm1, residual, pending, self.dtype)

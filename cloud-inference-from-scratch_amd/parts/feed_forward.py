@@ -38,6 +38,9 @@ class GatedMLP(Part):
         ).contiguous()
         self.w_down = tensors[prefix + "down_proj.weight"].contiguous()
 
+    def warm_up(self, rows: int) -> None:
+        self.forward(torch.zeros((rows, self.hidden_size), dtype=self.w_down.dtype, device=self.w_down.device))
+
     def forward(self, x, residual: Optional[torch.Tensor] = None):
         return linear(linear(x, self.w_gate_up, epilogue="silu"), self.w_down, into=residual)
 

@@ -93,6 +93,23 @@ class DecoderModel:
             block.bind(tensors, self.spec.layer_prefix.format(index=index), self.dtype, device)
         return self
 
+    def warm_up(self, row_counts) -> None:
+        """Run every part's products once on blank rows of the given counts, so that what a product
+        does at the first call of a shape (the library's products time their candidates) happens
+        before the first request.  Layers of one specification share their shapes: one of each runs."""
+        if self.dtype != torch.bfloat16 or self.device.type != "cuda":
+            return
+        seen = set()
+        for block in self.blocks:
+            key = repr(block.spec)
+            if key in seen:
+                continue
+            seen.add(key)
+            warm = getattr(block, "warm_up", None)
+            if warm is not None:
+                for rows in row_counts:
+                    warm(rows)
+
     def forward(self, batch, cache) -> torch.Tensor:
         """Run the step's tokens; float32 logits ``[len(logit_rows), vocab]``."""
         residual = ops.embed(self.embedding, batch.token_ids, feed=batch.token_feed, pool=batch.token_pool)
