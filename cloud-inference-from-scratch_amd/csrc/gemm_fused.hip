@@ -369,7 +369,55 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         }
     }
 
-    if (WAVES > 1) {  // sum the waves' partial tiles in wave order; wave 0 keeps the result
+    // With more than one row tile the waves share the end of the work: row tile mt belongs to wave
+    // mt % WAVES, which sums the other waves' partial tiles of that row tile and stores it (one wave
+    // doing all of it would take as long again as the product).
+    constexpr bool kSharedEnd = WAVES > 1 && MT > 1 && EPI != EPI_ROPE;
+    if constexpr (kSharedEnd) {
+        __syncthreads();  // every wave is done with its staging area
+        // slot of wave w for row tile mt: the waves other than the owner, in wave order
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int owner = mt % WAVES;
+            if (wave != owner) {
+                const int slot = wave < owner ? wave : wave - 1;
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        reduce[(((mt * (WAVES - 1) + slot) * NT + t) * 4 + i) * 64 + lane] = acc[mt][t][i];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (wave != mt % WAVES) continue;  // wave-uniform
+#pragma unroll 1
+            for (int slot = 0; slot < WAVES - 1; ++slot)
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[mt][t][i] += reduce[(((mt * (WAVES - 1) + slot) * NT + t) * 4 + i) * 64 + lane];
+            if constexpr (EPI == EPI_RESID) {
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    if ((tile_first + t) * 16 < cols) {  // wave-uniform
+                        const floatx4 column[1] = {acc[mt][t]};
+                        store_resid<1>(a, column, m0 + mt * 16, (tile_first + t) * 16 + r, tile_first + t, lane);
+                    }
+            } else if (EPI == EPI_SILU) {
+                store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, tile_first * 16 + r, tile_first, lane);
+            } else {
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    if ((tile_first + t) * 16 < cols)  // wave-uniform
+                        store_tile<EPI>(a, acc[mt][t], acc[mt][t], m0 + mt * 16, (tile_first + t) * 16 + r, tile_first + t, lane);
+            }
+        }
+        return;
+    }
+    if (WAVES > 1) {  // one row tile: sum the waves' partial tiles in wave order; wave 0 keeps the result
         __syncthreads();  // every wave is done with its staging area
         if (wave > 0) {
 #pragma unroll
@@ -382,9 +430,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         }
         __syncthreads();
         if (wave > 0) return;
-        // many tiles: one wave's partial tiles at a time, or the loads of all of them would not fit the registers
-        constexpr int kWavesAtOnce = (MT * NT > 2) ? 1 : WAVES;
-#pragma unroll kWavesAtOnce
+#pragma unroll
         for (int w = 1; w < WAVES; ++w)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
