@@ -158,7 +158,7 @@ struct RopeRows {
     float bias_lo, bias_hi;
 };
 
-__device__ __forceinline__ RopeRows rope_prefetch(const FusedArgs& a, int head, int j, int lane) {
+__device__ __forceinline__ RopeRows rope_prefetch(const FusedArgs& a, int head, int j, int lane, int m_base) {
     const RopeArgs& p = a.rope;
     const int r = lane & 15;
     const int g = lane >> 4;
@@ -171,7 +171,7 @@ __device__ __forceinline__ RopeRows rope_prefetch(const FusedArgs& a, int head, 
     rows.bias_hi = a.bias ? to_float(a.bias[head * p.head_dim + d + half]) : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int m = g * 4 + i;
+        const int m = m_base + g * 4 + i;
         rows.pos[i] = 0;
         rows.page[i] = -1;
         rows.c[i] = 1.f;
@@ -192,7 +192,7 @@ __device__ __forceinline__ RopeRows rope_prefetch(const FusedArgs& a, int head, 
 }
 
 __device__ __forceinline__ void store_rope(const FusedArgs& a, const floatx4& lo, const floatx4& hi, int head,
-                                           int j, int lane, const RopeRows& rows) {
+                                           int j, int lane, const RopeRows& rows, int m_base) {
     const RopeArgs& p = a.rope;
     const int r = lane & 15;
     const int g = lane >> 4;
@@ -204,7 +204,7 @@ __device__ __forceinline__ void store_rope(const FusedArgs& a, const floatx4& lo
     const int kv_head = is_query ? 0 : (head - p.q_heads) % p.kv_heads;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int m = g * 4 + i;
+        const int m = m_base + g * 4 + i;
         if (m >= a.M) continue;
         const float x_lo = to_float(from_float<bf16_t>(lo[i] + rows.bias_lo));
         const float x_hi = to_float(from_float<bf16_t>(hi[i] + rows.bias_hi));
@@ -243,7 +243,8 @@ constexpr int kStageTile = 16 * kStageRow;    // a wave's staging area
 template <int WAVES, int EPI, int MT, int NT>
 __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
-    static_assert(EPI != EPI_ROPE || (NT == 2 && MT == 1), "the ROPE epilogue pairs the two halves of a head");
+    static_assert(EPI != EPI_ROPE || NT == 2, "the ROPE epilogue pairs the two halves of a head");
+    static_assert(MT <= WAVES || WAVES == 1, "a wave ends at most one row tile");
     // slices of 128 k values whose weight loads are in flight together
     constexpr int U = (MT == 1 && NT == 1) ? 4 : (MT == 4) ? 1 : 2;
     // During the product every wave has a staging area of its own for one 16 x 128 piece of W (below);
@@ -310,7 +311,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
     RopeRows rope_rows;
-    if (EPI == EPI_ROPE && wave == 0) rope_rows = rope_prefetch(a, rope_head, rope_tile, lane);
+    // (the wave that will store row tile `wave`, below)
+    if (EPI == EPI_ROPE && wave < MT) rope_rows = rope_prefetch(a, rope_head, rope_tile, lane, m0 + wave * 16);
 
     const int k_begin = blockIdx.z * a.k_per_part;
     const int k_end = min(a.K, k_begin + a.k_per_part);
@@ -372,7 +374,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     // With more than one row tile the waves share the end of the work: row tile mt belongs to wave
     // mt % WAVES, which sums the other waves' partial tiles of that row tile and stores it (one wave
     // doing all of it would take as long again as the product).
-    constexpr bool kSharedEnd = WAVES > 1 && MT > 1 && EPI != EPI_ROPE;
+    constexpr bool kSharedEnd = WAVES > 1 && MT > 1;
     if constexpr (kSharedEnd) {
         __syncthreads();  // every wave is done with its staging area
         // slot of wave w for row tile mt: the waves other than the owner, in wave order
@@ -406,6 +408,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
                         const floatx4 column[1] = {acc[mt][t]};
                         store_resid<1>(a, column, m0 + mt * 16, (tile_first + t) * 16 + r, tile_first + t, lane);
                     }
+            } else if (EPI == EPI_ROPE) {
+                store_rope(a, acc[mt][0], acc[mt][NT - 1], rope_head, rope_tile, lane, rope_rows, m0 + mt * 16);
             } else if (EPI == EPI_SILU) {
                 store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, tile_first * 16 + r, tile_first, lane);
             } else {
@@ -454,7 +458,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         if (EPI == EPI_ROPE) {
-            store_rope(a, acc[mt][0], acc[mt][NT - 1], rope_head, rope_tile, lane, rope_rows);
+            store_rope(a, acc[mt][0], acc[mt][NT - 1], rope_head, rope_tile, lane, rope_rows, m0 + mt * 16);
         } else if (EPI == EPI_SILU) {
             store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, tile_first * 16 + r, tile_first, lane);
         } else {
@@ -553,16 +557,17 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     return CIE_BAD_ARGUMENT;
 }
 
-// q/k/v product of up to 16 rows with the ROPE epilogue: `w` [N, K] stacks the rows of q_heads query
+// q/k/v product of up to 64 rows with the ROPE epilogue: `w` [N, K] stacks the rows of q_heads query
 // heads, kv_heads key heads and kv_heads value heads of head_dim dimensions each (a multiple of 32);
 // `c` [M, N] receives the rotated queries (its key and value columns are left alone); rotated keys and
-// values go to the cache page of each row's position.  `waves` waves per workgroup share K (1, 2, 4, 8).
+// values go to the cache page of each row's position.  `waves` waves per workgroup share K (1, 2, 4, 8;
+// with more than 16 rows 4 or 8).
 CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
                               int M, int N, int K, int waves, const float* cos_table, const float* sin_table,
                               const int* positions, const int* seq_of_token, const int* seq_slot,
                               const int* block_table, int table_width, void* k_pool, void* v_pool, int q_heads,
                               int kv_heads, int head_dim, int page_size, int rotate, int write_kv) {
-    if (M <= 0 || M > 16 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
+    if (M <= 0 || M > 64 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
     if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 32 || page_size <= 0 || table_width <= 0 ||
         N != (q_heads + 2 * kv_heads) * head_dim)
         return CIE_BAD_ARGUMENT;
@@ -586,5 +591,8 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
                       static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads, head_dim,
                       page_size, rotate, write_kv};
     const dim3 grid((q_heads + 2 * kv_heads) * (head_dim / 32), 1, 1);
-    return launch_waves<EPI_ROPE, 1, 2>(static_cast<hipStream_t>(stream), waves, grid, f);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (M <= 16) return launch_waves<EPI_ROPE, 1, 2>(s, waves, grid, f);
+    if (M <= 32) return launch_waves<EPI_ROPE, 2, 2>(s, waves, grid, f);
+    return launch_waves<EPI_ROPE, 4, 2>(s, waves, grid, f);
 }

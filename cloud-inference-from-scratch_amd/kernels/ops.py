@@ -522,7 +522,7 @@ def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Te
                   block_table: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, q_heads: int,
                   kv_heads: int, head_dim: int, rotate: bool = True, write_kv: bool = True,
                   waves: Optional[int] = None) -> torch.Tensor:
-    """The q/k/v product of up to 16 rows fused with what ``rope_kv_write`` does:
+    """The q/k/v product of up to 64 rows fused with what ``rope_kv_write`` does:
     ``a @ weight.T + bias`` for weight [(Hq+2Hkv)*D, K], queries and keys rotated
     by each row's position, keys and values written into the cache.  Returns the
     buffer [M, (Hq+2Hkv)*D] whose query columns hold the rotated queries (its key
@@ -533,8 +533,8 @@ def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Te
     if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
         raise ValueError("a must be a bf16 GPU matrix with unit inner stride")
     m = a.shape[0]
-    if not (1 <= m <= 16 and a.shape[1] == k):
-        raise ValueError(f"a {tuple(a.shape)}: up to 16 rows of K={k}")
+    if not (1 <= m <= 64 and a.shape[1] == k):
+        raise ValueError(f"a {tuple(a.shape)}: up to 64 rows of K={k}")
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
     if not (k % 8 == 0 and lda % 8 == 0):
         raise ValueError(f"K and the row stride must be multiples of 8, are {k} and {lda}")
@@ -563,8 +563,8 @@ def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Te
     page_size = _check_pools(k_pool, v_pool, torch.bfloat16, kv_heads, head_dim)
     if waves is None:
         _, waves, _ = plan_fused(m, n // 32, k)
-    if not (waves in (1, 2, 4, 8)):
-        raise ValueError(f"{waves} waves per workgroup is not a form the kernel has")
+    if not (waves in ((1, 2, 4, 8) if m <= 16 else (4, 8))):
+        raise ValueError(f"{waves} waves per workgroup with {m} rows is not a form the kernel has")
     out = torch.empty((m, n), dtype=torch.bfloat16, device=weight.device)
     _run("cie_gemm_qkv_rope", load_library().cie_gemm_qkv_rope(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k), _i(waves), _ptr(cos),

@@ -21,7 +21,7 @@ from ..config.specs import PartSpec
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, build_part, register_part
-from .linear import FUSED_ROWS, linear
+from .linear import FUSED_ROWS, FUSED_SMALL_ROWS, FUSED_SMALL_WEIGHT, linear
 
 
 class Attention(Part):
@@ -89,9 +89,10 @@ class Attention(Part):
                 f"position {batch.max_context - 1} is beyond the rotary table of {self.position.max_position}"
             )
         rows = x.shape[0]
-        if (x.dtype == torch.bfloat16 and rows <= FUSED_ROWS and self.head_dim % 32 == 0
+        few = rows <= FUSED_ROWS or (rows <= FUSED_SMALL_ROWS and self.w_qkv.numel() <= FUSED_SMALL_WEIGHT)
+        if (x.dtype == torch.bfloat16 and few and self.head_dim % 32 == 0
                 and x.shape[1] % 8 == 0 and (rows == 1 or x.stride(0) % 8 == 0)):
-            # few rows: the product's epilogue rotates and writes the cache itself
+            # few rows (where the hand-written product is the faster one): its epilogue rotates and writes the cache
             qkv = ops.gemm_qkv_rope(self.w_qkv, x, self.b_qkv, self.cos, self.sin, batch.positions,
                                     batch.seq_of_token, batch.seq_slot, view.block_table, view.k_pool, view.v_pool,
                                     self.num_heads, self.num_kv_heads, self.head_dim,

@@ -427,7 +427,7 @@ def test_rope_kv_write(ops, dtype, geometry):
 
 
 @pytest.mark.parametrize("geometry", [(16, 2, 128, 16, 2048), (4, 2, 32, 8, 96), (3, 1, 64, 4, 328), (5, 5, 96, 32, 200)])
-@pytest.mark.parametrize("rows", [1, 7, 16])
+@pytest.mark.parametrize("rows", [1, 7, 16, 24, 40, 64])
 @pytest.mark.parametrize("waves", [None, 1, 8])
 def test_gemm_qkv_rope_equals_product_then_rotation(ops, geometry, rows, waves):
     """The q/k/v product whose epilogue rotates and writes the cache, against the plain
@@ -435,7 +435,10 @@ def test_gemm_qkv_rope_equals_product_then_rotation(ops, geometry, rows, waves):
     implementation above): rotated queries, touched cache rows and untouched ones."""
     q_heads, kv_heads, head_dim, page_size, hidden = geometry
     n = (q_heads + 2 * kv_heads) * head_dim
-    lengths = [40, 5, 100, 17][: max(1, min(4, rows))]  # every sequence has at least rows / 4 tokens
+    row_tiles = 1 if rows <= 16 else 2 if rows <= 32 else 4
+    if waves == 1 and row_tiles > 1:
+        waves = 4  # the fewest with more than 16 rows
+    lengths = [40, 25, 100, 17][: max(1, min(4, rows))]  # every sequence has at least rows / 4 tokens
     k_pool, v_pool, table, slots, _ = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=44)
     k_two, v_two = k_pool.clone(), v_pool.clone()
     # the rows: the last tokens of the sequences in turn (decode rows), several per sequence when rows > sequences
@@ -453,7 +456,7 @@ def test_gemm_qkv_rope_equals_product_then_rotation(ops, geometry, rows, waves):
     meta = (torch.tensor(positions, dtype=torch.int32).cuda(), torch.tensor(seq_of_token, dtype=torch.int32).cuda(),
             torch.tensor(slots, dtype=torch.int32).cuda(), table)
     fused = ops.gemm_qkv_rope(w, a, b, cos, sin, *meta, k_pool, v_pool, q_heads, kv_heads, head_dim, waves=waves)
-    plain_qkv = ops.gemm_fused(w, ops.EPI_BF16, a, bias=b, plan=None if waves is None else (1, waves, 1))
+    plain_qkv = ops.gemm_fused(w, ops.EPI_BF16, a, bias=b, plan=None if waves is None else (row_tiles, waves, 1))
     ops.rope_kv_write(plain_qkv, cos, sin, *meta, k_two, v_two, q_heads, kv_heads, head_dim)
     q_cols = q_heads * head_dim
     # one bf16 step at most (the two kernels may round a fused multiply-add differently)
@@ -468,7 +471,11 @@ def test_gemm_qkv_rope_equals_product_then_rotation(ops, geometry, rows, waves):
     if waves is None:  # the two plans may cut K differently: sums in another order
         torch.testing.assert_close(bare[:, :q_cols].float(), ops.gemm_fused(w, ops.EPI_BF16, a, bias=b)[:, :q_cols].float(), **step)
     else:
-        assert torch.equal(bare[:, :q_cols], ops.gemm_fused(w, ops.EPI_BF16, a, bias=b, plan=(1, waves, 1))[:, :q_cols])
+        same_plan = ops.gemm_fused(w, ops.EPI_BF16, a, bias=b, plan=(row_tiles, waves, 1))
+        if row_tiles == 1:
+            assert torch.equal(bare[:, :q_cols], same_plan[:, :q_cols])
+        else:  # a pair of column tiles per workgroup here, one there: the waves' sums meet in another order
+            torch.testing.assert_close(bare[:, :q_cols].float(), same_plan[:, :q_cols].float(), **step)
     assert torch.equal(k_pool, k_before) and torch.equal(v_pool, v_before)
     with pytest.raises(ValueError, match="steps of 32"):
         ops.gemm_qkv_rope(w[: 3 * 16], a, None, cos[:, :8].contiguous(), sin[:, :8].contiguous(), *meta,
