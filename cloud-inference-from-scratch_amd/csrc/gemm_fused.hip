@@ -19,13 +19,13 @@
 //               writes q to C[m, n], k and v into the paged cache (v transposed).
 //
 // One kernel: a workgroup owns one or two tiles of 16 columns (SILU: a gate tile and its up tile)
-// and 16, 32 or 64 rows; its WAVES waves cut K into slices of 128 and take them round-robin;
-// every lane loads its own rows of A and of W for the same k values straight into MFMA operands
-// (W from memory, once; the few rows of A from the cache); the waves' partial tiles are summed
-// through LDS in wave order.  v_mfma_f32_16x16x32_bf16 with A = activations (16 rows), B = weight
-// rows; the four lane groups of a wave read one contiguous 64-byte piece of each weight row per
-// load, and the same k values of A (the order of k inside a product is free as long as both
-// operands agree).
+// and 16, 32 or 64 rows; its WAVES waves cut K into slices of 128 and take them round-robin.
+// A wave fetches a 16 x 128 piece of W with loads that read whole 256-byte row segments and turns
+// it into the MFMA operand layout through a small staging area in LDS (with more than 16 rows the
+// rows of A too; with 16 the lanes load A as the MFMA wants it, from the cache); the waves' partial
+// tiles are summed through LDS in wave order, by wave 0 or, with more than one row tile, by one
+// wave per row tile.  v_mfma_f32_16x16x32_bf16 with A = activations (16 rows), B = weight rows
+// (the order of k inside a product is free as long as both operands agree).
 // No workgroup ever waits for another: a device-wide fence between workgroups costs more on
 // this GPU than the whole product.
 #include "common.h"

@@ -1,7 +1,8 @@
 """``x @ W^T + b`` for a Linear's weight ``[out, in]``, and its fused forms.
 
 float32: the hand-written true-float32 kernel, always.  bfloat16 with up to
-``FUSED_ROWS`` rows (decode steps, the output head): the hand-written
+``FUSED_ROWS`` rows (decode steps, the output head), and up to 64 rows where
+it is the faster one (a small weight, a long K): the hand-written
 matrix-core kernel that streams the weight once and takes over its neighbours'
 work: a SiLU-gate behind (``epilogue="silu"``), the add into the float32
 residual stream (``into=residual``), or float32 results for the logits.
