@@ -5,6 +5,7 @@ groups, head sizes in steps of 16)."""
 from __future__ import annotations
 
 import math
+import random
 
 import pytest
 import torch
@@ -567,6 +568,34 @@ def test_gemm_fused_epilogues(ops, shape, plan):
     padded[:, :n] = want
     torch.testing.assert_close(sumsq[:m].double(), padded.pow(2).view(m, parts, 16).sum(-1), rtol=1e-4, atol=1e-3)
     assert torch.isnan(sumsq[m:]).all()
+
+
+def test_gemm_fused_random_shapes(ops):
+    """Seeded random shapes (rows to 70, any column count, K any multiple of 8) through every
+    epilogue, against float64 products: the edges of row tiles, column tiles and K slices in
+    combinations the hand-picked shapes do not hold."""
+    rng = random.Random(1234)
+    for case in range(40):
+        m, n, k = rng.randint(1, 70), 2 * rng.randint(1, 150), 8 * rng.randint(1, 180)
+        k_parts = rng.choice([1, 1, 2, 3, 5])
+        a, w = rand((m, k), torch.bfloat16, 300 + case), rand((n, k), torch.bfloat16, 400 + case, 0.3)
+        b = rand((n,), torch.bfloat16, 500 + case)
+        exact = a.double() @ w.double().t()
+        tag = f"case {case}: m={m} n={n} k={k} parts={k_parts}"
+        out = ops.gemm_fused(w, ops.EPI_F32, a, bias=b)
+        torch.testing.assert_close(out.double(), exact + b.double(), rtol=1e-4, atol=2e-4 * math.sqrt(k), msg=lambda t: f"{tag}: {t}")
+        parts = ops.gemm_fused(w, ops.EPI_PARTIAL, a, bias=b, k_parts=k_parts)
+        torch.testing.assert_close(parts.double().sum(0), exact + b.double(), rtol=1e-4, atol=2e-4 * math.sqrt(k),
+                                   msg=lambda t: f"{tag}: {t}")
+        gated = ops.gemm_fused(w, ops.EPI_SILU, a)
+        want = torch.nn.functional.silu(exact[:, : n // 2]) * exact[:, n // 2:]
+        torch.testing.assert_close(gated.double(), want, rtol=1e-2, atol=1e-2 * float(want.abs().max()) + 1e-6,
+                                   msg=lambda t: f"{tag}: {t}")
+        residual = rand((m, n), torch.float32, 600 + case, 2.0)
+        want = residual.double() + exact + b.double()
+        sumsq = ops.gemm_fused(w, ops.EPI_RESID, a, bias=b, residual_out=residual)
+        torch.testing.assert_close(residual.double(), want, rtol=1e-4, atol=2e-4 * math.sqrt(k), msg=lambda t: f"{tag}: {t}")
+        torch.testing.assert_close(sumsq.double().sum(-1), want.pow(2).sum(-1), rtol=1e-3, atol=1e-3, msg=lambda t: f"{tag}: {t}")
 
 
 @pytest.mark.parametrize("shape", [(1, 64, 256), (8, 2048, 11008), (13, 96, 328), (16, 48, 1032), (40, 200, 1032),
