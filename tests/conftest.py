@@ -106,7 +106,7 @@ def sharpen(tensors: dict, factor: float = 8.0) -> dict:
     return out
 
 
-def make_folder(tmp: Path, raw: dict, seed: int, store_dtype: str = "bfloat16") -> tuple[Path, dict]:
+def make_folder(tmp: Path, raw: dict, seed: int, store_dtype: str = "bfloat16", factor: float = 8.0) -> tuple[Path, dict]:
     """Write config.json + model.safetensors; returns the folder and the stored tensors."""
     from cie_amd.config import config_from_dict
     from cie_amd.parts.model import expected_tensors
@@ -114,7 +114,7 @@ def make_folder(tmp: Path, raw: dict, seed: int, store_dtype: str = "bfloat16") 
 
     config = config_from_dict(raw)
     expected = expected_tensors(config.model_spec())
-    tensors = sharpen(RandomSource(seed).load(expected, store_dtype, "cpu"))
+    tensors = sharpen(RandomSource(seed).load(expected, store_dtype, "cpu"), factor)
     write_tensors(tmp, raw, tensors)
     return tmp, tensors
 

@@ -138,21 +138,26 @@ def by_position(steps: list[dict], outputs: dict[int, np.ndarray]) -> dict[str, 
     return rows
 
 
-def compare(rows: dict[str, dict[int, np.ndarray]], plain: dict[str, torch.Tensor], rtol: float, atol: float) -> float:
-    """Assert every position of every request against the plain logits; returns the worst abs difference."""
+def compare(rows: dict[str, dict[int, np.ndarray]], plain: dict[str, torch.Tensor], rtol: float, atol: float,
+            every_position: bool = True) -> float:
+    """Assert every position of every request (or, with ``every_position=False``, the
+    positions that were asked for) against the plain logits; returns the worst abs difference."""
     worst = 0.0
     for rid, expected in plain.items():
         got = rows[rid]
-        assert sorted(got) == list(range(expected.shape[0])), f"{rid}: positions {sorted(got)[:5]}..."
-        stacked = np.stack([got[p] for p in range(expected.shape[0])])
-        want = expected.numpy()
+        if every_position:
+            assert sorted(got) == list(range(expected.shape[0])), f"{rid}: positions {sorted(got)[:5]}..."
+        positions = sorted(got)
+        assert positions, f"{rid}: no logits"
+        stacked = np.stack([got[p] for p in positions])
+        want = expected.numpy()[positions]
         diff = np.abs(stacked - want)
         worst = max(worst, float(diff.max()))
         bad = diff > atol + rtol * np.abs(want)
         if bad.any():
-            pos = int(np.argwhere(bad.any(axis=1))[0][0])
+            pos = positions[int(np.argwhere(bad.any(axis=1))[0][0])]
             raise AssertionError(
                 f"request {rid}: first wrong position {pos} of {expected.shape[0]}, "
-                f"max |diff| there {diff[pos].max():.3e}, overall {diff.max():.3e}"
+                f"max |diff| there {diff[positions.index(pos)].max():.3e}, overall {diff.max():.3e}"
             )
     return worst

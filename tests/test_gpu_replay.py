@@ -279,3 +279,73 @@ def test_trace_run_program(tiny_folders, plain, tmp_path, dtype):
             assert not path.exists()
     rows = replay_util.by_position(steps, outputs)
     replay_util.compare(rows, expected, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape,layers", [("0.5b", 2), ("3b", 1)])
+def test_replay_at_the_sizes_of_real_models(tmp_path_factory, shape, layers, dtype):
+    """The widths, head counts and vocabulary of two models of the family (few layers,
+    random weights): the kernels meet the shapes that serving meets, not only the
+    tiny ones.  One request most of it at once and its tail token by token, another
+    in portions beside it; logits at the end of every step against the plain
+    implementation."""
+    from conftest import make_folder
+    from cie_amd.workloads import SHAPES
+
+    raw = dict(SHAPES[shape], architectures=["Qwen2ForCausalLM"], num_hidden_layers=layers)
+    # (at these widths the tiny models' factor of 8 on the query and key weights would make every softmax
+    # one-hot, and a bfloat16 rounding of a score could then swap the key it picks)
+    folder, tensors = make_folder(tmp_path_factory.mktemp(f"real_{shape}"), raw, seed=31, factor=1.5)
+    requests = {"long": random_tokens(190, raw["vocab_size"], seed=7), "cut": random_tokens(121, raw["vocab_size"], seed=8)}
+    weights = {k: v.float() for k, v in tensors.items()}
+    expected = {rid: plain_qwen2.forward(raw, weights, tokens) for rid, tokens in requests.items()}
+    # what float32 itself costs at these widths: the plain implementation with float64 layers
+    exact = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.float64) for rid, tokens in requests.items()}
+    del weights
+    steps = []
+
+    def step(entries, end=()):
+        steps.append({"step": len(steps), "end": list(end),
+                      "entries": [{"id": rid, "tokens": tokens, "want": [len(tokens) - 1]} for rid, tokens in entries]})
+
+    long, cut = requests["long"], requests["cut"]
+    step([("long", long[:150]), ("cut", cut[:64])])
+    fed = 64
+    for i, size in enumerate((33, 2, 17, 5)):  # the other request's portions beside single tokens of the first
+        step([("long", [long[150 + i]]), ("cut", cut[fed:fed + size])], end=["cut"] if fed + size == len(cut) else [])
+        fed += size
+    assert fed == len(cut)
+    for i in range(154, len(long)):
+        step([("long", [long[i]])], end=["long"] if i == len(long) - 1 else [])
+    runner = make_runner(folder, dtype, replay_util.max_live_tokens(steps, page=16), 16)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    if dtype == "float32":
+        # sums of thousands of float32 products: the engine may be as far from the exact logits as a few times
+        # what the plain float32 implementation is (its sums run in another order)
+        plain_error = max(float((expected[rid] - exact[rid]).abs().max()) for rid in requests)
+        print(f"plain float32 against float64 layers: {plain_error:.3e}", flush=True)
+        worst = replay_util.compare(rows, exact, every_position=False, rtol=0.0, atol=4 * plain_error + 1e-6)
+        print(f"{shape} x {layers} layers float32: worst |diff| to exact {worst:.3e}, plain float32 {plain_error:.3e}", flush=True)
+    else:
+        # bfloat16 keeps 8 bits, and at these widths a logit sums 896 to 2,048 rounded values: what that costs is
+        # measured, not assumed: the plain implementation run in bfloat16 throughout is the yardstick, and the
+        # engine (float32 residual stream, softmax and sums) has to be closer to the float32 logits than it is
+        def errors(logits_of):
+            square, count, worst = 0.0, 0, 0.0
+            for rid, by_pos in rows.items():
+                for pos in by_pos:
+                    diff = logits_of(rid, pos) - expected[rid][pos]
+                    square += float((diff ** 2).sum())
+                    count += diff.numel()
+                    worst = max(worst, float(diff.abs().max()))
+            return (square / count) ** 0.5, worst
+
+        weights = {k: v.float() for k, v in tensors.items()}
+        rough = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
+        del weights
+        plain_rms, plain_worst = errors(lambda rid, pos: rough[rid][pos])
+        rms, worst = errors(lambda rid, pos: torch.from_numpy(rows[rid][pos]))
+        print(f"{shape} x {layers} layers bfloat16: root mean square {rms:.3e} (plain in bfloat16 {plain_rms:.3e}), "
+              f"worst {worst:.3e} ({plain_worst:.3e})", flush=True)
+        assert rms <= plain_rms and worst <= 1.5 * plain_worst
+    assert runner.cache.stats().pages_used == 0
