@@ -282,17 +282,19 @@ def test_trace_run_program(tiny_folders, plain, tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape,layers", [("0.5b", 2), ("3b", 1)])
-def test_replay_at_the_sizes_of_real_models(tmp_path_factory, shape, layers, dtype):
-    """The widths, head counts and vocabulary of two models of the family (few layers,
-    random weights): the kernels meet the shapes that serving meets, not only the
-    tiny ones.  One request most of it at once and its tail token by token, another
+@pytest.mark.parametrize("shape,layers,vocab", [("0.5b", 2, None), ("3b", 1, None), ("7b", 1, 20011)])
+def test_replay_at_the_sizes_of_real_models(tmp_path_factory, shape, layers, vocab, dtype):
+    """The widths, head counts and vocabulary of models of the family (few layers,
+    random weights; the largest with a short vocabulary, to keep its files small): the
+    kernels meet the shapes that serving meets, not only the tiny ones.  One request most of it at once and its tail token by token, another
     in portions beside it; logits at the end of every step against the plain
     implementation."""
     from conftest import make_folder
     from cie_amd.workloads import SHAPES
 
     raw = dict(SHAPES[shape], architectures=["Qwen2ForCausalLM"], num_hidden_layers=layers)
+    if vocab is not None:
+        raw.update(vocab_size=vocab, eos_token_id=vocab - 1)
     # (at these widths the tiny models' factor of 8 on the query and key weights would make every softmax
     # one-hot, and a bfloat16 rounding of a score could then swap the key it picks)
     folder, tensors = make_folder(tmp_path_factory.mktemp(f"real_{shape}"), raw, seed=31, factor=1.5)
