@@ -63,6 +63,15 @@ struct FusedArgs {
     int M, N, K;
     int up_offset;         // SILU: rows of W between a gate row and its up row (N/2)
     int k_per_part;        // k values per grid.z part (a multiple of 128); K with one part
+    // An RMSNorm that follows the RESID product, folded into its neighbours: the RESID epilogue also
+    // writes scaled_out[m, n] = bf16(residual[m, n] * norm_weight[n]) (the norm's output short of the
+    // row's 1/rms), and a SILU product that reads such rows gets the sums of squares of the residual's
+    // rows (row_sumsq [M, sumsq_parts] partial sums) and multiplies its sums by 1/rms before the SiLU.
+    const float* norm_weight;  // RESID: [N] or null
+    bf16_t* scaled_out;        // RESID: [M, N] or null
+    const float* row_sumsq;    // SILU: [M, sumsq_parts] or null
+    int sumsq_parts;
+    float eps;
     RopeArgs rope;         // ROPE only
 };
 
@@ -70,7 +79,8 @@ struct FusedArgs {
 // `n` is the lane's column (of C, or of the SILU output), `m_base` the tile's first row.
 template <int EPI>
 __device__ __forceinline__ void store_tile(const FusedArgs& a, const floatx4& acc, const floatx4& acc_up,
-                                           int m_base, int n, int n_tile, int lane) {
+                                           int m_base, int n, int n_tile, int lane,
+                                           const float (&row_scale)[4] = {1.f, 1.f, 1.f, 1.f}) {
     const int r = lane & 15;
     const int g = lane >> 4;
     const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
@@ -82,9 +92,9 @@ __device__ __forceinline__ void store_tile(const FusedArgs& a, const floatx4& ac
         const bool ok = col_ok && m < a.M;
         if (EPI == EPI_SILU) {
             if (ok) {
-                const float gate = acc[i];
+                const float gate = acc[i] * row_scale[i];
                 static_cast<bf16_t*>(a.c)[static_cast<size_t>(m) * cols + n] =
-                    from_float<bf16_t>((gate / (1.0f + __expf(-gate))) * acc_up[i]);
+                    from_float<bf16_t>((gate / (1.0f + __expf(-gate))) * (acc_up[i] * row_scale[i]));
             }
         } else if (EPI == EPI_RESID) {
             float v = 0.f;
@@ -137,6 +147,8 @@ __device__ __forceinline__ void store_resid(const FusedArgs& a, const floatx4 (&
             const bool ok = col_ok && m < a.M;
             const float v = ok ? old[mt][i] + acc[mt][i] + add : 0.f;
             if (ok) a.residual[static_cast<size_t>(m) * a.N + n] = v;
+            if (ok && a.scaled_out)
+                a.scaled_out[static_cast<size_t>(m) * a.N + n] = from_float<bf16_t>(v * a.norm_weight[n]);
             float sq = v * v;  // sum over the tile's 16 columns: the lanes that share g
             sq += __shfl_xor(sq, 1, kWave);
             sq += __shfl_xor(sq, 2, kWave);
@@ -251,7 +263,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     // afterwards the same memory takes the waves' partial tiles.
     constexpr int kReduceBytes = WAVES > 1 ? (WAVES - 1) * MT * NT * 64 * 4 * 4 : 16;
     constexpr int kStageBytes = WAVES * kStageTile;
-    __shared__ __attribute__((aligned(16))) char shared[kReduceBytes > kStageBytes ? kReduceBytes : kStageBytes];
+    constexpr int kSharedBytes = kReduceBytes > kStageBytes ? kReduceBytes : kStageBytes;
+    __shared__ __attribute__((aligned(16))) char shared[kSharedBytes + 16 * sizeof(float)];  // + the rows' scales
     float* reduce = reinterpret_cast<float*>(shared);
     char* stage = shared + (threadIdx.x / kWave) * kStageTile;
 
@@ -313,6 +326,30 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     RopeRows rope_rows;
     // (the wave that will store row tile `wave`, below)
     if (EPI == EPI_ROPE && wave < MT) rope_rows = rope_prefetch(a, rope_head, rope_tile, lane, m0 + wave * 16);
+    // Rows that still lack their 1/rms (one row tile only): the waves share the 16 rows, 4 * WAVES lanes
+    // sum the partial sums of a row, and the scales meet in LDS for the wave that stores.  The loads are
+    // issued behind the wave's first loads of W, so that they add nothing to its start.
+    constexpr int kScaleLanes = 4 * WAVES;         // lanes per row
+    constexpr int kScaleRows = 16 / WAVES;         // rows per wave
+    float* scale_lds = reinterpret_cast<float*>(shared + kSharedBytes);
+    float row_scale[4] = {1.f, 1.f, 1.f, 1.f};
+    float sq_part = 0.f;
+    const bool scaled_rows = EPI == EPI_SILU && MT == 1 && a.row_sumsq != nullptr;
+    bool scale_pending = scaled_rows;
+    const int scale_row = wave * kScaleRows + lane / kScaleLanes;  // of the tile
+    auto sum_row_parts = [&]() {
+        if (m0 + scale_row >= a.M) return;
+        const float* row = a.row_sumsq + static_cast<size_t>(m0 + scale_row) * a.sumsq_parts;
+        const int sub = lane % kScaleLanes;
+        if (a.sumsq_parts % 4 == 0) {
+            for (int p = sub * 4; p < a.sumsq_parts; p += kScaleLanes * 4) {
+                const float4 v = *reinterpret_cast<const float4*>(row + p);
+                sq_part += (v.x + v.y) + (v.z + v.w);
+            }
+        } else {
+            for (int p = sub; p < a.sumsq_parts; p += kScaleLanes) sq_part += row[p];
+        }
+    };
 
     const int k_begin = blockIdx.z * a.k_per_part;
     const int k_end = min(a.K, k_begin + a.k_per_part);
@@ -327,6 +364,10 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     b[u][t][i] = (k0 + load_col < k_end) ? *reinterpret_cast<const uint4*>(w_rows[t][i] + k0) : uint4{0, 0, 0, 0};
+        }
+        if (scale_pending) {  // once, behind the wave's first loads of W
+            sum_row_parts();
+            scale_pending = false;
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -371,6 +412,16 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         }
     }
 
+    if (scaled_rows) {
+        if (scale_pending) sum_row_parts();  // (a K so short that this wave had no slice)
+#pragma unroll
+        for (int offset = kScaleLanes / 2; offset > 0; offset >>= 1) sq_part += __shfl_xor(sq_part, offset, kWave);
+        if (lane % kScaleLanes == 0) scale_lds[scale_row] = 1.0f / sqrtf(sq_part / static_cast<float>(a.K) + a.eps);
+        if (WAVES == 1) {  // (with more waves the barrier below stands between the write and the read)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) row_scale[i] = scale_lds[g * 4 + i];
+        }
+    }
     // With more than one row tile the waves share the end of the work: row tile mt belongs to wave
     // mt % WAVES, which sums the other waves' partial tiles of that row tile and stores it (one wave
     // doing all of it would take as long again as the product).
@@ -434,6 +485,10 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         }
         __syncthreads();
         if (wave > 0) return;
+        if (scaled_rows) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) row_scale[i] = scale_lds[g * 4 + i];
+        }
 #pragma unroll
         for (int w = 1; w < WAVES; ++w)
 #pragma unroll
@@ -460,7 +515,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         if (EPI == EPI_ROPE) {
             store_rope(a, acc[mt][0], acc[mt][NT - 1], rope_head, rope_tile, lane, rope_rows, m0 + mt * 16);
         } else if (EPI == EPI_SILU) {
-            store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, tile_first * 16 + r, tile_first, lane);
+            store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, tile_first * 16 + r, tile_first, lane, row_scale);
         } else {
 #pragma unroll
             for (int t = 0; t < NT; ++t)
@@ -522,9 +577,13 @@ int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, int k_part
 // column_tiles 1 or 2 tiles of 16 columns per workgroup (2 only with more than one row tile: the rows of
 // A that a wave loads then meet two tiles of W; the SiLU epilogue always takes a gate tile and its up tile).
 // K and lda must be multiples of 8 (16-byte loads); N is free.
+// norm_weight [N] float32 and scaled_out [M, N] bf16 (both or neither; RESID only): the epilogue also writes
+// the new residual times the weight.  row_sumsq [M, sumsq_parts] and eps (SILU with one row tile only): the
+// rows of `a` lack the factor rsqrt(sum of the row's partial sums / K + eps), applied before the SiLU.
 CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
                            float* residual, float* sumsq, int M, int N, int K, int epilogue, int row_tiles,
-                           int waves, int column_tiles, int k_parts) {
+                           int waves, int column_tiles, int k_parts, const float* norm_weight, void* scaled_out,
+                           const float* row_sumsq, int sumsq_parts, float eps) {
     if (M <= 0 || N <= 0 || K <= 0 || K % 8 || !a || !w || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
     if (row_tiles != 1 && row_tiles != 2 && row_tiles != 4) return CIE_BAD_ARGUMENT;
     if (waves != 1 && waves != 2 && waves != 4 && waves != 8) return CIE_BAD_ARGUMENT;
@@ -532,6 +591,11 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     if (epilogue == EPI_RESID && (!residual || !sumsq)) return CIE_BAD_ARGUMENT;
     if (epilogue != EPI_RESID && !c) return CIE_BAD_ARGUMENT;
     if (k_parts < 1 || k_parts > 64 || (k_parts > 1 && epilogue != EPI_PARTIAL)) return CIE_BAD_ARGUMENT;
+    // the folded norm: a scaled copy needs the weight and the RESID epilogue; rows that lack their scale
+    // are taken by the SILU epilogue of one row tile
+    if ((scaled_out != nullptr) != (norm_weight != nullptr) || (scaled_out && epilogue != EPI_RESID)) return CIE_BAD_ARGUMENT;
+    if (row_sumsq && (epilogue != EPI_SILU || row_tiles != 1 || M > 16 || sumsq_parts < 1 || !(eps > 0.f)))
+        return CIE_BAD_ARGUMENT;
     FusedArgs f;
     f.a = static_cast<const bf16_t*>(a);
     f.lda = lda;
@@ -545,6 +609,11 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     f.K = K;
     f.up_offset = (epilogue == EPI_SILU) ? N / 2 : 0;
     f.k_per_part = ((K + k_parts - 1) / k_parts + 127) / 128 * 128;
+    f.norm_weight = norm_weight;
+    f.scaled_out = static_cast<bf16_t*>(scaled_out);
+    f.row_sumsq = row_sumsq;
+    f.sumsq_parts = sumsq_parts;
+    f.eps = eps;
     f.rope = RopeArgs{};
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (epilogue) {
@@ -587,6 +656,11 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
     f.K = K;
     f.up_offset = 0;
     f.k_per_part = (K + 127) / 128 * 128;
+    f.norm_weight = nullptr;
+    f.scaled_out = nullptr;
+    f.row_sumsq = nullptr;
+    f.sumsq_parts = 0;
+    f.eps = 0.f;
     f.rope = RopeArgs{cos_table, sin_table, positions, seq_of_token, seq_slot, block_table, table_width,
                       static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads, head_dim,
                       page_size, rotate, write_kv};

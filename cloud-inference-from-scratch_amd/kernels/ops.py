@@ -404,7 +404,9 @@ def plan_fused(rows: int, column_tiles: int, k: int, k_parts: int = 1) -> tuple[
 
 def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optional[torch.Tensor] = None,
                residual_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None,
-               plan: Optional[tuple[int, int, int]] = None, k_parts: int = 1) -> torch.Tensor:
+               plan: Optional[tuple[int, int, int]] = None, k_parts: int = 1,
+               norm_weight: Optional[torch.Tensor] = None, scaled_out: Optional[torch.Tensor] = None,
+               row_sumsq: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
     """Few-row matrix product ``a @ weight.T`` (bf16 operands, float32 sums) fused
     with its neighbour.  ``epilogue``: ``EPI_BF16`` / ``EPI_F32`` return
     ``a W^T + bias``; ``EPI_SILU`` (weight = gate rows over up rows) returns
@@ -412,7 +414,12 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
     into ``residual_out`` (float32 [M, N]) and returns the partial sums of
     squares of its new rows [M, ceil(N/16)]; ``EPI_PARTIAL`` cuts K into
     ``k_parts`` parts and returns their float32 partial products
-    [k_parts, M, N] (bias in part 0), to be summed by ``add_parts_rmsnorm``."""
+    [k_parts, M, N] (bias in part 0), to be summed by ``add_parts_rmsnorm``.
+    An RMSNorm between an ``EPI_RESID`` product and an ``EPI_SILU`` product of up to 16
+    rows can ride along: with ``norm_weight`` (float32 [N]) and ``scaled_out`` (bf16
+    [M, N]) the former also writes the new residual times the weight, and the latter,
+    given these rows as ``a`` with ``row_sumsq`` (the former's result) and ``eps``,
+    multiplies its sums by each row's ``rsqrt(mean square + eps)`` before the SiLU."""
     _gpu("weight", weight, torch.bfloat16, 2)
     n, k = weight.shape
     if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
@@ -467,9 +474,23 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
         out, residual, sumsq = sumsq_out, residual_out, sumsq_out
     else:
         raise ValueError(f"unknown epilogue {epilogue}")
+    if (norm_weight is None) != (scaled_out is None) or (scaled_out is not None and epilogue != EPI_RESID):
+        raise ValueError("a scaled copy needs the norm's weight, its own rows and the residual epilogue")
+    if scaled_out is not None:
+        _gpu("norm_weight", norm_weight, torch.float32, 1)
+        _gpu("scaled_out", scaled_out, torch.bfloat16, 2)
+        if not (norm_weight.shape[0] == n and scaled_out.shape == (m, n)):
+            raise ValueError(f"norm_weight {tuple(norm_weight.shape)} / scaled_out {tuple(scaled_out.shape)} vs {(m, n)}")
+    parts_in = 0
+    if row_sumsq is not None:
+        _gpu("row_sumsq", row_sumsq, torch.float32, 2)
+        if not (epilogue == EPI_SILU and row_tiles == 1 and m <= 16 and row_sumsq.shape[0] >= m and eps > 0):
+            raise ValueError("rows that lack their scale go to the SiLU epilogue of up to 16 rows, with a positive eps")
+        parts_in = row_sumsq.shape[1]
     _run("cie_gemm_fused", load_library().cie_gemm_fused(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(None if epilogue == EPI_RESID else out),
-        _ptr(residual), _ptr(sumsq), _i(m), _i(n), _i(k), _i(epilogue), _i(row_tiles), _i(waves), _i(column_tiles), _i(k_parts)))
+        _ptr(residual), _ptr(sumsq), _i(m), _i(n), _i(k), _i(epilogue), _i(row_tiles), _i(waves), _i(column_tiles),
+        _i(k_parts), _ptr(norm_weight), _ptr(scaled_out), _ptr(row_sumsq), _i(parts_in), _f(eps)))
     return out
 
 

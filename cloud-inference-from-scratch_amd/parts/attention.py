@@ -27,6 +27,7 @@ from .linear import FUSED_ROWS, FUSED_SMALL_ROWS, FUSED_SMALL_WEIGHT, linear
 class Attention(Part):
     graph_safe = True
     adds_to_residual = True
+    folds_next_norm = True  # its output product can leave the next norm's rows short of their scale
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool, out_bias: bool, position: PartSpec, window: Optional[int] = None,
                  scale: Optional[float] = None) -> None:
@@ -83,7 +84,8 @@ class Attention(Part):
         linear(blank(self.hidden_size), self.w_qkv, self.b_qkv)
         linear(blank(self.num_heads * self.head_dim), self.w_o, self.b_o)
 
-    def forward(self, x, batch, view, writes: bool = True, residual: Optional[torch.Tensor] = None):
+    def forward(self, x, batch, view, writes: bool = True, residual: Optional[torch.Tensor] = None,
+                next_norm=None):
         if batch.max_context > self.position.max_position and self.position.rotates:
             raise ValueError(
                 f"position {batch.max_context - 1} is beyond the rotary table of {self.position.max_position}"
@@ -104,7 +106,7 @@ class Attention(Part):
                               self.head_dim, rotate=self.position.rotates, write_kv=writes)
         context = attend(qkv, batch, view, self.num_heads, self.num_kv_heads, self.head_dim,
                          self.window, self.scale)
-        return linear(context, self.w_o, self.b_o, into=residual)
+        return linear(context, self.w_o, self.b_o, into=residual, then_norm=next_norm)
 
 
 WIDE_DECODE_KEYS = 2048  # contexts from which decode rows go to the four-wave form

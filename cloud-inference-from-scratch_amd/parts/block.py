@@ -61,6 +61,9 @@ class PreNormBlock:
                 writes: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
         x = normalise(self.norm1, residual, pending, self.dtype)
         extra = {"residual": residual} if getattr(self.mixer, "adds_to_residual", False) else {}
+        if (extra and getattr(self.mixer, "folds_next_norm", False) and getattr(self.norm2, "folds_into_products", False)
+                and getattr(self.feed_forward, "takes_scaled_rows", False)):
+            extra["next_norm"] = self.norm2  # the norm between the two rides along with their products
         mixed = self.mixer.forward(x, batch, view, writes, **extra)
         x = normalise(self.norm2, residual, mixed, self.dtype)
         extra = {"residual": residual} if getattr(self.feed_forward, "adds_to_residual", False) else {}

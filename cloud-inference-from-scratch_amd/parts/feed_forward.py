@@ -18,6 +18,7 @@ from .linear import linear
 class GatedMLP(Part):
     graph_safe = True
     adds_to_residual = True
+    takes_scaled_rows = True  # its first product applies the scale of rows that come without it
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu") -> None:
         if activation != "silu":
             raise ValueError(f"gated feed-forward runs silu only, got {activation!r}")

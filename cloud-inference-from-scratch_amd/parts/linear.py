@@ -14,7 +14,7 @@ a library (src/cloud_engine/model.py:89-137), with the small kernels around it.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional, Union
+from typing import Any, Optional, Union
 
 import torch
 
@@ -44,9 +44,34 @@ PART_K = 2752
 class RowSumsq:
     """Stands where a branch output would: the branch was already added into the
     residual stream, and ``sumsq`` [rows, parts] holds partial sums of squares of
-    the residual's rows (what an RMSNorm needs of them)."""
+    the residual's rows (what an RMSNorm needs of them).  ``scaled``, if given, is
+    the new residual times the weight of ``norm`` in bf16: that norm's output
+    short of each row's 1/rms."""
 
     sumsq: torch.Tensor
+    scaled: Optional[torch.Tensor] = None
+    norm: Any = None
+
+
+@dataclass
+class ScaledRows:
+    """Stands where an RMSNorm's output would: ``rows`` [M, hidden] bf16 lack the
+    factor ``rsqrt(sum(sumsq[m]) / hidden + eps)`` of their row, which a product
+    that reads them applies to its sums (a product is linear in its rows)."""
+
+    rows: torch.Tensor
+    sumsq: torch.Tensor
+    eps: float
+    residual: torch.Tensor
+    norm: Any
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    def complete(self) -> torch.Tensor:
+        """The norm's output after all (for a reader that cannot apply the factor)."""
+        return ops.rmsnorm_from_sumsq(self.residual, self.sumsq, self.norm.weight, self.eps)
 
 
 @dataclass
@@ -61,9 +86,9 @@ def _fusable(rows: int, k: int, row_stride: int, weight: torch.Tensor) -> bool:
     return weight.dtype == torch.bfloat16 and rows >= 1 and k % 8 == 0 and row_stride % 8 == 0
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None, epilogue: Optional[str] = None,
-           into: Optional[torch.Tensor] = None) -> Union[torch.Tensor, RowSumsq, PartialSum]:
+           into: Optional[torch.Tensor] = None, then_norm: Any = None) -> Union[torch.Tensor, RowSumsq, PartialSum]:
     """``x @ weight.T + bias``.
 
     ``epilogue="silu"``: weight stacks gate rows over up rows; returns
@@ -71,7 +96,18 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     the float32 residual stream; if a fused kernel runs, either it adds it in
     place and a :class:`RowSumsq` comes back, or a :class:`PartialSum` of partial
     products comes back that the next norm kernel adds; otherwise the plain
-    result comes back and the caller adds it (the next norm kernel does)."""
+    result comes back and the caller adds it (the next norm kernel does).
+    ``then_norm`` (with ``into``): the norm that follows, if it can be folded into
+    this product and the next (``RMSNorm.folds_into_products``): the residual
+    epilogue then also leaves that norm's output short of the rows' scale.
+    ``x`` may be such rows (:class:`ScaledRows`): the SiLU product of few rows
+    applies the scale itself, any other reader gets the completed rows."""
+    if isinstance(x, ScaledRows):
+        rows, k = x.rows.shape
+        if (epilogue == "silu" and rows <= FUSED_ROWS and weight.shape[0] % 2 == 0
+                and _fusable(rows, k, x.rows.stride(0) if rows > 1 else k, weight)):
+            return ops.gemm_fused(weight, ops.EPI_SILU, x.rows, row_sumsq=x.sumsq, eps=x.eps)
+        x = x.complete()
     rows, k = x.shape
     n = weight.shape[0]
     silu = epilogue == "silu"
@@ -87,6 +123,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     small = rows <= FUSED_SMALL_ROWS and n * k <= FUSED_SMALL_WEIGHT and not silu
     if fusable and (rows <= FUSED_ROWS or wants_f32 or small):
         if into is not None:
+            if then_norm is not None and rows <= FUSED_ROWS:
+                scaled = torch.empty((rows, n), dtype=torch.bfloat16, device=x.device)
+                sumsq = ops.gemm_fused(weight, ops.EPI_RESID, x, bias=bias, residual_out=into,
+                                       norm_weight=then_norm.weight_f32, scaled_out=scaled)
+                return RowSumsq(sumsq, scaled, then_norm)
             return RowSumsq(ops.gemm_fused(weight, ops.EPI_RESID, x, bias=bias, residual_out=into))
         elif silu and n % 2 == 0:
             return ops.gemm_fused(weight, ops.EPI_SILU, x)

@@ -15,12 +15,15 @@ import torch
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, register_part
-from .linear import PartialSum, RowSumsq
+from .linear import PartialSum, RowSumsq, ScaledRows
 
 
 class RMSNorm(Part):
     graph_safe = True
     takes_row_sumsq = True
+    # between a product that adds into the residual and a product that reads the norm's output, the norm can
+    # ride along: the first writes residual * weight, the second applies the rows' 1 / rms to its sums
+    folds_into_products = True
     def __init__(self, size: int, eps: float) -> None:
         if size <= 0 or not eps > 0:
             raise ValueError(f"RMSNorm needs a positive size and eps, got {size}, {eps}")
@@ -34,6 +37,7 @@ class RMSNorm(Part):
     def bind(self, tensors, prefix, dtype, device) -> None:
         super().bind(tensors, prefix, dtype, device)
         self.weight = tensors[prefix + "weight"].contiguous()
+        self.weight_f32 = self.weight.float().contiguous()
 
     def forward(self, residual: torch.Tensor, branch, out_dtype: torch.dtype,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -44,6 +48,8 @@ class RMSNorm(Part):
         if isinstance(branch, PartialSum):
             return ops.add_parts_rmsnorm(residual, branch.parts, self.weight, self.eps, rows=rows)
         if isinstance(branch, RowSumsq):
+            if branch.scaled is not None and branch.norm is self and rows is None and out_dtype == torch.bfloat16:
+                return ScaledRows(branch.scaled, branch.sumsq, self.eps, residual, self)
             if rows is None and out_dtype == torch.bfloat16:
                 return ops.rmsnorm_from_sumsq(residual, branch.sumsq, self.weight, self.eps)
             branch = None

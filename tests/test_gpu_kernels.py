@@ -624,6 +624,39 @@ def test_gemm_fused_partial_products_and_their_norm(ops, shape, k_parts):
     torch.testing.assert_close(out.float().cpu(), want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("shape", [(1, 128, 64), (8, 2048, 2048), (13, 200, 328), (16, 96, 1032)])
+def test_norm_folded_into_the_products_around_it(ops, shape):
+    """o_proj adds into the residual and leaves residual * weight; the gate/up product
+    applies each row's 1 / rms to its sums: together the same as the residual product,
+    the norm kernel and the plain gate/up product."""
+    m, hidden, k = shape
+    inter = 2 * 88
+    a = rand((m, k), torch.bfloat16, 700)
+    w_o, b_o = rand((hidden, k), torch.bfloat16, 701, 0.3), rand((hidden,), torch.bfloat16, 702)
+    w_gu = rand((inter, hidden), torch.bfloat16, 703, 0.3)
+    norm_weight = (rand((hidden,), torch.float32, 704) + 1).to(torch.bfloat16)
+    eps = 1e-5
+    residual = rand((m, hidden), torch.float32, 705, 2.0)
+    apart = residual.clone()
+    sumsq = ops.gemm_fused(w_o, ops.EPI_RESID, a, bias=b_o, residual_out=apart)
+    normed = ops.rmsnorm_from_sumsq(apart, sumsq, norm_weight, eps)
+    want = ops.gemm_fused(w_gu, ops.EPI_SILU, normed)
+    scaled = torch.empty((m, hidden), dtype=torch.bfloat16).cuda()
+    folded_sumsq = ops.gemm_fused(w_o, ops.EPI_RESID, a, bias=b_o, residual_out=residual,
+                                  norm_weight=norm_weight.float().contiguous(), scaled_out=scaled)
+    assert torch.equal(residual, apart) and torch.equal(folded_sumsq, sumsq)
+    got = ops.gemm_fused(w_gu, ops.EPI_SILU, scaled, row_sumsq=folded_sumsq, eps=eps)
+    # the same values rounded to bf16 at another point (before instead of after the division by the rms)
+    exact = torch.nn.functional.silu(
+        plain_qwen2.rms_norm(residual.cpu(), norm_weight.float().cpu(), eps).double() @ w_gu.double().cpu().t()[:, : inter // 2]
+    ) * (plain_qwen2.rms_norm(residual.cpu(), norm_weight.float().cpu(), eps).double() @ w_gu.double().cpu().t()[:, inter // 2:])
+    bound = 1e-2 * float(exact.abs().max())
+    torch.testing.assert_close(got.double().cpu(), exact, rtol=2e-2, atol=bound)
+    torch.testing.assert_close(want.double().cpu(), exact, rtol=2e-2, atol=bound)
+    with pytest.raises(ValueError, match="scale"):
+        ops.gemm_fused(w_gu, ops.EPI_BF16, scaled, row_sumsq=folded_sumsq, eps=eps)
+
+
 @pytest.mark.parametrize("norm_dtype", [torch.bfloat16, torch.float32])
 def test_rmsnorm_from_sumsq(ops, norm_dtype):
     residual = rand((5, 1000), torch.float32, 90, 2.0)
