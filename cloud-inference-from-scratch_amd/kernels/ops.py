@@ -220,8 +220,12 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
         _i(q_heads), _i(kv_heads), _i(head_dim), _i(page_size), _i(1 if rotate else 0), _i(1 if write_kv else 0)))
 
 
-def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for gate_up [T, 2I]."""
+def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None, row_sumsq: Optional[torch.Tensor] = None,
+             hidden: int = 0, eps: float = 0.0) -> torch.Tensor:
+    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for gate_up [T, 2I].  With ``row_sumsq``
+    [T, parts] (partial sums of squares of rows of ``hidden`` values) both halves of
+    row t are first multiplied by ``rsqrt(sum(row_sumsq[t]) / hidden + eps)``: the
+    1/rms that the rows of the product behind ``gate_up`` lacked."""
     _gpu("gate_up", gate_up, dims=2)
     tokens, twice = gate_up.shape
     if not (twice % 2 == 0):
@@ -232,8 +236,15 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     _gpu("out", out, gate_up.dtype, 2)
     if not (out.shape == (tokens, inter)):
         raise ValueError(f"out must be {(tokens, inter)}, is {tuple(out.shape)}")
+    parts = 0
+    if row_sumsq is not None:
+        _gpu("row_sumsq", row_sumsq, torch.float32, 2)
+        if not (row_sumsq.shape[0] >= tokens and hidden > 0 and eps > 0):
+            raise ValueError("row_sumsq needs a row per token, the rows' width and a positive eps")
+        parts = row_sumsq.shape[1]
     _run("cie_silu_mul", load_library().cie_silu_mul(_stream(), _i(_code(gate_up.dtype)), _ptr(gate_up),
-                                                     _ptr(out), _i(tokens), _i(inter)))
+                                                     _ptr(out), _i(tokens), _i(inter), _ptr(row_sumsq), _i(parts),
+                                                     _i(hidden), _f(eps)))
     return out
 
 

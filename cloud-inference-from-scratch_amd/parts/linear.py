@@ -104,9 +104,13 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     applies the scale itself, any other reader gets the completed rows."""
     if isinstance(x, ScaledRows):
         rows, k = x.rows.shape
-        if (epilogue == "silu" and rows <= FUSED_ROWS and weight.shape[0] % 2 == 0
-                and _fusable(rows, k, x.rows.stride(0) if rows > 1 else k, weight)):
-            return ops.gemm_fused(weight, ops.EPI_SILU, x.rows, row_sumsq=x.sumsq, eps=x.eps)
+        if epilogue == "silu" and weight.shape[0] % 2 == 0 and bias is None and weight.dtype == torch.bfloat16:
+            if rows <= FUSED_ROWS and _fusable(rows, k, x.rows.stride(0) if rows > 1 else k, weight):
+                return ops.gemm_fused(weight, ops.EPI_SILU, x.rows, row_sumsq=x.sumsq, eps=x.eps)
+            # more rows: the library's product of the rows as they are, the scale in the SiLU kernel behind it
+            out = ops.gemm_library(x.rows, weight) if x.rows.stride(1) == 1 else None
+            if out is not None:
+                return ops.silu_mul(out, row_sumsq=x.sumsq, hidden=k, eps=x.eps)
         x = x.complete()
     rows, k = x.shape
     n = weight.shape[0]
@@ -123,7 +127,7 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     small = rows <= FUSED_SMALL_ROWS and n * k <= FUSED_SMALL_WEIGHT and not silu
     if fusable and (rows <= FUSED_ROWS or wants_f32 or small):
         if into is not None:
-            if then_norm is not None and rows <= FUSED_ROWS:
+            if then_norm is not None:
                 scaled = torch.empty((rows, n), dtype=torch.bfloat16, device=x.device)
                 sumsq = ops.gemm_fused(weight, ops.EPI_RESID, x, bias=bias, residual_out=into,
                                        norm_weight=then_norm.weight_f32, scaled_out=scaled)

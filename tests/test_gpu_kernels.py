@@ -624,6 +624,24 @@ def test_gemm_fused_partial_products_and_their_norm(ops, shape, k_parts):
     torch.testing.assert_close(out.float().cpu(), want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 8), (5, 200), (40, 4864), (3, 25)])
+def test_silu_mul_with_the_rows_scale(ops, dtype, shape):
+    """The SiLU-gate kernel applying the 1/rms that the rows of the product before it lacked."""
+    tokens, inter = shape
+    hidden, parts, eps = 96, 7, 1e-5
+    gate_up = rand((tokens, 2 * inter), dtype, 710, 3.0)
+    sumsq = rand((tokens, parts), torch.float32, 711).abs() * 40 + 1
+    factor = torch.rsqrt(sumsq.double().sum(-1, keepdim=True) / hidden + eps)
+    g, u = gate_up.double()[:, :inter] * factor, gate_up.double()[:, inter:] * factor
+    want = torch.nn.functional.silu(g) * u
+    got = ops.silu_mul(gate_up, row_sumsq=sumsq, hidden=hidden, eps=eps)
+    torch.testing.assert_close(got.double(), want, **({"rtol": 1e-2, "atol": 1e-3} if dtype == torch.bfloat16 else {"rtol": 1e-5, "atol": 1e-6}))
+    plain = torch.nn.functional.silu(gate_up.double()[:, :inter]) * gate_up.double()[:, inter:]
+    torch.testing.assert_close(ops.silu_mul(gate_up).double(), plain,
+                               **({"rtol": 1e-2, "atol": 1e-3} if dtype == torch.bfloat16 else {"rtol": 1e-5, "atol": 1e-6}))
+
+
 @pytest.mark.parametrize("shape", [(1, 128, 64), (8, 2048, 2048), (13, 200, 328), (16, 96, 1032)])
 def test_norm_folded_into_the_products_around_it(ops, shape):
     """o_proj adds into the residual and leaves residual * weight; the gate/up product
