@@ -110,6 +110,7 @@ class Attention(Part):
 
 
 WIDE_DECODE_KEYS = 2048  # contexts from which decode rows go to the four-wave form
+PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's keys are cut
 
 
 def plan_splits(units: int, max_keys: int, target_waves: int = 1024, min_keys: int = 128) -> tuple[int, int]:
@@ -177,12 +178,16 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
                                  n_tiles, *common, tokens_per_tile=1, row_tiles=1, n_splits=n_splits,
                                  keys_per_split=per_split, part_o=part_o, part_ml=part_ml, tile_waves=decode_waves)
     prompt_tokens = sum(n for n in batch.host_q_lens if n > 1)
+    cuts = 1
     if wide:
         # the prompt form: four waves share a tile's keys.  More rows per tile re-use each key more often,
-        # fewer tiles leave compute units idle: the most rows that still give most units a workgroup
+        # fewer tiles leave compute units idle: the most rows that still give most units a workgroup, where a
+        # short portion behind a long context also has its keys cut (256 tokens behind 3,840 keys, 2 kv heads:
+        # 34 us with 64 rows per tile and four parts, 48 us with 16 rows per tile and the keys whole)
         tile_waves = ops.TILE_WAVES
         row_tiles = 4 if head_dim <= 128 else 1
-        while row_tiles > 1 and -(-prompt_tokens * group // (16 * row_tiles)) * num_kv_heads < 192:
+        cuts = max(1, max_keys // PROMPT_SPLIT_KEYS) if window is None else 1  # (a window's keys stay whole)
+        while row_tiles > 1 and -(-prompt_tokens * group // (16 * row_tiles)) * num_kv_heads * cuts < 192:
             row_tiles //= 2
     else:
         # one wave per tile; fewer rows where that would leave SIMDs without a wave (about a thousand
@@ -196,8 +201,19 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     per_tile = (16 * row_tiles) // group
     tile_seq, tile_q0, n_tiles = batch.tiles(per_tile, decode=False)
     if n_tiles:
+        # few tiles and many keys: parts of the keys, about as many workgroups as compute units
+        n_splits, per_split, part_o, part_ml = 1, 0, None, None
+        wanted = min(cuts, int(256 / (n_tiles * num_kv_heads) + 0.5))
+        if wanted > 1:
+            per_split = -(-(-(-max_keys // wanted)) // 128) * 128
+            n_splits = -(-max_keys // per_split)
+        if n_splits > 1:
+            part_o, part_ml = _workspaces(qkv.device, n_tiles * num_kv_heads * n_splits, 16 * row_tiles, head_dim)
+        else:
+            per_split = 0
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
                                  n_tiles, *common, tokens_per_tile=per_tile, row_tiles=row_tiles,
+                                 n_splits=n_splits, keys_per_split=per_split, part_o=part_o, part_ml=part_ml,
                                  tile_waves=tile_waves)
     return out
 

@@ -297,6 +297,33 @@ def test_paged_attention_mfma_decode_splits(ops, geometry, splits, tile_waves):
             torch.testing.assert_close(out, torch.cat(expected), **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("geometry", [(16, 2, 128, 16), (6, 2, 32, 16), (5, 5, 64, 32)])
+@pytest.mark.parametrize("row_tiles", [1, 2, 4])
+@pytest.mark.parametrize("splits", [(3, 512), (5, 256), (9, 128)])
+def test_paged_attention_mfma_prompt_portions_with_their_keys_cut(ops, geometry, row_tiles, splits):
+    """Portions of prompts behind long contexts, tiles of 16 to 64 rows whose keys are cut into
+    parts (some of them empty for the shorter sequences, some ending inside the portion)."""
+    q_heads, kv_heads, head_dim, page_size = geometry
+    group = q_heads // kv_heads
+    if group > 16 * row_tiles:
+        pytest.skip("the group does not fit the tile")
+    n_splits, per_split = splits
+    contexts, q_lens = [1000, 0, 300, 37], [40, 70, 9, 33]
+    lengths = [c + n for c, n in zip(contexts, q_lens)]
+    k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=82)
+    scale = 1.0 / math.sqrt(head_dim)
+    g = torch.Generator().manual_seed(83)
+    qs, expected = [], []
+    for s, (c, n) in enumerate(zip(contexts, q_lens)):
+        q = (torch.randn((n, q_heads, head_dim), generator=g) * 2).to(torch.bfloat16).float()
+        qs.append(q.reshape(n, -1))
+        expected.append(plain_qwen2.causal_attention(q, *dense[s], scale, past_len=c))
+    per_tile = (16 * row_tiles) // group
+    out = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
+                   None, scale, per_tile, row_tiles, n_splits=n_splits, keys_per_split=per_split, tile_waves=4)
+    torch.testing.assert_close(out, torch.cat(expected), **tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("window", [5, 32, 100])
 def test_paged_attention_mfma_window(ops, window):
     q_heads, kv_heads, head_dim = 4, 2, 64

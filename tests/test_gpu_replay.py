@@ -351,3 +351,42 @@ def test_replay_at_the_sizes_of_real_models(tmp_path_factory, shape, layers, voc
               f"worst {worst:.3e} ({plain_worst:.3e})", flush=True)
         assert rms <= plain_rms and worst <= 1.5 * plain_worst
     assert runner.cache.stats().pages_used == 0
+
+
+def test_replay_with_the_keys_of_prompt_portions_cut(tiny_folders, monkeypatch):
+    """A short portion behind a long context has few tiles and many keys: its keys are cut
+    into parts that a second kernel joins (Tiny-B, the limit lowered so that 300 positions reach it)."""
+    from cie_amd.kernels import ops
+    from cie_amd.parts import attention
+
+    monkeypatch.setattr(attention, "PROMPT_SPLIT_KEYS", 64)
+    seen = []
+    real = ops.paged_attention_mfma
+
+    def spy(*args, **kwargs):
+        seen.append((kwargs.get("tokens_per_tile", 1), kwargs.get("n_splits", 1)))
+        return real(*args, **kwargs)
+
+    monkeypatch.setattr(ops, "paged_attention_mfma", spy)
+    folder, raw, tensors = tiny_folders["B"]
+    requests = {"r": random_tokens(300, raw["vocab_size"], seed=77), "s": random_tokens(150, raw["vocab_size"], seed=78)}
+    expected = plain_all(raw, tensors, requests)
+    steps, fed = [], {"r": 0, "s": 0}
+
+    def step(parts, end=()):
+        entries = []
+        for rid, size in parts:
+            tokens = requests[rid][fed[rid]: fed[rid] + size]
+            fed[rid] += size
+            entries.append({"id": rid, "tokens": tokens, "want": list(range(len(tokens)))})
+        steps.append({"step": len(steps), "entries": entries, "end": list(end)})
+
+    step([("r", 200)])
+    step([("r", 60), ("s", 120)])     # portions of two requests with different contexts in one step
+    step([("r", 38), ("s", 1)])       # beside a single token
+    step([("r", 2), ("s", 29)], end=["r", "s"])
+    runner = make_runner(folder, "bfloat16", replay_util.max_live_tokens(steps, page=16), 16)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    replay_util.compare(rows, expected, **TOL["bfloat16"])
+    assert any(per_tile > 1 and splits > 1 for per_tile, splits in seen), seen
+    assert runner.cache.stats().pages_used == 0
