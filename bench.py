@@ -166,7 +166,7 @@ def main(argv=None) -> int:
     value = args.batch * args.steps / elapsed
     achieved = decode_bytes(config, args.layers, args.batch, mean_context, elem) / (elapsed / args.steps) / 1e9
     line = {
-        "metric": "decode tokens/s, Qwen2.5-3B shape, batch 8, context to 4096",
+        "metric": f"decode tokens/s, Qwen2.5-3B shape, batch {args.batch}, context to {args.context}",
         "value": round(value, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
