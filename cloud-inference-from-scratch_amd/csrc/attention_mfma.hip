@@ -623,6 +623,16 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
     const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
     if (row >= n_tok * group) return;
     const size_t unit0 = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits;
+    // The thread's share of the first parts' sums is fetched before the weights are known: these loads
+    // depend on nothing and travel while the statistics are read and reduced (the dimension of the
+    // thread's first round and the first sixteen parts; a wider head and further parts are fetched afterwards).
+    constexpr int kEarly = 16;
+    const size_t stride = static_cast<size_t>(rows_per_tile) * head_dim;
+    const float* po_row = a.part_o + (unit0 * rows_per_tile + row) * head_dim;
+    const int d0 = threadIdx.x;
+    float early[kEarly];
+#pragma unroll
+    for (int u = 0; u < kEarly; ++u) early[u] = (u < a.n_splits && d0 < head_dim) ? po_row[u * stride + d0] : 0.f;
     float m_local = -INFINITY;
     for (int s = threadIdx.x; s < a.n_splits; s += blockDim.x)
         m_local = fmaxf(m_local, a.part_ml[((unit0 + s) * rows_per_tile + row) * 2]);
@@ -641,10 +651,15 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
                   static_cast<size_t>(kv_head * group + head) * head_dim;
     const float inv = 1.0f / den;
     for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-        const float* po = a.part_o + (unit0 * rows_per_tile + row) * head_dim + d;
-        const size_t stride = static_cast<size_t>(rows_per_tile) * head_dim;
         float num = 0.f;
-        for (int s = 0; s < a.n_splits; ++s) num += po[s * stride] * weight[s];
+        int s = 0;
+        if (d == d0) {
+#pragma unroll
+            for (int u = 0; u < kEarly; ++u)
+                if (u < a.n_splits) num += early[u] * weight[u];
+            s = min(a.n_splits, kEarly);
+        }
+        for (; s < a.n_splits; ++s) num += po_row[s * stride + d] * weight[s];
         dst[d] = from_float<bf16_t>(num * inv);
     }
 }
