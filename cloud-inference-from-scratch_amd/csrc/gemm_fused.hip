@@ -121,41 +121,48 @@ __device__ __forceinline__ void store_tile(const FusedArgs& a, const floatx4& ac
     }
 }
 
-// The RESID epilogue for the MT row tiles of one column tile: all old values of the residual are fetched
-// before the first new one is written (taken tile by tile, every load would wait behind the stores of
-// the tile before it, which the compiler must assume to alias: one round trip to memory per row).
-template <int MT>
-__device__ __forceinline__ void store_resid(const FusedArgs& a, const floatx4 (&acc)[MT], int m_base, int n, int n_tile,
-                                            int lane) {
+// The RESID epilogue for one 16 x 16 tile.  What it needs beside the product (the old values of the
+// residual, the bias, the weight of the norm that rides along) is fetched before the product starts, by
+// the wave that will store the tile, so that these loads travel while the weights stream instead of
+// standing between the product and its store.
+struct ResidRows {
+    float old[4];
+    float add, weight;
+};
+
+__device__ __forceinline__ ResidRows resid_prefetch(const FusedArgs& a, int m_base, int n, int lane) {
+    const int g = lane >> 4;
+    const bool col_ok = n < a.N;
+    ResidRows rows;
+    rows.add = (col_ok && a.bias) ? to_float(a.bias[n]) : 0.f;
+    rows.weight = (col_ok && a.scaled_out) ? a.norm_weight[n] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m_base + g * 4 + i;
+        rows.old[i] = (col_ok && m < a.M) ? a.residual[static_cast<size_t>(m) * a.N + n] : 0.f;
+    }
+    return rows;
+}
+
+__device__ __forceinline__ void store_resid(const FusedArgs& a, const floatx4& acc, const ResidRows& rows, int m_base,
+                                            int n, int n_tile, int lane) {
     const int r = lane & 15;
     const int g = lane >> 4;
     const bool col_ok = n < a.N;
-    const float add = (col_ok && a.bias) ? to_float(a.bias[n]) : 0.f;
-    float old[MT][4];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int m = m_base + mt * 16 + g * 4 + i;
-            old[mt][i] = (col_ok && m < a.M) ? a.residual[static_cast<size_t>(m) * a.N + n] : 0.f;
-        }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int m = m_base + mt * 16 + g * 4 + i;
-            const bool ok = col_ok && m < a.M;
-            const float v = ok ? old[mt][i] + acc[mt][i] + add : 0.f;
-            if (ok) a.residual[static_cast<size_t>(m) * a.N + n] = v;
-            if (ok && a.scaled_out)
-                a.scaled_out[static_cast<size_t>(m) * a.N + n] = from_float<bf16_t>(v * a.norm_weight[n]);
-            float sq = v * v;  // sum over the tile's 16 columns: the lanes that share g
-            sq += __shfl_xor(sq, 1, kWave);
-            sq += __shfl_xor(sq, 2, kWave);
-            sq += __shfl_xor(sq, 4, kWave);
-            sq += __shfl_xor(sq, 8, kWave);
-            if (r == 0 && m < a.M) a.sumsq[static_cast<size_t>(m) * ((a.N + 15) / 16) + n_tile] = sq;
-        }
+    for (int i = 0; i < 4; ++i) {
+        const int m = m_base + g * 4 + i;
+        const bool ok = col_ok && m < a.M;
+        const float v = ok ? rows.old[i] + acc[i] + rows.add : 0.f;
+        if (ok) a.residual[static_cast<size_t>(m) * a.N + n] = v;
+        if (ok && a.scaled_out) a.scaled_out[static_cast<size_t>(m) * a.N + n] = from_float<bf16_t>(v * rows.weight);
+        float sq = v * v;  // sum over the tile's 16 columns: the lanes that share g
+        sq += __shfl_xor(sq, 1, kWave);
+        sq += __shfl_xor(sq, 2, kWave);
+        sq += __shfl_xor(sq, 4, kWave);
+        sq += __shfl_xor(sq, 8, kWave);
+        if (r == 0 && m < a.M) a.sumsq[static_cast<size_t>(m) * ((a.N + 15) / 16) + n_tile] = sq;
+    }
 }
 
 // The ROPE epilogue for one pair of tiles: `lo` holds dimensions j*16 + r of head `head`, `hi` those
@@ -326,6 +333,11 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     RopeRows rope_rows;
     // (the wave that will store row tile `wave`, below)
     if (EPI == EPI_ROPE && wave < MT) rope_rows = rope_prefetch(a, rope_head, rope_tile, lane, m0 + wave * 16);
+    ResidRows resid_rows[NT];
+    if (EPI == EPI_RESID && wave < MT) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) resid_rows[t] = resid_prefetch(a, m0 + wave * 16, (tile_first + t) * 16 + r, lane);
+    }
     // Rows that still lack their 1/rms (one row tile only): the waves share the 16 rows, 4 * WAVES lanes
     // sum the partial sums of a row, and the scales meet in LDS for the wave that stores.  The loads are
     // issued behind the wave's first loads of W, so that they add nothing to its start.
@@ -455,10 +467,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
             if constexpr (EPI == EPI_RESID) {
 #pragma unroll
                 for (int t = 0; t < NT; ++t)
-                    if ((tile_first + t) * 16 < cols) {  // wave-uniform
-                        const floatx4 column[1] = {acc[mt][t]};
-                        store_resid<1>(a, column, m0 + mt * 16, (tile_first + t) * 16 + r, tile_first + t, lane);
-                    }
+                    if ((tile_first + t) * 16 < cols)  // wave-uniform
+                        store_resid(a, acc[mt][t], resid_rows[t], m0 + mt * 16, (tile_first + t) * 16 + r, tile_first + t, lane);
             } else if (EPI == EPI_ROPE) {
                 store_rope(a, acc[mt][0], acc[mt][NT - 1], rope_head, rope_tile, lane, rope_rows, m0 + mt * 16);
             } else if (EPI == EPI_SILU) {
@@ -499,15 +509,11 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
                     for (int i = 0; i < 4; ++i)
                         acc[mt][t][i] += reduce[((((w - 1) * MT + mt) * NT + t) * 4 + i) * 64 + lane];
     }
-    if constexpr (EPI == EPI_RESID) {
+    if constexpr (EPI == EPI_RESID) {  // (one row tile, or one wave: this wave fetched the tiles' old values)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
-            if ((tile_first + t) * 16 < cols) {  // wave-uniform
-                floatx4 column[MT];
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) column[mt] = acc[mt][t];
-                store_resid<MT>(a, column, m0, (tile_first + t) * 16 + r, tile_first + t, lane);
-            }
+            if ((tile_first + t) * 16 < cols)  // wave-uniform
+                store_resid(a, acc[0][t], resid_rows[t], m0, (tile_first + t) * 16 + r, tile_first + t, lane);
         return;
     }
 #pragma unroll
