@@ -177,6 +177,8 @@ struct RopeRows {
     float bias_lo, bias_hi;
 };
 
+// In two steps, because the second reads where the first points: positions and sequences of the rows
+// (and the bias) before the product starts; angles, slots and pages behind the wave's first loads of W.
 __device__ __forceinline__ RopeRows rope_prefetch(const FusedArgs& a, int head, int j, int lane, int m_base) {
     const RopeArgs& p = a.rope;
     const int r = lane & 15;
@@ -184,30 +186,44 @@ __device__ __forceinline__ RopeRows rope_prefetch(const FusedArgs& a, int head, 
     const int half = p.head_dim / 2;
     const int d = j * 16 + r;
     const bool is_query = head < p.q_heads;
-    const bool is_value = head >= p.q_heads + p.kv_heads;
     RopeRows rows;
     rows.bias_lo = a.bias ? to_float(a.bias[head * p.head_dim + d]) : 0.f;
     rows.bias_hi = a.bias ? to_float(a.bias[head * p.head_dim + d + half]) : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int m = m_base + g * 4 + i;
-        rows.pos[i] = 0;
-        rows.page[i] = -1;
+        rows.pos[i] = -1;   // no such row
+        rows.page[i] = -1;  // until the second step: the row's sequence, if its key or value is to be written
         rows.c[i] = 1.f;
         rows.s[i] = 0.f;
         if (m >= a.M) continue;
-        const int pos = p.positions[m];
-        rows.pos[i] = pos;
-        if (!is_value && p.rotate) {
+        rows.pos[i] = p.positions[m];
+        if (!is_query && p.write_kv) rows.page[i] = p.seq_of_token[m];
+    }
+    return rows;
+}
+
+__device__ __forceinline__ void rope_prefetch_rest(const FusedArgs& a, int head, int j, int lane, RopeRows& rows) {
+    const RopeArgs& p = a.rope;
+    const int half = p.head_dim / 2;
+    const int d = j * 16 + (lane & 15);
+    const bool is_value = head >= p.q_heads + p.kv_heads;
+    int slot[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int pos = rows.pos[i];
+        if (pos >= 0 && !is_value && p.rotate) {
             rows.c[i] = p.cos_table[static_cast<size_t>(pos) * half + d];
             rows.s[i] = p.sin_table[static_cast<size_t>(pos) * half + d];
         }
-        if (!is_query && p.write_kv) {
-            const int slot = p.seq_slot[p.seq_of_token[m]];
-            rows.page[i] = p.block_table[static_cast<size_t>(slot) * p.table_width + pos / p.page_size];
-        }
+        slot[i] = rows.page[i] >= 0 ? p.seq_slot[rows.page[i]] : -1;
     }
-    return rows;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (slot[i] >= 0)
+            rows.page[i] = p.block_table[static_cast<size_t>(slot[i]) * p.table_width + rows.pos[i] / p.page_size];
+        if (rows.pos[i] < 0) rows.pos[i] = 0;
+    }
 }
 
 __device__ __forceinline__ void store_rope(const FusedArgs& a, const floatx4& lo, const floatx4& hi, int head,
@@ -332,7 +348,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         for (int t = 0; t < NT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
     RopeRows rope_rows;
     // (the wave that will store row tile `wave`, below)
-    if (EPI == EPI_ROPE && wave < MT) rope_rows = rope_prefetch(a, rope_head, rope_tile, lane, m0 + wave * 16);
+    bool rope_pending = EPI == EPI_ROPE && wave < MT;
+    if (rope_pending) rope_rows = rope_prefetch(a, rope_head, rope_tile, lane, m0 + wave * 16);
     ResidRows resid_rows[NT];
     if (EPI == EPI_RESID && wave < MT) {
 #pragma unroll
@@ -381,6 +398,10 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
             sum_row_parts();
             scale_pending = false;
         }
+        if (rope_pending) {  // likewise
+            rope_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
+            rope_pending = false;
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             // the few rows of A come from the cache; their loads are issued slice by slice
@@ -424,8 +445,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         }
     }
 
+    if (rope_pending) rope_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);  // (a K so short that this wave had no slice)
     if (scaled_rows) {
-        if (scale_pending) sum_row_parts();  // (a K so short that this wave had no slice)
+        if (scale_pending) sum_row_parts();  // (likewise)
 #pragma unroll
         for (int offset = kScaleLanes / 2; offset > 0; offset >>= 1) sq_part += __shfl_xor(sq_part, offset, kWave);
         if (lane % kScaleLanes == 0) scale_lds[scale_row] = 1.0f / sqrtf(sq_part / static_cast<float>(a.K) + a.eps);
