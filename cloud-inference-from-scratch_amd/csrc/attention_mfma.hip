@@ -76,8 +76,8 @@ __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs 
     const int kv_head = blockIdx.y;
     const int split = blockIdx.z;
     const int group = a.q_heads / a.kv_heads;
-    const int seq = a.tile_seq[tile];
-    const int q0 = a.tile_q0[tile];
+    const int seq = a.tile_seq ? a.tile_seq[tile] : tile;  // (no lists: tile i is the first tile of sequence i)
+    const int q0 = a.tile_seq ? a.tile_q0[tile] : 0;
     const int start = a.seq_start[seq];
     const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
     const int n_rows = n_tok * group;
@@ -318,8 +318,8 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
     if (tile_index >= a.n_tiles) return;  // padding of the grid; the whole workgroup leaves
     const int tile = a.n_tiles - 1 - tile_index;
     const int group = a.q_heads / a.kv_heads;
-    const int seq = a.tile_seq[tile];
-    const int q0 = a.tile_q0[tile];
+    const int seq = a.tile_seq ? a.tile_seq[tile] : tile;  // (no lists: tile i is the first tile of sequence i)
+    const int q0 = a.tile_seq ? a.tile_q0[tile] : 0;
     const int start = a.seq_start[seq];
     const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
     const int n_rows = n_tok * group;
@@ -618,8 +618,8 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
     const int kv_head = blockIdx.y;
     const int row = blockIdx.z;
     const int group = a.q_heads / a.kv_heads;
-    const int seq = a.tile_seq[tile];
-    const int q0 = a.tile_q0[tile];
+    const int seq = a.tile_seq ? a.tile_seq[tile] : tile;  // (no lists: tile i is the first tile of sequence i)
+    const int q0 = a.tile_seq ? a.tile_q0[tile] : 0;
     const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
     if (row >= n_tok * group) return;
     const size_t unit0 = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits;

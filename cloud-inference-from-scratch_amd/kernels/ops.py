@@ -292,7 +292,8 @@ TILE_WAVES = 4  # waves per workgroup of the prompt form of the matrix-core atte
 
 
 def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
-                         block_table: torch.Tensor, tile_seq: torch.Tensor, tile_q0: torch.Tensor, n_tiles: int,
+                         block_table: torch.Tensor, tile_seq: Optional[torch.Tensor], tile_q0: Optional[torch.Tensor],
+                         n_tiles: int,
                          seq_slot: torch.Tensor, seq_start: torch.Tensor, seq_q_len: torch.Tensor,
                          q_start_loc: torch.Tensor, out: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int,
                          window: Optional[int], scale: float, tokens_per_tile: int, row_tiles: int,
@@ -302,7 +303,8 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
                          tile_waves: int = 1) -> None:
     """Matrix-core attention (bf16) for the tiles ``(tile_seq[i], tile_q0[i])``: tile i
     holds up to ``tokens_per_tile`` tokens of sequence ``tile_seq[i]`` from its
-    ``tile_q0[i]``-th token of this step on.  Rows of other tokens of ``out`` are left alone.
+    ``tile_q0[i]``-th token of this step on (both ``None``: tile i starts sequence i, as in
+    a step of single tokens; one dependent load less).  Rows of other tokens of ``out`` are left alone.
     With ``n_splits > 1`` every tile's keys are cut into parts of ``keys_per_split``
     (a multiple of 32; or, with ``max_context_dev``, derived on the device from the
     step's longest context) and merged through the workspaces.  ``tile_waves=4`` gives
@@ -325,10 +327,16 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
     if not (page_size >= 4 and page_size & (page_size - 1) == 0):
         raise ValueError(f"page size must be a power of two >= 4, is {page_size}")
     _gpu("block_table", block_table, torch.int32, 2)
+    if (tile_seq is None) != (tile_q0 is None):
+        raise ValueError("tile_seq and tile_q0 come together, or neither (tile i is then the first tile of sequence i)")
     for name, meta in (("tile_seq", tile_seq), ("tile_q0", tile_q0)):
+        if meta is None:
+            continue
         _gpu(name, meta, torch.int32, 1)
         if not (meta.shape[0] >= n_tiles):
             raise ValueError(f"{name} has {meta.shape[0]} entries for {n_tiles} tiles")
+    if tile_seq is None and seq_q_len.shape[0] < n_tiles:
+        raise ValueError(f"{n_tiles} tiles for {seq_q_len.shape[0]} sequences")
     for name, meta in (("seq_slot", seq_slot), ("seq_start", seq_start), ("seq_q_len", seq_q_len),
                        ("q_start_loc", q_start_loc)):
         _gpu(name, meta, torch.int32, 1)

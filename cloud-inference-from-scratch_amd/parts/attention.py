@@ -167,8 +167,9 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         part_o = part_ml = None
         if n_splits > 1:
             part_o, part_ml = _workspaces(qkv.device, batch.sequences * num_kv_heads * n_splits, 16, head_dim)
-        ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, plan.tile_seq,
-                                 plan.tile_q0, batch.sequences, *common, tokens_per_tile=1, row_tiles=1,
+        # (every sequence brings one token: tile i is sequence i, no tile lists)
+        ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, None,
+                                 None, batch.sequences, *common, tokens_per_tile=1, row_tiles=1,
                                  n_splits=n_splits, max_context_dev=plan.max_context, part_o=part_o, part_ml=part_ml,
                                  tile_waves=decode_waves)
         return out
