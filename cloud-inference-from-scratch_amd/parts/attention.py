@@ -110,6 +110,7 @@ class Attention(Part):
 
 
 WIDE_DECODE_KEYS = 2048  # contexts from which decode rows go to the four-wave form
+SHARED_DECODE_KEYS = 96  # contexts from which four waves share a decode row's keys without cutting them
 SPLIT_DECODE_KEYS = 192  # contexts from which the keys of decode rows are cut into parts at all
 PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's keys are cut
 
@@ -156,8 +157,12 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         if waves > 1:
             return waves, dict(target_waves=1024 // waves, min_keys=32 * waves)
         # one wave per part: parts down to one block of 32 keys (8 x 256 keys: 7.3 us in 8 parts, 10.2 us in 2;
-        # 8 x 512 keys: 8.1 us in 16 parts, 10.6 us in 4); below some 200 keys the merge costs more than it saves
-        return waves, dict(target_waves=1024, min_keys=32 if bound >= SPLIT_DECODE_KEYS else bound + 1)
+        # 8 x 512 keys: 8.1 us in 16 parts, 10.6 us in 4); below some 200 keys the merge costs more than it
+        # saves, and four waves that share a sequence's few blocks inside one workgroup do better than one
+        # wave that takes them in turn (8 x 128 keys: 6.5 against 6.9 us, 8 x 160: 7 against 11)
+        if bound >= SPLIT_DECODE_KEYS:
+            return 1, dict(target_waves=1024, min_keys=32)
+        return (ops.TILE_WAVES if wide and bound >= SHARED_DECODE_KEYS else 1), dict(target_waves=1024, min_keys=bound + 1)
 
     if batch.static_plan is not None:  # a captured decode step: the grid is fixed, lengths live on the device
         plan = batch.static_plan
