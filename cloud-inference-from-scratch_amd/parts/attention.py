@@ -110,6 +110,7 @@ class Attention(Part):
 
 
 WIDE_DECODE_KEYS = 2048  # contexts from which decode rows go to the four-wave form
+MANY_DECODE_UNITS = 96  # (sequence, kv head) pairs from which decode rows take the four-wave form at any context
 SHARED_DECODE_KEYS = 96  # contexts from which four waves share a decode row's keys without cutting them
 SPLIT_DECODE_KEYS = 192  # contexts from which the keys of decode rows are cut into parts at all
 PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's keys are cut
@@ -149,25 +150,29 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     max_keys = batch.max_context if window is None else min(batch.max_context, window + 64)
     wide = page_size >= 16 and scale > 0
 
-    def decode_form(bound: int) -> tuple[int, dict]:
-        # Decode rows.  Long contexts: four waves per (sequence, kv head, part of the keys) take the part's
-        # blocks in turn with their loads running ahead (15.8 against 18.1 us for 8 x 4,096 keys); short
-        # ones: one wave per part (9.1 against 10.9 us for 8 x 1,024 keys).
-        waves = ops.TILE_WAVES if wide and bound >= WIDE_DECODE_KEYS else 1
-        if waves > 1:
-            return waves, dict(target_waves=1024 // waves, min_keys=32 * waves)
-        # one wave per part: parts down to one block of 32 keys (8 x 256 keys: 7.3 us in 8 parts, 10.2 us in 2;
-        # 8 x 512 keys: 8.1 us in 16 parts, 10.6 us in 4); below some 200 keys the merge costs more than it
-        # saves, and four waves that share a sequence's few blocks inside one workgroup do better than one
-        # wave that takes them in turn (8 x 128 keys: 6.5 against 6.9 us, 8 x 160: 7 against 11)
+    def decode_form(bound: int, units: int) -> tuple[int, dict]:
+        # Decode rows, `units` (sequence, kv head) pairs over up to `bound` keys.  Long contexts: four waves
+        # per (sequence, kv head, part of the keys) take the part's blocks in turn with their loads running
+        # ahead (15.8 against 18.1 us for 8 x 4,096 keys).
+        if wide and bound >= WIDE_DECODE_KEYS:
+            return ops.TILE_WAVES, dict(target_waves=1024 // ops.TILE_WAVES, min_keys=32 * ops.TILE_WAVES)
+        # Many pairs fill the GPU by themselves: the same form with the keys whole or in large parts
+        # (64 sequences x 2 heads x 256 keys: 9.2 us against 11.1 us with one wave per part)
+        if wide and units >= MANY_DECODE_UNITS and bound >= SHARED_DECODE_KEYS:
+            return ops.TILE_WAVES, dict(target_waves=1024 // ops.TILE_WAVES, min_keys=512)
+        # Otherwise one wave per part, parts down to one block of 32 keys (8 x 256 keys: 7.3 us in 8 parts,
+        # 10.2 us in 2; 8 x 512 keys: 8.1 us in 16 parts, 10.6 us in 4) ...
         if bound >= SPLIT_DECODE_KEYS:
             return 1, dict(target_waves=1024, min_keys=32)
+        # ... and below some 200 keys, where the merge costs more than it saves, four waves that share a
+        # sequence's few blocks inside one workgroup instead of one wave that takes them in turn
+        # (8 x 128 keys: 6.5 against 6.9 us, 8 x 160: 7 against 11)
         return (ops.TILE_WAVES if wide and bound >= SHARED_DECODE_KEYS else 1), dict(target_waves=1024, min_keys=bound + 1)
 
     if batch.static_plan is not None:  # a captured decode step: the grid is fixed, lengths live on the device
         plan = batch.static_plan
         bound = plan.max_keys if window is None else min(plan.max_keys, window + 64)
-        decode_waves, split_options = decode_form(bound)
+        decode_waves, split_options = decode_form(bound, batch.sequences * num_kv_heads)
         n_splits, _ = plan_splits(batch.sequences * num_kv_heads, bound, **split_options)
         part_o = part_ml = None
         if n_splits > 1:
@@ -180,7 +185,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         return out
     tile_seq, tile_q0, n_tiles = batch.tiles(1, decode=True)
     if n_tiles:
-        decode_waves, split_options = decode_form(max_keys)
+        decode_waves, split_options = decode_form(max_keys, n_tiles * num_kv_heads)
         n_splits, per_split = plan_splits(n_tiles * num_kv_heads, max_keys, **split_options)
         part_o = part_ml = None
         if n_splits > 1:
