@@ -18,7 +18,7 @@ from __future__ import annotations
 import json
 import random
 import time
-from dataclasses import dataclass, field
+from dataclasses import dataclass, field, replace
 from typing import Any
 
 # Model shapes of the Qwen2.5 family (their config.json values); weights are random.
@@ -180,11 +180,17 @@ def main(argv: list[str] | None = None) -> int:
     parser.add_argument("--shape", choices=sorted(SHAPES), default=None, help="another model shape than the profile's")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--requests", type=int, default=None, help="another number of requests than the profile's")
     parser.add_argument("--verify", type=int, default=0, metavar="N",
                         help="afterwards run the first N requests alone and compare their tokens "
                              "(float32: must be equal; bfloat16: reported)")
     args = parser.parse_args(argv)
-    record = run_profile(PROFILES[args.name], layers=args.layers, dtype=args.dtype, seed=args.seed, shape=args.shape,
+    profile = PROFILES[args.name]
+    if args.requests is not None:
+        if args.requests < 1:
+            parser.error("--requests must be positive")
+        profile = replace(profile, requests=args.requests, lead_requests=min(profile.lead_requests, args.requests))
+    record = run_profile(profile, layers=args.layers, dtype=args.dtype, seed=args.seed, shape=args.shape,
                          verify=args.verify)
     print(json.dumps(record))
     return 0
