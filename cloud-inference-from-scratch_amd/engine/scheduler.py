@@ -372,13 +372,6 @@ class Scheduler:
         return True
 
     # -- internals -----------------------------------------------------------------
-    def _room_for(self, request: Request) -> bool:
-        free_tokens = getattr(self.runner, "free_tokens", None)
-        if free_tokens is None:
-            return False
-        known = len(request.prompt_token_ids) + request.generated_count
-        return free_tokens() >= known + 1
-
     def _room_beside_admitted(self, request: Request) -> bool:
         """Whether the pool holds what is known of ``request`` beside what is known
         of the admitted requests (the part of it that they have not taken yet)."""
@@ -397,8 +390,11 @@ class Scheduler:
         progressed = False
         while self.waiting and len(self.active) < self.config.max_running:
             candidate = self.waiting[0]
-            if candidate.preemption_count and self.active and not self._room_for(candidate):
-                break  # wait for room instead of thrashing; keeps its place at the head
+            if candidate.preemption_count and self.active and not self._room_beside_admitted(candidate):
+                # wait for room instead of thrashing; keeps its place at the head.  Room beside what the admitted
+                # requests still have to take: the pages it has just given back are free, and taking them
+                # again at once would starve the same requests again, for ever
+                break
             if self.config.admit_within_pool and self.active and not self._room_beside_admitted(candidate):
                 break  # admitted now it would push another request out, or be pushed out, and be computed twice
             self.waiting.popleft()
