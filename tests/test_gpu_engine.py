@@ -1,6 +1,7 @@
 """GPU: the whole engine through its entry points: greedy generation against the
 plain implementation, long decoding, the first tokens of a sequence, temperature
-sampling, cache pressure with recompute preemption, prefix reuse, the command line."""
+sampling, cache pressure with recompute preemption, prefix reuse, random requests
+through a small pool against each request alone, the command line."""
 
 from __future__ import annotations
 
@@ -179,6 +180,51 @@ def test_prefix_is_shared_with_a_request_that_arrives_while_the_first_still_deco
     # tokens run through the model: both prompts less the 32 shared tokens, plus the decoded tokens fed back
     assert engine.snapshot_metrics()["tokens"]["input_total"] <= len(prompt) + len(sibling) - 32 + 2 * 12
     engine.runner.cache.assert_invariants()
+
+
+def test_random_requests_through_a_small_pool_equal_each_request_alone(tiny_folders):
+    """Forty random requests (shared prefixes, greedy and seeded temperature sampling, end
+    tokens) arrive a few per step at an engine whose pool holds one and a half full sequences: with
+    preemption, prefix sharing, captured decode steps and tokens fed back on the device, every
+    request ends with the tokens it gets when it runs alone, and the pool drains."""
+    import random
+
+    from cie_amd import GenerationConfig
+
+    folder, raw, _ = tiny_folders["B"]
+    rng = random.Random(3)
+    limit, vocab = raw["max_position_embeddings"], raw["vocab_size"]
+    prefix = [rng.randrange(vocab) for _ in range(40)]
+    requests = []
+    for _ in range(40):
+        count = rng.randint(2, limit // 2)
+        prompt = prefix[: rng.randint(0, min(40, count - 1))] if rng.random() < 0.5 else []
+        prompt = prompt + [rng.randrange(vocab) for _ in range(count - len(prompt))]
+        gen = GenerationConfig(max_output_tokens=rng.randint(1, min(40, limit - count - 1)),
+                               eos_token_id=rng.choice([None, None, rng.randrange(vocab)]),
+                               temperature=rng.choice([0.0, 0.0, 0.7, 1.3]), seed=rng.randrange(1000))
+        requests.append((prompt, gen))
+    busy = make_engine(folder, page_size=8, kv_tokens=3 * limit // 2, max_running=8, max_queue_size=64,
+                       max_model_len=limit, max_output_tokens=64, token_budget=64, prefill_chunk=7,
+                       prefix_cache_pages=16, admit_within_pool=False)
+    handles, pending, steps = [], list(requests), 0
+    while pending or busy.has_work():
+        for _ in range(rng.randint(0, 3)):
+            if pending:
+                handles.append(busy.submit(*pending.pop(0)))
+        busy.step()
+        steps += 1
+        assert steps < 4000, "the engine does not drain"
+    results = [busy.result_of(handle) for handle in handles]
+    metrics = busy.snapshot_metrics()
+    assert metrics["requests"]["preempted_total"] > 0 and metrics["kv_cache"]["prefix_cache_hits"] > 0
+    assert metrics["kv_cache"]["request_pages_used"] == 0
+    busy.runner.cache.assert_invariants()
+    alone = make_engine(folder, page_size=16, kv_tokens=2 * limit, max_running=1, max_model_len=limit,
+                        max_output_tokens=64, graph_decode=False, async_decode=False)
+    for (prompt, gen), got in zip(requests, results):
+        want = alone.generate([prompt], gen)[0]
+        assert (want.token_ids, want.finish_reason) == (got.token_ids, got.finish_reason), (len(prompt), gen)
 
 
 def test_warm_up_captures_every_decode_bucket_once(tiny_folders):
