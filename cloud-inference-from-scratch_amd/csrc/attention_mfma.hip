@@ -606,14 +606,17 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
 }
 
 // Merge the splits of every (tile, kv head): out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M).
-// One workgroup per (tile, kv head, row); the splits' weights are made once in LDS, then every thread
-// sums its head dimensions over the splits with independent loads.
+// One workgroup per (tile, kv head, row).  The parts' weights are made once in LDS; the threads are
+// laid out as (group, four head dimensions): group g sums parts g, g + groups, ... with independent
+// 16-byte loads, and the groups' sums meet in LDS.
 constexpr int kMergeMaxSplits = 1024;
+constexpr int kMergeThreads = 256;
 
-__global__ void __launch_bounds__(128)
+__global__ void __launch_bounds__(kMergeThreads)
 attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
     __shared__ float weight[kMergeMaxSplits];
     __shared__ float scratch[16];
+    __shared__ floatx4 group_sum[kMergeThreads];
     const int tile = blockIdx.x;
     const int kv_head = blockIdx.y;
     const int row = blockIdx.z;
@@ -623,16 +626,23 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
     const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
     if (row >= n_tok * group) return;
     const size_t unit0 = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits;
-    // The thread's share of the first parts' sums is fetched before the weights are known: these loads
-    // depend on nothing and travel while the statistics are read and reduced (the dimension of the
-    // thread's first round and the first sixteen parts; a wider head and further parts are fetched afterwards).
-    constexpr int kEarly = 16;
-    const size_t stride = static_cast<size_t>(rows_per_tile) * head_dim;
-    const float* po_row = a.part_o + (unit0 * rows_per_tile + row) * head_dim;
-    const int d0 = threadIdx.x;
-    float early[kEarly];
+    const int per_row = head_dim / 4;            // threads that cover a row of sums
+    const int groups = kMergeThreads / per_row;  // parts summed side by side
+    const int mine = threadIdx.x / per_row;
+    const int chunk = threadIdx.x - mine * per_row;
+    const bool active = mine < groups;
+    // The thread's share of its first parts' sums is fetched before the weights are known: these loads
+    // depend on nothing and travel while the statistics are read and reduced.
+    constexpr int kEarly = 4;
+    const size_t stride = static_cast<size_t>(rows_per_tile) * per_row;
+    const floatx4* po_row =
+        reinterpret_cast<const floatx4*>(a.part_o + (unit0 * rows_per_tile + row) * head_dim) + chunk;
+    floatx4 early[kEarly];
 #pragma unroll
-    for (int u = 0; u < kEarly; ++u) early[u] = (u < a.n_splits && d0 < head_dim) ? po_row[u * stride + d0] : 0.f;
+    for (int u = 0; u < kEarly; ++u) {
+        const int s = mine + u * groups;
+        early[u] = (active && s < a.n_splits) ? po_row[s * stride] : floatx4{0.f, 0.f, 0.f, 0.f};
+    }
     float m_local = -INFINITY;
     for (int s = threadIdx.x; s < a.n_splits; s += blockDim.x)
         m_local = fmaxf(m_local, a.part_ml[((unit0 + s) * rows_per_tile + row) * 2]);
@@ -645,23 +655,29 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
         den_local += ml[1] * w;
     }
     const float den = block_sum(den_local, scratch);  // its barriers also publish weight[]
+    floatx4 num = {0.f, 0.f, 0.f, 0.f};
+    if (active) {
+#pragma unroll
+        for (int u = 0; u < kEarly; ++u) {
+            const int s = mine + u * groups;
+            if (s < a.n_splits) num += early[u] * weight[s];
+        }
+#pragma unroll 4
+        for (int s = mine + kEarly * groups; s < a.n_splits; s += groups) num += po_row[s * stride] * weight[s];
+    }
+    group_sum[threadIdx.x] = num;
+    __syncthreads();
+    if (threadIdx.x >= per_row) return;
+    for (int g = 1; g < groups; ++g) num += group_sum[g * per_row + chunk];
     const int tok = row / group;
     const int head = row - tok * group;
     bf16_t* dst = a.out + static_cast<size_t>(a.q_start_loc[seq] + q0 + tok) * a.q_heads * head_dim +
-                  static_cast<size_t>(kv_head * group + head) * head_dim;
+                  static_cast<size_t>(kv_head * group + head) * head_dim + 4 * chunk;
     const float inv = 1.0f / den;
-    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-        float num = 0.f;
-        int s = 0;
-        if (d == d0) {
-#pragma unroll
-            for (int u = 0; u < kEarly; ++u)
-                if (u < a.n_splits) num += early[u] * weight[u];
-            s = min(a.n_splits, kEarly);
-        }
-        for (; s < a.n_splits; ++s) num += po_row[s * stride + d] * weight[s];
-        dst[d] = from_float<bf16_t>(num * inv);
-    }
+    uint2 packed;
+    packed.x = from_float<bf16_t>(num[0] * inv).bits | (static_cast<uint32_t>(from_float<bf16_t>(num[1] * inv).bits) << 16);
+    packed.y = from_float<bf16_t>(num[2] * inv).bits | (static_cast<uint32_t>(from_float<bf16_t>(num[3] * inv).bits) << 16);
+    *reinterpret_cast<uint2*>(dst) = packed;
 }
 
 template <int D>
@@ -762,6 +778,6 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
         default: return CIE_BAD_ARGUMENT;
     }
     if (rc != CIE_OK || n_splits == 1) return rc;
-    attention_merge_kernel<<<dim3(n_tiles, kv_heads, tokens_per_tile * group), 128, 0, s>>>(a, head_dim, 16 * row_tiles);
+    attention_merge_kernel<<<dim3(n_tiles, kv_heads, tokens_per_tile * group), kMergeThreads, 0, s>>>(a, head_dim, 16 * row_tiles);
     return cie_after_launch();
 }

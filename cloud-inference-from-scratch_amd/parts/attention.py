@@ -110,6 +110,7 @@ class Attention(Part):
 
 
 WIDE_DECODE_KEYS = 2048  # contexts from which decode rows go to the four-wave form
+FEW_DECODE_UNITS = 8  # (sequence, kv head) pairs below which they do not: parts of one wave fill the GPU better
 MANY_DECODE_UNITS = 96  # (sequence, kv head) pairs from which decode rows take the four-wave form at any context
 SHARED_DECODE_KEYS = 96  # contexts from which four waves share a decode row's keys without cutting them
 SPLIT_DECODE_KEYS = 192  # contexts from which the keys of decode rows are cut into parts at all
@@ -153,8 +154,10 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     def decode_form(bound: int, units: int) -> tuple[int, dict]:
         # Decode rows, `units` (sequence, kv head) pairs over up to `bound` keys.  Long contexts: four waves
         # per (sequence, kv head, part of the keys) take the part's blocks in turn with their loads running
-        # ahead (15.8 against 18.1 us for 8 x 4,096 keys).
-        if wide and bound >= WIDE_DECODE_KEYS:
+        # ahead (15.8 against 18.1 us for 8 x 4,096 keys).  A few pairs do not fill the GPU that way: they take the
+        # one-wave form below, whose parts are smaller (one sequence of the 3B shape over 32,000 keys: 333 -> 363
+        # tokens/s; from four sequences on the forms are level).
+        if wide and bound >= WIDE_DECODE_KEYS and units >= FEW_DECODE_UNITS:
             return ops.TILE_WAVES, dict(target_waves=1024 // ops.TILE_WAVES, min_keys=32 * ops.TILE_WAVES)
         # Many pairs fill the GPU by themselves: the same form with the keys whole or in large parts
         # (64 sequences x 2 heads x 256 keys: 9.2 us against 11.1 us with one wave per part)

@@ -352,6 +352,29 @@ def test_paged_attention_mfma_window(ops, window):
             torch.testing.assert_close(split[rows], want[rows], **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("geometry", [(16, 2, 128, 16), (16, 1, 96, 32), (12, 4, 256, 16), (6, 6, 64, 16)])
+def test_paged_attention_mfma_decode_hundreds_of_parts(ops, geometry):
+    """Two single tokens over 9,000 and 3,100 keys cut into parts of 32 and 64 keys: the merge sums
+    up to 282 parts per row, most of them in its loop behind the parts it fetches early; one far key
+    carries the weight of the first sequence, so a part lost or counted twice shows."""
+    q_heads, kv_heads, head_dim, page_size = geometry
+    group = q_heads // kv_heads
+    lengths, far = [9000, 3100], 7777
+    k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=91)
+    scale = 1.0 / math.sqrt(head_dim)
+    g = torch.Generator().manual_seed(92)
+    qs = [torch.stack([dense[0][0][far, h // group] * 2.0 for h in range(q_heads)])[None].to(torch.bfloat16).float(),
+          (torch.randn((1, q_heads, head_dim), generator=g) * 2).to(torch.bfloat16).float()]
+    contexts = [n - 1 for n in lengths]
+    expected = torch.cat([plain_qwen2.causal_attention(q, *dense[s], scale, past_len=contexts[s])
+                          for s, q in enumerate(qs)])
+    for n_splits, per_split, tile_waves in [(282, 32, 1), (141, 64, 1), (71, 128, 4)]:
+        out = run_mfma(ops, torch.cat([q.reshape(1, -1) for q in qs]), contexts, [1, 1], k_pool, v_pool, table, slots,
+                       q_heads, kv_heads, head_dim, None, scale, 1, 1, n_splits=n_splits, keys_per_split=per_split,
+                       tile_waves=tile_waves)
+        torch.testing.assert_close(out, expected, **tol(torch.bfloat16))
+
+
 def test_paged_attention_mfma_far_key(ops):
     """One key among two thousand carries the weight: output = its value row, in
     the tiled form and in every split layout."""

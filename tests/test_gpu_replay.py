@@ -114,12 +114,14 @@ def test_replay_with_the_four_wave_prompt_attention(tiny_folders, plain, monkeyp
 
 @pytest.mark.parametrize("graph", [False, True])
 def test_replay_with_the_four_wave_decode_attention(tiny_folders, plain, monkeypatch, graph):
-    """Decode rows go to the four-wave attention form only for long contexts; make
-    every context long enough, eagerly and in captured steps."""
+    """Decode rows go to the four-wave attention form only for long contexts and not for
+    a few sequences; make every context long enough and every batch large enough, eagerly
+    and in captured steps."""
     from cie_amd.kernels import ops
     from cie_amd.parts import attention
 
     monkeypatch.setattr(attention, "WIDE_DECODE_KEYS", 0)
+    monkeypatch.setattr(attention, "FEW_DECODE_UNITS", 0)
     seen = []
     real = ops.paged_attention_mfma
 
