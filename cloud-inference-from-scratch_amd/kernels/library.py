@@ -105,9 +105,11 @@ def build_library(force: bool = True) -> Path:
     files = sources()
     _log(f"compiling {len(files)} HIP sources for {ARCH} into {folder}")
     started = time.time()
+    # objects of this build alone: two processes that build at once do not write each other's files
+    objects_dir = Path(tempfile.mkdtemp(prefix="objects_", dir=folder))
 
     def compile_one(path: Path) -> Path:
-        obj = folder / (path.stem + ".o")
+        obj = objects_dir / (path.stem + ".o")
         cmd = [hipcc, *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(path), "-o", str(obj)]
         done = subprocess.run(cmd, env=env, capture_output=True, text=True)
         if done.returncode != 0:
@@ -116,14 +118,17 @@ def build_library(force: bool = True) -> Path:
         return obj
 
     workers = max(1, min(len(files), os.cpu_count() or 4, 8))
-    with ThreadPoolExecutor(max_workers=workers) as pool:
-        objects = list(pool.map(compile_one, files))
-    scratch = folder / f"{LIB_NAME}.{os.getpid()}.tmp"
-    link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(scratch), *map(str, objects), *LINK_LIBS]
-    done = subprocess.run(link, env=env, capture_output=True, text=True)
-    if done.returncode != 0:
-        raise KernelLibraryError(f"linking {LIB_NAME} failed:\n{done.stderr[-4000:]}")
-    os.replace(scratch, target)
+    try:
+        with ThreadPoolExecutor(max_workers=workers) as pool:
+            objects = list(pool.map(compile_one, files))
+        scratch = objects_dir / LIB_NAME
+        link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(scratch), *map(str, objects), *LINK_LIBS]
+        done = subprocess.run(link, env=env, capture_output=True, text=True)
+        if done.returncode != 0:
+            raise KernelLibraryError(f"linking {LIB_NAME} failed:\n{done.stderr[-4000:]}")
+        os.replace(scratch, target)  # (same file system: the finished library appears at once)
+    finally:
+        shutil.rmtree(objects_dir, ignore_errors=True)
     stamp.write_text(wanted + "\n")
     _log(f"built {target} in {time.time() - started:.0f}s")
     return target
@@ -148,14 +153,8 @@ def load_library() -> ctypes.CDLL:
             return _library
         path = find_built(check_stamp=True)
         if path is None:
-            stale = find_built(check_stamp=False)
-            try:
-                path = build_library(force=False)
-            except KernelLibraryError:
-                if stale is None:
-                    raise
-                _log(f"sources changed but rebuilding failed; loading the stale {stale}")
-                path = stale
+            # (a library built from other sources is never loaded: its entry points may take other arguments)
+            path = build_library(force=False)
         try:
             _library = ctypes.CDLL(str(path))
         except OSError as exc:
