@@ -35,6 +35,10 @@ class EngineConfig:
     kv_cache_bytes: int = 4 << 30
     prefix_cache_pages: int = 256  # reference: prefix_cache_max_blocks
     graph_decode: bool = True  # reference: cuda_graph_decode
+    # steps of up to 128 rows that bring prompt portions are captured too, from the second time a shape comes
+    # (bucket of the decode rows, lengths of the portions); this many shapes are kept, the least recently used
+    # are dropped; 0: such steps always run launch by launch
+    graph_mixed_steps: int = 16
     # a captured decode step is started before the tokens of the step before it have reached the host (it takes
     # them on the device); a request that ends on an end-of-sequence token then has run one step too many
     async_decode: bool = True
@@ -54,6 +58,8 @@ class EngineConfig:
             raise ValueError(f"page_size must be a power of two, got {config.page_size}")
         if config.prefix_cache_pages < 0:
             raise ValueError("prefix_cache_pages must be non-negative")
+        if config.graph_mixed_steps < 0:
+            raise ValueError("graph_mixed_steps must be non-negative")
         if config.kv_tokens is not None and config.kv_tokens < config.page_size:
             raise ValueError("kv_tokens too small for even one page")
         return config

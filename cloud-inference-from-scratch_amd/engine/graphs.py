@@ -13,7 +13,9 @@ cleared with a memset inside the graph.
 
 from __future__ import annotations
 
-from collections.abc import Sequence
+import contextlib
+import gc
+from collections.abc import Iterator, Sequence
 from dataclasses import dataclass
 from typing import Any
 
@@ -27,10 +29,26 @@ class StaticPlan:
     """What kernel planning may use during a captured step: only bounds known at
     capture time and device tensors."""
 
-    tile_seq: torch.Tensor      # int32 [bucket] = 0..bucket-1 (one query tile per sequence)
-    tile_q0: torch.Tensor       # int32 [bucket] = 0
+    tile_seq: torch.Tensor | None  # int32 [bucket] = 0..bucket-1 (one query tile per sequence)
+    tile_q0: torch.Tensor | None   # int32 [bucket] = 0
     max_context: torch.Tensor   # int32 [1], the step's longest context, rewritten before each replay
-    max_keys: int               # upper bound of any context (max_model_len)
+    max_keys: int               # upper bound of any context (max_model_len, or the bound a captured step was made for)
+    decode_rows: int | None = None  # the step's first sequences that bring one token each; None: all of them
+
+
+@contextlib.contextmanager
+def _collector_off() -> Iterator[None]:
+    """Around a capture.  A runner and its graphs refer to each other, so a runner that is gone waits for
+    the cyclic collector with its captured graphs; a graph destroyed while another is being captured aborts
+    the process.  What waits is collected now, and the collector stays off until the capture has ended."""
+    gc.collect()
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        yield
+    finally:
+        if was_enabled:
+            gc.enable()
 
 
 class _Bucket:
@@ -127,7 +145,7 @@ class DecodeGraphs:
         graph = torch.cuda.CUDAGraph()
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
-        with torch.cuda.graph(graph, pool=self.pool):
+        with _collector_off(), torch.cuda.graph(graph, pool=self.pool):
             bucket.logits = runner.model.forward(bucket.batch, runner.device_cache)
         bucket.graph = graph
         self.buckets[size] = bucket
@@ -163,3 +181,180 @@ class DecodeGraphs:
         if rows == list(range(len(entries))):
             return bucket.logits[: len(entries)]
         return bucket.logits[torch.tensor(rows, dtype=torch.long, device=runner.device)]
+
+
+@dataclass
+class _CapturedStep:
+    """A captured step of single tokens beside prompt portions, and the buffer its replays rewrite."""
+
+    decode_rows: int
+    portions: tuple[int, ...]
+    host: torch.Tensor
+    dev: torch.Tensor
+    offsets: dict[str, int]
+    batch: StepBatch
+    graph: Any = None
+    logits: torch.Tensor | None = None
+
+
+class MixedGraphs:
+    """Steps that bring short prompt portions (beside decode tokens or alone) as captured graphs.
+
+    Such a step is a few hundred launches too, and with few tokens the host cannot queue them as fast as the
+    GPU runs them (8 decode rows and a 64-token portion of the 3B shape: 5.6 ms launch by launch, 4.7 ms
+    replayed; with a 256-token portion the GPU is the slower one either way, 7.6 ms).  A capture costs as
+    much as ten such steps, so only shapes that come again are captured: a step's shape is (bucket of its
+    single-token rows, the lengths of its portions); one that comes a second time (the portions of one
+    long prompt beside the same decoding requests do) is captured from that very step, with its real
+    tokens, slots and pages, and replayed from then on.  As in captured decode steps, the parts of the
+    keys are sized on the device from the step's longest context.  The least recently used shapes beyond
+    ``limit`` are dropped.  The reference captures decode steps only (src/cloud_engine/engine.py:316-437)."""
+
+    MAX_PORTIONS = 4
+    MAX_TOKENS = 128  # rows of a step (decode bucket and portions) up to which the host is the slower side
+
+    def __init__(self, runner: Any, decode_graphs: "DecodeGraphs", limit: int) -> None:
+        self.runner = runner
+        self.decode_graphs = decode_graphs
+        self.limit = limit
+        self.steps: dict[tuple, _CapturedStep] = {}   # in order of last use
+        self.seen: dict[tuple, int] = {}
+        self.captures = 0
+        self.replays = 0
+
+    def shape_of(self, entries: Sequence[Any]) -> tuple | None:
+        """The step's shape if a captured graph may run it, else None: at most MAX_PORTIONS portions, and
+        logits wanted at no other place than a portion's last token."""
+        single = [e for e in entries if len(e.tokens) == 1]
+        portions = [e for e in entries if len(e.tokens) > 1]
+        if not portions or len(portions) > self.MAX_PORTIONS or len(single) > self.decode_graphs.largest:
+            return None
+        bucket = DecodeGraphs.bucket_of(len(single)) if single else 0
+        if bucket + sum(len(e.tokens) for e in portions) > self.MAX_TOKENS:
+            return None
+        for e in portions:
+            if tuple(e.want) not in ((), (len(e.tokens) - 1,)):
+                return None
+        if any(len(e.want) > 1 for e in single):
+            return None
+        return bucket, tuple(len(e.tokens) for e in portions)
+
+    def wants(self, entries: Sequence[Any]) -> tuple | None:
+        """The shape if this step is to run from a graph now (captured already, or seen before)."""
+        if self.limit < 1:
+            return None
+        shape = self.shape_of(entries)
+        if shape is None:
+            return None
+        if shape in self.steps:
+            return shape
+        self.seen[shape] = self.seen.get(shape, 0) + 1
+        if len(self.seen) > 4096:
+            self.seen.clear()
+        return shape if self.seen[shape] >= 2 else None
+
+    def _layout(self, shape: tuple) -> _CapturedStep:
+        decode_rows, portions = shape
+        runner = self.runner
+        bound = runner.config.max_model_len
+        sequences = decode_rows + len(portions)
+        tokens = decode_rows + sum(portions)
+        offsets: dict[str, int] = {}
+        offset = 0
+        for name, length in (("token_ids", tokens), ("positions", tokens), ("seq_of_token", tokens),
+                             ("seq_slot", sequences), ("seq_start", sequences), ("seq_q_len", sequences),
+                             ("q_start_loc", sequences + 1), ("logit_rows", sequences), ("max_context", 1)):
+            offsets[name] = offset
+            offset += length
+        host = torch.zeros(offset, dtype=torch.int32)
+        q_lens = [1] * decode_rows + list(portions)
+        starts = [0]
+        for count in q_lens:
+            starts.append(starts[-1] + count)
+        o = offsets
+        host[o["seq_of_token"]: o["seq_of_token"] + tokens] = torch.tensor(
+            [index for index, count in enumerate(q_lens) for _ in range(count)], dtype=torch.int32)
+        host[o["seq_q_len"]: o["seq_q_len"] + sequences] = torch.tensor(q_lens, dtype=torch.int32)
+        host[o["q_start_loc"]: o["q_start_loc"] + sequences + 1] = torch.tensor(starts, dtype=torch.int32)
+        # logits: every single-token row, and the last token of every portion
+        host[o["logit_rows"]: o["logit_rows"] + sequences] = torch.tensor(
+            [start + count - 1 for start, count in zip(starts, q_lens)], dtype=torch.int32)
+        dev = torch.zeros(offset, dtype=torch.int32, device=runner.device)
+
+        def view(name: str, length: int) -> torch.Tensor:
+            return dev[o[name]: o[name] + length]
+
+        pad = runner.device_cache.pad_slot
+        batch = StepBatch(
+            tokens=tokens, sequences=sequences, token_ids=view("token_ids", tokens), positions=view("positions", tokens),
+            seq_of_token=view("seq_of_token", tokens), seq_slot=view("seq_slot", sequences),
+            seq_start=view("seq_start", sequences), seq_q_len=view("seq_q_len", sequences),
+            q_start_loc=view("q_start_loc", sequences + 1), logit_rows=view("logit_rows", sequences),
+            host_slots=[pad] * sequences, host_starts=[0] * sequences, host_q_lens=q_lens,
+            static_plan=StaticPlan(None, None, view("max_context", 1), bound, decode_rows=decode_rows),
+        )
+        return _CapturedStep(decode_rows, portions, host, dev, offsets, batch)
+
+    def _fill(self, step: _CapturedStep, single: Sequence[Any], portions: Sequence[Any]) -> None:
+        """Real single-token rows first, padding up to the bucket (token 0 at position 0 of the pad slot),
+        then the portions."""
+        cache = self.runner.cache
+        pad = step.decode_rows - len(single)
+        tokens = [e.tokens[0] for e in single] + [0] * pad
+        positions = [e.start_pos for e in single] + [0] * pad
+        slots = [cache.slot(e.request_id) for e in single] + [self.runner.device_cache.pad_slot] * pad
+        starts = list(positions)
+        for e in portions:
+            tokens.extend(e.tokens)
+            positions.extend(range(e.start_pos, e.start_pos + len(e.tokens)))
+            slots.append(cache.slot(e.request_id))
+            starts.append(e.start_pos)
+        o, host = step.offsets, step.host
+        host[o["token_ids"]: o["token_ids"] + len(tokens)] = torch.tensor(tokens, dtype=torch.int32)
+        host[o["positions"]: o["positions"] + len(positions)] = torch.tensor(positions, dtype=torch.int32)
+        host[o["seq_slot"]: o["seq_slot"] + len(slots)] = torch.tensor(slots, dtype=torch.int32)
+        host[o["seq_start"]: o["seq_start"] + len(starts)] = torch.tensor(starts, dtype=torch.int32)
+        host[o["max_context"]] = max(e.start_pos + len(e.tokens) for e in list(single) + list(portions))
+        step.dev.copy_(to_device_staging(host, self.runner.device), non_blocking=True)
+
+    def _capture(self, step: _CapturedStep) -> None:
+        """Capture from the buffer as it is filled: the step's own tokens, slots and pages (the cache has
+        room for them already), so that the run before the capture and the first replay write what the
+        step has to write anyway."""
+        runner = self.runner
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):  # outside capture: libraries set themselves up, tile lists are made
+            runner.model.forward(step.batch, runner.device_cache)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        if self.decode_graphs.pool is None:
+            self.decode_graphs.pool = torch.cuda.graph_pool_handle()
+        with _collector_off(), torch.cuda.graph(graph, pool=self.decode_graphs.pool):
+            step.logits = runner.model.forward(step.batch, runner.device_cache)
+        step.graph = graph
+        self.captures += 1
+
+    def run(self, shape: tuple, entries: Sequence[Any]) -> torch.Tensor:
+        """Replay (after capturing, if need be) the graph of this shape; logits [wanted, vocab] in the order
+        of the entries."""
+        single = [e for e in entries if len(e.tokens) == 1]
+        portions = [e for e in entries if len(e.tokens) > 1]
+        step = self.steps.pop(shape, None)
+        fresh = step is None
+        if fresh:
+            step = self._layout(shape)
+        self.steps[shape] = step  # (last in the order of use)
+        self._fill(step, single, portions)
+        if fresh:
+            self._capture(step)
+            while len(self.steps) > self.limit:
+                del self.steps[next(iter(self.steps))]
+        step.graph.replay()
+        self.replays += 1
+        row_of = {id(e): index for index, e in enumerate(single)}
+        row_of.update({id(e): step.decode_rows + index for index, e in enumerate(portions)})
+        rows = [row_of[id(e)] for e in entries for _ in e.want]
+        return step.logits[torch.tensor(rows, dtype=torch.long, device=self.runner.device)]

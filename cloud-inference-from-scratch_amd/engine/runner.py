@@ -25,7 +25,7 @@ from ..profiling import trace_range
 from ..sampling.sampler import Sampler
 from .batch import StepBatch, to_device_staging
 from .device_cache import DeviceCache
-from .graphs import DecodeGraphs
+from .graphs import DecodeGraphs, MixedGraphs
 
 
 @dataclass(frozen=True)
@@ -76,6 +76,8 @@ class Runner:
         self.forward_plans: deque[tuple[tuple[str, int, int, int], ...]] = deque(maxlen=256)
         self.sampler = Sampler(config.seed)
         self.graphs = DecodeGraphs(self) if config.graph_decode and getattr(model, "graph_safe", False) else None
+        self.mixed_graphs = (MixedGraphs(self, self.graphs, config.graph_mixed_steps)
+                             if self.graphs is not None and config.graph_mixed_steps > 0 else None)
         self._staging = [None, None]
         self._staging_turn = 0
 
@@ -125,6 +127,14 @@ class Runner:
     @property
     def graph_replays(self) -> int:
         return self.graphs.replays if self.graphs is not None else 0
+
+    @property
+    def mixed_graph_captures(self) -> int:
+        return self.mixed_graphs.captures if self.mixed_graphs is not None else 0
+
+    @property
+    def mixed_graph_replays(self) -> int:
+        return self.mixed_graphs.replays if self.mixed_graphs is not None else 0
 
     def free_tokens(self) -> int:
         """Tokens the pool could take now (free pages of the scarcest group)."""
@@ -277,10 +287,15 @@ class Runner:
         decode = all(len(e.tokens) == 1 for e in entries)
         tokens = sum(len(e.tokens) for e in entries)
         with trace_range(f"ragged.forward.{'decode' if decode else 'mixed'}.requests_{len(entries)}.tokens_{tokens}"):
+            shape = None
+            if not decode and feed is None and self.mixed_graphs is not None:
+                shape = self.mixed_graphs.wants(entries)
             if decode and self.graphs is not None and self.graphs.takes(len(entries)):
                 logits = self.graphs.run(entries, feed)
             elif feed is not None:
                 raise ValueError("tokens can be fed on the device to captured decode steps only")
+            elif shape is not None:
+                logits = self.mixed_graphs.run(shape, entries)
             else:
                 logits = self.model.forward(self.pack(entries), self.device_cache)
         with trace_range("ragged.kv.commit"):

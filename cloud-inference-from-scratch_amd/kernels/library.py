@@ -14,6 +14,7 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -22,6 +23,7 @@ import threading
 import time
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
+from typing import Any
 
 CSRC = Path(__file__).resolve().parent.parent / "csrc"
 LIB_NAME = "libcie_kernels.so"
@@ -145,6 +147,33 @@ def find_built(check_stamp: bool = True) -> Path | None:
     return None
 
 
+_C_TYPES = {"int": ctypes.c_int, "long": ctypes.c_long, "size_t": ctypes.c_size_t, "float": ctypes.c_float}
+_ENTRY_POINT = re.compile(r"CIE_API\s+int\s+(\w+)\s*\(([^)]*)\)")
+
+
+def entry_point_signatures() -> dict[str, list[Any]]:
+    """The argument types of every ``CIE_API int name(...)`` in the sources, read from their text (the
+    library that is loaded was built from exactly these sources): a pointer of any kind is an address,
+    scalars are ``int``, ``long``, ``size_t`` or ``float``.  Anything else is an error, not a guess."""
+    found: dict[str, list[Any]] = {}
+    for path in sources():
+        for name, params in _ENTRY_POINT.findall(path.read_text()):
+            types: list[Any] = []
+            for param in params.split(","):
+                words = param.replace("*", " * ").split()
+                if "*" in words:
+                    types.append(ctypes.c_void_p)
+                    continue
+                kind = [w for w in words[:-1] if w not in ("const", "unsigned")]
+                if len(kind) != 1 or kind[0] not in _C_TYPES or "unsigned" in words:
+                    raise KernelLibraryError(f"{path.name}: cannot read the parameter '{param.strip()}' of {name}")
+                types.append(_C_TYPES[kind[0]])
+            if name in found:
+                raise KernelLibraryError(f"entry point {name} is defined twice")
+            found[name] = types
+    return found
+
+
 def load_library() -> ctypes.CDLL:
     """The loaded kernel library; built first if nothing current is there."""
     global _library
@@ -159,5 +188,11 @@ def load_library() -> ctypes.CDLL:
             _library = ctypes.CDLL(str(path))
         except OSError as exc:
             raise KernelLibraryError(f"cannot load {path}: {exc}") from exc
+        # declared once: calls then pass plain Python numbers and addresses, which costs a fraction of
+        # building a ctypes object per argument
+        for name, types in entry_point_signatures().items():
+            function = getattr(_library, name)
+            function.argtypes = types
+            function.restype = ctypes.c_int
         _library.cie_path = str(path)  # type: ignore[attr-defined]
         return _library

@@ -8,7 +8,6 @@ on operands it was not written for.  Kernels run on torch's current stream.
 
 from __future__ import annotations
 
-import ctypes
 from typing import Optional
 
 import torch
@@ -44,13 +43,15 @@ def _gpu(name: str, tensor: torch.Tensor, dtype: Optional[torch.dtype] = None, d
             raise ValueError(f"{name} must have {dims} dims, has shape {tuple(tensor.shape)}")
 
 
-def _ptr(tensor: Optional[torch.Tensor]) -> ctypes.c_void_p:
-    return ctypes.c_void_p(0 if tensor is None else tensor.data_ptr())
+# Arguments go to the library as plain Python numbers: the entry points' argument types are declared
+# when the library is loaded (kernels/library.py), and ctypes converts them itself.
+def _ptr(tensor: Optional[torch.Tensor]) -> Optional[int]:
+    return None if tensor is None else tensor.data_ptr()
 
 
-def _stream() -> ctypes.c_void_p:
+def _stream() -> int:
     # the raw handle of torch's current stream (also the capturing one), without building a Stream object
-    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 def _run(name: str, code: int) -> None:
@@ -58,12 +59,8 @@ def _run(name: str, code: int) -> None:
         raise KernelError(f"{name}: {_ERRORS.get(code, f'error {code}')}")
 
 
-def _i(value: int) -> ctypes.c_int:
-    return ctypes.c_int(int(value))
-
-
-def _f(value: float) -> ctypes.c_float:
-    return ctypes.c_float(float(value))
+_i = int
+_f = float
 
 
 def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, dtype: torch.dtype, kv_heads: int,
@@ -549,7 +546,7 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     out = torch.empty((m, n), dtype=out_dtype, device=device)
     code = load_library().cie_gemm_library(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k),
-        _i(1 if out_dtype == torch.float32 else 0), _ptr(workspace), ctypes.c_size_t(workspace.numel()),
+        _i(1 if out_dtype == torch.float32 else 0), _ptr(workspace), workspace.numel(),
         _i(1 if (m >= LIBRARY_TUNE_ROWS and m % 256 == 0) or (m >= 32 and m & (m - 1) == 0) else 0))
     if code == 1:
         return None

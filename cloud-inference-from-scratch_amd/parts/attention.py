@@ -172,21 +172,30 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         # (8 x 128 keys: 6.5 against 6.9 us, 8 x 160: 7 against 11)
         return (ops.TILE_WAVES if wide and bound >= SHARED_DECODE_KEYS else 1), dict(target_waves=1024, min_keys=bound + 1)
 
-    if batch.static_plan is not None:  # a captured decode step: the grid is fixed, lengths live on the device
-        plan = batch.static_plan
-        bound = plan.max_keys if window is None else min(plan.max_keys, window + 64)
-        decode_waves, split_options = decode_form(bound, batch.sequences * num_kv_heads)
-        n_splits, _ = plan_splits(batch.sequences * num_kv_heads, bound, **split_options)
-        part_o = part_ml = None
-        if n_splits > 1:
-            part_o, part_ml = _workspaces(qkv.device, batch.sequences * num_kv_heads * n_splits, 16, head_dim)
-        # (every sequence brings one token: tile i is sequence i, no tile lists)
-        ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, None,
-                                 None, batch.sequences, *common, tokens_per_tile=1, row_tiles=1,
-                                 n_splits=n_splits, max_context_dev=plan.max_context, part_o=part_o, part_ml=part_ml,
-                                 tile_waves=decode_waves)
-        return out
-    tile_seq, tile_q0, n_tiles = batch.tiles(1, decode=True)
+    plan = batch.static_plan
+    longest_dev = None
+    if plan is not None:
+        # a captured step: grids are fixed, lengths live on the device.  Its first sequences bring one token
+        # each (tile i is sequence i, no tile lists); the sizes of the keys' parts follow the step's longest
+        # context, which the device knows, within the bound the step was captured for
+        max_keys = plan.max_keys if window is None else min(plan.max_keys, window + 64)
+        longest_dev = plan.max_context
+        decode_rows = batch.sequences if plan.decode_rows is None else plan.decode_rows
+        if decode_rows:
+            decode_waves, split_options = decode_form(max_keys, decode_rows * num_kv_heads)
+            n_splits, _ = plan_splits(decode_rows * num_kv_heads, max_keys, **split_options)
+            part_o = part_ml = None
+            if n_splits > 1:
+                part_o, part_ml = _workspaces(qkv.device, decode_rows * num_kv_heads * n_splits, 16, head_dim)
+            ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, None,
+                                     None, decode_rows, *common, tokens_per_tile=1, row_tiles=1,
+                                     n_splits=n_splits, max_context_dev=longest_dev, part_o=part_o, part_ml=part_ml,
+                                     tile_waves=decode_waves)
+        if decode_rows == batch.sequences:
+            return out
+        n_tiles = 0  # (of the eager decode form below)
+    else:
+        tile_seq, tile_q0, n_tiles = batch.tiles(1, decode=True)
     if n_tiles:
         decode_waves, split_options = decode_form(max_keys, n_tiles * num_kv_heads)
         n_splits, per_split = plan_splits(n_tiles * num_kv_heads, max_keys, **split_options)
@@ -233,7 +242,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
                                  n_tiles, *common, tokens_per_tile=per_tile, row_tiles=row_tiles,
                                  n_splits=n_splits, keys_per_split=per_split, part_o=part_o, part_ml=part_ml,
-                                 tile_waves=tile_waves)
+                                 tile_waves=tile_waves, max_context_dev=longest_dev if n_splits > 1 else None)
     return out
 
 

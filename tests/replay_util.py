@@ -86,6 +86,32 @@ def mixed(requests: dict[str, list[int]], live: int = 4, chunk_sizes=(5, 12, 2, 
     return steps
 
 
+def fixed_portions(requests: dict[str, list[int]], portion: int = 8, live: int = 3, decode_tail: int = 12) -> list[dict]:
+    """As a scheduler cuts them: every prompt in portions of one size (its rest last), the last
+    ``decode_tail`` tokens one by one, up to ``live`` requests side by side; logits are wanted where a
+    sampler would look, at the last token of every portion and at every single token.  The same shapes
+    of steps come again and again."""
+    waiting = list(requests.items())
+    active: list[list] = []
+    steps = []
+    while waiting or active:
+        if waiting and len(active) < live:  # (one newcomer per step: prompts start at different steps)
+            rid, tokens = waiting.pop(0)
+            active.append([rid, tokens, 0])
+        entries, ended = [], []
+        for state in active:
+            rid, tokens, fed = state
+            left = len(tokens) - fed
+            size = 1 if left <= decode_tail else min(portion, left - decode_tail)
+            state[2] = fed + size
+            entries.append({"id": rid, "tokens": tokens[fed:fed + size], "want": [size - 1]})
+            if state[2] == len(tokens):
+                ended.append(rid)
+        active = [s for s in active if s[2] < len(s[1])]
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+    return steps
+
+
 def max_live_tokens(steps: list[dict], page: int = 64) -> int:
     """Most tokens live requests hold at any time, each rounded up to ``page``."""
     held: dict[str, int] = {}

@@ -143,6 +143,53 @@ def test_replay_with_the_four_wave_decode_attention(tiny_folders, plain, monkeyp
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_captured_steps_with_prompt_portions_match_plain(tiny_folders, plain, name, dtype):
+    """Steps that bring prompt portions beside decode tokens are captured when their shape comes a second
+    time and replayed from then on, with other tokens, slots, pages and lengths at every replay (pages of
+    finished requests are used again): every wanted row against the plain model, and against the same
+    schedule run launch by launch."""
+    folder, raw, _ = tiny_folders[name]
+    requests, expected = plain[name]
+    page = 16 if name == "A" else 8
+    steps = replay_util.fixed_portions(requests, portion=8 if name == "B" else 5)
+    pool = replay_util.max_live_tokens(steps, page=page)
+    runner = make_runner(folder, dtype, pool, page, graph_decode=True)
+    assert runner.mixed_graphs is not None
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    replay_util.compare(rows, expected, every_position=False, **TOL[dtype])
+    assert runner.mixed_graph_captures >= 2 and runner.mixed_graph_replays >= 8, (
+        runner.mixed_graph_captures, runner.mixed_graph_replays)
+    assert runner.cache.stats().pages_used == 0
+    eager = make_runner(folder, dtype, pool, page, graph_decode=False)
+    assert eager.mixed_graphs is None
+    eager_rows = replay_util.by_position(steps, replay_util.drive_runner(eager, steps))
+    for rid, positions in rows.items():
+        for position, row in positions.items():
+            if dtype == "float32":  # the same kernels on the same rows: the same bits
+                assert np.array_equal(row, eager_rows[rid][position]), (rid, position)
+            else:  # (the parts of a portion's keys may be cut elsewhere)
+                np.testing.assert_allclose(row, eager_rows[rid][position], **TOL[dtype])
+
+
+def test_shapes_beyond_the_limit_drop_the_least_recently_used(tiny_folders, plain):
+    from cie_amd.config import build_engine_config
+    from cie_amd.engine import Runner, load_model
+
+    folder, raw, _ = tiny_folders["A"]
+    requests, expected = plain["A"]
+    model, config = load_model(folder, "float32", "cuda:0")
+    steps = replay_util.fixed_portions(requests, portion=5)
+    pool = replay_util.max_live_tokens(steps, page=16)
+    runner = Runner(model, build_engine_config(dtype="float32", page_size=16, kv_tokens=pool, max_running=8,
+                                               max_model_len=min(config.max_position_embeddings, pool), prefix_cache_pages=0,
+                                               graph_mixed_steps=1), "cuda:0")
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    replay_util.compare(rows, expected, every_position=False, **TOL["float32"])
+    assert len(runner.mixed_graphs.steps) == 1 and runner.mixed_graph_captures >= 2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_captured_decode_steps_match_plain(tiny_folders, plain, name, dtype):
     """Decode steps replayed from captured graphs (buckets 1, 2 and 4, padded

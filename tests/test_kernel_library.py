@@ -1,0 +1,29 @@
+"""The kernel library's host side without a GPU: the entry points' argument types are read from the sources."""
+
+from __future__ import annotations
+
+import ctypes
+
+import pytest
+
+from cie_amd.kernels import library
+
+
+def test_signatures_of_all_entry_points_are_read_from_the_sources():
+    found = library.entry_point_signatures()
+    text = "".join(path.read_text() for path in library.sources())
+    assert len(found) == text.count("CIE_API int ") >= 14
+    # (stream, dtype, gate_up, out, tokens, intermediate, row_sumsq, parts, hidden, eps)
+    p, i, f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    assert found["cie_silu_mul"] == [p, i, p, p, i, i, p, i, i, f]
+    assert found["cie_gemm_library"][-2:] == [ctypes.c_size_t, i]
+    assert all(types[0] is p for types in found.values())  # every entry point takes the stream first
+
+
+@pytest.mark.parametrize("params", ["void* stream, double x", "void* stream, unsigned int n", "void* stream, int"])
+def test_a_parameter_that_is_not_understood_is_an_error(tmp_path, monkeypatch, params):
+    source = tmp_path / "odd.hip"
+    source.write_text(f"CIE_API int cie_odd({params}) {{ return 0; }}\n")
+    monkeypatch.setattr(library, "sources", lambda: [source])
+    with pytest.raises(library.KernelLibraryError, match="cie_odd"):
+        library.entry_point_signatures()
