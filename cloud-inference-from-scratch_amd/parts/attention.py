@@ -110,6 +110,7 @@ class Attention(Part):
 
 
 WIDE_DECODE_KEYS = 2048  # contexts from which decode rows go to the four-wave form
+WIDE_TARGET_WORKGROUPS = 256  # workgroups the four-wave form cuts long contexts for
 FEW_DECODE_UNITS = 8  # (sequence, kv head) pairs below which they do not: parts of one wave fill the GPU better
 MANY_DECODE_UNITS = 96  # (sequence, kv head) pairs from which decode rows take the four-wave form at any context
 SHARED_DECODE_KEYS = 96  # contexts from which four waves share a decode row's keys without cutting them
@@ -158,7 +159,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         # one-wave form below, whose parts are smaller (one sequence of the 3B shape over 32,000 keys: 333 -> 363
         # tokens/s; from four sequences on the forms are level).
         if wide and bound >= WIDE_DECODE_KEYS and units >= FEW_DECODE_UNITS:
-            return ops.TILE_WAVES, dict(target_waves=1024 // ops.TILE_WAVES, min_keys=32 * ops.TILE_WAVES)
+            return ops.TILE_WAVES, dict(target_waves=WIDE_TARGET_WORKGROUPS, min_keys=32 * ops.TILE_WAVES)
         # Many pairs fill the GPU by themselves: the same form with the keys whole or in large parts
         # (64 sequences x 2 heads x 256 keys: 9.2 us against 11.1 us with one wave per part)
         if wide and units >= MANY_DECODE_UNITS and bound >= SHARED_DECODE_KEYS:
