@@ -142,6 +142,49 @@ def test_replay_with_the_four_wave_decode_attention(tiny_folders, plain, monkeyp
         assert runner.graph_replays >= 20
 
 
+ODD_SIZES = [  # hidden, heads, kv heads, head_dim, intermediate, vocabulary
+    (75, 3, 1, 16, 77, 97),      # an odd width: no 16-byte rows anywhere
+    (90, 6, 2, 48, 50, 1001),
+    (34, 2, 2, 80, 33, 130),     # heads wider than the model
+    (200, 24, 8, 16, 12, 50),    # many small heads, a feed-forward narrower than a tile
+    (30, 3, 1, 8, 50, 101),      # the smallest head the kernels take
+    (64, 2, 1, 136, 12, 50),     # a head size in steps of 8 that the matrix-core attention does not take
+    (128, 2, 1, 256, 64, 300),   # the widest head
+]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("sizes", ODD_SIZES, ids=lambda s: "x".join(map(str, s)))
+def test_replay_at_odd_sizes(tmp_path, sizes, dtype):
+    """Widths, head sizes and vocabularies that no fast path was written for run through the kernels
+    that take every size, in a mixed schedule with reused pages, to the plain model's logits."""
+    from conftest import TINY_C, make_folder
+
+    hidden, heads, kv_heads, head_dim, intermediate, vocab = sizes
+    raw = dict(TINY_C, hidden_size=hidden, num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=head_dim,
+               intermediate_size=intermediate, vocab_size=vocab, eos_token_id=1)
+    folder, tensors = make_folder(tmp_path, raw, seed=3)
+    requests = {f"r{i}": random_tokens(n, vocab, seed=50 + i) for i, n in enumerate((5, 33, 70))}
+    expected = plain_all(raw, tensors, requests)
+    steps = replay_util.mixed(requests, live=3)
+    pool = replay_util.max_live_tokens(steps, page=16)
+    runner = make_runner(folder, dtype, pool, 16, max_running=4)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    replay_util.compare(rows, expected, **TOL[dtype])
+    assert runner.cache.stats().pages_used == 0
+
+
+def test_a_head_size_the_kernels_do_not_take_is_refused_when_the_model_is_built(tmp_path):
+    from conftest import TINY_C
+    from cie_amd.config import config_from_dict
+    from cie_amd.parts.model import expected_tensors
+
+    for head_dim in (20, 264):
+        config = config_from_dict(dict(TINY_C, head_dim=head_dim))
+        with pytest.raises(ValueError, match="head_dim must be a multiple of 8 up to 256"):
+            expected_tensors(config.model_spec())
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_captured_steps_with_prompt_portions_match_plain(tiny_folders, plain, name, dtype):
