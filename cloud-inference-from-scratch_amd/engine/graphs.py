@@ -346,12 +346,12 @@ class MixedGraphs:
         fresh = step is None
         if fresh:
             step = self._layout(shape)
-        self.steps[shape] = step  # (last in the order of use)
         self._fill(step, single, portions)
         if fresh:
-            self._capture(step)
-            while len(self.steps) > self.limit:
-                del self.steps[next(iter(self.steps))]
+            self._capture(step)  # (a capture that fails leaves no half-made entry behind)
+        self.steps[shape] = step  # last in the order of use
+        while len(self.steps) > self.limit:
+            del self.steps[next(iter(self.steps))]
         step.graph.replay()
         self.replays += 1
         row_of = {id(e): index for index, e in enumerate(single)}
