@@ -63,9 +63,10 @@ class StepBatch:
     def max_q_len(self) -> int:
         return max(self.host_q_lens, default=0)
 
-    def tiles(self, tokens_per_tile: int, decode: bool) -> tuple[torch.Tensor, torch.Tensor, int]:
+    def tiles(self, tokens_per_tile: int, decode: bool | None) -> tuple[torch.Tensor, torch.Tensor, int]:
         """Query tiles of at most ``tokens_per_tile`` consecutive tokens of one
-        sequence, for the sequences that bring one token (``decode``) or more:
+        sequence, for the sequences that bring one token (``decode``), more (``decode=False``)
+        or any number (``decode=None``):
         (sequence index of each tile, its first token within the sequence's
         portion, number of tiles), the two lists as int32 device tensors."""
         key = (tokens_per_tile, decode)
@@ -73,7 +74,7 @@ class StepBatch:
             seqs: list[int] = []
             firsts: list[int] = []
             for index, count in enumerate(self.host_q_lens):
-                if (count == 1) != decode:
+                if decode is not None and (count == 1) != decode:
                     continue
                 for first in range(0, count, tokens_per_tile):
                     seqs.append(index)

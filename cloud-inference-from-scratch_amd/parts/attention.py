@@ -115,6 +115,7 @@ FEW_DECODE_UNITS = 8  # (sequence, kv head) pairs below which they do not: parts
 MANY_DECODE_UNITS = 96  # (sequence, kv head) pairs from which decode rows take the four-wave form at any context
 SHARED_DECODE_KEYS = 96  # contexts from which four waves share a decode row's keys without cutting them
 SPLIT_DECODE_KEYS = 192  # contexts from which the keys of decode rows are cut into parts at all
+JOINED_DECODE_ROWS = 32  # up to this many single-token sequences beside prompt portions ride in the prompt form's launch
 PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's keys are cut
 
 
@@ -182,7 +183,8 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         max_keys = plan.max_keys if window is None else min(plan.max_keys, window + 64)
         longest_dev = plan.max_context
         decode_rows = batch.sequences if plan.decode_rows is None else plan.decode_rows
-        if decode_rows:
+        joined = wide and 0 < decode_rows <= JOINED_DECODE_ROWS and decode_rows < batch.sequences
+        if decode_rows and not joined:
             decode_waves, split_options = decode_form(max_keys, decode_rows * num_kv_heads)
             n_splits, _ = plan_splits(decode_rows * num_kv_heads, max_keys, **split_options)
             part_o = part_ml = None
@@ -197,7 +199,11 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         n_tiles = 0  # (of the eager decode form below)
     else:
         tile_seq, tile_q0, n_tiles = batch.tiles(1, decode=True)
-    if n_tiles:
+        # A few single tokens beside prompt portions: one launch (and one merge) of the prompt form for all
+        # sequences instead of two of each (8 decode rows and a 64-token portion of the 3B shape: 4.84 -> 4.49 ms
+        # a step; 32 rows over 3,000 keys and 256 tokens: 8.9 -> 8.2 ms; with 64 such rows the forms are level)
+        joined = wide and 0 < n_tiles <= JOINED_DECODE_ROWS and n_tiles < batch.sequences
+    if n_tiles and not joined:
         decode_waves, split_options = decode_form(max_keys, n_tiles * num_kv_heads)
         n_splits, per_split = plan_splits(n_tiles * num_kv_heads, max_keys, **split_options)
         part_o = part_ml = None
@@ -228,7 +234,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     while 16 * row_tiles < group:
         row_tiles *= 2
     per_tile = (16 * row_tiles) // group
-    tile_seq, tile_q0, n_tiles = batch.tiles(per_tile, decode=False)
+    tile_seq, tile_q0, n_tiles = batch.tiles(per_tile, decode=None if joined else False)
     if n_tiles:
         # few tiles and many keys: parts of the keys, about as many workgroups as compute units
         n_splits, per_split, part_o, part_ml = 1, 0, None, None

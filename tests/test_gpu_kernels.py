@@ -375,6 +375,52 @@ def test_paged_attention_mfma_decode_hundreds_of_parts(ops, geometry):
         torch.testing.assert_close(out, expected, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("joined_rows", [0, 32])
+@pytest.mark.parametrize("geometry", [(16, 2, 128, 16), (28, 4, 128, 16), (6, 2, 64, 32)])
+def test_attention_planning_of_steps_with_single_tokens_beside_portions(ops, geometry, joined_rows, monkeypatch):
+    """The planner of the attention part on a step as a scheduler makes it: four sequences that bring one
+    token over 1 to 3,001 keys beside two prompt portions (one behind 2,000 cached keys), once with two
+    launches (decode form and prompt form) and once with the single tokens riding in the prompt form's
+    launch, against plain attention per sequence."""
+    from cie_amd.engine.batch import PagedView, StepBatch
+    from cie_amd.parts import attention
+
+    monkeypatch.setattr(attention, "JOINED_DECODE_ROWS", joined_rows)
+    q_heads, kv_heads, head_dim, page_size = geometry
+    contexts = [0, 31, 600, 3000, 100, 2000]
+    q_lens = [1, 1, 1, 1, 40, 70]
+    lengths = [c + n for c, n in zip(contexts, q_lens)]
+    k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=95)
+    scale = 1.0 / math.sqrt(head_dim)
+    g = torch.Generator().manual_seed(96)
+    total = sum(q_lens)
+    width = (q_heads + 2 * kv_heads) * head_dim
+    qkv = torch.zeros((total, width), dtype=torch.bfloat16)
+    expected, row = [], 0
+    for s, (c, n) in enumerate(zip(contexts, q_lens)):
+        q = (torch.randn((n, q_heads, head_dim), generator=g) * 2).to(torch.bfloat16)
+        qkv[row: row + n, : q_heads * head_dim] = q.reshape(n, -1)
+        expected.append(plain_qwen2.causal_attention(q.float(), *dense[s], scale, past_len=c))
+        row += n
+    as_dev = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")  # noqa: E731
+    loc = [0]
+    for n in q_lens:
+        loc.append(loc[-1] + n)
+    positions = [c + i for c, n in zip(contexts, q_lens) for i in range(n)]
+    seq_of_token = [s for s, n in enumerate(q_lens) for _ in range(n)]
+    batch = StepBatch(tokens=total, sequences=len(q_lens), token_ids=as_dev([0] * total), positions=as_dev(positions),
+                      seq_of_token=as_dev(seq_of_token), seq_slot=as_dev(slots), seq_start=as_dev(contexts),
+                      seq_q_len=as_dev(q_lens), q_start_loc=as_dev(loc), logit_rows=as_dev([0]),
+                      host_slots=list(slots), host_starts=contexts, host_q_lens=q_lens)
+    view = PagedView(k_pool, v_pool, table, page_size)
+    launches = []
+    real = ops.paged_attention_mfma
+    monkeypatch.setattr(ops, "paged_attention_mfma", lambda *a, **k: (launches.append(k["tokens_per_tile"]), real(*a, **k))[1])
+    out = attention.attend(qkv.cuda(), batch, view, q_heads, kv_heads, head_dim, None, scale)
+    assert len(launches) == (1 if joined_rows else 2), launches
+    torch.testing.assert_close(out.float().cpu(), torch.cat(expected), **tol(torch.bfloat16))
+
+
 def test_paged_attention_mfma_far_key(ops):
     """One key among two thousand carries the weight: output = its value row, in
     the tiled form and in every split layout."""
