@@ -654,7 +654,8 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     return CIE_BAD_ARGUMENT;
 }
 
-// q/k/v product of up to 64 rows with the ROPE epilogue: `w` [N, K] stacks the rows of q_heads query
+// q/k/v product with the ROPE epilogue (64 rows per workgroup; more rows run as more workgroup rows, each
+// streaming the weight again): `w` [N, K] stacks the rows of q_heads query
 // heads, kv_heads key heads and kv_heads value heads of head_dim dimensions each (a multiple of 32);
 // `c` [M, N] receives the rotated queries (its key and value columns are left alone); rotated keys and
 // values go to the cache page of each row's position.  `waves` waves per workgroup share K (1, 2, 4, 8;
@@ -664,7 +665,7 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
                               const int* positions, const int* seq_of_token, const int* seq_slot,
                               const int* block_table, int table_width, void* k_pool, void* v_pool, int q_heads,
                               int kv_heads, int head_dim, int page_size, int rotate, int write_kv) {
-    if (M <= 0 || M > 64 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
+    if (M <= 0 || (M + 63) / 64 > 65535 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
     if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 32 || page_size <= 0 || table_width <= 0 ||
         N != (q_heads + 2 * kv_heads) * head_dim)
         return CIE_BAD_ARGUMENT;
@@ -692,7 +693,7 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
     f.rope = RopeArgs{cos_table, sin_table, positions, seq_of_token, seq_slot, block_table, table_width,
                       static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads, head_dim,
                       page_size, rotate, write_kv};
-    const dim3 grid((q_heads + 2 * kv_heads) * (head_dim / 32), 1, 1);
+    const dim3 grid((q_heads + 2 * kv_heads) * (head_dim / 32), M <= 64 ? 1 : (M + 63) / 64, 1);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (M <= 16) return launch_waves<EPI_ROPE, 1, 2>(s, waves, grid, f);
     if (M <= 32) return launch_waves<EPI_ROPE, 2, 2>(s, waves, grid, f);

@@ -559,7 +559,7 @@ def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Te
                   block_table: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, q_heads: int,
                   kv_heads: int, head_dim: int, rotate: bool = True, write_kv: bool = True,
                   waves: Optional[int] = None) -> torch.Tensor:
-    """The q/k/v product of up to 64 rows fused with what ``rope_kv_write`` does:
+    """The q/k/v product of a few rows (64 per workgroup) fused with what ``rope_kv_write`` does:
     ``a @ weight.T + bias`` for weight [(Hq+2Hkv)*D, K], queries and keys rotated
     by each row's position, keys and values written into the cache.  Returns the
     buffer [M, (Hq+2Hkv)*D] whose query columns hold the rotated queries (its key
@@ -570,8 +570,8 @@ def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Te
     if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
         raise ValueError("a must be a bf16 GPU matrix with unit inner stride")
     m = a.shape[0]
-    if not (1 <= m <= 64 and a.shape[1] == k):
-        raise ValueError(f"a {tuple(a.shape)}: up to 64 rows of K={k}")
+    if not (m >= 1 and a.shape[1] == k):
+        raise ValueError(f"a {tuple(a.shape)}: rows of K={k}")
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
     if not (k % 8 == 0 and lda % 8 == 0):
         raise ValueError(f"K and the row stride must be multiples of 8, are {k} and {lda}")

@@ -1,7 +1,7 @@
 """``x @ W^T + b`` for a Linear's weight ``[out, in]``, and its fused forms.
 
 float32: the hand-written true-float32 kernel, always.  bfloat16 with up to
-``FUSED_ROWS`` rows (decode steps, the output head), and up to 64 rows where
+``FUSED_ROWS`` rows (decode steps, the output head), and up to 64 or 128 rows where
 it is the faster one (a small weight, a long K): the hand-written
 matrix-core kernel that streams the weight once and takes over its neighbours'
 work: a SiLU-gate behind (``epilogue="silu"``), the add into the float32
@@ -26,10 +26,12 @@ from ..kernels import ops
 # product loses from 32 rows on (34 us against 26 + 5 us at 64 rows: every workgroup re-reads the rows of A).
 FUSED_ROWS = 16
 FUSED_PARTS_ROWS = 64
-# With 17 to 64 rows it also wins where the weight is small (q/k/v and o_proj of the 3B shape: 7-9 us against
-# the library's 12-18 us inside a step, and the residual add rides along); from about 6M weight values on the
-# library is faster (7B o_proj at 64 rows: 12.6 us against 11.1 us).
-FUSED_SMALL_ROWS = 64
+# With 17 to 128 rows it also wins where the weight is small (q/k/v and o_proj of the 3B shape: 7-9 us against
+# the library's 12-18 us inside a step at up to 64 rows, 9.3 and 8.2 us against 9.5-12.4 and 9.1 us at 72 and 128
+# rows, where the weight is streamed twice; and the rotation, the cache write, the residual add and the next
+# norm ride along); from about 6M weight values on the library is faster (7B o_proj at 64 rows: 12.6 us against
+# 11.1 us).
+FUSED_SMALL_ROWS = 128
 FUSED_SMALL_WEIGHT = 6 << 20
 # float32 logits of more rows than this go to the library (the hand-written kernel streams the weight once per
 # 64 rows; up to 64 rows it is one pass either way)

@@ -524,7 +524,7 @@ def test_rope_kv_write(ops, dtype, geometry):
 
 
 @pytest.mark.parametrize("geometry", [(16, 2, 128, 16, 2048), (4, 2, 32, 8, 96), (3, 1, 64, 4, 328), (5, 5, 96, 32, 200)])
-@pytest.mark.parametrize("rows", [1, 7, 16, 24, 40, 64])
+@pytest.mark.parametrize("rows", [1, 7, 16, 24, 40, 64, 72, 100, 128])
 @pytest.mark.parametrize("waves", [None, 1, 8])
 def test_gemm_qkv_rope_equals_product_then_rotation(ops, geometry, rows, waves):
     """The q/k/v product whose epilogue rotates and writes the cache, against the plain
@@ -535,7 +535,7 @@ def test_gemm_qkv_rope_equals_product_then_rotation(ops, geometry, rows, waves):
     row_tiles = 1 if rows <= 16 else 2 if rows <= 32 else 4
     if waves == 1 and row_tiles > 1:
         waves = 4  # the fewest with more than 16 rows
-    lengths = [40, 25, 100, 17][: max(1, min(4, rows))]  # every sequence has at least rows / 4 tokens
+    lengths = [40, 35, 100, 33][: max(1, min(4, rows))]  # every sequence has at least rows / 4 tokens
     k_pool, v_pool, table, slots, _ = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=44)
     k_two, v_two = k_pool.clone(), v_pool.clone()
     # the rows: the last tokens of the sequences in turn (decode rows), several per sequence when rows > sequences
