@@ -201,8 +201,8 @@ class MixedGraphs:
     """Steps that bring short prompt portions (beside decode tokens or alone) as captured graphs.
 
     Such a step is a few hundred launches too, and with few tokens the host cannot queue them as fast as the
-    GPU runs them (8 decode rows and a 64-token portion of the 3B shape: 5.6 ms launch by launch, 4.7 ms
-    replayed; with a 256-token portion the GPU is the slower one either way, 7.6 ms).  A capture costs as
+    GPU runs them (8 decode rows and a 32-token portion of the 3B shape: 4.1 ms launch by launch, 3.6 ms
+    replayed; with a 64-token portion 4.4 and 4.2 ms; with 256 tokens the GPU is the slower one either way).  A capture costs as
     much as ten such steps, so only shapes that come again are captured: a step's shape is (bucket of its
     single-token rows, the lengths of its portions); one that comes a second time (the portions of one
     long prompt beside the same decoding requests do) is captured from that very step, with its real
