@@ -411,7 +411,7 @@ def plan_fused(rows: int, column_tiles: int, k: int, k_parts: int = 1) -> tuple[
     takes to fill the GPU, each with at least one 128-wide slice."""
     row_tiles = 1 if rows <= 16 else 2 if rows <= 32 else 4
     pair = row_tiles > 1 and column_tiles * k_parts >= 2 * FUSED_PAIR_WORKGROUPS
-    groups = (-(-column_tiles // 2) if pair else column_tiles) * k_parts
+    groups = (-(-column_tiles // 2) if pair else column_tiles) * k_parts * -(-rows // FUSED_MAX_ROWS)
     waves = 1 if row_tiles == 1 else 4
     while waves < 8 and groups * waves < FUSED_TARGET_WAVES and waves * 2 * 128 <= k:
         waves *= 2

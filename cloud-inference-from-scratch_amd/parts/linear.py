@@ -26,6 +26,11 @@ from ..kernels import ops
 # product loses from 32 rows on (34 us against 26 + 5 us at 64 rows: every workgroup re-reads the rows of A).
 FUSED_ROWS = 16
 FUSED_PARTS_ROWS = 64
+# ... and up to 128 rows where the weight has few columns, which leave the library few tiles to spread (a step
+# of 72 rows: 3B shape, 128 column tiles, 4.38 -> 4.17 ms; 7B, 224 tiles, 7.5 -> 6.4 ms; 14B, 320 tiles,
+# 10.8 -> 11.6 ms: there the library stays)
+FUSED_PARTS_ROWS_NARROW = 128
+PARTS_NARROW_TILES = 256
 # With 17 to 128 rows it also wins where the weight is small (q/k/v and o_proj of the 3B shape: 7-9 us against
 # the library's 12-18 us inside a step at up to 64 rows, 9.3 and 8.2 us against 9.5-12.4 and 9.1 us at 72 and 128
 # rows, where the weight is streamed twice; and the rotation, the cache write, the residual add and the next
@@ -120,7 +125,7 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     wants_f32 = out_dtype == torch.float32
     fusable = _fusable(rows, k, x.stride(0) if rows > 1 else k, weight)
     cut_k = into is not None and -(-n // 16) < PART_BELOW_TILES and k >= 2 * PART_K
-    if fusable and cut_k and rows <= FUSED_PARTS_ROWS:
+    if fusable and cut_k and rows <= (FUSED_PARTS_ROWS_NARROW if -(-n // 16) < PARTS_NARROW_TILES else FUSED_PARTS_ROWS):
         return PartialSum(ops.gemm_fused(weight, ops.EPI_PARTIAL, x, bias=bias, k_parts=-(-k // PART_K)))
     if fusable and wants_f32 and rows > FUSED_LOGIT_ROWS and into is None and not silu and bias is None:
         out = ops.gemm_library(x, weight, out_dtype=torch.float32)  # logits of many rows: one pass over the weight

@@ -695,7 +695,8 @@ def test_gemm_fused_random_shapes(ops):
 
 
 @pytest.mark.parametrize("shape", [(1, 64, 256), (8, 2048, 11008), (13, 96, 328), (16, 48, 1032), (40, 200, 1032),
-                                   (64, 2048, 2752), (5, 50, 264), (8, 3584, 1024)])
+                                   (64, 2048, 2752), (5, 50, 264), (8, 3584, 1024), (72, 2048, 11008), (100, 200, 1032),
+                                   (128, 96, 328), (200, 48, 264)])
 @pytest.mark.parametrize("k_parts", [1, 3, 4])
 def test_gemm_fused_partial_products_and_their_norm(ops, shape, k_parts):
     """K cut into parts: the float32 partial products sum to the product (bias once), and the
