@@ -171,5 +171,7 @@ class Engine:
             "max_forward_request_count": getattr(runner, "max_forward_request_count", 0),
             "graph_captures": getattr(runner, "graph_captures", 0),
             "graph_replays": getattr(runner, "graph_replays", 0),
+            "mixed_graph_captures": getattr(runner, "mixed_graph_captures", 0),
+            "mixed_graph_replays": getattr(runner, "mixed_graph_replays", 0),
         }
         return snapshot

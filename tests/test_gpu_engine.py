@@ -219,6 +219,8 @@ def test_random_requests_through_a_small_pool_equal_each_request_alone(tiny_fold
     metrics = busy.snapshot_metrics()
     assert metrics["requests"]["preempted_total"] > 0 and metrics["kv_cache"]["prefix_cache_hits"] > 0
     assert metrics["kv_cache"]["request_pages_used"] == 0
+    # (portions of 7 tokens beside the same few decoding requests: shapes of steps that come again and are captured)
+    assert metrics["runner"]["mixed_graph_replays"] > 0 and metrics["runner"]["graph_replays"] > 0
     busy.runner.cache.assert_invariants()
     alone = make_engine(folder, page_size=16, kv_tokens=2 * limit, max_running=1, max_model_len=limit,
                         max_output_tokens=64, graph_decode=False, async_decode=False)
