@@ -158,7 +158,7 @@ def test_attention_part_whole_and_in_portions(dtype, rotary):
 
 
 @pytest.mark.parametrize("part_k", [None, 32])
-@pytest.mark.parametrize("rows", [13, 40])
+@pytest.mark.parametrize("rows", [13, 40, 72, 100])
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_block_part(dtype, rows, part_k, monkeypatch):
     """norm -> mixer -> add -> norm -> feed-forward, the add of the second branch left pending
@@ -172,7 +172,7 @@ def test_block_part(dtype, rows, part_k, monkeypatch):
 
     raw = dict(model_type="qwen2", hidden_size=48, num_hidden_layers=1, num_attention_heads=3,
                num_key_value_heads=3, intermediate_size=88, vocab_size=32, rms_norm_eps=1e-5, rope_theta=1e4,
-               max_position_embeddings=64)
+               max_position_embeddings=128)
     spec = Qwen2Config.from_hf_config(raw).model_spec().layers[0]
     block = PreNormBlock(spec)
     w = bound(block, "model.layers.0.", dtype, 5, scale=0.3)
