@@ -187,3 +187,25 @@ def compare(rows: dict[str, dict[int, np.ndarray]], plain: dict[str, torch.Tenso
                 f"max |diff| there {diff[positions.index(pos)].max():.3e}, overall {diff.max():.3e}"
             )
     return worst
+
+
+def closer_than_plain_bfloat16(rows: dict[str, dict[int, np.ndarray]], plain: dict[str, torch.Tensor],
+                               rough: dict[str, torch.Tensor]) -> tuple[float, float, float, float]:
+    """What bfloat16 costs at a model's widths is measured, not assumed: ``rough`` are the logits of the plain
+    implementation run in bfloat16 throughout, ``plain`` those in float32.  The engine (float32 residual
+    stream, softmax and sums) has to be closer to the float32 logits than that: root mean square no larger,
+    worst difference at most 1.5 times.  Returns (rms, worst, plain rms, plain worst)."""
+    def errors(logits_of):
+        square, count, worst = 0.0, 0, 0.0
+        for rid, by_pos in rows.items():
+            for pos in by_pos:
+                diff = logits_of(rid, pos) - plain[rid][pos]
+                square += float((diff ** 2).sum())
+                count += diff.numel()
+                worst = max(worst, float(diff.abs().max()))
+        return (square / count) ** 0.5, worst
+
+    plain_rms, plain_worst = errors(lambda rid, pos: rough[rid][pos].float())
+    rms, worst = errors(lambda rid, pos: torch.from_numpy(rows[rid][pos]))
+    assert rms <= plain_rms and worst <= 1.5 * plain_worst, (rms, worst, plain_rms, plain_worst)
+    return rms, worst, plain_rms, plain_worst

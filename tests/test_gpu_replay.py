@@ -153,6 +153,42 @@ ODD_SIZES = [  # hidden, heads, kv heads, head_dim, intermediate, vocabulary
 ]
 
 
+HEAD_SIZES = [  # head sizes and group sizes the matrix-core attention takes (pages of 16 tokens: its four-wave forms)
+    (64, 2, 1, 32, 40, 97),      # two heads on one key head
+    (192, 3, 3, 64, 100, 300),   # no grouping
+    (96, 7, 1, 96, 64, 211),     # seven heads on one key head: rows of a tile that are no power of two
+    (256, 16, 2, 128, 300, 515),
+    (128, 10, 2, 64, 72, 130),   # groups of five
+    (512, 16, 1, 32, 64, 97),    # sixteen heads on one key head: a tile's rows are one token
+]
+
+
+@pytest.mark.parametrize("schedule", ["portions", "mixed"])
+@pytest.mark.parametrize("sizes", HEAD_SIZES, ids=lambda s: "x".join(map(str, s)))
+def test_replay_at_the_head_sizes_of_the_matrix_core_attention(tmp_path, sizes, schedule):
+    """bfloat16 with pages of 16 tokens, where prompt portions and decode rows take the tiled attention
+    forms (and, side by side, one launch for both): portions of changing size and a mixed schedule with
+    reused pages at several head and group sizes, to the plain model's logits."""
+    from conftest import TINY_C, make_folder
+
+    hidden, heads, kv_heads, head_dim, intermediate, vocab = sizes
+    raw = dict(TINY_C, hidden_size=hidden, num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=head_dim,
+               intermediate_size=intermediate, vocab_size=vocab, eos_token_id=1, attention_bias=True)
+    folder, tensors = make_folder(tmp_path, raw, seed=4)
+    requests = {f"r{i}": random_tokens(n, vocab, seed=60 + i) for i, n in enumerate((9, 47, 130, 200))}
+    expected = plain_all(raw, tensors, requests)
+    steps = SCHEDULES[schedule](requests)
+    pool = replay_util.max_live_tokens(steps, page=16)
+    runner = make_runner(folder, "bfloat16", pool, 16, max_running=4)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    # (peaked softmaxes at widths of hundreds: the yardstick is the plain implementation run in bfloat16)
+    weights = {k: v.float() for k, v in tensors.items()}
+    rough = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
+    print(sizes, schedule, "rms %.3e worst %.3e, plain in bfloat16 %.3e %.3e"
+          % replay_util.closer_than_plain_bfloat16(rows, expected, rough), flush=True)
+    assert runner.cache.stats().pages_used == 0
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("sizes", ODD_SIZES, ids=lambda s: "x".join(map(str, s)))
 def test_replay_at_odd_sizes(tmp_path, sizes, dtype):
@@ -425,24 +461,12 @@ def test_replay_at_the_sizes_of_real_models(tmp_path_factory, shape, layers, voc
         # bfloat16 keeps 8 bits, and at these widths a logit sums 896 to 2,048 rounded values: what that costs is
         # measured, not assumed: the plain implementation run in bfloat16 throughout is the yardstick, and the
         # engine (float32 residual stream, softmax and sums) has to be closer to the float32 logits than it is
-        def errors(logits_of):
-            square, count, worst = 0.0, 0, 0.0
-            for rid, by_pos in rows.items():
-                for pos in by_pos:
-                    diff = logits_of(rid, pos) - expected[rid][pos]
-                    square += float((diff ** 2).sum())
-                    count += diff.numel()
-                    worst = max(worst, float(diff.abs().max()))
-            return (square / count) ** 0.5, worst
-
         weights = {k: v.float() for k, v in tensors.items()}
         rough = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
         del weights
-        plain_rms, plain_worst = errors(lambda rid, pos: rough[rid][pos])
-        rms, worst = errors(lambda rid, pos: torch.from_numpy(rows[rid][pos]))
+        rms, worst, plain_rms, plain_worst = replay_util.closer_than_plain_bfloat16(rows, expected, rough)
         print(f"{shape} x {layers} layers bfloat16: root mean square {rms:.3e} (plain in bfloat16 {plain_rms:.3e}), "
               f"worst {worst:.3e} ({plain_worst:.3e})", flush=True)
-        assert rms <= plain_rms and worst <= 1.5 * plain_worst
     assert runner.cache.stats().pages_used == 0
 
 
