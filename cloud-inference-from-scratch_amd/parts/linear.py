@@ -123,6 +123,8 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     n = weight.shape[0]
     silu = epilogue == "silu"
     wants_f32 = out_dtype == torch.float32
+    if rows == 0 and into is None:  # nothing to multiply: no kernel, and no widened copy of the weight
+        return torch.empty((0, n // 2 if silu else n), dtype=torch.float32 if wants_f32 else x.dtype, device=x.device)
     fusable = _fusable(rows, k, x.stride(0) if rows > 1 else k, weight)
     cut_k = into is not None and -(-n // 16) < PART_BELOW_TILES and k >= 2 * PART_K
     if fusable and cut_k and rows <= (FUSED_PARTS_ROWS_NARROW if -(-n // 16) < PARTS_NARROW_TILES else FUSED_PARTS_ROWS):

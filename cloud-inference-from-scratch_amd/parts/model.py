@@ -117,5 +117,7 @@ class DecoderModel:
         for call in self.spec.order:
             residual, pending = self.blocks[call.layer].forward(
                 residual, pending, batch, cache.view(call.cache), call.writes)
+        if batch.logit_rows.shape[0] == 0:  # a step of prompt portions that end before their prompts do
+            return torch.empty((0, self.head.shape[0]), dtype=torch.float32, device=residual.device)
         selected = normalise(self.final_norm, residual, pending, self.dtype, rows=batch.logit_rows)
         return linear(selected, self.head, None, out_dtype=torch.float32)
