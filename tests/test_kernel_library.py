@@ -27,3 +27,18 @@ def test_a_parameter_that_is_not_understood_is_an_error(tmp_path, monkeypatch, p
     monkeypatch.setattr(library, "sources", lambda: [source])
     with pytest.raises(library.KernelLibraryError, match="cie_odd"):
         library.entry_point_signatures()
+
+
+def test_a_product_of_no_rows_launches_nothing_and_widens_nothing():
+    """Steps of prompt portions that end before their prompts want no logits: the output head is given no
+    rows.  No kernel runs (none could, here without a GPU) and the weight is not touched."""
+    import torch
+
+    from cie_amd.parts.linear import linear
+
+    weight = torch.zeros((32, 16), dtype=torch.bfloat16)
+    rows = torch.empty((0, 16), dtype=torch.bfloat16)
+    logits = linear(rows, weight, None, out_dtype=torch.float32)
+    assert logits.shape == (0, 32) and logits.dtype == torch.float32
+    gated = linear(rows, weight, None, epilogue="silu")
+    assert gated.shape == (0, 16) and gated.dtype == torch.bfloat16
