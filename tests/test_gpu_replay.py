@@ -386,14 +386,17 @@ def test_trace_run_program(tiny_folders, plain, tmp_path, dtype):
     steps = replay_util.mixed(requests, live=4, seed=3)
     pool = replay_util.max_live_tokens(steps, page=64)
     out_dir = tmp_path / "out"
-    text = "\n".join(json.dumps(step) for step in steps) + "\n"
+    # (first a step whose only request brings nothing and ends: it is answered and leaves no file)
+    idle = {"step": 999, "entries": [{"id": "ghost", "tokens": [], "want": []}], "end": ["ghost"]}
+    text = "\n".join(json.dumps(step) for step in [idle] + steps) + "\n"
     done = subprocess.run(
         [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype", dtype,
          "--out", str(out_dir), "--max-tokens", str(pool)],
         input=text, capture_output=True, text=True, timeout=600)
     assert done.returncode == 0, done.stderr[-3000:]
     lines = [line for line in done.stdout.splitlines() if line.startswith("done ")]
-    assert lines == [f"done {step['step']}" for step in steps]
+    assert lines == ["done 999"] + [f"done {step['step']}" for step in steps]
+    assert not (out_dir / "999.f32").exists()
     vocab = raw["vocab_size"]
     outputs = {}
     for step in steps:
