@@ -114,6 +114,7 @@ WIDE_TARGET_WORKGROUPS = 256  # workgroups the four-wave form cuts long contexts
 FEW_DECODE_UNITS = 8  # (sequence, kv head) pairs below which they do not: parts of one wave fill the GPU better
 MANY_DECODE_UNITS = 96  # (sequence, kv head) pairs from which decode rows take the four-wave form at any context
 SHARED_DECODE_KEYS = 96  # contexts from which four waves share a decode row's keys without cutting them
+SPLIT_MIN_KEYS = 32  # the fewest keys of a one-wave part
 SPLIT_DECODE_KEYS = 192  # contexts from which the keys of decode rows are cut into parts at all
 JOINED_DECODE_ROWS = 32  # up to this many single-token sequences beside prompt portions ride in the prompt form's launch
 PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's keys are cut
@@ -168,7 +169,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         # Otherwise one wave per part, parts down to one block of 32 keys (8 x 256 keys: 7.3 us in 8 parts,
         # 10.2 us in 2; 8 x 512 keys: 8.1 us in 16 parts, 10.6 us in 4) ...
         if bound >= SPLIT_DECODE_KEYS:
-            return 1, dict(target_waves=1024, min_keys=32)
+            return 1, dict(target_waves=1024, min_keys=SPLIT_MIN_KEYS)
         # ... and below some 200 keys, where the merge costs more than it saves, four waves that share a
         # sequence's few blocks inside one workgroup instead of one wave that takes them in turn
         # (8 x 128 keys: 6.5 against 6.9 us, 8 x 160: 7 against 11)
