@@ -68,7 +68,7 @@ def make_engine(config, dtype, batch, context, prefill_tokens, seed=0):
         max_output_tokens=context, token_budget=max(2048, batch), prefill_chunk=2048,
         prefix_cache_pages=0, draw_device="cuda",
         # fill all caches before decoding starts, so that the timed steps are pure decode steps
-        scheduling_priority=lambda candidate: (candidate.phase == "decode",),
+        plan_order=lambda standing: (standing.decoding,),
     )
 
 
@@ -101,8 +101,8 @@ def time_decode(engine, config, batch: int, context: int, steps: int, warmup: in
     elapsed = time.perf_counter() - start
     for r in requests:
         # (with decode steps started ahead of their tokens, the last step's token is still on its way)
-        assert not r.is_terminal and r.generated_count >= warmup + steps - 1, (r.state, r.generated_count)
-    mean_context = sum(r.tokens_fed for r in requests) / batch - steps / 2.0
+        assert not r.is_final and len(r.output) >= warmup + steps - 1, (r.state, len(r.output))
+    mean_context = sum(r.cached for r in requests) / batch - steps / 2.0
     for r in requests:
         engine.scheduler.cancel(r)
     return elapsed, mean_context
@@ -120,7 +120,7 @@ def time_prefill(engine, config, tokens: int, seed: int, repeats: int = 3):
         request = engine.submit(prompt, GenerationConfig(max_output_tokens=1, eos_token_id=None))
         torch.cuda.synchronize()
         start = time.perf_counter()
-        while not request.is_terminal:
+        while not request.is_final:
             engine.step()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - start

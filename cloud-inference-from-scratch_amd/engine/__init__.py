@@ -1,25 +1,13 @@
 from .batch import PagedView, StateView, StepBatch
 from .engine import Engine, GenerationResult
 from .loading import build_model, load_model, random_model
+from .plan import Portion, Standing, StepPlan, decodes_before_prompts, most_resident_gives_way
+from .request import GenerationConfig, Refusal, RejectedError, Request, RequestState
 from .runner import Runner, StepEntry
-from .scheduler import (
-    BatchItem,
-    BatchPlan,
-    GenerationConfig,
-    PreemptionCandidate,
-    RejectedError,
-    RejectionReason,
-    Request,
-    RequestState,
-    Scheduler,
-    SchedulingCandidate,
-    decode_first_priority,
-    largest_sequence_preemption,
-)
+from .scheduler import Scheduler
 
 __all__ = [
-    "BatchItem", "BatchPlan", "Engine", "GenerationConfig", "GenerationResult", "PagedView",
-    "PreemptionCandidate", "RejectedError", "RejectionReason", "Request", "RequestState", "Runner",
-    "Scheduler", "SchedulingCandidate", "StateView", "StepBatch", "StepEntry", "build_model",
-    "decode_first_priority", "largest_sequence_preemption", "load_model", "random_model",
+    "Engine", "GenerationConfig", "GenerationResult", "PagedView", "Portion", "Refusal", "RejectedError",
+    "Request", "RequestState", "Runner", "Scheduler", "Standing", "StateView", "StepBatch", "StepEntry",
+    "StepPlan", "build_model", "decodes_before_prompts", "load_model", "most_resident_gives_way", "random_model",
 ]

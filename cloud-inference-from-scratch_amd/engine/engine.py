@@ -19,14 +19,9 @@ from ..config.engine_config import EngineConfig, build_engine_config
 from ..metrics import Metrics
 from .loading import load_model, random_model
 from .runner import Runner
-from .scheduler import (
-    GenerationConfig,
-    Request,
-    RequestState,
-    Scheduler,
-    decode_first_priority,
-    largest_sequence_preemption,
-)
+from .plan import decodes_before_prompts, most_resident_gives_way
+from .request import GenerationConfig, Request, RequestState
+from .scheduler import Scheduler
 
 
 @dataclass
@@ -50,7 +45,7 @@ class Engine:
                  engine_config: EngineConfig | None = None, device: str = "cuda:0",
                  draw_device: str = "cpu",
                  runner_factory: Callable[[EngineConfig], Any] | None = None,
-                 scheduling_priority=decode_first_priority, preemption_priority=largest_sequence_preemption,
+                 plan_order=decodes_before_prompts, victim_order=most_resident_gives_way,
                  **options: Any) -> None:
         self.engine_config = build_engine_config(engine_config, **options)
         self.model_dir = Path(model_dir) if model_dir is not None else None
@@ -74,8 +69,7 @@ class Engine:
             self.runner = Runner(self.model, self.engine_config, device)
         self.metrics = Metrics()
         self.scheduler = Scheduler(self.engine_config, self.runner, self.metrics,
-                                   scheduling_priority=scheduling_priority,
-                                   preemption_priority=preemption_priority)
+                                   plan_order=plan_order, victim_order=victim_order)
 
     # -- text ------------------------------------------------------------------------
     def _tokenizer(self) -> Any:
@@ -125,17 +119,17 @@ class Engine:
 
     def result_of(self, request: Request) -> GenerationResult:
         if request.state is not RequestState.COMPLETED:
-            raise RuntimeError(f"generation {request.state.value}: {request.error_detail or request.finish_reason}")
-        end = request.finish_ns or time.monotonic_ns()
+            raise RuntimeError(f"generation {request.state.value}: {request.error or request.finish_reason}")
+        end = request.ended_ns or time.monotonic_ns()
         return GenerationResult(
             request_id=request.request_id,
-            text=self.detokenize(request.generated_token_ids),
-            token_ids=list(request.generated_token_ids),
-            input_tokens=len(request.prompt_token_ids),
-            output_tokens=request.generated_count,
+            text=self.detokenize(request.output),
+            token_ids=list(request.output),
+            input_tokens=len(request.prompt),
+            output_tokens=len(request.output),
             finish_reason=request.finish_reason,
-            ttft_ms=(request.first_token_ns - request.arrival_ns) / 1e6 if request.first_token_ns else None,
-            e2e_ms=(end - request.arrival_ns) / 1e6,
+            ttft_ms=(request.first_token_ns - request.arrived_ns) / 1e6 if request.first_token_ns else None,
+            e2e_ms=(end - request.arrived_ns) / 1e6,
         )
 
     def generate(self, prompts: Sequence[str | Sequence[int]],

@@ -94,10 +94,10 @@ class Runner:
 
     # -- what the scheduler calls ------------------------------------------------
     def admit(self, request: Any) -> None:
-        request.tokens_fed = self.cache.admit(request.request_id, request.prompt_token_ids)
+        request.cached = self.cache.admit(request.request_id, request.prompt)
 
     def release(self, request: Any, preempted: bool = False) -> None:
-        self.cache.release(request.request_id, None if preempted else request.prompt_token_ids)
+        self.cache.release(request.request_id, None if preempted else request.prompt)
 
     def warm_up(self) -> int:
         """Do now what the first steps would otherwise do on the clock: capture the decode graphs of
@@ -115,7 +115,7 @@ class Runner:
     def publish_prefix(self, request: Any) -> None:
         """The request's prompt is in the cache: offer its full pages to the prefix index now, not only
         when it ends (the reference stores at release, src/cloud_engine/engine.py:224-226)."""
-        self.cache.publish_prefix(request.request_id, request.prompt_token_ids)
+        self.cache.publish_prefix(request.request_id, request.prompt)
 
     def allocated_tokens(self, request: Any) -> int:
         return self.cache.allocated_tokens(request.request_id)
@@ -144,24 +144,24 @@ class Runner:
         """Run a scheduler's plan and sample where it asks to (the reference's
         ``execute_batch``, src/cloud_engine/engine.py:439-488)."""
         entries = [
-            StepEntry(item.request.request_id, item.token_ids, item.start_pos,
-                      (item.query_length - 1,) if item.sample else ())
-            for item in plan.items
+            StepEntry(portion.request.request_id, portion.tokens, portion.start,
+                      (portion.length - 1,) if portion.samples else ())
+            for portion in plan.portions
         ]
         logits = self.run(entries)
-        for item in plan.items:
-            item.request.tokens_fed = item.end_pos
-        sampled = [item.request for item in plan.items if item.sample]
-        if not sampled:
+        for portion in plan.portions:
+            portion.request.cached = portion.end
+        sampling = [portion.request for portion in plan.portions if portion.samples]
+        if not sampling:
             return {}
         with trace_range("ragged.sample"):
             tokens = self.sampler.sample(
                 logits,
-                [r.config.temperature for r in sampled],
-                [self.sampler.uniform(r.config.seed, r.serial, r.generated_count) if r.config.temperature > 0 else 0.0
-                 for r in sampled],
+                [r.gen.temperature for r in sampling],
+                [self.sampler.uniform(r.gen.seed, r.serial, len(r.output)) if r.gen.temperature > 0 else 0.0
+                 for r in sampling],
             )
-        return {r.request_id: token for r, token in zip(sampled, tokens)}
+        return {r.request_id: token for r, token in zip(sampling, tokens)}
 
     # -- decode steps that do not wait for their tokens -----------------------------------
     def can_launch_decode(self, requests: int) -> bool:
@@ -171,22 +171,22 @@ class Runner:
     def launch_decode(self, plan: Any, feed: Sequence[int], token_indices: Sequence[int]) -> "PendingTokens":
         """Start a step in which every request brings one token and samples, and return at once.
 
-        ``feed[i] >= 0``: item i's token is the one the launch before this sampled at that place (it is
-        still on the device; the item's own token id is a placeholder).  ``token_indices[i]`` is the index of
-        the token item i is about to generate (what its random draw depends on).  The sampled tokens stay
+        ``feed[i] >= 0``: portion i's token is the one the launch before this sampled at that place (it is
+        still on the device; the portion's own token id is a placeholder).  ``token_indices[i]`` is the index of
+        the token portion i is about to sample (what its random draw depends on).  The sampled tokens stay
         on the device for the next launch and travel to the host behind the step;
         :meth:`PendingTokens.tokens` waits for them."""
-        assert self.graphs is not None and all(item.query_length == 1 and item.sample for item in plan.items)
-        entries = [StepEntry(item.request.request_id, item.token_ids, item.start_pos, (0,)) for item in plan.items]
+        assert self.graphs is not None and all(p.length == 1 and p.samples for p in plan.portions)
+        entries = [StepEntry(p.request.request_id, p.tokens, p.start, (0,)) for p in plan.portions]
         logits = self.run(entries, feed=feed)
-        requests = [item.request for item in plan.items]
-        for item in plan.items:
-            item.request.tokens_fed = item.end_pos
+        requests = [p.request for p in plan.portions]
+        for p in plan.portions:
+            p.request.cached = p.end
         with trace_range("ragged.sample"):
             pool = self.graphs.token_pool[: len(requests)]
             self.sampler.sample_on_device(
-                logits, [r.config.temperature for r in requests],
-                [self.sampler.uniform(r.config.seed, r.serial, index) if r.config.temperature > 0 else 0.0
+                logits, [r.gen.temperature for r in requests],
+                [self.sampler.uniform(r.gen.seed, r.serial, index) if r.gen.temperature > 0 else 0.0
                  for r, index in zip(requests, token_indices)],
                 out=pool)
             host = torch.empty(len(requests), dtype=torch.int32, pin_memory=True)

@@ -1,25 +1,33 @@
-"""Request lifecycle and the iteration-level scheduler.
+"""The iteration-level scheduler: which requests run in the next step, with how
+many tokens each, and what happens when the pool cannot hold them.
 
-The policy is the reference's packed scheduler (src/cloud_engine/scheduler.py):
-one state machine ``waiting -> prefill -> decoding -> completed | cancelled |
-failed`` (:29-46); FIFO admission up to ``max_running`` (:438-457); each
-iteration builds one plan under a shared token budget, decodes first, prompts
-cut into portions of at most ``prefill_chunk`` tokens (:459-518); a sampled
-token becomes the next iteration's one-token input (:581-607); EOS or
-``max_output_tokens`` finishes a request (:593-605).  It is synchronous: the
-caller drives :meth:`Scheduler.step`; streams, time-outs and the asyncio loop of
-the reference belong to its server and are not here.
+The policy is that of the reference's packed scheduler
+(src/cloud_engine/scheduler.py): requests are admitted in the order they came,
+up to ``max_running`` (:438-457); every iteration shares one token budget, the
+requests that decode go first and prompts are cut into portions of at most
+``prefill_chunk`` tokens (:459-518); only a portion that reaches the request's
+last known token samples (:513); the sampled token is the next iteration's
+one-token portion, and an end-of-sequence token or ``max_output_tokens`` ends
+the request (:581-607).  The loop is the caller's: :meth:`Scheduler.step` is one
+iteration.  Streams, time-outs and the asyncio task of the reference belong to
+its server and are not here.
 
-When pages run out (:527-553): the step raised a capacity error before changing
-anything; the live request with the largest ``preemption_priority`` (most
-resident tokens first) gives back all its pages and slot, keeps its generated
-tokens, and goes to the *front* of the waiting queue with ``tokens_fed = 0``; it
-is recomputed (prompt and generated tokens fed as prompt portions, sampling only
-at the tail) once the pool has room for it again or nothing else is running.
-The reference re-admits it only when nothing else runs and blocks the queue
-behind it meanwhile (:443-446); here the queue is blocked too (a preempted
-request keeps its seniority), but room in the pool suffices.  If a single live
-request cannot get its pages, it fails with ``rejected`` set.
+**When pages run out** the step function has refused the plan before it changed
+anything.  The live request that ranks highest under ``victim_order`` (most
+resident tokens, as in the reference, :197-199, :527-553) gives back its pages
+and its slot, keeps the tokens it has produced, and returns to the *front* of
+the waiting queue; it comes back when the pool has room for everything known of
+it beside what the admitted requests still have to take, or when nothing else
+runs, and then rebuilds its cache from prompt + output as prompt portions.  (The
+reference puts it at the back and lets it in only once nothing runs, :443-446.)
+While it waits nobody behind it is admitted: it keeps its seniority.  A lone
+request that cannot get its pages fails as ``rejected``.
+
+**Decode steps in flight** (``async_decode``): a plan of single sampled tokens is
+only started; the next call first starts the step that follows it, whose rows
+take their tokens from the device, and then collects the tokens of the step
+before.  Requests leave the follow-up in time when their token limit is in
+sight; an end-of-sequence token is seen one step late and costs one dropped row.
 """
 
 from __future__ import annotations
@@ -28,513 +36,340 @@ import inspect
 import time
 from collections import deque
 from collections.abc import Callable, Sequence
-from dataclasses import dataclass, field
-from enum import Enum
 from typing import Any
 
 from ..profiling import trace_range
+from .plan import Portion, Standing, StepPlan, decodes_before_prompts, most_resident_gives_way
+from .request import GenerationConfig, Refusal, RejectedError, Request, RequestState
+
+__all__ = ["GenerationConfig", "Portion", "Refusal", "RejectedError", "Request", "RequestState", "Scheduler",
+           "Standing", "StepPlan", "decodes_before_prompts", "most_resident_gives_way"]
+
+Order = Callable[[Standing], tuple[Any, ...]]
 
 
-class RequestState(Enum):
-    WAITING = "waiting"
-    PREFILL = "prefill"
-    DECODING = "decoding"
-    COMPLETED = "completed"
-    CANCELLED = "cancelled"
-    FAILED = "failed"
+def _is_shortage(error: BaseException) -> bool:
+    """The step function marks "no pages left" with an attribute, not a type, so that a
+    scheduler needs nothing of the cache's modules (src/cloud_engine/scheduler.py:384)."""
+    return bool(getattr(error, "is_capacity_error", False))
 
 
-TERMINAL_STATES = frozenset({RequestState.COMPLETED, RequestState.CANCELLED, RequestState.FAILED})
+class _InFlight:
+    """A started decode step: its plan, and the handle its tokens arrive through."""
 
+    __slots__ = ("plan", "handle")
 
-class RejectionReason(Enum):
-    QUEUE_FULL = "queue_full"
-    KV_CAPACITY = "capacity_exhausted"
-    CONTEXT_OVERFLOW = "context_length_exceeded"
-
-
-class RejectedError(RuntimeError):
-    def __init__(self, reason: RejectionReason, detail: str = "") -> None:
-        super().__init__(detail or reason.value)
-        self.reason = reason
-
-
-@dataclass
-class GenerationConfig:
-    """``temperature == 0`` is greedy (all the reference samples with,
-    src/cloud_engine/scheduler.py:63-71); ``temperature > 0`` draws from
-    softmax(logits / temperature) with a generator keyed by ``seed`` and the
-    token's index, so a request's draws do not depend on its batch.
-    ``eos_token_id is None`` ignores EOS."""
-
-    max_output_tokens: int
-    temperature: float = 0.0
-    eos_token_id: int | None = None
-    seed: int | None = None
-
-    def __post_init__(self) -> None:
-        if self.max_output_tokens < 1:
-            raise ValueError("max_output_tokens must be positive")
-        if not self.temperature >= 0:
-            raise ValueError("temperature must be zero (greedy) or positive")
-
-
-@dataclass
-class Request:
-    request_id: str
-    prompt_token_ids: list[int]
-    config: GenerationConfig
-    arrival_ns: int
-    serial: int = 0
-    label: str = ""
-    state: RequestState = RequestState.WAITING
-    generated_token_ids: list[int] = field(default_factory=list)
-    tokens_fed: int = 0
-    first_token_ns: int | None = None
-    last_token_ns: int | None = None
-    finish_ns: int | None = None
-    finish_reason: str = ""
-    error_detail: str = ""
-    rejected: bool = False
-    preemption_count: int = 0
-    recomputed_tokens: int = 0
-    recompute_until: int = 0
-    on_token: Callable[["Request", int], None] | None = None
-
-    @property
-    def is_terminal(self) -> bool:
-        return self.state in TERMINAL_STATES
-
-    @property
-    def generated_count(self) -> int:
-        return len(self.generated_token_ids)
-
-
-@dataclass(frozen=True)
-class BatchItem:
-    """One sequence's token slice in a shared iteration."""
-
-    request: Request
-    token_ids: tuple[int, ...]
-    start_pos: int
-    sample: bool
-    is_decode: bool
-
-    @property
-    def query_length(self) -> int:
-        return len(self.token_ids)
-
-    @property
-    def end_pos(self) -> int:
-        return self.start_pos + self.query_length
-
-
-@dataclass(frozen=True)
-class BatchPlan:
-    items: tuple[BatchItem, ...]
-
-    @property
-    def token_count(self) -> int:
-        return sum(item.query_length for item in self.items)
-
-    @property
-    def request_ids(self) -> tuple[str, ...]:
-        return tuple(item.request.request_id for item in self.items)
-
-
-@dataclass(frozen=True)
-class SchedulingCandidate:
-    request_id: str
-    phase: str
-    remaining_tokens: int
-    prompt_tokens: int
-    generated_tokens: int
-    arrival_ns: int
-
-
-@dataclass(frozen=True)
-class PreemptionCandidate:
-    request_id: str
-    allocated_tokens: int
-    tokens_fed: int
-    generated_tokens: int
-    arrival_ns: int
-
-
-def decode_first_priority(candidate: SchedulingCandidate) -> tuple[Any, ...]:
-    """Decode before prefill; the stable sort keeps admission order inside each."""
-    return (candidate.phase != "decode",)
-
-
-def largest_sequence_preemption(candidate: PreemptionCandidate) -> tuple[Any, ...]:
-    """Reclaim the most resident work first."""
-    return (candidate.allocated_tokens, candidate.tokens_fed, candidate.arrival_ns)
+    def __init__(self, plan: StepPlan, handle: Any) -> None:
+        self.plan = plan
+        self.handle = handle
 
 
 class Scheduler:
-    def __init__(
-        self,
-        config: Any,
-        runner: Any,
-        metrics: Any,
-        clock: Callable[[], int] = time.monotonic_ns,
-        scheduling_priority: Callable[[SchedulingCandidate], tuple[Any, ...]] = decode_first_priority,
-        preemption_priority: Callable[[PreemptionCandidate], tuple[Any, ...]] = largest_sequence_preemption,
-    ) -> None:
+    def __init__(self, config: Any, runner: Any, metrics: Any, clock: Callable[[], int] = time.monotonic_ns,
+                 plan_order: Order = decodes_before_prompts, victim_order: Order = most_resident_gives_way) -> None:
         self.config = config
         self.runner = runner
         self.metrics = metrics
         self.clock = clock
-        self.scheduling_priority = scheduling_priority
-        self.preemption_priority = preemption_priority
+        self.plan_order = plan_order
+        self.victim_order = victim_order
         self.waiting: deque[Request] = deque()
         self.active: list[Request] = []
         self.finished: deque[Request] = deque(maxlen=4096)
-        self._counter = 0
-        self._release_takes_flag = "preempted" in inspect.signature(runner.release).parameters
-        self._publish_prefix = getattr(runner, "publish_prefix", None)
-        # decode steps that are started before the tokens of the step before have arrived (see step())
-        self._launch_decode = getattr(runner, "launch_decode", None)
-        self._can_launch_decode = getattr(runner, "can_launch_decode", None)
-        self.async_decode = bool(getattr(config, "async_decode", False)) and self._launch_decode is not None \
-            and self._can_launch_decode is not None
-        self._in_flight: tuple[BatchPlan, Any] | None = None  # (plan, its pending tokens)
-        self._resolving = False
+        self._submitted = 0
+        # what the runner offers beyond admit / release / execute_batch
+        self._release_knows_preemption = "preempted" in inspect.signature(runner.release).parameters
+        self._resident = getattr(runner, "allocated_tokens", None)
+        self._free = getattr(runner, "free_tokens", None)
+        self._publish = getattr(runner, "publish_prefix", None)
+        self._launch = getattr(runner, "launch_decode", None)
+        self._launchable = getattr(runner, "can_launch_decode", None)
+        self.async_decode = (bool(getattr(config, "async_decode", False))
+                             and self._launch is not None and self._launchable is not None)
+        self._flying: _InFlight | None = None
+        self._collecting = False
 
-    # -- public ------------------------------------------------------------------
-    def submit(self, prompt_token_ids: Sequence[int], gen_config: GenerationConfig, label: str = "",
+    # ---------------------------------------------------------------- callers
+    def submit(self, prompt: Sequence[int], gen: GenerationConfig, label: str = "",
                on_token: Callable[[Request, int], None] | None = None) -> Request:
-        if len(prompt_token_ids) == 0:
-            raise RejectedError(RejectionReason.CONTEXT_OVERFLOW, "empty prompt")
-        if len(prompt_token_ids) + gen_config.max_output_tokens > self.config.max_model_len:
-            raise RejectedError(RejectionReason.CONTEXT_OVERFLOW)
-        if len(self.waiting) >= self.config.max_queue_size:
-            raise RejectedError(RejectionReason.QUEUE_FULL)
-        self._counter += 1
-        request = Request(
-            request_id=f"req-{self._counter:08d}",
-            prompt_token_ids=[int(t) for t in prompt_token_ids],
-            config=gen_config,
-            arrival_ns=self.clock(),
-            serial=self._counter,
-            label=label,
-            on_token=on_token,
-        )
+        """Queue a request, or refuse it (src/cloud_engine/scheduler.py:233-254): no
+        prompt, prompt + output beyond ``max_model_len``, queue full."""
+        limits = self.config
+        if not len(prompt):
+            raise RejectedError(Refusal.TOO_LONG, "empty prompt")
+        if len(prompt) + gen.max_output_tokens > limits.max_model_len:
+            raise RejectedError(Refusal.TOO_LONG)
+        if len(self.waiting) >= limits.max_queue_size:
+            raise RejectedError(Refusal.QUEUE_FULL)
+        self._submitted += 1
+        serial = self._submitted
+        request = Request(request_id="req-%08d" % serial, serial=serial, prompt=tuple(int(t) for t in prompt),
+                          gen=gen, arrived_ns=self.clock(), label=label, on_token=on_token)
         self.waiting.append(request)
         return request
 
     def cancel(self, request: Request) -> None:
-        """Idempotent; the request's pages go back at once."""
-        if request.is_terminal:
+        """End a request now; its pages go back at once.  A second call does nothing."""
+        if request.is_final:
             return
-        if self._in_flight is not None and not self._resolving:
-            self._take_in_flight()  # what it has generated so far is kept
-            if request.is_terminal:
+        if self._flying is not None and not self._collecting:
+            self._collect()  # the token under way is kept
+            if request.is_final:
                 return
-        request.state = RequestState.CANCELLED
-        request.finish_reason = "cancelled"
-        self._finalize(request)
+        self._retire(request, RequestState.CANCELLED, "cancelled")
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.active or self._in_flight is not None)
+        return bool(self.waiting) or bool(self.active) or self._flying is not None
 
     def run_until_done(self, max_iterations: int | None = None) -> None:
-        iterations = 0
+        done = 0
         while self.has_work():
             self.step()
-            iterations += 1
-            if max_iterations is not None and iterations >= max_iterations:
+            done += 1
+            if max_iterations is not None and done >= max_iterations:
                 raise RuntimeError(f"scheduler did not drain in {max_iterations} iterations")
 
     def step(self) -> bool:
-        """One iteration: admit, plan, run the plan, take the tokens.  Returns
-        whether anything progressed.
-
-        With ``async_decode`` a plan in which every request decodes one token is
-        only started; its tokens are taken by the next call, after that call has
-        started the step that follows (whose rows take their tokens on the device).
-        The GPU then never waits for the host between two decode steps.  What the
-        host cannot know in time is an end-of-sequence token: such a request runs
-        one step more than needed, and that step's token is dropped."""
-        if self._in_flight is not None:
-            return self._step_behind_in_flight()
-        progressed = self._admit_waiting()
+        """One iteration.  Returns whether anything moved."""
+        if self._flying is not None:
+            self._step_behind()
+            return True
+        moved = self._admit()
         with trace_range("scheduler.build_batch_plan"):
-            plan = self._build_batch_plan()
-        if not plan.items:
-            return progressed
-        if self._may_launch(plan):
-            try:
-                with trace_range("scheduler.launch_decode"):
-                    pending = self._launch_decode(plan, [-1] * len(plan.items),
-                                                  [item.request.generated_count for item in plan.items])
-            except Exception as exc:
-                self._plan_failed(plan, exc)
-                return True
-            self._in_flight = (plan, pending)
-            return True
-        try:
-            with trace_range("scheduler.execute_batch"):
-                outputs = self.runner.execute_batch(plan)
-        except Exception as exc:
-            self._plan_failed(plan, exc)
-            return True
-        self._take_outputs(plan, outputs)
+            plan = self._plan()
+        if not plan:
+            return moved
+        if self.async_decode and plan.all_decode and self._launchable(len(plan.portions)):
+            self._start(plan)
+        else:
+            self._run(plan)
         return True
 
-    def _plan_failed(self, plan: BatchPlan, exc: Exception) -> None:
-        if bool(getattr(exc, "is_capacity_error", False)):
-            if not self._preempt_for_capacity(plan):
-                for item in plan.items:
-                    if not item.request.is_terminal:
-                        self._fail(item.request,
-                                   f"KV capacity cannot fit one runnable sequence: {exc}", rejected=True)
-            return
-        for item in plan.items:
-            if not item.request.is_terminal:
-                self._fail(item.request, f"packed forward failed: {exc}")
-
-    def _take_outputs(self, plan: BatchPlan, outputs: dict[str, int]) -> None:
-        stamp = self.clock()
-        self.metrics.record_input_tokens(plan.token_count)
-        for item in plan.items:
-            request = item.request
-            if request.is_terminal:
+    # ---------------------------------------------------------------- admission
+    def _fits_beside_admitted(self, request: Request) -> bool:
+        """Whether the pool has room for all that is known of ``request`` once the admitted
+        requests have taken what is known of them (plus the token each is about to sample)."""
+        if self._free is None:
+            return True
+        spoken_for = 0
+        for other in self.active:
+            if other.is_final:
                 continue
-            recomputed = max(0, min(item.end_pos, request.recompute_until) - item.start_pos)
-            if recomputed:
-                request.recomputed_tokens += recomputed
-                self.metrics.record_recomputed_tokens(recomputed)
-            if item.sample:
-                token_id = outputs.get(request.request_id)
-                if token_id is None:
-                    self._fail(request, "packed runner omitted sampled token")
-                    continue
-                self._after_token(request, int(token_id), stamp)
-            else:
-                request.state = RequestState.PREFILL
-        self.metrics.record_iteration(len(plan.items))
+            held = self._resident(other) if self._resident is not None else 0
+            spoken_for += max(0, other.known + 1 - held)
+        return self._free() - spoken_for >= request.known + 1
 
-    # -- decode steps whose tokens are taken one call later ------------------------------
-    def _may_launch(self, plan: BatchPlan) -> bool:
-        return (self.async_decode and all(item.is_decode and item.sample for item in plan.items)
-                and self._can_launch_decode(len(plan.items)))
+    def _admit(self) -> bool:
+        moved = False
+        while self.waiting and len(self.active) < self.config.max_running:
+            head = self.waiting[0]
+            # A preempted request that came back the moment its own pages were free would take them from
+            # the same requests again, for ever.  A newcomer that does not fit would push someone out or
+            # be pushed out, and be computed twice.  Both wait at the head; alone, anything may try.
+            guarded = head.preemptions > 0 or self.config.admit_within_pool
+            if guarded and self.active and not self._fits_beside_admitted(head):
+                break
+            self.waiting.popleft()
+            try:
+                self.runner.admit(head)
+            except Exception as error:
+                self._retire(head, RequestState.FAILED, "failed", error=f"admission refused: {error}",
+                             rejected=_is_shortage(error))
+                continue
+            head.state = RequestState.PREFILL
+            self.active.append(head)
+            moved = True
+        return moved
 
-    def _take_in_flight(self) -> None:
-        """Wait for the tokens of the step in flight and hand them to their requests."""
-        plan, pending = self._in_flight
-        self._in_flight = None
-        self._resolving = True
+    # ---------------------------------------------------------------- planning
+    def _plan(self) -> StepPlan:
+        runnable = [r for r in self.active if not r.is_final and r.pending > 0]
+        standings = {id(r): Standing.of(r) for r in runnable}
+        runnable.sort(key=lambda r: self.plan_order(standings[id(r)]))
+        left = self.config.token_budget
+        portions: list[Portion] = []
+        for request in runnable:
+            if left <= 0:
+                break
+            most = 1 if standings[id(request)].decoding else self.config.prefill_chunk
+            take = min(request.pending, most, left)
+            start = request.cached
+            portions.append(Portion(request, start, request.tokens(start, start + take),
+                                    samples=start + take == request.known))
+            left -= take
+        return StepPlan(tuple(portions))
+
+    # ---------------------------------------------------------------- running a plan
+    def _run(self, plan: StepPlan) -> None:
         try:
-            self._take_outputs(plan, pending.tokens())
-        finally:
-            self._resolving = False
+            with trace_range("scheduler.execute_batch"):
+                sampled = self.runner.execute_batch(plan)
+        except Exception as error:
+            if not (_is_shortage(error) and self._make_room(error)):
+                self._fail_plan(plan, error)
+            return
+        self._account(plan, sampled)
 
-    def _follow_up(self, plan: BatchPlan) -> tuple[BatchPlan, list[int], list[int]] | None:
-        """The step after the one in flight, if it can be planned without that step's tokens: the same
-        requests, less those that reach their token limit with the token in flight; each row takes its
-        token from the place of its request in the step in flight."""
-        if self.waiting and len(self.active) < self.config.max_running:
-            return None  # a request wants in: let the step in flight end, then admit
-        in_flight = {id(item.request) for item in plan.items}
-        if any(id(request) not in in_flight for request in self.active if not request.is_terminal):
-            return None  # someone still has a prompt to run: the next step is a mixed one
-        items, feed, indices = [], [], []
-        for place, item in enumerate(plan.items):
-            request = item.request
-            if request.is_terminal or request.generated_count + 1 >= request.config.max_output_tokens:
+    def _start(self, plan: StepPlan) -> None:
+        """Start a decode step without waiting for its tokens: no row has a token on the device yet."""
+        placeholder = [-1] * len(plan.portions)
+        next_index = [len(portion.request.output) for portion in plan.portions]
+        try:
+            with trace_range("scheduler.launch_decode"):
+                handle = self._launch(plan, placeholder, next_index)
+        except Exception as error:
+            if not (_is_shortage(error) and self._make_room(error)):
+                self._fail_plan(plan, error)
+            return
+        self._flying = _InFlight(plan, handle)
+
+    def _fail_plan(self, plan: StepPlan, error: Exception) -> None:
+        if _is_shortage(error):
+            reason, rejected = f"KV capacity cannot fit one runnable sequence: {error}", True
+        else:
+            reason, rejected = f"packed forward failed: {error}", False
+        for portion in plan.portions:
+            if not portion.request.is_final:
+                self._retire(portion.request, RequestState.FAILED, "failed", error=reason, rejected=rejected)
+
+    def _account(self, plan: StepPlan, sampled: dict[str, int]) -> None:
+        now = self.clock()
+        for portion in plan.portions:
+            request = portion.request
+            if request.is_final:
                 continue
-            items.append(BatchItem(request=request, token_ids=(0,), start_pos=request.tokens_fed, sample=True,
-                                   is_decode=True))
-            feed.append(place)
-            indices.append(request.generated_count + 1)
-        if not items or not self._can_launch_decode(len(items)):
-            return None
-        return BatchPlan(tuple(items)), feed, indices
+            again = min(portion.end, request.redo_below) - portion.start
+            if again > 0:
+                request.recomputed += again
+                self.metrics.totals.recomputed_tokens += again
+            if not portion.samples:
+                request.state = RequestState.PREFILL
+            elif request.request_id in sampled:
+                self._token_arrived(request, int(sampled[request.request_id]), now)
+            else:
+                self._retire(request, RequestState.FAILED, "failed", error="packed runner omitted sampled token")
+        self.metrics.iteration(len(plan.portions), plan.token_count)
 
-    def _step_behind_in_flight(self) -> bool:
-        plan, _ = self._in_flight
-        follow = self._follow_up(plan) if self.async_decode else None
-        launched = None
-        failure: Exception | None = None
+    def _token_arrived(self, request: Request, token: int, now: int) -> None:
+        prompt_just_ended = request.state is RequestState.PREFILL
+        request.output.append(token)
+        if request.first_token_ns is None:
+            request.first_token_ns = now
+            self.metrics.first_token_ms.add((now - request.arrived_ns) * 1e-6)
+        else:
+            self.metrics.between_tokens_ms.add((now - request.latest_token_ns) * 1e-6)
+        request.latest_token_ns = now
+        self.metrics.totals.output_tokens += 1
+        gen = request.gen
+        if gen.eos_token_id is not None and token == gen.eos_token_id:
+            # the id stays in ``output`` (ids are what a recomputation feeds) but is not streamed
+            self._retire(request, RequestState.COMPLETED, "eos_token_reached")
+            return
+        if request.on_token is not None:
+            request.on_token(request, token)
+        if len(request.output) >= gen.max_output_tokens:
+            self._retire(request, RequestState.COMPLETED, "max_output_tokens_reached")
+            return
+        request.state = RequestState.DECODING
+        if prompt_just_ended and self._publish is not None:
+            # the prompt's full pages will not change again: requests that arrive while this one
+            # decodes may share them already
+            self._publish(request)
+
+    # ---------------------------------------------------------------- decode steps in flight
+    def _collect(self) -> None:
+        """Wait for the tokens of the step in flight and give them to their requests."""
+        flying, self._flying = self._flying, None
+        self._collecting = True
+        try:
+            self._account(flying.plan, flying.handle.tokens())
+        finally:
+            self._collecting = False
+
+    def _follow_up(self, flying: StepPlan) -> tuple[StepPlan, list[int], list[int]] | None:
+        """The step behind the one in flight, where it can be planned without that step's tokens:
+        the same requests, less those whose token limit the token in flight reaches.  Row i takes
+        its token from row ``feed[i]`` of the step in flight."""
+        if self.waiting and len(self.active) < self.config.max_running:
+            return None  # someone wants in: let the flight land, then admit
+        aboard = {id(portion.request) for portion in flying.portions}
+        if any(id(r) not in aboard for r in self.active if not r.is_final):
+            return None  # someone has prompt left: the next step is a mixed one
+        portions, feed, token_index = [], [], []
+        for row, portion in enumerate(flying.portions):
+            request = portion.request
+            after_flight = len(request.output) + 1
+            if request.is_final or after_flight >= request.gen.max_output_tokens:
+                continue
+            portions.append(Portion(request, request.cached, (0,), samples=True))
+            feed.append(row)
+            token_index.append(after_flight)
+        if not portions or not self._launchable(len(portions)):
+            return None
+        return StepPlan(tuple(portions)), feed, token_index
+
+    def _step_behind(self) -> None:
+        follow = self._follow_up(self._flying.plan)
+        handle = problem = None
         if follow is not None:
             try:
                 with trace_range("scheduler.launch_decode"):
-                    launched = self._launch_decode(*follow)
-            except Exception as exc:  # nothing was started; the tokens in flight are taken first
-                failure = exc
-        self._take_in_flight()
-        if launched is not None:
-            self._in_flight = (follow[0], launched)
-        elif failure is not None and not bool(getattr(failure, "is_capacity_error", False)):
-            self._plan_failed(follow[0], failure)
-        # (a shortage of pages shows again in the next call, which plans with the tokens in hand and preempts)
-        return True
+                    handle = self._launch(*follow)
+            except Exception as error:  # nothing was started
+                problem = error
+        self._collect()
+        if handle is not None:
+            self._flying = _InFlight(follow[0], handle)
+        elif problem is not None and not _is_shortage(problem):
+            self._fail_plan(follow[0], problem)
+        # a shortage is left alone here: the next call plans with every token in hand and makes room
 
-    # -- internals -----------------------------------------------------------------
-    def _room_beside_admitted(self, request: Request) -> bool:
-        """Whether the pool holds what is known of ``request`` beside what is known
-        of the admitted requests (the part of it that they have not taken yet)."""
-        free_tokens = getattr(self.runner, "free_tokens", None)
-        if free_tokens is None:
-            return True
-        allocated_tokens = getattr(self.runner, "allocated_tokens", lambda _r: 0)
-        owed = 0
-        for admitted in self.active:
-            if not admitted.is_terminal:
-                known = len(admitted.prompt_token_ids) + admitted.generated_count + 1
-                owed += max(0, known - allocated_tokens(admitted))
-        return free_tokens() - owed >= len(request.prompt_token_ids) + request.generated_count + 1
-
-    def _admit_waiting(self) -> bool:
-        progressed = False
-        while self.waiting and len(self.active) < self.config.max_running:
-            candidate = self.waiting[0]
-            if candidate.preemption_count and self.active and not self._room_beside_admitted(candidate):
-                # wait for room instead of thrashing; keeps its place at the head.  Room beside what the admitted
-                # requests still have to take: the pages it has just given back are free, and taking them
-                # again at once would starve the same requests again, for ever
-                break
-            if self.config.admit_within_pool and self.active and not self._room_beside_admitted(candidate):
-                break  # admitted now it would push another request out, or be pushed out, and be computed twice
-            self.waiting.popleft()
-            try:
-                self.runner.admit(candidate)
-            except Exception as exc:
-                self._fail(candidate, f"admission refused: {exc}",
-                           rejected=bool(getattr(exc, "is_capacity_error", False)))
-                continue
-            candidate.state = RequestState.PREFILL
-            self.active.append(candidate)
-            progressed = True
-        return progressed
-
-    def _build_batch_plan(self) -> BatchPlan:
-        budget = self.config.token_budget
-        candidates: list[tuple[SchedulingCandidate, Request]] = []
-        for request in self.active:
-            if request.is_terminal:
-                continue
-            known = len(request.prompt_token_ids) + request.generated_count
-            remaining = known - request.tokens_fed
-            if remaining <= 0:
-                continue
-            phase = "decode" if request.state is RequestState.DECODING and remaining == 1 else "prefill"
-            candidates.append((
-                SchedulingCandidate(request.request_id, phase, remaining, len(request.prompt_token_ids),
-                                    request.generated_count, request.arrival_ns),
-                request,
-            ))
-        items: list[BatchItem] = []
-        for candidate, request in sorted(candidates, key=lambda pair: self.scheduling_priority(pair[0])):
-            if budget <= 0:
-                break
-            prompt, generated = request.prompt_token_ids, request.generated_token_ids
-            known = len(prompt) + len(generated)
-            remaining = known - request.tokens_fed
-            limit = 1 if candidate.phase == "decode" else self.config.prefill_chunk
-            query_length = min(remaining, limit, budget)
-            start = request.tokens_fed
-            end = start + query_length
-            # the portion's tokens, without joining the two lists (a decode step would copy the whole context)
-            if start >= len(prompt):
-                token_ids = tuple(generated[start - len(prompt): end - len(prompt)])
-            elif end <= len(prompt):
-                token_ids = tuple(prompt[start:end])
-            else:
-                token_ids = tuple(prompt[start:]) + tuple(generated[: end - len(prompt)])
-            items.append(BatchItem(
-                request=request,
-                token_ids=token_ids,
-                start_pos=start,
-                sample=end == known,
-                is_decode=query_length == 1 and start >= len(prompt),
-            ))
-            budget -= query_length
-        return BatchPlan(tuple(items))
-
-    def _preempt_for_capacity(self, plan: BatchPlan) -> bool:
-        candidates = [request for request in self.active if not request.is_terminal]
-        if len(candidates) <= 1:
+    # ---------------------------------------------------------------- giving way and ending
+    def _make_room(self, _error: Exception | None = None) -> bool:
+        """Preempt one live request.  ``False`` if there is at most one, which then cannot run at all."""
+        live = [r for r in self.active if not r.is_final]
+        if len(live) < 2:
             return False
-        allocated_tokens = getattr(self.runner, "allocated_tokens", lambda _r: 0)
-        victim = max(
-            candidates,
-            key=lambda request: self.preemption_priority(PreemptionCandidate(
-                request.request_id, allocated_tokens(request), request.tokens_fed,
-                request.generated_count, request.arrival_ns)),
-        )
+        resident = self._resident if self._resident is not None else (lambda _request: 0)
+        victim = max(live, key=lambda r: self.victim_order(Standing.of(r, resident(r))))
         self.active.remove(victim)
-        self._release(victim, preempted=True)
-        victim.recompute_until = victim.tokens_fed
-        victim.tokens_fed = 0
-        victim.preemption_count += 1
+        self._give_back(victim, preempted=True)
+        victim.redo_below, victim.cached = victim.cached, 0
+        victim.preemptions += 1
         victim.state = RequestState.WAITING
         self.waiting.appendleft(victim)
-        self.metrics.inc_preempted()
+        self.metrics.totals.preempted += 1
         return True
 
-    def _release(self, request: Request, preempted: bool = False) -> None:
-        if self._release_takes_flag:
+    def _give_back(self, request: Request, preempted: bool = False) -> None:
+        if self._release_knows_preemption:
             self.runner.release(request, preempted=preempted)
         else:
             self.runner.release(request)
 
-    def _after_token(self, request: Request, token_id: int, now: int) -> None:
-        finished_prompt = request.state is RequestState.PREFILL
-        request.generated_token_ids.append(token_id)
-        if request.first_token_ns is None:
-            request.first_token_ns = now
-            self.metrics.record_ttft_ms((now - request.arrival_ns) / 1e6)
-        else:
-            self.metrics.record_itl_ms((now - (request.last_token_ns or now)) / 1e6)
-        request.last_token_ns = now
-        self.metrics.record_output_token(1)
-        eos_hit = request.config.eos_token_id is not None and token_id == request.config.eos_token_id
-        limit_hit = request.generated_count >= request.config.max_output_tokens
-        if eos_hit:
-            request.finish_reason = "eos_token_reached"
-        elif limit_hit:
-            request.finish_reason = "max_output_tokens_reached"
-        if request.on_token is not None and not eos_hit:
-            request.on_token(request, token_id)
-        if eos_hit or limit_hit:
-            request.state = RequestState.COMPLETED
-            self._finalize(request)
-        else:
-            request.state = RequestState.DECODING
-            if finished_prompt and self._publish_prefix is not None:
-                # the prompt's full pages are final from here on: requests that arrive while this one
-                # still decodes can already share them
-                self._publish_prefix(request)
-
-    def _fail(self, request: Request, detail: str, rejected: bool = False) -> None:
-        if request.is_terminal:
+    def _retire(self, request: Request, state: RequestState, reason: str, error: str = "",
+                rejected: bool = False) -> None:
+        """Every way a request ends passes here once: out of the queues, cache given back, counted."""
+        if request.is_final:
             return
-        request.rejected = rejected
-        request.state = RequestState.FAILED
-        request.error_detail = detail
-        request.finish_reason = "failed"
-        self._finalize(request)
-
-    def _finalize(self, request: Request) -> None:
-        """The one terminal funnel: leave the queues, give the cache back, count."""
-        if request in self.active:
-            self.active.remove(request)
-        if request in self.waiting:
-            self.waiting.remove(request)
+        request.state, request.finish_reason = state, reason
+        request.error, request.rejected = error, rejected
+        for queue in (self.active, self.waiting):
+            if request in queue:
+                queue.remove(request)
         try:
-            self._release(request)
-        except Exception as exc:  # release must never break teardown
-            request.error_detail = f"release error: {exc}"
-        request.finish_ns = self.clock()
+            self._give_back(request)
+        except Exception as problem:  # an ending request must end, whatever the cache says
+            request.error = f"release error: {problem}"
+        request.ended_ns = self.clock()
         self.finished.append(request)
-        if request.state is RequestState.COMPLETED:
-            self.metrics.record_e2e_ms((request.finish_ns - request.arrival_ns) / 1e6)
-            self.metrics.inc_completed()
-        elif request.state is RequestState.CANCELLED:
-            self.metrics.inc_cancelled()
-        elif request.rejected:
-            self.metrics.inc_rejected()
+        totals = self.metrics.totals
+        if state is RequestState.COMPLETED:
+            totals.completed += 1
+            self.metrics.whole_request_ms.add((request.ended_ns - request.arrived_ns) * 1e-6)
+        elif state is RequestState.CANCELLED:
+            totals.cancelled += 1
+        elif rejected:
+            totals.rejected += 1
         else:
-            self.metrics.inc_failed()
+            totals.failed += 1

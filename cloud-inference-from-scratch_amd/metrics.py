@@ -1,108 +1,99 @@
-"""Bounded counters and latency windows, after the reference's ``Metrics``
-(src/cloud_engine/metrics.py:52-200): TTFT / ITL / E2E samples in fixed-capacity
-windows, totals for requests and tokens, batch sizes per iteration."""
+"""What the engine counts while it serves: totals since the last reset, and the
+latest latencies in windows of bounded length.
+
+The figures are those of the reference's ``Metrics``
+(src/cloud_engine/metrics.py:52-200): time to the first token, time between
+tokens and whole-request time with their percentiles; requests by outcome;
+tokens taken in, produced and computed twice; the size of each iteration's
+batch.  The scheduler writes into :class:`Totals` and the :class:`Window`
+objects directly.
+"""
 
 from __future__ import annotations
 
+import math
 from collections import deque
+from collections.abc import Iterable
+from dataclasses import asdict, dataclass
 from typing import Any
 
 
-def percentile(values: list[float], pct: float) -> float:
-    """Linear interpolation on a sorted copy; empty input gives 0 (metrics.py:19-31)."""
-    if not values:
+def quantile(samples: Iterable[float], fraction: float) -> float:
+    """The value at ``fraction`` (0..1) of the way through the sorted samples,
+    weighted between the two neighbours it falls between; 0 for no samples."""
+    ranked = sorted(samples)
+    if not ranked:
         return 0.0
-    ordered = sorted(values)
-    if len(ordered) == 1:
-        return ordered[0]
-    rank = (len(ordered) - 1) * (pct / 100.0)
-    lower = int(rank)
-    upper = min(lower + 1, len(ordered) - 1)
-    return ordered[lower] + (ordered[upper] - ordered[lower]) * (rank - lower)
+    place = min(max(fraction, 0.0), 1.0) * (len(ranked) - 1)
+    under = math.floor(place)
+    weight = place - under
+    if weight == 0.0:
+        return ranked[under]
+    return (1.0 - weight) * ranked[under] + weight * ranked[under + 1]
+
+
+class Window:
+    """The latest ``length`` samples of one latency."""
+
+    def __init__(self, length: int) -> None:
+        self._samples: deque[float] = deque(maxlen=length)
+
+    def add(self, value: float) -> None:
+        self._samples.append(value)
+
+    def __len__(self) -> int:
+        return len(self._samples)
+
+    def summary(self) -> dict[str, float]:
+        out: dict[str, float] = {"count": len(self._samples)}
+        for name, fraction in (("p50", 0.50), ("p95", 0.95), ("p99", 0.99)):
+            out[name] = quantile(self._samples, fraction)
+        return out
+
+
+@dataclass
+class Totals:
+    completed: int = 0
+    failed: int = 0
+    cancelled: int = 0
+    rejected: int = 0
+    preempted: int = 0
+    iterations: int = 0
+    input_tokens: int = 0
+    output_tokens: int = 0
+    recomputed_tokens: int = 0
 
 
 class Metrics:
-    def __init__(self, latency_capacity: int = 4096) -> None:
-        self._latency_capacity = latency_capacity
+    def __init__(self, latency_samples: int = 4096, batch_samples: int = 16_384) -> None:
+        self._lengths = (latency_samples, batch_samples)
         self.reset()
 
     def reset(self) -> None:
-        """Forget everything recorded so far (after a warm-up, before a measured run)."""
-        latency_capacity = self._latency_capacity
-        self._ttft: deque[float] = deque(maxlen=latency_capacity)
-        self._itl: deque[float] = deque(maxlen=latency_capacity)
-        self._e2e: deque[float] = deque(maxlen=latency_capacity)
-        self._batch_sizes: deque[int] = deque(maxlen=16_384)
-        self.completed_total = 0
-        self.failed_total = 0
-        self.cancelled_total = 0
-        self.rejected_total = 0
-        self.preempted_total = 0
-        self.iterations_total = 0
-        self.input_tokens_total = 0
-        self.output_tokens_total = 0
-        self.recomputed_tokens_total = 0
+        """Start counting afresh (after a warm-up, before a measured run)."""
+        latency_samples, batch_samples = self._lengths
+        self.totals = Totals()
+        self.first_token_ms = Window(latency_samples)
+        self.between_tokens_ms = Window(latency_samples)
+        self.whole_request_ms = Window(latency_samples)
+        self.batch_sizes: deque[int] = deque(maxlen=batch_samples)
 
-    def record_ttft_ms(self, value: float) -> None:
-        self._ttft.append(value)
-
-    def record_itl_ms(self, value: float) -> None:
-        self._itl.append(value)
-
-    def record_e2e_ms(self, value: float) -> None:
-        self._e2e.append(value)
-
-    def record_iteration(self, batch_size: int) -> None:
-        self.iterations_total += 1
-        self._batch_sizes.append(batch_size)
-
-    def record_input_tokens(self, count: int) -> None:
-        self.input_tokens_total += count
-
-    def record_output_token(self, count: int = 1) -> None:
-        self.output_tokens_total += count
-
-    def record_recomputed_tokens(self, count: int) -> None:
-        self.recomputed_tokens_total += count
-
-    def inc_completed(self) -> None:
-        self.completed_total += 1
-
-    def inc_failed(self) -> None:
-        self.failed_total += 1
-
-    def inc_cancelled(self) -> None:
-        self.cancelled_total += 1
-
-    def inc_rejected(self) -> None:
-        self.rejected_total += 1
-
-    def inc_preempted(self) -> None:
-        self.preempted_total += 1
-
-    @staticmethod
-    def _summary(samples: deque) -> dict[str, float]:
-        values = list(samples)
-        return {"count": len(values), "p50": percentile(values, 50), "p95": percentile(values, 95),
-                "p99": percentile(values, 99)}
+    def iteration(self, requests: int, tokens: int) -> None:
+        self.totals.iterations += 1
+        self.totals.input_tokens += tokens
+        self.batch_sizes.append(requests)
 
     def snapshot(self) -> dict[str, Any]:
-        sizes = list(self._batch_sizes)
+        totals = asdict(self.totals)
+        sizes = self.batch_sizes
         return {
-            "latency_ms": {"ttft": self._summary(self._ttft), "itl": self._summary(self._itl),
-                           "e2e": self._summary(self._e2e)},
-            "requests": {
-                "completed_total": self.completed_total, "failed_total": self.failed_total,
-                "cancelled_total": self.cancelled_total, "rejected_total": self.rejected_total,
-                "preempted_total": self.preempted_total,
-            },
-            "tokens": {
-                "input_total": self.input_tokens_total, "output_total": self.output_tokens_total,
-                "recomputed_total": self.recomputed_tokens_total,
-            },
-            "scheduler": {
-                "iterations_total": self.iterations_total,
-                "mean_batch_size": sum(sizes) / len(sizes) if sizes else 0.0,
-                "max_batch_size": max(sizes, default=0),
-            },
+            "latency_ms": {"ttft": self.first_token_ms.summary(), "itl": self.between_tokens_ms.summary(),
+                           "e2e": self.whole_request_ms.summary()},
+            "requests": {f"{outcome}_total": totals[outcome]
+                         for outcome in ("completed", "failed", "cancelled", "rejected", "preempted")},
+            "tokens": {"input_total": totals["input_tokens"], "output_total": totals["output_tokens"],
+                       "recomputed_total": totals["recomputed_tokens"]},
+            "scheduler": {"iterations_total": totals["iterations"],
+                          "mean_batch_size": sum(sizes) / len(sizes) if sizes else 0.0,
+                          "max_batch_size": max(sizes, default=0)},
         }

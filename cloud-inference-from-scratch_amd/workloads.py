@@ -119,7 +119,7 @@ def run_profile(profile: Profile, *, layers: int | None = None, dtype: str = "bf
     warm = [engine.submit(list(range(1, 49)), GenerationConfig(max_output_tokens=4, eos_token_id=None)) for _ in range(2)]
     while engine.has_work():
         engine.step()
-    assert all(r.is_terminal for r in warm)
+    assert all(r.is_final for r in warm)
     engine.metrics.reset()
     torch.cuda.synchronize()
 
@@ -129,7 +129,7 @@ def run_profile(profile: Profile, *, layers: int | None = None, dtype: str = "bf
 
     steps = 0
     handles = submit(requests[: profile.lead_requests])
-    while any(h.generated_count == 0 and not h.is_terminal for h in handles):
+    while any(len(h.output) == 0 and not h.is_final for h in handles):
         engine.step()
         steps += 1
     handles += submit(requests[profile.lead_requests:])

@@ -166,7 +166,7 @@ def test_prefix_is_shared_with_a_request_that_arrives_while_the_first_still_deco
     gen = GenerationConfig(max_output_tokens=12, eos_token_id=None)
     engine = make_engine(folder, page_size=16, prefix_cache_pages=8)
     first = engine.submit(prompt, gen)
-    while first.generated_count < 3:
+    while len(first.output) < 3:
         engine.step()
     assert first.state is RequestState.DECODING
     second = engine.submit(sibling, gen)

@@ -7,7 +7,7 @@ import pytest
 
 from cie_amd.config import build_engine_config
 from cie_amd.engine.scheduler import (
-    GenerationConfig, RejectedError, RejectionReason, RequestState, Scheduler,
+    GenerationConfig, RejectedError, Refusal, RequestState, Scheduler,
 )
 from cie_amd.metrics import Metrics
 
@@ -25,7 +25,7 @@ class FakeRunner:
         if request.request_id in self.resident:
             raise RuntimeError("duplicate admission")
         self.resident[request.request_id] = 0
-        request.tokens_fed = 0
+        request.cached = 0
 
     def release(self, request, preempted: bool = False) -> None:
         if request.request_id in self.resident:
@@ -43,21 +43,21 @@ class FakeRunner:
             error, self.fail_next = self.fail_next, None
             raise error
         required = dict(self.resident)
-        for item in plan.items:
-            required[item.request.request_id] = max(required[item.request.request_id], item.end_pos)
+        for item in plan.portions:
+            required[item.request.request_id] = max(required[item.request.request_id], item.end)
         if sum(required.values()) > self.token_capacity:
             error = RuntimeError("fake KV capacity exhausted")
             error.is_capacity_error = True
             raise error
         self.resident = required
         self.plans.append(plan)
-        self.traces.append((plan.request_ids, tuple(item.query_length for item in plan.items)))
+        self.traces.append((plan.request_ids, tuple(item.length for item in plan.portions)))
         outputs = {}
-        for item in plan.items:
-            assert item.start_pos == item.request.tokens_fed, "a portion must start where the cache ends"
-            item.request.tokens_fed = item.end_pos
-            if item.sample:
-                outputs[item.request.request_id] = 100 + item.request.generated_count
+        for item in plan.portions:
+            assert item.start == item.request.cached, "a portion must start where the cache ends"
+            item.request.cached = item.end
+            if item.samples:
+                outputs[item.request.request_id] = 100 + len(item.request.output)
         return outputs
 
 
@@ -72,7 +72,7 @@ def test_requests_share_one_forward():
     scheduler = make(runner)
     requests = [scheduler.submit([i + 1] * 3, GenerationConfig(max_output_tokens=2)) for i in range(3)]
     scheduler.run_until_done(100)
-    assert [r.generated_token_ids for r in requests] == [[100, 101]] * 3
+    assert [r.output for r in requests] == [[100, 101]] * 3
     assert any(len(ids) == 3 for ids, _ in runner.traces)
     assert all(r.state is RequestState.COMPLETED and r.finish_reason == "max_output_tokens_reached" for r in requests)
     assert not runner.resident
@@ -83,9 +83,9 @@ def test_prefill_is_cut_into_portions_under_the_budget():
     scheduler = make(runner, token_budget=5, prefill_chunk=4)
     request = scheduler.submit(list(range(11)), GenerationConfig(max_output_tokens=1))
     scheduler.run_until_done(100)
-    assert request.generated_token_ids == [100]
+    assert request.output == [100]
     assert [lengths[0] for _, lengths in runner.traces][:3] == [4, 4, 3]
-    samples = [item.sample for plan in runner.plans for item in plan.items]
+    samples = [item.samples for plan in runner.plans for item in plan.portions]
     assert samples == [False, False, True]  # logits only where the portion reaches the tail
 
 
@@ -98,23 +98,23 @@ def test_decode_goes_first_and_budget_is_shared():
     scheduler.step()
     plan = runner.plans[-1]
     assert plan.request_ids == (first.request_id, late.request_id)
-    assert [item.query_length for item in plan.items] == [1, 4] and plan.items[0].is_decode
-    assert not plan.items[1].is_decode and plan.token_count <= 6
+    assert [item.length for item in plan.portions] == [1, 4] and plan.portions[0].is_decode
+    assert not plan.portions[1].is_decode and plan.token_count <= 6
     scheduler.run_until_done(100)
     for plan in runner.plans:
         assert plan.token_count <= 6 and len(set(plan.request_ids)) == len(plan.request_ids)
-        phases = [item.is_decode for item in plan.items]
+        phases = [item.is_decode for item in plan.portions]
         assert phases == sorted(phases, reverse=True), "decode items come before prefill items"
 
 
 def test_custom_priority_reorders_but_cannot_exceed_budget():
     runner = FakeRunner()
     scheduler = make(runner, token_budget=4)
-    scheduler.scheduling_priority = lambda candidate: (candidate.remaining_tokens,)
+    scheduler.plan_order = lambda standing: (standing.pending_tokens,)
     long = scheduler.submit([1] * 8, GenerationConfig(max_output_tokens=1))
     short = scheduler.submit([2] * 2, GenerationConfig(max_output_tokens=1))
-    scheduler._admit_waiting()
-    plan = scheduler._build_batch_plan()
+    scheduler._admit()
+    plan = scheduler._plan()
     assert plan.request_ids == (short.request_id, long.request_id) and plan.token_count == 4
 
 
@@ -123,8 +123,8 @@ def test_pressure_preempts_then_recomputes_without_token_drift():
     scheduler = make(runner, token_budget=8, prefill_chunk=4)
     requests = [scheduler.submit([i + 1] * 4, GenerationConfig(max_output_tokens=3)) for i in range(2)]
     scheduler.run_until_done(200)
-    assert [r.generated_token_ids for r in requests] == [[100, 101, 102]] * 2
-    assert sum(r.preemption_count for r in requests) > 0 and sum(r.recomputed_tokens for r in requests) > 0
+    assert [r.output for r in requests] == [[100, 101, 102]] * 2
+    assert sum(r.preemptions for r in requests) > 0 and sum(r.recomputed for r in requests) > 0
     snapshot = scheduler.metrics.snapshot()
     assert snapshot["requests"]["preempted_total"] > 0 and snapshot["tokens"]["recomputed_total"] > 0
     assert snapshot["requests"]["completed_total"] == 2
@@ -141,19 +141,19 @@ def test_preempted_request_keeps_generated_tokens_and_its_place():
     scheduler.config = build_engine_config(scheduler.config, max_running=2)
     scheduler.step()  # a and b prefilled: 10 resident; each has its first token
     scheduler.step()  # 12 resident
-    assert (a.generated_count, b.generated_count) == (2, 2)
+    assert (len(a.output), len(b.output)) == (2, 2)
     scheduler.step()  # 14 > 12: the larger one (tie: the later arrival) is preempted
-    assert b.state is RequestState.WAITING and b.preemption_count == 1 and b.tokens_fed == 0
-    assert b.generated_token_ids == [100, 101] and b.recompute_until == 6
+    assert b.state is RequestState.WAITING and b.preemptions == 1 and b.cached == 0
+    assert b.output == [100, 101] and b.redo_below == 6
     assert scheduler.waiting[0] is b, "the preempted request waits at the head, before the newcomer"
     scheduler.step()  # a decodes alone: 7 resident, 5 free; b needs 5 + 2 + 1 = 8: still waiting, c behind it
     assert b.state is RequestState.WAITING and c.state is RequestState.WAITING
     scheduler.run_until_done(200)
-    assert [r.generated_token_ids for r in (a, b, c)] == [[100, 101, 102, 103]] * 2 + [[100]]
+    assert [r.output for r in (a, b, c)] == [[100, 101, 102, 103]] * 2 + [[100]]
     # the recompute fed prompt and generated tokens as prompt portions and sampled only at the tail
-    recompute = [item for plan in runner.plans for item in plan.items
-                 if item.request is b and item.start_pos == 0 and item.query_length > 5]
-    assert recompute and recompute[0].token_ids == (2, 2, 2, 2, 2, 100, 101) and recompute[0].sample
+    recompute = [item for plan in runner.plans for item in plan.portions
+                 if item.request is b and item.start == 0 and item.length > 5]
+    assert recompute and recompute[0].tokens == (2, 2, 2, 2, 2, 100, 101) and recompute[0].samples
 
 
 def test_long_prompts_are_admitted_only_while_the_pool_holds_them():
@@ -167,8 +167,8 @@ def test_long_prompts_are_admitted_only_while_the_pool_holds_them():
         scheduler.step()
         admitted = len(scheduler.active)
         scheduler.run_until_done(200)
-        assert [r.generated_token_ids for r in requests] == [[100, 101]] * 3 and not runner.resident
-        return admitted, sum(r.preemption_count for r in requests), sum(r.recomputed_tokens for r in requests)
+        assert [r.output for r in requests] == [[100, 101]] * 3 and not runner.resident
+        return admitted, sum(r.preemptions for r in requests), sum(r.recomputed for r in requests)
 
     assert run(True) == (2, 0, 0)
     admitted, preempted, recomputed = run(False)
@@ -183,8 +183,8 @@ def test_a_request_larger_than_what_is_left_is_admitted_when_nothing_else_runs()
     scheduler.step()
     assert [r.request_id for r in scheduler.active] == [first.request_id] and scheduler.waiting[0] is second
     scheduler.run_until_done(100)
-    assert first.generated_token_ids == second.generated_token_ids == [100, 101]
-    assert first.preemption_count == second.preemption_count == 0
+    assert first.output == second.output == [100, 101]
+    assert first.preemptions == second.preemptions == 0
 
 
 def test_over_subscribed_pools_drain_under_random_loads():
@@ -204,20 +204,20 @@ def test_over_subscribed_pools_drain_under_random_loads():
                     for i in range(30)]
         scheduler.run_until_done(5000)
         for request in requests:
-            assert request.state is RequestState.COMPLETED, (seed, request.state, request.error_detail)
-            assert request.generated_token_ids == [100 + i for i in range(request.config.max_output_tokens)], seed
+            assert request.state is RequestState.COMPLETED, (seed, request.state, request.error)
+            assert request.output == [100 + i for i in range(request.gen.max_output_tokens)], seed
         assert not runner.resident, seed
 
 
 def test_custom_preemption_policy_selects_victim():
     runner = FakeRunner(token_capacity=10)
     scheduler = make(runner, token_budget=8, prefill_chunk=4)
-    scheduler.preemption_priority = lambda candidate: (-candidate.arrival_ns,)
+    scheduler.victim_order = lambda standing: (-standing.arrived_ns,)
     requests = [scheduler.submit([i + 1] * 4, GenerationConfig(max_output_tokens=3)) for i in range(2)]
-    scheduler._admit_waiting()
+    scheduler._admit()
     runner.resident = {r.request_id: 4 for r in requests}
-    assert scheduler._preempt_for_capacity(scheduler._build_batch_plan())
-    assert (requests[0].preemption_count, requests[1].preemption_count) == (1, 0)
+    assert scheduler._make_room()
+    assert (requests[0].preemptions, requests[1].preemptions) == (1, 0)
 
 
 def test_single_request_that_cannot_fit_is_rejected():
@@ -226,7 +226,7 @@ def test_single_request_that_cannot_fit_is_rejected():
     request = scheduler.submit([1] * 8, GenerationConfig(max_output_tokens=2))
     scheduler.run_until_done(10)
     assert request.state is RequestState.FAILED and request.rejected
-    assert "KV capacity cannot fit one runnable sequence" in request.error_detail
+    assert "KV capacity cannot fit one runnable sequence" in request.error
     assert scheduler.metrics.snapshot()["requests"]["rejected_total"] == 1 and not runner.resident
 
 
@@ -234,15 +234,15 @@ def test_submit_time_rejections():
     scheduler = make(FakeRunner(), max_queue_size=2, max_model_len=16)
     with pytest.raises(RejectedError) as caught:
         scheduler.submit([], GenerationConfig(max_output_tokens=1))
-    assert caught.value.reason is RejectionReason.CONTEXT_OVERFLOW
+    assert caught.value.reason is Refusal.TOO_LONG
     with pytest.raises(RejectedError) as caught:
         scheduler.submit([1] * 10, GenerationConfig(max_output_tokens=7))
-    assert caught.value.reason is RejectionReason.CONTEXT_OVERFLOW
+    assert caught.value.reason is Refusal.TOO_LONG
     scheduler.submit([1] * 10, GenerationConfig(max_output_tokens=6))
     scheduler.submit([1], GenerationConfig(max_output_tokens=1))
     with pytest.raises(RejectedError) as caught:
         scheduler.submit([1], GenerationConfig(max_output_tokens=1))
-    assert caught.value.reason is RejectionReason.QUEUE_FULL
+    assert caught.value.reason is Refusal.QUEUE_FULL
     assert [r.request_id for r in scheduler.waiting] == ["req-00000001", "req-00000002"]
 
 
@@ -262,9 +262,9 @@ def test_eos_finishes_and_is_kept_but_not_streamed():
                                on_token=lambda r, t: streamed.append(t))
     ignoring = scheduler.submit([1, 2], GenerationConfig(max_output_tokens=4, eos_token_id=None))
     scheduler.run_until_done(100)
-    assert request.generated_token_ids == [100, 101, 102] and request.finish_reason == "eos_token_reached"
+    assert request.output == [100, 101, 102] and request.finish_reason == "eos_token_reached"
     assert streamed == [100, 101]
-    assert ignoring.generated_token_ids == [100, 101, 102, 103]
+    assert ignoring.output == [100, 101, 102, 103]
 
 
 def test_active_limit_and_fifo_admission():
@@ -299,10 +299,10 @@ def test_forward_failure_fails_the_plan_and_the_loop_goes_on():
     doomed = scheduler.submit([1] * 3, GenerationConfig(max_output_tokens=2))
     runner.fail_next = RuntimeError("kernel exploded")
     scheduler.step()
-    assert doomed.state is RequestState.FAILED and not doomed.rejected and "kernel exploded" in doomed.error_detail
+    assert doomed.state is RequestState.FAILED and not doomed.rejected and "kernel exploded" in doomed.error
     later = scheduler.submit([1] * 3, GenerationConfig(max_output_tokens=2))
     scheduler.run_until_done(100)
-    assert later.generated_token_ids == [100, 101] and not runner.resident
+    assert later.output == [100, 101] and not runner.resident
 
 
 def test_admission_failure_is_counted():
@@ -315,7 +315,7 @@ def test_admission_failure_is_counted():
     scheduler = make(Refusing())
     request = scheduler.submit([1], GenerationConfig(max_output_tokens=1))
     scheduler.step()
-    assert request.state is RequestState.FAILED and request.rejected and "admission refused" in request.error_detail
+    assert request.state is RequestState.FAILED and request.rejected and "admission refused" in request.error
 
 
 def test_prompt_is_published_once_its_last_portion_has_run():
@@ -328,8 +328,8 @@ def test_prompt_is_published_once_its_last_portion_has_run():
             self.published = []
 
         def publish_prefix(self, request) -> None:
-            assert request.tokens_fed >= len(request.prompt_token_ids)
-            self.published.append((request.request_id, request.generated_count))
+            assert request.cached >= len(request.prompt)
+            self.published.append((request.request_id, len(request.output)))
 
     runner = Publishing()
     scheduler = make(runner)
@@ -360,25 +360,25 @@ class AsyncFakeRunner(FakeRunner):
 
     def execute_batch(self, plan):
         outputs = super().execute_batch(plan)
-        return {item.request.request_id: self._token(item.request, item.request.generated_count)
-                for item in plan.items if item.request.request_id in outputs}
+        return {item.request.request_id: self._token(item.request, len(item.request.output))
+                for item in plan.portions if item.request.request_id in outputs}
 
     def launch_decode(self, plan, feed, token_indices):
         required = dict(self.resident)
-        for item in plan.items:
-            required[item.request.request_id] = max(required[item.request.request_id], item.end_pos)
+        for item in plan.portions:
+            required[item.request.request_id] = max(required[item.request.request_id], item.end)
         if sum(required.values()) > self.token_capacity:
             error = RuntimeError("fake KV capacity exhausted")
             error.is_capacity_error = True
             raise error
         self.resident = required
         fed_tokens = []
-        for item, source in zip(plan.items, feed):
-            assert item.start_pos == item.request.tokens_fed and item.query_length == 1
-            fed_tokens.append(self.device_tokens[source] if source >= 0 else item.token_ids[0])
-            item.request.tokens_fed = item.end_pos
+        for item, source in zip(plan.portions, feed):
+            assert item.start == item.request.cached and item.length == 1
+            fed_tokens.append(self.device_tokens[source] if source >= 0 else item.tokens[0])
+            item.request.cached = item.end
         self.launches.append((plan.request_ids, tuple(fed_tokens)))
-        self.device_tokens = [self._token(item.request, index) for item, index in zip(plan.items, token_indices)]
+        self.device_tokens = [self._token(item.request, index) for item, index in zip(plan.portions, token_indices)]
         produced = dict(zip(plan.request_ids, self.device_tokens))
 
         class Pending:
@@ -404,12 +404,12 @@ def test_async_decode_gives_the_same_tokens_with_one_launch_per_token():
     sync_runner, a0, b0 = run(lambda r: make(r, async_decode=False))
     runner, a, b = run(make_async)
     assert not sync_runner.launches and runner.launches
-    assert a.generated_token_ids == a0.generated_token_ids == [100, 101, 102, 103, 104]
-    assert b.generated_token_ids == b0.generated_token_ids == [100, 101, 102]
+    assert a.output == a0.output == [100, 101, 102, 103, 104]
+    assert b.output == b0.output == [100, 101, 102]
     # the first token of each comes with its prompt; every further token is one row of one launch, no more:
     # b leaves the launches when its limit is in sight, nothing runs for a token that is not wanted
     launched_rows = sum(len(ids) for ids, _ in runner.launches)
-    sampled_with_prompts = sum(item.sample for plan in runner.plans for item in plan.items)
+    sampled_with_prompts = sum(item.samples for plan in runner.plans for item in plan.portions)
     assert launched_rows + sampled_with_prompts == 5 + 3
     # from the second launch on, rows are fed the token the launch before made, not a placeholder
     assert runner.launches[1][1][0] == 101
@@ -421,13 +421,13 @@ def test_async_decode_tokens_arrive_one_call_late():
     scheduler = make_async(runner)
     request = scheduler.submit(list(range(4)), GenerationConfig(max_output_tokens=6))
     scheduler.step()                    # the prompt, with its first token
-    assert request.generated_count == 1
+    assert len(request.output) == 1
     scheduler.step()                    # launches token 2; nothing has arrived
-    assert request.generated_count == 1 and scheduler.has_work()
+    assert len(request.output) == 1 and scheduler.has_work()
     scheduler.step()                    # launches token 3, takes token 2
-    assert request.generated_count == 2
+    assert len(request.output) == 2
     scheduler.run_until_done()
-    assert request.generated_token_ids == [100, 101, 102, 103, 104, 105]
+    assert request.output == [100, 101, 102, 103, 104, 105]
 
 
 def test_async_decode_end_of_sequence_costs_one_dropped_step():
@@ -436,8 +436,8 @@ def test_async_decode_end_of_sequence_costs_one_dropped_step():
     stops = scheduler.submit(list(range(4)), GenerationConfig(max_output_tokens=10, eos_token_id=7))
     goes_on = scheduler.submit(list(range(4)), GenerationConfig(max_output_tokens=6))
     scheduler.run_until_done()
-    assert stops.generated_token_ids == [100, 101, 7] and stops.finish_reason == "eos_token_reached"
-    assert goes_on.generated_token_ids == [100, 101, 102, 103, 104, 105]
+    assert stops.output == [100, 101, 7] and stops.finish_reason == "eos_token_reached"
+    assert goes_on.output == [100, 101, 102, 103, 104, 105]
     launched_for_stops = sum(stops.request_id in ids for ids, _ in runner.launches)
     assert launched_for_stops == 3  # tokens 2 and 3, and one step more that was under way when token 7 arrived
     assert not runner.resident and (stops.request_id, False) in runner.released
@@ -451,8 +451,8 @@ def test_async_decode_lets_a_new_request_in_and_survives_a_shortage():
         scheduler.step()
     late = scheduler.submit(list(range(8)), GenerationConfig(max_output_tokens=12))  # both need 20: one must wait
     scheduler.run_until_done(max_iterations=200)
-    assert first.generated_token_ids == [100 + i for i in range(12)]
-    assert late.generated_token_ids == [100 + i for i in range(12)]
+    assert first.output == [100 + i for i in range(12)]
+    assert late.output == [100 + i for i in range(12)]
     assert scheduler.metrics.snapshot()["requests"]["preempted_total"] >= 1
     assert not runner.resident
 
@@ -463,7 +463,7 @@ def test_async_decode_cancel_takes_what_is_in_flight_first():
     request = scheduler.submit(list(range(4)), GenerationConfig(max_output_tokens=9))
     for _ in range(3):
         scheduler.step()
-    assert request.generated_count == 2
+    assert len(request.output) == 2
     scheduler.cancel(request)
-    assert request.state is RequestState.CANCELLED and request.generated_count == 3 and not scheduler.has_work()
+    assert request.state is RequestState.CANCELLED and len(request.output) == 3 and not scheduler.has_work()
     assert not runner.resident
