@@ -35,13 +35,39 @@ from .allocator import CacheCapacityFull, PageAllocator
 PREFIX_HOLDER = "\0prefix-index"
 
 
+UNBOUNDED_TOKENS = 1 << 62   # what a cache without pages reports as free
+
+
 @dataclass(frozen=True)
 class PagedKV:
-    """A mixer that appends ``kv_heads * head_dim`` keys and values per token."""
+    """A mixer that appends per token, for each of ``kv_heads`` heads, a key of
+    ``head_dim`` numbers and, if ``values``, a value of ``value_dim`` numbers
+    (``None``: as wide as the key).  ``values=False`` is a cache of one vector
+    per token and head (a latent that keys and values are both made from, or
+    keys alone).  With a ``window`` only that many latest tokens are read."""
 
     kv_heads: int
     head_dim: int
     window: int | None = None
+    values: bool = True
+    value_dim: int | None = None
+
+    def __post_init__(self) -> None:
+        if self.kv_heads < 1 or self.head_dim < 1:
+            raise ValueError("a paged cache needs at least one head of at least one number")
+        if self.value_dim is not None and (not self.values or self.value_dim < 1):
+            raise ValueError("value_dim needs values=True and a positive width")
+
+    @property
+    def value_width(self) -> int:
+        """Numbers per value vector; 0 where none are stored."""
+        if not self.values:
+            return 0
+        return self.head_dim if self.value_dim is None else self.value_dim
+
+    @property
+    def numbers_per_token(self) -> int:
+        return self.kv_heads * (self.head_dim + self.value_width)
 
 
 @dataclass(frozen=True)
@@ -53,6 +79,24 @@ class FixedState:
 
 
 @dataclass(frozen=True)
+class GroupBytes:
+    """One group's memory, as the reference's cache reports it for its single pool
+    (src/cloud_engine/cache.py:503-526): ``reserved`` is what the used pages take in
+    all the group's units, ``occupied`` what the tokens in them take, the rest is
+    lost inside pages that are not full."""
+
+    units: int
+    pages_total: int
+    pages_used: int
+    reserved_bytes: int
+    occupied_bytes: int
+
+    @property
+    def internal_fragmentation_bytes(self) -> int:
+        return self.reserved_bytes - self.occupied_bytes
+
+
+@dataclass(frozen=True)
 class CacheStats:
     pages_total: int
     pages_used: int
@@ -61,10 +105,23 @@ class CacheStats:
     prefix_cache_hits: int
     prefix_cache_misses: int
     slots_used: int
+    groups: tuple[GroupBytes, ...] = ()
 
     @property
     def utilization(self) -> float:
         return self.pages_used / self.pages_total if self.pages_total else 0.0
+
+    @property
+    def reserved_bytes(self) -> int:
+        return sum(group.reserved_bytes for group in self.groups)
+
+    @property
+    def occupied_bytes(self) -> int:
+        return sum(group.occupied_bytes for group in self.groups)
+
+    @property
+    def internal_fragmentation_bytes(self) -> int:
+        return self.reserved_bytes - self.occupied_bytes
 
 
 class _Group:
@@ -98,6 +155,7 @@ class CacheManager:
         max_model_len: int,
         prefill_chunk: int = 256,
         prefix_cache_pages: int = 0,
+        element_bytes: int = 2,
     ) -> None:
         if page_size < 1 or page_size & (page_size - 1):
             raise ValueError(f"page_size must be a power of two, got {page_size}")
@@ -106,6 +164,7 @@ class CacheManager:
         self.page_size = page_size
         self.max_running = max_running
         self.max_model_len = max_model_len
+        self.element_bytes = element_bytes  # of one cached number; only the byte statistics use it
         self.table_width = -(-max_model_len // page_size)
         self.unit_specs = tuple(unit_specs)
         self.groups: list[_Group] = []
@@ -164,6 +223,23 @@ class CacheManager:
             return 0
         held = max((sum(1 for p in g.tables[request_id] if p >= 0) for g in self.groups), default=0)
         return held * self.page_size
+
+    def free_tokens(self) -> int:
+        """Tokens the pool could take now: the free pages of the scarcest group, and with them the
+        pages that only the prefix index holds, which growth evicts when it needs them.  A cache
+        without pages (every unit a fixed state, or none) is never the limit."""
+        if not self.groups:
+            return UNBOUNDED_TOKENS
+        pages = []
+        for index, group in enumerate(self.groups):
+            free = group.allocator.free_count
+            if index == 0 and self._prefix:
+                # a page that a request shares keeps its ancestors shared too, so every page held by
+                # the index alone can be evicted, leaves first
+                free += sum(1 for node in self._prefix.values()
+                            if group.allocator.holders_of(node.page) == (PREFIX_HOLDER,))
+            pages.append(free)
+        return min(pages) * self.page_size
 
     def take_dirty_rows(self) -> list[tuple[int, int, list[int]]]:
         """(group, slot, table) of every block-table row that changed since the last call."""
@@ -366,24 +442,39 @@ class CacheManager:
             pass
 
     # -- accounting -------------------------------------------------------------
+    def _group_bytes(self, index: int, group: _Group) -> GroupBytes:
+        """Tokens are counted once per page, however many hold it; a shared page is a full one."""
+        size = self.page_size
+        filled: dict[int, int] = {}
+        for request_id, table in group.tables.items():
+            length = self._length.get(request_id, 0)
+            for place, page in enumerate(table):
+                if page >= 0:
+                    filled[page] = max(filled.get(page, 0), min(size, max(0, length - place * size)))
+        if index == 0:
+            for node in self._prefix.values():
+                filled[node.page] = size
+        token_bytes = group.spec.numbers_per_token * self.element_bytes * len(group.units)
+        used = group.allocator.used_count
+        return GroupBytes(units=len(group.units), pages_total=group.allocator.total_pages, pages_used=used,
+                          reserved_bytes=used * size * token_bytes,
+                          occupied_bytes=sum(filled.values()) * token_bytes)
+
     def stats(self) -> CacheStats:
-        total = sum(g.allocator.total_pages for g in self.groups)
-        used = sum(g.allocator.used_count for g in self.groups)
-        prefix_pages = len(self._prefix)
-        request_pages = sum(
-            1
-            for g in self.groups
-            for page in list(g.allocator._holders)
-            if any(h != PREFIX_HOLDER for h in g.allocator.holders_of(page))
-        )
+        request_pages = 0
+        for group in self.groups:
+            allocator = group.allocator
+            request_pages += sum(1 for page in list(allocator._holders)
+                                 if any(holder != PREFIX_HOLDER for holder in allocator.holders_of(page)))
         return CacheStats(
-            pages_total=total,
-            pages_used=used,
+            pages_total=sum(g.allocator.total_pages for g in self.groups),
+            pages_used=sum(g.allocator.used_count for g in self.groups),
             request_pages_used=request_pages,
-            prefix_pages_used=prefix_pages,
+            prefix_pages_used=len(self._prefix),
             prefix_cache_hits=self.prefix_cache_hits,
             prefix_cache_misses=self.prefix_cache_misses,
             slots_used=len(self._slots),
+            groups=tuple(self._group_bytes(i, g) for i, g in enumerate(self.groups)),
         )
 
     def assert_invariants(self) -> None:

@@ -1,5 +1,5 @@
 from .engine_config import EngineConfig, build_engine_config, canonical_dtype
-from .qwen2 import ConfigError, Qwen2Config
+from .qwen2 import Qwen2Config
 from .registry import (
     ARCHITECTURES,
     Architecture,
@@ -8,7 +8,10 @@ from .registry import (
     load_config,
     register_architecture,
 )
-from .specs import LayerCall, LayerSpec, ModelSpec, PartSpec
+from .specs import ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpec
+
+# the architectures this package brings; others register themselves the same way from outside
+register_architecture("Qwen2ForCausalLM", Qwen2Config, model_type="qwen2")
 
 __all__ = [
     "ARCHITECTURES", "Architecture", "ConfigError", "EngineConfig", "LayerCall", "LayerSpec",

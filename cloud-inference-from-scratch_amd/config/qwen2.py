@@ -14,7 +14,7 @@ from __future__ import annotations
 from dataclasses import dataclass, fields
 from typing import Any
 
-from .specs import LayerCall, LayerSpec, ModelSpec, PartSpec
+from .specs import ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpec
 
 _REQUIRED = (
     "hidden_size",
@@ -25,10 +25,6 @@ _REQUIRED = (
     "vocab_size",
     "rms_norm_eps",
 )
-
-
-class ConfigError(ValueError):
-    """A ``config.json`` that this engine does not run."""
 
 
 @dataclass(frozen=True)

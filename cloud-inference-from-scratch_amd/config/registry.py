@@ -14,7 +14,7 @@ from dataclasses import dataclass
 from pathlib import Path
 from typing import Any, Callable
 
-from .qwen2 import ConfigError, Qwen2Config
+from .specs import ConfigError
 
 
 @dataclass(frozen=True)
@@ -63,5 +63,3 @@ def load_config(model_dir: str | Path) -> Any:
     with open(path, encoding="utf-8") as handle:
         return config_from_dict(json.load(handle))
 
-
-register_architecture("Qwen2ForCausalLM", Qwen2Config, model_type="qwen2")

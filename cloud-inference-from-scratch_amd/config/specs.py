@@ -15,6 +15,11 @@ from dataclasses import dataclass, field
 from typing import Any
 
 
+class ConfigError(ValueError):
+    """A ``config.json`` that no registered architecture can run: an unknown name, a key
+    that is missing, a value outside what the parts take."""
+
+
 @dataclass(frozen=True)
 class PartSpec:
     """``kind`` selects the part class; ``params`` are its constructor arguments."""

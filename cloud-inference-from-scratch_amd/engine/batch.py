@@ -96,7 +96,7 @@ class PagedView:
     """One cache unit of paged keys and values, as a mixer sees it."""
 
     k_pool: torch.Tensor         # [pages, kv_heads, page_size, head_dim]
-    v_pool: torch.Tensor         # [pages, kv_heads, head_dim, page_size]  (transposed)
+    v_pool: torch.Tensor | None  # [pages, kv_heads, value_width, page_size]  (transposed); None: keys only
     block_table: torch.Tensor    # int32 [max_running, width] of the unit's group
     page_size: int
 

@@ -1,12 +1,13 @@
 """Device side of the cache: page pools, block tables and state rows.
 
-For every group of the :class:`~cie_amd.cache.manager.CacheManager` one pool
-``[units, 2, pages, kv_heads, page_size * head_dim]`` (keys at index 0 of the
-second axis as ``[page_size, head_dim]``, values at index 1 transposed as
-``[head_dim, page_size]``, the layouts the matrix-core attention reads with plain
-vector loads; a page of one head is contiguous) and one int32 block
-table ``[max_running, width]`` whose row ``slot`` holds the request's host
-table in its first entries.  The reference keeps ``[layers, pages, page_size, kv_heads, head_dim]``
+For every group of the :class:`~cie_amd.cache.manager.CacheManager` a pool of
+keys ``[units, pages, kv_heads, page_size, head_dim]`` and, where the group's
+need stores values, a pool of values ``[units, pages, kv_heads, value_width,
+page_size]``, transposed: the layouts the matrix-core attention reads with plain
+vector loads, a page of one head contiguous.  (A need with ``values=False`` has
+the key pool only; its mixer decides what the one vector per token means.)
+Beside them one int32 block table ``[max_running, width]`` whose row ``slot``
+holds the request's host table in its first entries.  The reference keeps ``[layers, pages, page_size, kv_heads, head_dim]``
 pools (src/cloud_engine/cache.py:266-274) and uploads padded tables every step
 (src/cloud_engine/engine.py:264-278); here only rows that changed are copied.
 
@@ -34,15 +35,19 @@ class DeviceCache:
         self.manager = manager
         self.dtype = dtype
         self.device = device
-        self.pools: list[torch.Tensor] = []
+        self.key_pools: list[torch.Tensor] = []
+        self.value_pools: list[torch.Tensor | None] = []
         self.tables: list[torch.Tensor] = []
         self.pad_slot = manager.max_running
         self._row_seen: dict[tuple[int, int], tuple[int, int]] = {}  # (group, slot) -> (slot serial, entries copied)
         for group in manager.groups:
             spec = group.spec
             pad_page = group.allocator.total_pages
-            shape = (len(group.units), 2, pad_page + 1, spec.kv_heads, manager.page_size, spec.head_dim)
-            self.pools.append(torch.zeros(shape, dtype=dtype, device=device))
+            units, pages, size = len(group.units), pad_page + 1, manager.page_size
+            self.key_pools.append(torch.zeros((units, pages, spec.kv_heads, size, spec.head_dim),
+                                              dtype=dtype, device=device))
+            self.value_pools.append(torch.zeros((units, pages, spec.kv_heads, spec.value_width, size),
+                                                dtype=dtype, device=device) if spec.values else None)
             table = torch.zeros((manager.max_running + 1, manager.table_width), dtype=torch.int32, device=device)
             table[self.pad_slot] = pad_page
             self.tables.append(table)
@@ -56,11 +61,10 @@ class DeviceCache:
             if unit in manager.unit_group:
                 index = manager.unit_group[unit]
                 local = manager.groups[index].units.index(unit)
-                pool = self.pools[index]
-                spec = manager.groups[index].spec
-                pages = manager.groups[index].allocator.total_pages + 1
-                values = pool[local, 1].view(pages, spec.kv_heads, spec.head_dim, manager.page_size)
-                self._views[unit] = PagedView(pool[local, 0], values, self.tables[index], manager.page_size)
+                values = self.value_pools[index]
+                self._views[unit] = PagedView(self.key_pools[index][local],
+                                              values[local] if values is not None else None,
+                                              self.tables[index], manager.page_size)
             elif unit in self.states:
                 self._views[unit] = StateView(self.states[unit])
             else:
@@ -70,7 +74,8 @@ class DeviceCache:
         return self._views[unit]
 
     def bytes(self) -> int:
-        return sum(p.numel() * p.element_size() for p in self.pools)
+        pools = self.key_pools + [p for p in self.value_pools if p is not None]
+        return sum(p.numel() * p.element_size() for p in pools)
 
     def sync(self) -> None:
         """Bring the device block tables up to the host's; clear the state of

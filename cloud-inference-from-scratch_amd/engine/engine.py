@@ -159,6 +159,14 @@ class Engine:
                 "utilization": round(stats.utilization, 4),
                 "request_pages_used": stats.request_pages_used, "prefix_pages_used": stats.prefix_pages_used,
                 "prefix_cache_hits": stats.prefix_cache_hits, "prefix_cache_misses": stats.prefix_cache_misses,
+                "reserved_bytes": stats.reserved_bytes, "occupied_bytes": stats.occupied_bytes,
+                "internal_fragmentation_bytes": stats.internal_fragmentation_bytes,
+                "groups": [
+                    {"units": g.units, "pages_total": g.pages_total, "pages_used": g.pages_used,
+                     "reserved_bytes": g.reserved_bytes, "occupied_bytes": g.occupied_bytes,
+                     "internal_fragmentation_bytes": g.internal_fragmentation_bytes}
+                    for g in stats.groups
+                ],
             }
         snapshot["runner"] = {
             "forward_invocations": getattr(runner, "forward_invocations", 0),

@@ -19,7 +19,7 @@ from typing import Any
 
 import torch
 
-from ..cache.manager import CacheManager
+from ..cache.manager import CacheManager, PagedKV
 from ..config.engine_config import EngineConfig
 from ..profiling import trace_range
 from ..sampling.sampler import Sampler
@@ -69,6 +69,7 @@ class Runner:
         self.cache = CacheManager(
             needs, config.page_size, kv_tokens, config.max_running, config.max_model_len,
             prefill_chunk=config.prefill_chunk, prefix_cache_pages=config.prefix_cache_pages,
+            element_bytes=torch.tensor([], dtype=self.dtype).element_size(),
         )
         self.device_cache = DeviceCache(self.cache, self.dtype, self.device)
         self.forward_invocations = 0
@@ -83,7 +84,7 @@ class Runner:
 
     def _tokens_from_bytes(self, needs: list[Any]) -> int:
         element = torch.tensor([], dtype=self.dtype).element_size()
-        per_token = sum(2 * n.kv_heads * n.head_dim * element for n in needs if hasattr(n, "kv_heads"))
+        per_token = sum(n.numbers_per_token * element for n in needs if isinstance(n, PagedKV))
         if per_token == 0:
             return self.config.page_size
         page = self.config.page_size
@@ -137,8 +138,8 @@ class Runner:
         return self.mixed_graphs.replays if self.mixed_graphs is not None else 0
 
     def free_tokens(self) -> int:
-        """Tokens the pool could take now (free pages of the scarcest group)."""
-        return min((g.allocator.free_count for g in self.cache.groups), default=0) * self.cache.page_size
+        """Tokens the pool could take now (see :meth:`CacheManager.free_tokens`)."""
+        return self.cache.free_tokens()
 
     def execute_batch(self, plan: Any) -> dict[str, int]:
         """Run a scheduler's plan and sample where it asks to (the reference's

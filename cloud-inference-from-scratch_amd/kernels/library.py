@@ -16,6 +16,7 @@ import hashlib
 import os
 import re
 import shutil
+import stat
 import subprocess
 import sys
 import tempfile
@@ -66,9 +67,26 @@ def _hipcc() -> str | None:
     return str(candidate) if candidate.is_file() else None
 
 
+def _fallback_dir() -> Path:
+    return Path(tempfile.gettempdir()) / f"cie_amd_build_{os.getuid()}"
+
+
+def _private_to_this_user(folder: Path) -> bool:
+    """The fallback folder has a name anyone can guess, in a place anyone can write: it is used only if
+    it is a real folder of this user's that nobody else can write into.  Otherwise another user could
+    have put a library there that this process would load and run."""
+    try:
+        folder.mkdir(mode=0o700, exist_ok=True)
+        info = folder.lstat()
+    except OSError:
+        return False
+    return stat.S_ISDIR(info.st_mode) and info.st_uid == os.getuid() and not info.st_mode & 0o022
+
+
 def _build_dirs() -> list[Path]:
-    fallback = Path(tempfile.gettempdir()) / f"cie_amd_build_{os.getuid()}"
-    return [CSRC / "_build", fallback]
+    """Where a built library may lie: in the tree, else in this user's own folder under the temporary directory."""
+    fallback = _fallback_dir()
+    return [CSRC / "_build"] + ([fallback] if _private_to_this_user(fallback) else [])
 
 
 def _log(message: str) -> None:

@@ -102,6 +102,9 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = 
     return out
 
 
+MAX_NORM_WIDTH = 16384  # a row of the norm kernels is held in 64 KB of LDS as float32
+
+
 def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -117,8 +120,8 @@ def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: 
         raise ValueError(f"weight must be [{hidden}], is {tuple(weight.shape)}")
     if not (weight.dtype in (out_dtype, torch.float32)):
         raise ValueError(f"weight dtype {weight.dtype} does not fit {out_dtype}")
-    if not (hidden * 4 <= 64 * 1024):
-        raise ValueError(f"hidden size {hidden} exceeds the norm kernel's 16384")
+    if not (hidden <= MAX_NORM_WIDTH):
+        raise ValueError(f"hidden size {hidden} exceeds the norm kernel's {MAX_NORM_WIDTH}")
     if not (eps > 0):
         raise ValueError(f"eps must be positive, is {eps}")
     if branch is not None:
@@ -152,7 +155,7 @@ def add_parts_rmsnorm(residual: torch.Tensor, parts: torch.Tensor, weight: torch
     _gpu("weight", weight, dims=1)
     if not (weight.shape[0] == hidden and weight.dtype in (torch.bfloat16, torch.float32)):
         raise ValueError("norm weight does not fit")
-    if not (hidden * 4 <= 64 * 1024 and eps > 0):
+    if not (hidden <= MAX_NORM_WIDTH and eps > 0):
         raise ValueError(f"hidden {hidden} or eps {eps} out of range")
     if rows is not None:
         _gpu("rows", rows, torch.int32, 1)

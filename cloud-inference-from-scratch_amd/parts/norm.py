@@ -27,6 +27,8 @@ class RMSNorm(Part):
     def __init__(self, size: int, eps: float) -> None:
         if size <= 0 or not eps > 0:
             raise ValueError(f"RMSNorm needs a positive size and eps, got {size}, {eps}")
+        if size > ops.MAX_NORM_WIDTH:
+            raise ValueError(f"the norm kernels take rows of up to {ops.MAX_NORM_WIDTH} numbers, not {size}")
         self.size = size
         self.eps = eps
         self.weight: Optional[torch.Tensor] = None

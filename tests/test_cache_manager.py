@@ -346,3 +346,73 @@ def test_shared_pages_survive_index_pressure():
         m.ensure_capacity_batch({"c": 28})  # 7 pages, 6 free: b's shared pages cannot be evicted
     assert m.block_table(0, "b")[0] in [p for p in range(8) if PREFIX_HOLDER in m.groups[0].allocator.holders_of(p)]
     m.assert_invariants()
+
+
+# -- what a paged need stores, byte statistics, room in the pool ---------------------------
+def test_a_paged_need_says_what_it_stores():
+    assert PagedKV(2, 16).numbers_per_token == 2 * (16 + 16) and PagedKV(2, 16).value_width == 16
+    keys_only = PagedKV(1, 24, values=False)
+    assert keys_only.value_width == 0 and keys_only.numbers_per_token == 24
+    assert PagedKV(4, 8, value_dim=20).numbers_per_token == 4 * 28
+    assert PagedKV(2, 16) != PagedKV(2, 16, value_dim=8), "another width is another group"
+    with pytest.raises(ValueError):
+        PagedKV(2, 16, values=False, value_dim=8)
+    with pytest.raises(ValueError):
+        PagedKV(0, 16)
+    m = manager(unit_specs=[PagedKV(2, 16), PagedKV(2, 16, values=False), PagedKV(2, 16)])
+    assert [g.units for g in m.groups] == [[0, 2], [1]]
+
+
+def test_byte_statistics_follow_pages_and_tokens():
+    """The reference's figures (src/cloud_engine/cache.py:503-526): reserved = used pages x page bytes over
+    all layers, occupied = tokens x token bytes, the difference is lost inside pages that are not full."""
+    m = manager(unit_specs=[PagedKV(2, 16)] * 3, element_bytes=2, prefix_cache_pages=8)  # pages of 4 tokens
+    token_bytes = 2 * (16 + 16) * 2 * 3
+    assert m.stats().reserved_bytes == m.stats().occupied_bytes == 0
+    prompt = list(range(9))
+    m.admit("a", prompt)
+    m.ensure_capacity_batch({"a": 9})
+    stats = m.stats()
+    assert stats.reserved_bytes == 3 * 4 * token_bytes and stats.occupied_bytes == 0  # reserved before the step ran
+    m.commit_lengths({"a": 9})
+    stats = m.stats()
+    assert stats.occupied_bytes == 9 * token_bytes
+    assert stats.internal_fragmentation_bytes == 3 * token_bytes == stats.groups[0].internal_fragmentation_bytes
+    # a page that the index and two requests share is counted once
+    m.publish_prefix("a", prompt)
+    assert m.admit("b", prompt[:8] + [70]) == 8
+    m.ensure_capacity_batch({"b": 9})
+    m.commit_lengths({"b": 9})
+    stats = m.stats()
+    assert stats.pages_used == 4 and stats.reserved_bytes == 16 * token_bytes and stats.occupied_bytes == 10 * token_bytes
+    m.release("a", prompt), m.release("b")
+    stats = m.stats()
+    assert stats.reserved_bytes == stats.occupied_bytes == 8 * token_bytes  # the two indexed pages are full ones
+    # groups report their own: a keys-only group of one unit in float32 beside keys and values
+    two = manager(unit_specs=[PagedKV(2, 16), PagedKV(1, 8, values=False)], element_bytes=4)
+    two.admit("x")
+    two.ensure_capacity_batch({"x": 5})
+    two.commit_lengths({"x": 5})
+    first, second = two.stats().groups
+    assert (first.reserved_bytes, first.occupied_bytes) == (8 * 64 * 4, 5 * 64 * 4)
+    assert (second.reserved_bytes, second.occupied_bytes) == (8 * 8 * 4, 5 * 8 * 4)
+    assert two.stats().internal_fragmentation_bytes == 3 * (64 + 8) * 4
+
+
+def test_free_tokens_count_what_the_index_would_give_back():
+    m = manager(kv_tokens=32, prefix_cache_pages=8)  # 8 pages of 4
+    assert m.free_tokens() == 32
+    prompt = list(range(13))
+    m.admit("a", prompt)
+    m.ensure_capacity_batch({"a": 13})
+    m.commit_lengths({"a": 13})
+    assert m.free_tokens() == 16
+    m.release("a", prompt)  # three full pages stay in the index
+    assert m.groups[0].allocator.free_count == 5 and m.free_tokens() == 32
+    assert m.admit("b", prompt[:8] + [99]) == 8  # two of them are shared now: only the third can be evicted
+    assert m.free_tokens() == 24
+    m.ensure_capacity_batch({"b": 9 + 20})  # 6 more pages: 5 free and the evicted one
+    assert m.free_tokens() == 0 and m.stats().prefix_pages_used == 2
+    m.assert_invariants()
+    only_state = manager(unit_specs=[FixedState((3,))])
+    assert only_state.free_tokens() > 1 << 40, "a cache without pages never limits admission"

@@ -42,3 +42,20 @@ def test_a_product_of_no_rows_launches_nothing_and_widens_nothing():
     assert logits.shape == (0, 32) and logits.dtype == torch.float32
     gated = linear(rows, weight, None, epilogue="silu")
     assert gated.shape == (0, 16) and gated.dtype == torch.bfloat16
+
+
+def test_the_fallback_build_folder_must_be_this_users_own(tmp_path, monkeypatch):
+    """The folder under the temporary directory has a name anyone can guess: one that others can write
+    into (or that is no folder of this user's) is neither built into nor loaded from."""
+    import os
+
+    folder = tmp_path / "cie_amd_build_me"
+    monkeypatch.setattr(library, "_fallback_dir", lambda: folder)
+    assert library._build_dirs()[-1] == folder and folder.stat().st_mode & 0o777 == 0o700
+    os.chmod(folder, 0o777)  # as if someone else had made it before us
+    assert folder not in library._build_dirs()
+    os.chmod(folder, 0o755)
+    assert folder in library._build_dirs()
+    folder.rmdir()
+    folder.symlink_to(tmp_path)  # a link is no folder of ours, wherever it points
+    assert folder not in library._build_dirs()

@@ -467,3 +467,65 @@ def test_async_decode_cancel_takes_what_is_in_flight_first():
     scheduler.cancel(request)
     assert request.state is RequestState.CANCELLED and len(request.output) == 3 and not scheduler.has_work()
     assert not runner.resident
+
+
+# -- a runner that keeps a real cache manager (no tensors): what admission sees of the pool -------------
+class ManagerRunner:
+    def __init__(self, manager) -> None:
+        self.cache = manager
+        self.most_side_by_side = 0
+
+    def admit(self, request) -> None:
+        request.cached = self.cache.admit(request.request_id, request.prompt)
+
+    def release(self, request, preempted: bool = False) -> None:
+        self.cache.release(request.request_id, None if preempted else request.prompt)
+
+    def allocated_tokens(self, request) -> int:
+        return self.cache.allocated_tokens(request.request_id)
+
+    def free_tokens(self) -> int:
+        return self.cache.free_tokens()
+
+    def execute_batch(self, plan):
+        need = {p.request.request_id: p.end for p in plan.portions}
+        self.cache.ensure_capacity_batch(need)
+        self.cache.commit_lengths(need)
+        self.most_side_by_side = max(self.most_side_by_side, len(plan.portions))
+        for portion in plan.portions:
+            portion.request.cached = portion.end
+        return {p.request.request_id: 100 + len(p.request.output) for p in plan.portions if p.samples}
+
+
+def test_pages_that_only_the_prefix_index_holds_do_not_block_admission():
+    """Earlier requests have left the index full; the free list alone holds one newcomer.  The
+    newcomers still run side by side: what the index holds alone is evicted when they grow."""
+    from cie_amd.cache.manager import CacheManager, PagedKV
+
+    manager = CacheManager([PagedKV(1, 8)], page_size=4, kv_tokens=64, max_running=8, max_model_len=64,
+                           prefix_cache_pages=12)
+    runner = ManagerRunner(manager)
+    scheduler = make(runner, max_model_len=64, max_running=8, token_budget=64, prefill_chunk=16)
+    for i in range(3):  # three prompts of 17 tokens leave four full pages each
+        scheduler.submit([i + 1] * 17, GenerationConfig(max_output_tokens=1))
+    scheduler.run_until_done(50)
+    assert manager.stats().prefix_pages_used == 12 and manager.groups[0].allocator.free_count == 4
+    runner.most_side_by_side = 0
+    fresh = [scheduler.submit([50 + i] * 9, GenerationConfig(max_output_tokens=3)) for i in range(4)]
+    scheduler.run_until_done(50)
+    assert runner.most_side_by_side == 4, "each needs 3 pages; 4 are free, 12 more can be evicted"
+    assert all(r.output == [100, 101, 102] and r.preemptions == 0 for r in fresh)
+    manager.assert_invariants()
+
+
+def test_a_cache_without_pages_admits_side_by_side():
+    """Every unit a state of fixed size: nothing is paged, so the pool never makes a request wait."""
+    from cie_amd.cache.manager import CacheManager, FixedState
+
+    runner = ManagerRunner(CacheManager([FixedState((4,))], page_size=4, kv_tokens=4, max_running=4, max_model_len=64))
+    scheduler = make(runner, max_model_len=64, max_running=4, admit_within_pool=True)
+    requests = [scheduler.submit([i + 1] * 6, GenerationConfig(max_output_tokens=4)) for i in range(4)]
+    scheduler.step()
+    assert len(scheduler.active) == 4
+    scheduler.run_until_done(50)
+    assert runner.most_side_by_side == 4 and all(r.output == [100, 101, 102, 103] for r in requests)
