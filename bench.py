@@ -1,22 +1,33 @@
 #!/usr/bin/env python3
-"""Serving benchmark on one MI355X: decode tokens per second of the Qwen2.5-3B
-shape with random weights, plus prefill and roofline figures.
+"""Serving benchmark on one MI355X: decode tokens per second of a Qwen2.5 shape
+(default: the 3B one) with random weights, plus prefill and roofline figures.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 36]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
+                    [--shape 3b|7b|14b] [--layers N] [--long-contexts 16384,32768]
 
 A "step" is one decode step of the whole engine (scheduler iteration: plan,
-step function, sampling, token hand-over).  The run fills the cache of ``batch``
-requests so that the timed steps end at ``context`` tokens, does W untimed and
-exactly K timed steps bracketed by ``torch.cuda.synchronize()``, and prints ONE
-JSON line.  Protocol after the reference's benchmark (benchmarks/run.py:3-8,
-205-207, 241-256): fresh engine, untimed warm-up, wall-clock output tokens per
-second; prompts are seeded uniform-random token ids, EOS is ignored.
+step function, sampling, token hand-over).  Protocol after the reference's
+benchmark (benchmarks/run.py:3-8, 205-207, 241-256): a fresh engine per
+measured point, two unmeasured warm-up runs, three measured runs, every run
+reported and the median taken; wall-clock output tokens per second; prompts are
+seeded uniform-random token ids, EOS is ignored.
+
+A *run* of the headline figure is a window of exactly K decode steps between two
+``torch.cuda.synchronize()``; the windows follow one another in the same batch
+of requests, after W untimed steps, and the last one ends at ``--context``
+tokens, so all of them sit at the heavy end of the range that the configuration
+states ("2,048-token prefill, then decode to 4,096").  The whole range is
+measured beside it (``range``): prompts of ``--prefill-tokens``, then every
+decode step up to ``--context``, one warm-up run and three measured ones.
+``prefill`` is one prompt of ``--prefill-tokens`` run to its first token.
+ONE JSON line is printed.
 """
 
 from __future__ import annotations
 
 import argparse
 import json
+import statistics
 import sys
 import time
 
@@ -25,13 +36,9 @@ HBM_GBPS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 SLACK = 16  # tokens a request may run past the nominal context (requests start decoding a step or two apart)
-
-SHAPE_3B = dict(
-    model_type="qwen2", hidden_size=2048, num_hidden_layers=36, num_attention_heads=16,
-    num_key_value_heads=2, intermediate_size=11008, vocab_size=151936, rope_theta=1e6,
-    rms_norm_eps=1e-6, attention_bias=True, tie_word_embeddings=True, use_sliding_window=False,
-    max_position_embeddings=32768, eos_token_id=151643,
-)
+WARM_WINDOWS = 2
+MEASURED_WINDOWS = 3
+PAGE = 16
 
 
 def linear_params_per_layer(c) -> int:
@@ -44,7 +51,7 @@ def decode_bytes(c, layers: int, batch: int, context: float, elem: int) -> float
     """Bytes one decode step has to read: every weight once, and the cache of the live requests."""
     weights = layers * (linear_params_per_layer(c) + 2 * c.hidden_size
                         + (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim) * elem
-    weights += c.vocab_size * c.hidden_size * elem + c.hidden_size * elem  # head (tied: the embedding) + final norm
+    weights += c.vocab_size * c.hidden_size * elem + c.hidden_size * elem  # the head (tied or not: read once) + final norm
     kv = batch * context * layers * 2 * c.num_key_value_heads * c.head_dim * elem
     return weights + kv
 
@@ -59,11 +66,10 @@ def prefill_flops(c, layers: int, tokens: int) -> float:
 def make_engine(config, dtype, batch, context, prefill_tokens, seed=0):
     from cie_amd import Engine
 
-    page = 16
-    per_request = -(-(context + SLACK) // page) * page
-    kv_tokens = max(batch * per_request, -(-prefill_tokens // page) * page) + 4 * page
+    per_request = -(-(context + SLACK) // PAGE) * PAGE
+    kv_tokens = max(batch * per_request, -(-prefill_tokens // PAGE) * PAGE) + 4 * PAGE
     return Engine(
-        config=config, seed=seed, dtype=dtype, page_size=page, kv_tokens=kv_tokens,
+        config=config, seed=seed, dtype=dtype, page_size=PAGE, kv_tokens=kv_tokens,
         max_running=max(batch, 1), max_queue_size=max(batch, 1) + 1, max_model_len=context + SLACK,
         max_output_tokens=context, token_budget=max(2048, batch), prefill_chunk=2048,
         prefix_cache_pages=0, draw_device="cuda",
@@ -72,60 +78,94 @@ def make_engine(config, dtype, batch, context, prefill_tokens, seed=0):
     )
 
 
-def time_decode(engine, config, batch: int, context: int, steps: int, warmup: int, seed: int):
-    """Fill ``batch`` requests so that warm-up plus timed steps end at ``context``; time the steps."""
+def random_prompts(config, count: int, length: int, seed: int) -> list[list[int]]:
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, config.vocab_size, (length,), generator=g).tolist() for _ in range(count)]
+
+
+def decode_windows(engine, config, batch: int, context: int, steps: int, warmup: int, seed: int):
+    """``batch`` requests whose last window ends at ``context``: W untimed steps, then
+    ``WARM_WINDOWS`` unmeasured and ``MEASURED_WINDOWS`` measured windows of exactly ``steps`` steps.
+    Returns [(seconds, mean context of the window)] of the measured ones."""
     import torch
 
     from cie_amd import GenerationConfig
-
-    prompt_len = context - steps - warmup
-    if prompt_len < 1:
-        raise ValueError(f"context {context} too short for {steps}+{warmup} steps")
-    g = torch.Generator().manual_seed(seed)
-    gen = GenerationConfig(max_output_tokens=steps + warmup + SLACK, eos_token_id=None)
-    requests = [
-        engine.submit(torch.randint(0, config.vocab_size, (prompt_len,), generator=g).tolist(), gen)
-        for _ in range(batch)
-    ]
     from cie_amd.engine import RequestState
 
+    windows = WARM_WINDOWS + MEASURED_WINDOWS
+    prompt_len = context - warmup - windows * steps
+    if prompt_len < 1:
+        raise ValueError(f"context {context} too short for {warmup} + {windows} x {steps} steps")
+    gen = GenerationConfig(max_output_tokens=warmup + windows * steps + SLACK, eos_token_id=None)
+    requests = [engine.submit(prompt, gen) for prompt in random_prompts(config, batch, prompt_len, seed)]
     while any(r.state is not RequestState.DECODING for r in requests):
         engine.step()  # prefill portions; the last one yields each request's first token
     for _ in range(warmup - 1):
         engine.step()
-    torch.cuda.synchronize()
-    start = time.perf_counter()
-    for _ in range(steps):
-        engine.step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - start
+    measured = []
+    for window in range(windows):
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        for _ in range(steps):
+            engine.step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - start
+        if window >= WARM_WINDOWS:
+            measured.append((elapsed, sum(r.cached for r in requests) / batch - steps / 2.0))
     for r in requests:
         # (with decode steps started ahead of their tokens, the last step's token is still on its way)
-        assert not r.is_final and len(r.output) >= warmup + steps - 1, (r.state, len(r.output))
-    mean_context = sum(r.cached for r in requests) / batch - steps / 2.0
-    for r in requests:
+        assert not r.is_final and len(r.output) >= warmup + windows * steps - 1, (r.state, len(r.output))
         engine.scheduler.cancel(r)
-    return elapsed, mean_context
+    return measured
 
 
-def time_prefill(engine, config, tokens: int, seed: int, repeats: int = 3):
+def decode_range(engine, config, batch: int, first: int, last: int, seed: int, warm_steps: int = 48):
+    """Prompts of ``first`` tokens, then every decode step until the requests hold ``last`` tokens:
+    one short unmeasured run, ``MEASURED_WINDOWS`` measured ones.  Returns [(seconds, decode steps)]."""
+    import torch
+
+    from cie_amd import GenerationConfig
+    from cie_amd.engine import RequestState
+
+    out = []
+    for run in range(1 + MEASURED_WINDOWS):
+        tokens = min(warm_steps, last - first) if run == 0 else last - first
+        gen = GenerationConfig(max_output_tokens=tokens, eos_token_id=None)
+        requests = [engine.submit(prompt, gen) for prompt in random_prompts(config, batch, first, seed + run)]
+        while any(r.state is not RequestState.DECODING for r in requests):
+            engine.step()
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        while engine.has_work():
+            engine.step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - start
+        assert all(len(r.output) == tokens for r in requests)
+        if run:
+            out.append((elapsed, tokens - 1))  # the first token came with the prompt
+    return out
+
+
+def time_prefill(engine, config, tokens: int, seed: int) -> list[float]:
+    """Seconds of each measured run: one prompt from submission to its first token."""
     import torch
 
     from cie_amd import GenerationConfig
 
-    g = torch.Generator().manual_seed(seed)
-    best = None
-    for _ in range(repeats + 1):  # the first is the warm-up
-        prompt = torch.randint(0, config.vocab_size, (tokens,), generator=g).tolist()
+    seconds = []
+    prompts = random_prompts(config, WARM_WINDOWS + MEASURED_WINDOWS, tokens, seed)
+    for run, prompt in enumerate(prompts):
         request = engine.submit(prompt, GenerationConfig(max_output_tokens=1, eos_token_id=None))
         torch.cuda.synchronize()
         start = time.perf_counter()
         while not request.is_final:
             engine.step()
         torch.cuda.synchronize()
-        elapsed = time.perf_counter() - start
-        best = elapsed if best is None or _ == 1 else min(best, elapsed)
-    return best
+        if run >= WARM_WINDOWS:
+            seconds.append(time.perf_counter() - start)
+    return seconds
 
 
 def main(argv=None) -> int:
@@ -135,11 +175,14 @@ def main(argv=None) -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=4096)
-    parser.add_argument("--layers", type=int, default=SHAPE_3B["num_hidden_layers"])
+    parser.add_argument("--shape", default="3b", choices=["3b", "7b", "14b"])
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
     parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--no-range", action="store_true", help="skip the run over the whole range of contexts")
+    parser.add_argument("--long-contexts", default="", help="further decode points of the main batch, e.g. 16384,32768")
     args = parser.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not run (this engine is single-GPU)")
@@ -148,30 +191,35 @@ def main(argv=None) -> int:
     import torch
 
     from cie_amd.config import Qwen2Config
+    from cie_amd.workloads import SHAPES
 
-    raw = dict(SHAPE_3B, num_hidden_layers=args.layers)
-    config = Qwen2Config.from_hf_config(raw)
+    shape = SHAPES[args.shape]
+    full_layers = shape["num_hidden_layers"]
+    layers = args.layers or full_layers
+    config = Qwen2Config.from_hf_config(dict(shape, num_hidden_layers=layers))
     elem = 2 if args.dtype == "bf16" else 4
-    full_layers = SHAPE_3B["num_hidden_layers"]
+    steps, warmup = args.steps, max(args.warmup, 1)
 
-    def decode_point(batch: int, steps: int, warmup: int):
-        engine = make_engine(config, args.dtype, batch, args.context, args.prefill_tokens)
-        elapsed, mean_context = time_decode(engine, config, batch, args.context, steps, warmup, seed=batch)
+    def point(batch: int, context: int):
+        """(tokens/s of each measured window, the median window's ms per step and roofline share)."""
+        engine = make_engine(config, args.dtype, batch, context, args.prefill_tokens)
+        measured = decode_windows(engine, config, batch, context, steps, warmup, seed=batch)
         del engine
         torch.cuda.empty_cache()
-        return elapsed, mean_context
+        rates = [batch * steps / seconds for seconds, _ in measured]
+        seconds, mean_context = sorted(measured)[len(measured) // 2]
+        achieved = decode_bytes(config, layers, batch, mean_context, elem) / (seconds / steps) / 1e9
+        return rates, seconds / steps * 1e3, achieved
 
-    elapsed, mean_context = decode_point(args.batch, args.steps, max(args.warmup, 1))
-    ms_per_step = elapsed / args.steps * 1e3
-    value = args.batch * args.steps / elapsed
-    achieved = decode_bytes(config, args.layers, args.batch, mean_context, elem) / (elapsed / args.steps) / 1e9
+    rates, ms_per_step, achieved = point(args.batch, args.context)
+    name = f"Qwen2.5-{args.shape.upper()} shape"
     line = {
-        "metric": f"decode tokens/s, Qwen2.5-3B shape, batch {args.batch}, context to {args.context}",
-        "value": round(value, 2),
+        "metric": f"decode tokens/s, {name}, batch {args.batch}, context to {args.context}",
+        "value": round(statistics.median(rates), 2),
         "unit": "tokens/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": max(args.warmup, 1),
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -179,35 +227,64 @@ def main(argv=None) -> int:
         "dtype": args.dtype,
         "data": "synthetic (seeded uniform-random token ids, random weights N(0, 0.02))",
         "config": {
-            "model": "Qwen2.5-3B shape (Qwen2ForCausalLM)", "layers": args.layers, "layers_full": full_layers,
+            "model": f"{name} (Qwen2ForCausalLM)", "layers": layers, "layers_full": full_layers,
             "hidden": config.hidden_size, "heads": config.num_attention_heads,
             "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
             "intermediate": config.intermediate_size, "vocab": config.vocab_size,
             "global_batch": args.batch, "seq_len": args.context, "prefill_tokens": args.prefill_tokens,
-            "page_size": 16, "rope_theta": config.rope_theta, "rms_norm_eps": config.rms_norm_eps,
+            "page_size": PAGE, "rope_theta": config.rope_theta, "rms_norm_eps": config.rms_norm_eps,
             "tie_word_embeddings": config.tie_word_embeddings, "attention_bias": config.attention_bias,
             "parallelism": "single GPU",
         },
+        "protocol": f"fresh engine per point, {WARM_WINDOWS} unmeasured and {MEASURED_WINDOWS} measured windows of "
+                    f"{steps} steps after {warmup} warm-up steps; value is the median window",
+        "runs": [round(r, 2) for r in rates],
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_GBPS, 4)},
     }
+    if not args.no_range and args.context > args.prefill_tokens + 1:
+        engine = make_engine(config, args.dtype, args.batch, args.context, args.prefill_tokens)
+        runs = decode_range(engine, config, args.batch, args.prefill_tokens, args.context, seed=7)
+        del engine
+        torch.cuda.empty_cache()
+        range_rates = [args.batch * n / seconds for seconds, n in runs]
+        seconds, n = sorted(runs)[len(runs) // 2]
+        mean_context = (args.prefill_tokens + args.context) / 2.0
+        through = decode_bytes(config, layers, args.batch, mean_context, elem) / (seconds / n) / 1e9
+        line["range"] = {
+            "from": args.prefill_tokens, "to": args.context, "steps": n,
+            "value": round(statistics.median(range_rates), 2), "runs": [round(r, 2) for r in range_rates],
+            "ms_per_step": round(seconds / n * 1e3, 4), "frac": round(through / HBM_GBPS, 4),
+        }
     if not args.no_prefill:
         engine = make_engine(config, args.dtype, 1, args.prefill_tokens + 1, args.prefill_tokens)
         seconds = time_prefill(engine, config, args.prefill_tokens, seed=99)
         del engine
         torch.cuda.empty_cache()
-        flops = prefill_flops(config, args.layers, args.prefill_tokens)
+        median = statistics.median(seconds)
+        flops = prefill_flops(config, layers, args.prefill_tokens)
         line["prefill"] = {
-            "value": round(args.prefill_tokens / seconds, 1), "tokens": args.prefill_tokens,
-            "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4),
+            "value": round(args.prefill_tokens / median, 1), "tokens": args.prefill_tokens,
+            "ms": round(median * 1e3, 3), "frac": round(flops / median / PEAK_FLOPS[args.dtype], 4),
+            "runs_ms": [round(s * 1e3, 3) for s in seconds],
         }
+    points, fractions, all_runs = {}, {}, {}
     if not args.no_points:
-        points = {}
         for batch in (1, 64):
-            steps = max(8, args.steps // 2)
-            elapsed, _ = decode_point(batch, steps, 4)
-            points[f"decode_b{batch}"] = round(batch * steps / elapsed, 2)
+            rates, _, achieved = point(batch, args.context)
+            points[f"decode_b{batch}"] = round(statistics.median(rates), 2)
+            fractions[f"decode_b{batch}"] = round(achieved / HBM_GBPS, 4)
+            all_runs[f"decode_b{batch}"] = [round(r, 2) for r in rates]
+    for context in [int(c) for c in args.long_contexts.split(",") if c]:
+        rates, _, achieved = point(args.batch, context)
+        key = f"decode_b{args.batch}_ctx{context}"
+        points[key] = round(statistics.median(rates), 2)
+        fractions[key] = round(achieved / HBM_GBPS, 4)
+        all_runs[key] = [round(r, 2) for r in rates]
+    if points:
         line["points"] = points
+        line["points_frac"] = fractions
+        line["points_runs"] = all_runs
     print(json.dumps(line))
     return 0
 

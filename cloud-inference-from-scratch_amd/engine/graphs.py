@@ -164,9 +164,12 @@ class DecodeGraphs:
             size *= 2
         return made
 
-    def run(self, entries: Sequence[Any], feed: Sequence[int] | None = None) -> torch.Tensor:
+    def run(self, entries: Sequence[Any], feed: Sequence[int] | None = None, borrow: bool = False) -> torch.Tensor:
         """Replay the bucket's graph for single-token entries; logits [wanted, vocab].  ``feed[i] >= 0``:
-        entry i's token is the one at that place of ``token_pool`` (its own ``tokens`` are ignored)."""
+        entry i's token is the one at that place of ``token_pool`` (its own ``tokens`` are ignored).
+        The graph writes its logits into one buffer of its own, which the bucket's next replay overwrites:
+        the caller gets a copy, unless it ``borrow``s the buffer (sampling that is queued on the same
+        stream right behind the replay has read it before the next replay can start)."""
         runner = self.runner
         size = self.bucket_of(len(entries))
         bucket = self.buckets.get(size) or self._capture(size)
@@ -179,7 +182,8 @@ class DecodeGraphs:
         self.replays += 1
         rows = [index for index, e in enumerate(entries) for _ in e.want]
         if rows == list(range(len(entries))):
-            return bucket.logits[: len(entries)]
+            view = bucket.logits[: len(entries)]
+            return view if borrow else view.clone()
         return bucket.logits[torch.tensor(rows, dtype=torch.long, device=runner.device)]
 
 

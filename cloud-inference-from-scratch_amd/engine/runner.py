@@ -149,7 +149,7 @@ class Runner:
                       (portion.length - 1,) if portion.samples else ())
             for portion in plan.portions
         ]
-        logits = self.run(entries)
+        logits = self.run(entries, borrow_logits=True)  # (sampled from at once, below)
         for portion in plan.portions:
             portion.request.cached = portion.end
         sampling = [portion.request for portion in plan.portions if portion.samples]
@@ -179,7 +179,7 @@ class Runner:
         :meth:`PendingTokens.tokens` waits for them."""
         assert self.graphs is not None and all(p.length == 1 and p.samples for p in plan.portions)
         entries = [StepEntry(p.request.request_id, p.tokens, p.start, (0,)) for p in plan.portions]
-        logits = self.run(entries, feed=feed)
+        logits = self.run(entries, feed=feed, borrow_logits=True)
         requests = [p.request for p in plan.portions]
         for p in plan.portions:
             p.request.cached = p.end
@@ -270,11 +270,14 @@ class Runner:
         )
 
     # -- the step ------------------------------------------------------------------
-    def run(self, entries: Sequence[StepEntry], feed: Sequence[int] | None = None) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], feed: Sequence[int] | None = None,
+            borrow_logits: bool = False) -> torch.Tensor:
         """One step.  Returns float32 logits ``[sum(len(e.want)), vocab]`` on the
-        device, in the order of the entries and of their ``want``.  Raises
-        ``CacheCapacityFull`` before anything changes if pages run out.
-        ``feed`` (captured decode steps only): see :meth:`launch_decode`."""
+        device, in the order of the entries and of their ``want``; they are the
+        caller's to keep.  Raises ``CacheCapacityFull`` before anything changes if
+        pages run out.  ``feed`` (captured decode steps only): see
+        :meth:`launch_decode`, which also borrows a captured step's own logits
+        buffer instead of a copy (``borrow_logits``)."""
         self.check(entries)
         required = {e.request_id: e.start_pos + len(e.tokens) for e in entries}
         with trace_range("ragged.kv.ensure_capacity"):
@@ -292,7 +295,7 @@ class Runner:
             if not decode and feed is None and self.mixed_graphs is not None:
                 shape = self.mixed_graphs.wants(entries)
             if decode and self.graphs is not None and self.graphs.takes(len(entries)):
-                logits = self.graphs.run(entries, feed)
+                logits = self.graphs.run(entries, feed, borrow=borrow_logits)
             elif feed is not None:
                 raise ValueError("tokens can be fed on the device to captured decode steps only")
             elif shape is not None:

@@ -56,7 +56,10 @@ class Sampler:
         """The same, left on the GPU (int32 [n], in ``out`` if given): nothing waits for the result."""
         if all(t == 0 for t in temperatures):
             return ops.sample(logits, out=out)
-        device = logits.device
-        temperature = torch.tensor(list(temperatures), dtype=torch.float32).to(device)
-        uniform = torch.tensor(list(uniforms), dtype=torch.float32).to(device)
-        return ops.sample(logits, temperature, uniform, out=out)
+        # one page-locked block for both, copied without waiting: the decode steps that are started ahead of
+        # their tokens must not stop the host here (a copy from pageable memory would)
+        rows = len(temperatures)
+        pinned = logits.device.type == "cuda"
+        staged = torch.tensor([*temperatures, *uniforms], dtype=torch.float32, pin_memory=pinned)
+        on_device = staged.to(logits.device, non_blocking=True)
+        return ops.sample(logits, on_device[:rows], on_device[rows:], out=out)

@@ -209,3 +209,47 @@ def closer_than_plain_bfloat16(rows: dict[str, dict[int, np.ndarray]], plain: di
     rms, worst = errors(lambda rid, pos: torch.from_numpy(rows[rid][pos]))
     assert rms <= plain_rms and worst <= 1.5 * plain_worst, (rms, worst, plain_rms, plain_worst)
     return rms, worst, plain_rms, plain_worst
+
+
+def greedy_tokens_follow_plain(plain_forward, prompt: list[int], got: list[int], rough_forward=None,
+                               floor: float = 1e-4) -> int:
+    """Every generated token against the plain model, teacher-forced on what was generated: token i must
+    be the arg-max of the plain logits after ``prompt + got[:i]``, or, where 16-bit rounding may turn a
+    near-tie, lie within twice the distance between the plain logits in float32 and in bfloat16
+    (``rough_forward``) of that maximum.  Returns how many tokens were near-ties that went the other way."""
+    turned = 0
+    for index, token in enumerate(got):
+        context = list(prompt) + list(got[:index])
+        row = plain_forward(context)[-1].float()
+        best = int(row.argmax())
+        if token == best:
+            continue
+        margin = floor
+        if rough_forward is not None:
+            margin = max(floor, 2.0 * float((rough_forward(context)[-1].float() - row).abs().max()))
+        gap = float(row[best] - row[token])
+        assert gap <= margin, f"token {index}: got {token} (logit {float(row[token]):.5f}), plain picks {best} " \
+                              f"({float(row[best]):.5f}); gap {gap:.2e} exceeds {margin:.2e}"
+        turned += 1
+    return turned
+
+
+def drawn_tokens_follow_plain(plain_forward, prompt: list[int], got: list[int], temperature: float,
+                              uniforms: list[float], slack: float = 1e-4) -> int:
+    """Temperature sampling end to end: token i must be the first index at which the running sum of
+    softmax(plain logits / temperature) passes ``uniforms[i]``, or a neighbour of it when the number
+    falls within ``slack`` of the boundary between the two.  Returns the boundary cases."""
+    close = 0
+    for index, (token, u) in enumerate(zip(got, uniforms)):
+        row = plain_forward(list(prompt) + list(got[:index]))[-1].double()
+        p = torch.softmax(row / temperature, dim=-1)
+        cdf = torch.cumsum(p, dim=-1)
+        expected = int(torch.searchsorted(cdf, torch.tensor(u, dtype=torch.float64), right=True))
+        expected = min(expected, row.numel() - 1)
+        if token == expected:
+            continue
+        low = float(cdf[token - 1]) if token > 0 else 0.0
+        assert low - slack <= u < float(cdf[token]) + slack, \
+            f"token {index}: got {token} whose share of [0, 1) is [{low:.6f}, {float(cdf[token]):.6f}), the number is {u:.6f}"
+        close += 1
+    return close

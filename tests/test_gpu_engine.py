@@ -109,6 +109,30 @@ def test_temperature_sampling_is_seeded_and_independent_of_the_batch(tiny_folder
     assert greedy[0].token_ids != together[0].token_ids  # the draws are not all argmax
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_temperature_tokens_are_the_inverse_cdf_of_the_plain_logits(tiny_folders, dtype):
+    """Not engine against engine: the expected ids come from the plain model's logits, the uniform number
+    the sampler documents for (seed, token index), and a plain inverse CDF."""
+    import replay_util
+    from cie_amd import GenerationConfig
+    from cie_amd.sampling.sampler import uniform_for
+
+    folder, raw, tensors = tiny_folders["A"]
+    weights = float_weights(tensors)
+    prompts = [random_tokens(n, raw["vocab_size"], 450 + n) for n in (6, 21, 37)]
+    gens = [GenerationConfig(max_output_tokens=16, temperature=t, eos_token_id=None, seed=90 + i)
+            for i, t in enumerate((0.7, 1.0, 1.6))]
+    results = make_engine(folder, dtype=dtype, page_size=16, token_budget=24).generate(prompts, gens)
+    slack = 1e-4 if dtype == "float32" else 2e-2  # (of the unit interval: what a logit's rounding moves a boundary by)
+    boundary = 0
+    for prompt, gen, result in zip(prompts, gens, results):
+        uniforms = [uniform_for(gen.seed, 0, i) for i in range(16)]
+        boundary += replay_util.drawn_tokens_follow_plain(
+            lambda tokens: plain.forward(raw, weights, tokens), prompt, result.token_ids, gen.temperature, uniforms, slack)
+        assert len(set(result.token_ids)) > 4, "draws, not one token over and over"
+    assert boundary <= (0 if dtype == "float32" else 6)
+
+
 def test_pressure_preempts_and_recomputes_to_the_same_tokens(tiny_folders):
     """A pool too small for two requests at once (reference
     tests/remote_ragged_gpu_tests.py:294-332): preemptions > 0, recomputed tokens
@@ -182,6 +206,34 @@ def test_prefix_is_shared_with_a_request_that_arrives_while_the_first_still_deco
     engine.runner.cache.assert_invariants()
 
 
+def test_bfloat16_under_pressure_with_shared_prefixes_follows_the_plain_model(tiny_folders):
+    """bfloat16 with everything on at once: a pool that forces preemption, prompts that share their first
+    pages, captured decode steps started ahead of their tokens.  Every request's tokens follow the plain
+    model, near-ties that bfloat16 may turn aside."""
+    import replay_util
+    from cie_amd import GenerationConfig
+
+    folder, raw, tensors = tiny_folders["A"]
+    weights = float_weights(tensors)
+    shared = random_tokens(32, raw["vocab_size"], 650)
+    prompts = [shared + random_tokens(8 + 3 * i, raw["vocab_size"], 651 + i) for i in range(4)]
+    gen = GenerationConfig(max_output_tokens=14, eos_token_id=None)
+    tight = make_engine(folder, dtype="bfloat16", page_size=16, kv_tokens=160, max_running=4, prefix_cache_pages=4,
+                        token_budget=32, prefill_chunk=16, admit_within_pool=False, max_model_len=128)
+    results = tight.generate(prompts, gen)
+    metrics = tight.snapshot_metrics()
+    assert metrics["requests"]["preempted_total"] > 0 and metrics["kv_cache"]["prefix_cache_hits"] > 0
+    assert metrics["runner"]["graph_replays"] > 0 and metrics["kv_cache"]["request_pages_used"] == 0
+    tight.runner.cache.assert_invariants()
+    turned = 0
+    for prompt, result in zip(prompts, results):
+        assert len(result.token_ids) == 14
+        turned += replay_util.greedy_tokens_follow_plain(
+            lambda tokens: plain.forward(raw, weights, tokens), prompt, result.token_ids,
+            lambda tokens: plain.forward(raw, weights, tokens, dtype=torch.bfloat16))
+    assert turned <= 6
+
+
 def test_random_requests_through_a_small_pool_equal_each_request_alone(tiny_folders):
     """Forty random requests (shared prefixes, greedy and seeded temperature sampling, end
     tokens) arrive a few per step at an engine whose pool holds one and a half full sequences: with
@@ -240,11 +292,17 @@ def test_warm_up_captures_every_decode_bucket_once(tiny_folders):
     results = engine.generate(prompts, GenerationConfig(max_output_tokens=10, eos_token_id=None))
     runner = engine.snapshot_metrics()["runner"]
     assert runner["graph_captures"] == 4 and runner["graph_replays"] >= 9
+    import replay_util
+
     weights = float_weights(tensors)
+    turned = 0
     for prompt, result in zip(prompts, results):
-        # bfloat16 may flip a near-tie: the first token at least is the plain model's, and all are valid ids
-        assert result.token_ids[0] == plain.generate_greedy(raw, weights, prompt, 1)[0]
+        # every token is the plain model's after the same context, or a near-tie that bfloat16 may turn
         assert len(result.token_ids) == 10
+        turned += replay_util.greedy_tokens_follow_plain(
+            lambda tokens: plain.forward(raw, weights, tokens), prompt, result.token_ids,
+            lambda tokens: plain.forward(raw, weights, tokens, dtype=torch.bfloat16))
+    assert turned <= 5, "most of the 50 tokens are the plain model's own"
 
 
 def test_step_refuses_what_it_cannot_run(tiny_folders):

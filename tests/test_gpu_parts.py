@@ -45,6 +45,25 @@ def harness(needs, lengths, page_size=8, dtype=torch.float32):
     return manager, device_cache
 
 
+def test_device_pools_follow_what_each_need_stores():
+    """Keys and values of one width share a group; a need without values has a key pool only; values of
+    another width get a pool of that width (transposed, as the attention kernels read values)."""
+    from cie_amd.cache import PagedKV
+
+    needs = [PagedKV(2, 16), PagedKV(1, 24, values=False), PagedKV(2, 16), PagedKV(2, 16, value_dim=8)]
+    manager, device_cache = harness(needs, [5])
+    pages = 512 // 8 + 1  # (one page beyond the pool's for padded rows of captured steps)
+    assert [tuple(p.shape) for p in device_cache.key_pools] == [(2, pages, 2, 8, 16), (1, pages, 1, 8, 24), (1, pages, 2, 8, 16)]
+    assert device_cache.value_pools[1] is None
+    assert tuple(device_cache.value_pools[0].shape) == (2, pages, 2, 16, 8)
+    assert tuple(device_cache.value_pools[2].shape) == (1, pages, 2, 8, 8)
+    latent = device_cache.view(1)
+    assert latent.v_pool is None and tuple(latent.k_pool.shape) == (pages, 1, 8, 24)
+    assert device_cache.view(2).k_pool.data_ptr() == device_cache.key_pools[0][1].data_ptr()
+    stats = manager.stats()
+    assert [g.reserved_bytes for g in stats.groups] == [8 * 64 * 2 * 2, 8 * 24 * 2, 8 * 48 * 2]
+
+
 def batch_of(manager, portions):
     """StepBatch for portions [(request index, start, count)], built by hand."""
     from cie_amd.engine.batch import StepBatch
@@ -255,12 +274,25 @@ def register_toy():
                 order=(LayerCall(0, 0), LayerCall(1, 1), LayerCall(0, 2)),
                 final_norm=base.final_norm, tie_word_embeddings=True, max_position=self.max_position_embeddings)
 
+    class OnlyStateConfig(ToyConfig):
+        """Every layer the running sum: a model that caches nothing in pages."""
+
+        architecture = "ToyOnlyStateForCausalLM"
+
+        def model_spec(self) -> ModelSpec:
+            mixed = super().model_spec()
+            return ModelSpec(
+                architecture=self.architecture, vocab_size=self.vocab_size, hidden_size=self.hidden_size,
+                layers=mixed.layers[:1], order=(LayerCall(0, 0), LayerCall(0, 1)),
+                final_norm=mixed.final_norm, tie_word_embeddings=True, max_position=self.max_position_embeddings)
+
     register_part("mixer", "running_sum", RunningSum)
     register_architecture("ToyRunningSumForCausalLM", ToyConfig)
+    register_architecture("ToyOnlyStateForCausalLM", OnlyStateConfig)
     return ToyConfig
 
 
-def toy_plain(raw, weights, tokens):
+def toy_plain(raw, weights, tokens, order=(0, 1, 0)):
     """Whole-sequence reference of the toy model, from the plain parts."""
     eps = raw["rms_norm_eps"]
     h = weights["model.embed_tokens.weight"][torch.tensor(tokens)]
@@ -279,7 +311,7 @@ def toy_plain(raw, weights, tokens):
         return plain.swiglu(x, weights[p + "mlp.gate_proj.weight"], weights[p + "mlp.up_proj.weight"],
                             weights[p + "mlp.down_proj.weight"])
 
-    for layer in (0, 1, 0):
+    for layer in order:
         p = f"model.layers.{layer}."
         a = plain.rms_norm(h, weights[p + "input_layernorm.weight"], eps)
         if layer == 0:
@@ -322,6 +354,36 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         replay_util.compare(rows, reference, rtol=1e-4, atol=2e-5)
     # a slot handed to a new request starts from a cleared state (slots were reused above)
     assert runner.cache.stats().slots_used == 0
+
+
+def test_a_model_of_fixed_states_only_runs_its_requests_side_by_side(tmp_path):
+    """No unit of this model is paged: the pool has nothing to say about admission, and four requests
+    run in the same steps under ``admit_within_pool``, each to the plain toy model's greedy tokens."""
+    from cie_amd import Engine, GenerationConfig
+    from cie_amd.config import load_config
+    from cie_amd.parts.model import expected_tensors
+    from cie_amd.weights import RandomSource, write_tensors
+
+    register_toy()
+    raw = dict(architectures=["ToyOnlyStateForCausalLM"], model_type="qwen2", hidden_size=32, num_hidden_layers=1,
+               num_attention_heads=2, num_key_value_heads=1, intermediate_size=40, vocab_size=64,
+               rms_norm_eps=1e-6, rope_theta=1e4, max_position_embeddings=128, tie_word_embeddings=True)
+    write_tensors(tmp_path, raw, {})
+    tensors = RandomSource(12, std=0.15).load(expected_tensors(load_config(tmp_path).model_spec()), "float32", "cpu")
+    write_tensors(tmp_path, raw, tensors)
+    engine = Engine(tmp_path, dtype="float32", page_size=8, kv_tokens=8, max_running=4, max_model_len=128,
+                    token_budget=64, prefill_chunk=16, admit_within_pool=True)
+    assert not engine.runner.cache.groups and set(engine.runner.cache.state_units) == {0, 1}
+    prompts = [random_tokens(n, 64, 80 + n) for n in (5, 12, 21, 9)]
+    results = engine.generate(prompts, GenerationConfig(max_output_tokens=6, eos_token_id=None))
+    assert engine.snapshot_metrics()["runner"]["max_forward_request_count"] == 4
+    for prompt, result in zip(prompts, results):
+        tokens, expected = list(prompt), []
+        for _ in range(6):
+            expected.append(int(toy_plain(raw, tensors, tokens, order=(0, 0))[-1].argmax()))
+            tokens.append(expected[-1])
+        assert result.token_ids == expected
+    assert engine.runner.cache.stats().slots_used == 0
 
 
 # ----------------------------------------------------------------------------------------------------

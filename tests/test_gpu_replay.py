@@ -50,6 +50,19 @@ def make_runner(folder, dtype, kv_tokens, page_size, max_running=8, graph_decode
     return Runner(model, engine_config, "cuda:0")
 
 
+_ROUGH: dict = {}
+
+
+def rough_all(name, tiny_folders, requests):
+    """The plain implementation in bfloat16 throughout, once per configuration."""
+    if name not in _ROUGH:
+        _, raw, tensors = tiny_folders[name]
+        weights = {k: v.float() for k, v in tensors.items()}
+        _ROUGH[name] = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16)
+                        for rid, tokens in requests.items()}
+    return _ROUGH[name]
+
+
 @pytest.fixture(scope="module")
 def plain(tiny_folders):
     out = {}
@@ -83,6 +96,10 @@ def test_replay_matches_plain(tiny_folders, plain, name, schedule, dtype):
     rows = replay_util.by_position(steps, outputs)
     worst = replay_util.compare(rows, expected, **TOL[dtype])
     print(f"worst |diff| {worst:.3e}", flush=True)
+    if dtype == "bfloat16":
+        # the stricter yardstick: closer to the float32 logits than the plain model run in bfloat16 is
+        print("rms %.3e worst %.3e, plain in bfloat16 %.3e %.3e"
+              % replay_util.closer_than_plain_bfloat16(rows, expected, rough_all(name, tiny_folders, requests)), flush=True)
     assert runner.cache.stats().pages_used == 0
 
 
@@ -142,6 +159,24 @@ def test_replay_with_the_four_wave_decode_attention(tiny_folders, plain, monkeyp
         assert runner.graph_replays >= 20
 
 
+def test_logits_of_a_captured_step_are_the_callers_to_keep(tiny_folders):
+    """A captured decode step writes into a buffer of its graph's; what ``run`` returns must not change
+    when the same graph is replayed for the next step."""
+    folder, raw, _ = tiny_folders["A"]
+    tokens = random_tokens(20, raw["vocab_size"], seed=77)
+    from cie_amd.engine.runner import StepEntry
+
+    runner = make_runner(folder, "bfloat16", 64, 16, graph_decode=True)
+    runner.cache.admit("k")
+    runner.run([StepEntry("k", tokens[:18], 0, ())])
+    first = runner.run([StepEntry("k", tokens[18:19], 18, (0,))])
+    kept = first.cpu().clone()
+    second = runner.run([StepEntry("k", tokens[19:20], 19, (0,))])
+    assert runner.graph_replays == 2
+    assert torch.equal(first.cpu(), kept) and not torch.equal(second.cpu(), kept)
+    runner.cache.release("k")
+
+
 ODD_SIZES = [  # hidden, heads, kv heads, head_dim, intermediate, vocabulary
     (75, 3, 1, 16, 77, 97),      # an odd width: no 16-byte rows anywhere
     (90, 6, 2, 48, 50, 1001),
@@ -160,6 +195,7 @@ HEAD_SIZES = [  # head sizes and group sizes the matrix-core attention takes (pa
     (256, 16, 2, 128, 300, 515),
     (128, 10, 2, 64, 72, 130),   # groups of five
     (512, 16, 1, 32, 64, 97),    # sixteen heads on one key head: a tile's rows are one token
+    (160, 40, 8, 128, 96, 130),  # forty heads on eight key heads (groups of five at the widest common head size)
 ]
 
 
@@ -369,13 +405,32 @@ def test_steps_queued_behind_a_busy_gpu_keep_their_own_metadata(tiny_folders, pl
 
 
 def test_mixed_reuses_pages(tiny_folders, plain):
-    """The mixed schedule runs in a pool smaller than the sum of all requests."""
-    _, raw, _ = tiny_folders["B"]
-    requests, _ = plain["B"]
-    steps = replay_util.mixed(requests, live=3)
+    """The mixed schedule as the replays run it (four live requests, a pool of exactly the peak): the
+    engine's allocator hands pages that one request gave back to a later one, while other requests are
+    in the middle of their sequences, and the logits written through those pages are the plain model's."""
+    folder, raw, _ = tiny_folders["B"]
+    requests, expected = plain["B"]
+    steps = replay_util.mixed(requests, live=4)
     pool = replay_util.max_live_tokens(steps, page=8)
-    total = sum(-(-len(t) // 8) * 8 for t in requests.values())
-    assert pool < total
+    assert pool < sum(-(-len(t) // 8) * 8 for t in requests.values())
+    runner = make_runner(folder, "float32", pool, 8)
+    allocator = runner.cache.groups[0].allocator
+    owners: dict[int, list[str]] = {}
+    real = allocator.allocate
+
+    def spy(holder, n_pages):
+        pages = real(holder, n_pages)
+        for page in pages:
+            owners.setdefault(page, []).append(holder)
+        return pages
+
+    allocator.allocate = spy
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    replay_util.compare(rows, expected, **F32_TOL)
+    reused = {page: who for page, who in owners.items() if len(set(who)) > 1}
+    assert len(reused) >= 4, f"pages handed to a second request: {reused}"
+    assert sum(len(who) for who in owners.values()) > allocator.total_pages, "more pages handed out than the pool has"
+    assert runner.cache.stats().pages_used == 0
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -410,6 +465,36 @@ def test_trace_run_program(tiny_folders, plain, tmp_path, dtype):
             assert not path.exists()
     rows = replay_util.by_position(steps, outputs)
     replay_util.compare(rows, expected, **TOL[dtype])
+
+
+def test_trace_run_takes_many_short_requests_and_names_a_step_that_does_not_fit(tiny_folders, plain, tmp_path):
+    """Fourteen requests live at once, each well inside the token bound: the program has a slot for every
+    page of its pool.  A step that the pool cannot hold ends the run with a message that names the step."""
+    folder, raw, tensors = tiny_folders["A"]
+    weights = {k: v.float() for k, v in tensors.items()}
+    requests = {f"s{i}": random_tokens(3 + i % 4, raw["vocab_size"], seed=900 + i) for i in range(14)}
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": tokens[:2], "want": [1]} for rid, tokens in requests.items()],
+              "end": []},
+             {"step": 1, "entries": [{"id": rid, "tokens": tokens[2:], "want": list(range(len(tokens) - 2))}
+                                     for rid, tokens in requests.items()], "end": list(requests)}]
+    pool = replay_util.max_live_tokens(steps, page=64)
+    out_dir = tmp_path / "out"
+    text = "\n".join(json.dumps(step) for step in steps) + "\n"
+    command = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype", "float32",
+               "--out", str(out_dir)]
+    done = subprocess.run(command + ["--max-tokens", str(pool)], input=text, capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr[-3000:]
+    assert [line for line in done.stdout.splitlines() if line.startswith("done ")] == ["done 0", "done 1"]
+    vocab = raw["vocab_size"]
+    outputs = {n: np.fromfile(out_dir / f"{n}.f32", dtype="<f4").reshape(-1, vocab) for n in (0, 1)}
+    rows = replay_util.by_position(steps, outputs)
+    expected = {rid: plain_qwen2.forward(raw, weights, tokens) for rid, tokens in requests.items()}
+    replay_util.compare(rows, expected, every_position=False, **F32_TOL)
+    # too small a pool (pages of 8: two pages hold two requests) and too few slots: a message, not a traceback
+    for extra in (["--max-tokens", "16", "--page-size", "8"], ["--max-tokens", str(pool), "--max-requests", "5"]):
+        short = subprocess.run(command + extra, input=text, capture_output=True, text=True, timeout=600)
+        assert short.returncode == 1 and "step 0 does not fit" in short.stderr and "Traceback" not in short.stderr, \
+            short.stderr[-2000:]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
