@@ -13,6 +13,8 @@ enum {
     CIE_OK = 0,
     CIE_BAD_ARGUMENT = 1,   // a size or option the kernel does not take
     CIE_LAUNCH_FAILED = 2,  // hipGetLastError() after the launch
+    CIE_TOO_LARGE = 3,      // more than the fixed scratch memory of an entry point that allocates nothing holds
+    CIE_SETUP_FAILED = 4,   // the library's own device memory could not be found on this device
 };
 
 constexpr int kWave = 64;

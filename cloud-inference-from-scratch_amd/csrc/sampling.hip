@@ -5,11 +5,41 @@
 // [0, 1) the token is the first i whose running sum of p exceeds u * sum(p).
 // u is made on the host from (seed, request, step), so a draw depends neither
 // on the batch nor on the thread layout.  T <= 0 means greedy.
+#include <mutex>
+
+#include "cie_no_alloc.h"
 #include "common.h"
+
+// Partial results of cie_argmax_static's first stage: CIE_ARGMAX_STATIC_MAX_ENTRIES best values (float),
+// then as many indices (int).  Host code never passes this name to a kernel: in host code it is a stand-in,
+// not a device address.  It asks for the array's address on the current device once (static_scratch) and
+// uses that pointer.
+static __device__ __align__(256) unsigned char scratch[CIE_ARGMAX_STATIC_MAX_ENTRIES * (sizeof(float) + sizeof(int))];
 
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kMaxDevices = 64;
+
+std::mutex scratch_lock;
+void* scratch_on_device[kMaxDevices];  // the array's address on each device, once it has been asked for
+
+// The address of `scratch` on the current device (every GPU holds its own copy at its own address).
+int static_scratch(unsigned char** out) {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return CIE_SETUP_FAILED;
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (scratch_on_device[device] == nullptr) {
+        void* found = nullptr;
+        if (hipGetSymbolAddress(&found, HIP_SYMBOL(scratch)) != hipSuccess || found == nullptr) {
+            (void)hipGetLastError();  // (so that the next launch check does not report this one)
+            return CIE_SETUP_FAILED;
+        }
+        scratch_on_device[device] = found;
+    }
+    *out = static_cast<unsigned char*>(scratch_on_device[device]);
+    return CIE_OK;
+}
 
 __device__ __forceinline__ void argmax_block(const float* row, int vocab, float* s_val, int* s_idx,
                                              float& best_out, int& idx_out) {
@@ -46,7 +76,7 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
               const float* __restrict__ uniform, int* __restrict__ out, int vocab, int ld) {
     __shared__ float s_val[kThreads];
     __shared__ int s_idx[kThreads];
-    __shared__ float scratch[16];
+    __shared__ float s_target;
     const int r = blockIdx.x;
     const float* row = logits + static_cast<size_t>(r) * ld;
     float best;
@@ -77,12 +107,12 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
         int owner = 0;  // the last non-empty span that starts at or below the target
         for (int t = 1; t < kThreads; ++t)
             if (t * span < vocab && s_val[t] <= target) owner = t;
-        scratch[0] = target;
+        s_target = target;
         s_idx[0] = owner;
     }
     __syncthreads();
     if (threadIdx.x != s_idx[0]) return;
-    const float target = scratch[0];
+    const float target = s_target;
     float running = s_val[threadIdx.x];
     int pick = end - 1;  // if rounding leaves the target unreached inside the span: its last token
     for (int i = begin; i < end; ++i) {
@@ -160,6 +190,25 @@ CIE_API int cie_argmax(void* stream, const float* logits, float* chunk_val, int*
     argmax_chunks_kernel<<<dim3(chunks, rows), kThreads, 0, s>>>(logits, chunk_val, chunk_idx, vocab, ld, chunk);
     if (cie_after_launch() != CIE_OK) return CIE_LAUNCH_FAILED;
     argmax_final_kernel<<<rows, kThreads, 0, s>>>(chunk_val, chunk_idx, out, chunks);
+    return cie_after_launch();
+}
+
+// The same without a workspace from the caller and without any allocation: see cie_no_alloc.h.
+CIE_API int cie_argmax_static(void* stream, const float* logits, int* out, int rows, int vocab, int ld, int chunk) {
+    if (rows < 0 || vocab <= 0 || ld < vocab || chunk <= 0 || rows > 65535 || !logits || !out) return CIE_BAD_ARGUMENT;
+    if (rows == 0) return CIE_OK;
+    const long chunks = (static_cast<long>(vocab) + chunk - 1) / chunk;
+    if (chunks * rows > CIE_ARGMAX_STATIC_MAX_ENTRIES) return CIE_TOO_LARGE;
+    unsigned char* base = nullptr;
+    const int found = static_scratch(&base);
+    if (found != CIE_OK) return found;
+    float* chunk_val = reinterpret_cast<float*>(base);
+    int* chunk_idx = reinterpret_cast<int*>(base + CIE_ARGMAX_STATIC_MAX_ENTRIES * sizeof(float));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    argmax_chunks_kernel<<<dim3(static_cast<unsigned>(chunks), rows), kThreads, 0, s>>>(logits, chunk_val, chunk_idx,
+                                                                                      vocab, ld, chunk);
+    if (cie_after_launch() != CIE_OK) return CIE_LAUNCH_FAILED;
+    argmax_final_kernel<<<rows, kThreads, 0, s>>>(chunk_val, chunk_idx, out, static_cast<int>(chunks));
     return cie_after_launch();
 }
 

@@ -16,7 +16,8 @@ from .library import load_library
 
 F32, BF16 = 0, 1
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
-_ERRORS = {1: "bad argument (a size or option the kernel does not take)", 2: "kernel launch failed"}
+_ERRORS = {1: "bad argument (a size or option the kernel does not take)", 2: "kernel launch failed",
+           3: "more than the entry point's fixed scratch memory holds", 4: "the library's device memory was not found"}
 
 
 class KernelError(RuntimeError):
