@@ -202,6 +202,7 @@ def main(argv=None) -> int:
 
     def point(batch: int, context: int):
         """(tokens/s of each measured window, the median window's ms per step and roofline share)."""
+        context = min(context, config.max_position_embeddings - SLACK)  # (the last positions are the slack's)
         engine = make_engine(config, args.dtype, batch, context, args.prefill_tokens)
         measured = decode_windows(engine, config, batch, context, steps, warmup, seed=batch)
         del engine

@@ -1,0 +1,52 @@
+// What the matrix-core attention kernels share: operand types, the block size of the key loop, and the
+// argument record that the entry point fills for every form (decode parts, tiled prompt forms, merge).
+#pragma once
+
+#include "common.h"
+
+namespace cie_attention {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kKeysPerBlock = 32;
+constexpr int kTileWaves = 4;  // waves of a workgroup in the prompt form
+constexpr float kLazyRescale = 8.f;  // base-2 units a score may pass a row's reference before it moves
+
+struct AttentionArgs {
+    const bf16_t* q;
+    int q_row_stride;
+    const bf16_t* k_pool;
+    const bf16_t* v_pool;
+    const int* block_table;
+    int table_width;
+    const int* tile_seq;
+    const int* tile_q0;
+    const int* seq_slot;
+    const int* seq_start;
+    const int* seq_q_len;
+    const int* q_start_loc;
+    bf16_t* out;
+    float* part_o;   // [tiles, kv_heads, splits, rows, D]
+    float* part_ml;  // [tiles, kv_heads, splits, rows, 2]
+    int q_heads;
+    int kv_heads;
+    int page_shift;
+    int window;
+    float scale;
+    int n_splits;
+    int tokens_per_tile;
+    int keys_per_split;  // multiple of kKeysPerBlock; 0 with one split
+    int n_tiles;
+    int xcds_per_head;  // prompt form: > 0 if every kv head has that many of the 8 XCDs (and their L2) to itself
+    const int* max_context_dev;  // if set (a captured graph replays with other lengths): keys per split are
+                                 // derived from this device value, the longest context of the step
+};
+
+// The prompt form of eight waves per 128-row tile (csrc/attention_prompt.hip); returns a CIE_* code.
+int launch_prompt_form(hipStream_t stream, const AttentionArgs& a, int head_dim);
+
+constexpr int kPromptWaves = 8;       // waves of a workgroup in that form
+constexpr int kPromptTileRows = 128;  // (token, head) rows of its tiles
+
+}  // namespace cie_attention

@@ -23,46 +23,12 @@
 // Scores, running maximum, sums and the output accumulator are float32.  The softmax runs in base 2:
 // scores are scaled by scale * log2(e) once, so that each probability is one v_exp_f32; the
 // accumulator is rescaled only in blocks where some row's running maximum moved.
+#include "attention_args.h"
 #include "common.h"
 
+using namespace cie_attention;
+
 namespace {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
-constexpr int kKeysPerBlock = 32;
-constexpr int kTileWaves = 4;  // waves of a workgroup in the prompt form
-constexpr float kLazyRescale = 8.f;  // base-2 units a score may pass a row's reference before it moves
-
-struct AttentionArgs {
-    const bf16_t* q;
-    int q_row_stride;
-    const bf16_t* k_pool;
-    const bf16_t* v_pool;
-    const int* block_table;
-    int table_width;
-    const int* tile_seq;
-    const int* tile_q0;
-    const int* seq_slot;
-    const int* seq_start;
-    const int* seq_q_len;
-    const int* q_start_loc;
-    bf16_t* out;
-    float* part_o;   // [tiles, kv_heads, splits, rows, D]
-    float* part_ml;  // [tiles, kv_heads, splits, rows, 2]
-    int q_heads;
-    int kv_heads;
-    int page_shift;
-    int window;
-    float scale;
-    int n_splits;
-    int tokens_per_tile;
-    int keys_per_split;  // multiple of kKeysPerBlock; 0 with one split
-    int n_tiles;
-    int xcds_per_head;  // prompt form: > 0 if every kv head has that many of the 8 XCDs (and their L2) to itself
-    const int* max_context_dev;  // if set (a captured graph replays with other lengths): keys per split are
-                                 // derived from this device value, the longest context of the step
-};
 
 template <int D, int RT>
 __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs a) {
@@ -712,6 +678,8 @@ int launch_for_dim(hipStream_t s, const AttentionArgs& a, int n_tiles, int row_t
 
 }  // namespace
 
+// tile_waves: 1 (one wave per tile and part), 4 (four waves take a tile's key blocks in turn; row_tiles 1, 2 or 4)
+// or 8 (csrc/attention_prompt.hip: tiles of 128 rows, row_tiles = 8, keys and values shared through LDS).
 // Workspace sizes (floats) the caller provides when n_splits > 1:
 //   part_o  n_tiles * kv_heads * n_splits * 16*row_tiles * head_dim
 //   part_ml n_tiles * kv_heads * n_splits * 16*row_tiles * 2
@@ -732,8 +700,10 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     if (n_splits > kMergeMaxSplits) return CIE_BAD_ARGUMENT;
     // the prompt form takes maxima before scaling, which needs a positive scale, and keeps the 16 keys of a
     // product in one page
-    if (tile_waves != 1 && (tile_waves != kTileWaves || !(scale > 0.f) || page_size < 16))
+    if (tile_waves != 1 && ((tile_waves != kTileWaves && tile_waves != kPromptWaves) || !(scale > 0.f) || page_size < 16))
         return CIE_BAD_ARGUMENT;
+    // the form of eight waves has tiles of 128 rows, no fewer, and heads of up to 128 dimensions
+    if (tile_waves == kPromptWaves && (16 * row_tiles != kPromptTileRows || head_dim > 128)) return CIE_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml ||
                          (!max_context_dev && (keys_per_split <= 0 || keys_per_split % kKeysPerBlock))))
         return CIE_BAD_ARGUMENT;
@@ -769,6 +739,12 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     a.xcds_per_head = (kv_heads <= 8 && 8 % kv_heads == 0) ? 8 / kv_heads : 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;
+    if (tile_waves == kPromptWaves) {
+        rc = launch_prompt_form(s, a, head_dim);
+        if (rc != CIE_OK || n_splits == 1) return rc;
+        attention_merge_kernel<<<dim3(n_tiles, kv_heads, tokens_per_tile * group), kMergeThreads, 0, s>>>(a, head_dim, kPromptTileRows);
+        return cie_after_launch();
+    }
     switch (head_dim) {
         case 32: rc = launch_for_dim<32>(s, a, n_tiles, row_tiles, tile_waves); break;
         case 64: rc = launch_for_dim<64>(s, a, n_tiles, row_tiles, tile_waves); break;

@@ -290,6 +290,7 @@ def paged_attention_generic(q: torch.Tensor, q_row_stride: int, k_pool: torch.Te
 
 MFMA_HEAD_DIMS = (32, 64, 96, 128, 256)
 TILE_WAVES = 4  # waves per workgroup of the prompt form of the matrix-core attention
+PROMPT_WAVES = 8  # ... and of its form with tiles of 128 rows whose keys and values go through LDS
 
 
 def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
@@ -310,7 +311,9 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
     (a multiple of 32; or, with ``max_context_dev``, derived on the device from the
     step's longest context) and merged through the workspaces.  ``tile_waves=4`` gives
     every tile (and every part of its keys) a workgroup of four waves that take the
-    blocks of 32 keys in turn; it needs pages of at least 16 keys."""
+    blocks of 32 keys in turn; it needs pages of at least 16 keys.  ``tile_waves=8`` (with
+    ``row_tiles=8``: tiles of 128 rows, heads of up to 128 dimensions) gives every tile eight waves that
+    share the tile's keys and values through LDS."""
     if not (
         q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 2 and q.stride(1) == 1 and q.stride(0) == q_row_stride
     ):
@@ -322,7 +325,7 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
     if not (q_heads % kv_heads == 0):
         raise ValueError(f"{q_heads} query heads are no multiple of {kv_heads} key heads")
     group = q_heads // kv_heads
-    if not (row_tiles in (1, 2, 4) and 1 <= tokens_per_tile and tokens_per_tile * group <= 16 * row_tiles):
+    if not (row_tiles in (1, 2, 4, 8) and 1 <= tokens_per_tile and tokens_per_tile * group <= 16 * row_tiles):
         raise ValueError(f"{tokens_per_tile} tokens of {group} heads do not fit {row_tiles} row tiles")
     page_size = _check_pools(k_pool, v_pool, torch.bfloat16, kv_heads, head_dim)
     if not (page_size >= 4 and page_size & (page_size - 1) == 0):
@@ -347,8 +350,10 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
     if not (1 <= n_splits <= 65535):
         raise ValueError(f"n_splits {n_splits} out of range")
     if not (
-        tile_waves == 1
-        or (tile_waves == TILE_WAVES and scale > 0 and page_size >= 16 and (row_tiles == 1 or head_dim <= 128))
+        (tile_waves == 1 and row_tiles <= 4)
+        or (tile_waves == TILE_WAVES and scale > 0 and page_size >= 16 and row_tiles <= 4
+            and (row_tiles == 1 or head_dim <= 128))
+        or (tile_waves == PROMPT_WAVES and scale > 0 and page_size >= 16 and row_tiles == 8 and head_dim <= 128)
     ):
         raise ValueError(f"tile_waves {tile_waves} with {n_splits} splits, {row_tiles} row tiles, head size {head_dim}, "
                          f"pages of {page_size}")

@@ -118,6 +118,13 @@ SPLIT_MIN_KEYS = 32  # the fewest keys of a one-wave part
 SPLIT_DECODE_KEYS = 192  # contexts from which the keys of decode rows are cut into parts at all
 JOINED_DECODE_ROWS = 32  # up to this many single-token sequences beside prompt portions ride in the prompt form's launch
 PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's keys are cut
+# Tiles of 128 rows x kv heads from which prompt portions take the form of eight waves: enough to give most
+# compute units a workgroup without cutting the keys (whose parts, 64 KB of sums per tile and kv head, cost that
+# form more than they gain it: 512 tokens behind 1,536 keys, 7B heads, 60 us in two parts against 40 us in the form
+# of four waves).  Measured at head size 128 (us, four waves -> eight): 2,048 tokens of one prompt 55.7 -> 51.4
+# (3B heads), 101 -> 58 (7B), 144 -> 84 (14B); behind 2,048 keys 108 -> 91, 195 -> 135, 284 -> 201; beside 8 single
+# tokens 108 -> 64, 138 -> 75, 182 -> 111.
+EIGHT_WAVE_TILES = 192
 
 
 def plan_splits(units: int, max_keys: int, target_waves: int = 1024, min_keys: int = 128) -> tuple[int, int]:
@@ -153,6 +160,15 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
               head_dim, window, scale)
     max_keys = batch.max_context if window is None else min(batch.max_context, window + 64)
     wide = page_size >= 16 and scale > 0
+    # Prompt portions with enough rows take tiles of 128 rows and eight waves, whose keys and values pass
+    # through LDS once per tile.  (A short portion behind a long context also has its keys cut into parts.)
+    prompt_tokens = sum(n for n in batch.host_q_lens if n > 1)
+    bound = batch.static_plan.max_keys if batch.static_plan is not None else max_keys
+    cuts = max(1, bound // PROMPT_SPLIT_KEYS) if wide and window is None else 1  # (a window's keys stay whole)
+    big_tiles = -(-prompt_tokens * group // 128) * num_kv_heads
+    # (heads of 128 dimensions: with 64 the form of four waves is the faster one, 2,048 tokens behind 6,144
+    # keys 114 against 140 us, since the softmax arithmetic per key is the same and the products are half)
+    eight = wide and head_dim == 128 and group <= 128 and big_tiles >= EIGHT_WAVE_TILES
 
     def decode_form(bound: int, units: int) -> tuple[int, dict]:
         # Decode rows, `units` (sequence, kv head) pairs over up to `bound` keys.  Long contexts: four waves
@@ -184,7 +200,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         max_keys = plan.max_keys if window is None else min(plan.max_keys, window + 64)
         longest_dev = plan.max_context
         decode_rows = batch.sequences if plan.decode_rows is None else plan.decode_rows
-        joined = wide and 0 < decode_rows <= JOINED_DECODE_ROWS and decode_rows < batch.sequences
+        joined = wide and not eight and 0 < decode_rows <= JOINED_DECODE_ROWS and decode_rows < batch.sequences
         if decode_rows and not joined:
             decode_waves, split_options = decode_form(max_keys, decode_rows * num_kv_heads)
             n_splits, _ = plan_splits(decode_rows * num_kv_heads, max_keys, **split_options)
@@ -203,7 +219,8 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         # A few single tokens beside prompt portions: one launch (and one merge) of the prompt form for all
         # sequences instead of two of each (8 decode rows and a 64-token portion of the 3B shape: 4.84 -> 4.49 ms
         # a step; 32 rows over 3,000 keys and 256 tokens: 8.9 -> 8.2 ms; with 64 such rows the forms are level)
-        joined = wide and 0 < n_tiles <= JOINED_DECODE_ROWS and n_tiles < batch.sequences
+        # (not beside the form of eight waves, where a tile of one token would leave six of them idle)
+        joined = wide and not eight and 0 < n_tiles <= JOINED_DECODE_ROWS and n_tiles < batch.sequences
     if n_tiles and not joined:
         decode_waves, split_options = decode_form(max_keys, n_tiles * num_kv_heads)
         n_splits, per_split = plan_splits(n_tiles * num_kv_heads, max_keys, **split_options)
@@ -213,18 +230,18 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
                                  n_tiles, *common, tokens_per_tile=1, row_tiles=1, n_splits=n_splits,
                                  keys_per_split=per_split, part_o=part_o, part_ml=part_ml, tile_waves=decode_waves)
-    prompt_tokens = sum(n for n in batch.host_q_lens if n > 1)
-    cuts = 1
     if wide:
-        # the prompt form: four waves share a tile's keys.  More rows per tile re-use each key more often,
+        # the prompt forms: waves share a tile's keys.  More rows per tile re-use each key more often,
         # fewer tiles leave compute units idle: the most rows that still give most units a workgroup, where a
         # short portion behind a long context also has its keys cut (256 tokens behind 3,840 keys, 2 kv heads:
         # 34 us with 64 rows per tile and four parts, 48 us with 16 rows per tile and the keys whole)
-        tile_waves = ops.TILE_WAVES
-        row_tiles = 4 if head_dim <= 128 else 1
-        cuts = max(1, max_keys // PROMPT_SPLIT_KEYS) if window is None else 1  # (a window's keys stay whole)
-        while row_tiles > 1 and -(-prompt_tokens * group // (16 * row_tiles)) * num_kv_heads * cuts < 192:
-            row_tiles //= 2
+        if eight:
+            tile_waves, row_tiles = ops.PROMPT_WAVES, 8
+        else:
+            tile_waves = ops.TILE_WAVES
+            row_tiles = 4 if head_dim <= 128 else 1
+            while row_tiles > 1 and -(-prompt_tokens * group // (16 * row_tiles)) * num_kv_heads * cuts < 192:
+                row_tiles //= 2
     else:
         # one wave per tile; fewer rows where that would leave SIMDs without a wave (about a thousand
         # waves fill the GPU) or where the accumulators of a wide head would spill

@@ -129,6 +129,42 @@ def test_replay_with_the_four_wave_prompt_attention(tiny_folders, plain, monkeyp
     assert runner.cache.stats().pages_used == 0
 
 
+@pytest.mark.parametrize("schedule", ["whole", "portions", "mixed"])
+@pytest.mark.parametrize("heads", [(16, 2), (28, 4), (10, 2)])
+def test_replay_with_the_eight_wave_prompt_attention(tmp_path, monkeypatch, schedule, heads):
+    """Prompt portions of many rows go to tiles of 128 rows and eight waves (heads of 128 dimensions).
+    The tiny requests here never have that many rows: the threshold is lowered so that every portion
+    takes that form, with groups of 8, 7 and 5 heads (tiles of 16, 18 and 25 tokens)."""
+    from conftest import TINY_C, make_folder
+    from cie_amd.kernels import ops
+    from cie_amd.parts import attention
+
+    monkeypatch.setattr(attention, "EIGHT_WAVE_TILES", 1)
+    seen = []
+    real = ops.paged_attention_mfma
+
+    def spy(*args, **kwargs):
+        seen.append(kwargs.get("tile_waves", 1))
+        return real(*args, **kwargs)
+
+    monkeypatch.setattr(ops, "paged_attention_mfma", spy)
+    q_heads, kv_heads = heads
+    raw = dict(TINY_C, hidden_size=128, num_attention_heads=q_heads, num_key_value_heads=kv_heads, head_dim=128,
+               intermediate_size=96, vocab_size=211, eos_token_id=1, attention_bias=True)
+    folder, tensors = make_folder(tmp_path, raw, seed=5)
+    requests = {f"r{i}": random_tokens(n, 211, seed=80 + i) for i, n in enumerate((9, 47, 130, 200))}
+    expected = plain_all(raw, tensors, requests)
+    steps = SCHEDULES[schedule](requests)
+    runner = make_runner(folder, "bfloat16", replay_util.max_live_tokens(steps, page=16), 16, max_running=4)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    weights = {k: v.float() for k, v in tensors.items()}
+    rough = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
+    print(heads, schedule, "rms %.3e worst %.3e, plain in bfloat16 %.3e %.3e"
+          % replay_util.closer_than_plain_bfloat16(rows, expected, rough), flush=True)
+    assert ops.PROMPT_WAVES in seen
+    assert runner.cache.stats().pages_used == 0
+
+
 @pytest.mark.parametrize("graph", [False, True])
 def test_replay_with_the_four_wave_decode_attention(tiny_folders, plain, monkeypatch, graph):
     """Decode rows go to the four-wave attention form only for long contexts and not for
