@@ -10,6 +10,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kKeysPerBlock = 32;
+constexpr int kXcds = 8;  // an MI355X has 8 XCDs of 32 compute units, each with an L2 of its own; the
+                          // hardware hands workgroup b of a launch to XCD b % 8
 constexpr int kTileWaves = 4;  // waves of a workgroup in the prompt form
 constexpr float kLazyRescale = 8.f;  // base-2 units a score may pass a row's reference before it moves
 
@@ -38,7 +40,7 @@ struct AttentionArgs {
     int tokens_per_tile;
     int keys_per_split;  // multiple of kKeysPerBlock; 0 with one split
     int n_tiles;
-    int xcds_per_head;  // prompt form: > 0 if every kv head has that many of the 8 XCDs (and their L2) to itself
+    int xcds_per_head;  // prompt forms: > 0 if every kv head has that many of the kXcds XCDs (and their L2) to itself
     const int* max_context_dev;  // if set (a captured graph replays with other lengths): keys per split are
                                  // derived from this device value, the longest context of the step
 };

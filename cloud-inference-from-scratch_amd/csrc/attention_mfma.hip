@@ -274,9 +274,9 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
     // tiles are given to its own XCDs: that L2 then holds one head's cache instead of every head's.
     int tile_index, kv_head;
     if (a.xcds_per_head > 0) {
-        const int xcd = blockIdx.x & 7;
+        const int xcd = blockIdx.x % kXcds;
         kv_head = xcd % a.kv_heads;
-        tile_index = (blockIdx.x >> 3) * a.xcds_per_head + xcd / a.kv_heads;
+        tile_index = (blockIdx.x / kXcds) * a.xcds_per_head + xcd / a.kv_heads;
     } else {
         kv_head = blockIdx.x % a.kv_heads;
         tile_index = blockIdx.x / a.kv_heads;
@@ -650,7 +650,7 @@ template <int D>
 int launch_for_dim(hipStream_t s, const AttentionArgs& a, int n_tiles, int row_tiles, int tile_waves) {
     dim3 grid(n_tiles, a.kv_heads, a.n_splits);
     if (tile_waves == kTileWaves) {
-        grid = a.xcds_per_head > 0 ? dim3(8 * ((n_tiles + a.xcds_per_head - 1) / a.xcds_per_head), a.n_splits)
+        grid = a.xcds_per_head > 0 ? dim3(kXcds * ((n_tiles + a.xcds_per_head - 1) / a.xcds_per_head), a.n_splits)
                                    : dim3(static_cast<unsigned>(n_tiles) * a.kv_heads, a.n_splits);
         if (row_tiles == 1)
             paged_attention_tile_kernel<D, 1, kTileWaves><<<grid, 64 * kTileWaves, 0, s>>>(a);
@@ -736,7 +736,7 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     a.keys_per_split = n_splits > 1 ? keys_per_split : 0;
     a.max_context_dev = n_splits > 1 ? max_context_dev : nullptr;
     a.n_tiles = n_tiles;
-    a.xcds_per_head = (kv_heads <= 8 && 8 % kv_heads == 0) ? 8 / kv_heads : 0;
+    a.xcds_per_head = (kv_heads <= kXcds && kXcds % kv_heads == 0) ? kXcds / kv_heads : 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;
     if (tile_waves == kPromptWaves) {

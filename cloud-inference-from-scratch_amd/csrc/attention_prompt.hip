@@ -88,9 +88,9 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
     // tiles of a kv head go to that head's XCDs where the heads divide the 8 XCDs (see attention_mfma.hip)
     int tile_index, kv_head;
     if (a.xcds_per_head > 0) {
-        const int xcd = blockIdx.x & 7;
+        const int xcd = blockIdx.x % kXcds;
         kv_head = xcd % a.kv_heads;
-        tile_index = (blockIdx.x >> 3) * a.xcds_per_head + xcd / a.kv_heads;
+        tile_index = (blockIdx.x / kXcds) * a.xcds_per_head + xcd / a.kv_heads;
     } else {
         kv_head = blockIdx.x % a.kv_heads;
         tile_index = blockIdx.x / a.kv_heads;
@@ -422,7 +422,7 @@ int launch(hipStream_t s, const AttentionArgs& a) {
     constexpr int kLdsBytes = 2 * L::kStageBytes > kMeetBytes ? 2 * L::kStageBytes : kMeetBytes;
     static_assert(kLdsBytes <= 64 * 1024, "a workgroup's LDS without asking for more");
     const dim3 grid = a.xcds_per_head > 0
-                          ? dim3(8 * ((a.n_tiles + a.xcds_per_head - 1) / a.xcds_per_head), a.n_splits)
+                          ? dim3(kXcds * ((a.n_tiles + a.xcds_per_head - 1) / a.xcds_per_head), a.n_splits)
                           : dim3(static_cast<unsigned>(a.n_tiles) * a.kv_heads, a.n_splits);
     paged_attention_prompt_kernel<D><<<grid, kThreadsP, kLdsBytes, s>>>(a);
     return cie_after_launch();

@@ -71,12 +71,51 @@ __device__ __forceinline__ void argmax_block(const float* row, int vocab, float*
     __syncthreads();
 }
 
+// Temperature sampling walks the row in chunks of kChunk numbers, a thread's four neighbours at a time, so that
+// a wave's loads are whole cache lines.  The running sum has a fixed order all the same: a chunk's sum is
+// made by one fixed tree, the chunks are added one after the other, and inside the chunk that holds the
+// target the numbers are added in the order of their indices.
+constexpr int kChunk = kThreads * 4;
+constexpr int kMaxChunks = 2048;  // of a row: vocabularies up to 2,097,152
+
+__device__ __forceinline__ float4 exp_of_four(const float* row, int first, int vocab, float best, float inv_t) {
+    float4 e = {0.f, 0.f, 0.f, 0.f};
+    if (first + 3 < vocab && (reinterpret_cast<uintptr_t>(row + first) & 15) == 0) {
+        const float4 v = *reinterpret_cast<const float4*>(row + first);
+        e.x = expf((v.x - best) * inv_t);
+        e.y = expf((v.y - best) * inv_t);
+        e.z = expf((v.z - best) * inv_t);
+        e.w = expf((v.w - best) * inv_t);
+    } else {
+        if (first < vocab) e.x = expf((row[first] - best) * inv_t);
+        if (first + 1 < vocab) e.y = expf((row[first + 1] - best) * inv_t);
+        if (first + 2 < vocab) e.z = expf((row[first + 2] - best) * inv_t);
+        if (first + 3 < vocab) e.w = expf((row[first + 3] - best) * inv_t);
+    }
+    return e;
+}
+
+// Sum over the workgroup's threads in one fixed order; every thread gets the result (contains barriers).
+__device__ __forceinline__ float fixed_block_sum(float v, float* s_val) {
+    s_val[threadIdx.x] = v;
+    __syncthreads();
+    for (int stride = kThreads / 2; stride > 0; stride >>= 1) {
+        if (threadIdx.x < stride) s_val[threadIdx.x] += s_val[threadIdx.x + stride];
+        __syncthreads();
+    }
+    const float total = s_val[0];
+    __syncthreads();
+    return total;
+}
+
 __global__ void __launch_bounds__(kThreads)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
               const float* __restrict__ uniform, int* __restrict__ out, int vocab, int ld) {
     __shared__ float s_val[kThreads];
     __shared__ int s_idx[kThreads];
+    __shared__ float s_chunk[kMaxChunks];
     __shared__ float s_target;
+    __shared__ int s_pick;
     const int r = blockIdx.x;
     const float* row = logits + static_cast<size_t>(r) * ld;
     float best;
@@ -87,42 +126,57 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
         if (threadIdx.x == 0) out[r] = best_idx;
         return;
     }
-    // Each thread owns one contiguous span of the row, so the running sum has a fixed order.
-    const int span = (vocab + kThreads - 1) / kThreads;
-    const int begin = min(threadIdx.x * span, vocab);
-    const int end = min(begin + span, vocab);
     const float inv_t = 1.0f / temp;
-    float local = 0.f;
-    for (int i = begin; i < end; ++i) local += expf((row[i] - best) * inv_t);
-    s_val[threadIdx.x] = local;
+    const int chunks = (vocab + kChunk - 1) / kChunk;
+    for (int c = 0; c < chunks; ++c) {
+        const float4 e = exp_of_four(row, c * kChunk + threadIdx.x * 4, vocab, best, inv_t);
+        const float sum = fixed_block_sum((e.x + e.y) + (e.z + e.w), s_val);
+        if (threadIdx.x == 0) s_chunk[c] = sum;
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
+        float total = 0.f;
+        for (int c = 0; c < chunks; ++c) total += s_chunk[c];
+        const float target = uniform[r] * total;
         float running = 0.f;
-        for (int t = 0; t < kThreads; ++t) {  // exclusive prefix over the spans
-            const float v = s_val[t];
-            s_val[t] = running;
-            running += v;
+        int owner = chunks - 1;  // if rounding leaves the target unreached: the last chunk (and its last token)
+        for (int c = 0; c < chunks; ++c) {
+            if (running + s_chunk[c] > target) {
+                owner = c;
+                break;
+            }
+            running += s_chunk[c];
         }
-        const float target = uniform[r] * running;
-        int owner = 0;  // the last non-empty span that starts at or below the target
-        for (int t = 1; t < kThreads; ++t)
-            if (t * span < vocab && s_val[t] <= target) owner = t;
-        s_target = target;
+        s_target = target - running;  // what is left to reach inside the chunk
         s_idx[0] = owner;
+        s_pick = min(vocab, (owner + 1) * kChunk) - 1;
     }
     __syncthreads();
-    if (threadIdx.x != s_idx[0]) return;
+    const int owner = s_idx[0];
     const float target = s_target;
-    float running = s_val[threadIdx.x];
-    int pick = end - 1;  // if rounding leaves the target unreached inside the span: its last token
-    for (int i = begin; i < end; ++i) {
-        running += expf((row[i] - best) * inv_t);
-        if (running > target) {
-            pick = i;
-            break;
-        }
+    __syncthreads();
+    // inside the chunk: the sums of the threads before this one (in index order), then the thread's own four
+    const int first = owner * kChunk + threadIdx.x * 4;
+    const float4 e = exp_of_four(row, first, vocab, best, inv_t);
+    s_val[threadIdx.x] = (e.x + e.y) + (e.z + e.w);
+    __syncthreads();
+    for (int offset = 1; offset < kThreads; offset <<= 1) {  // running sums over the threads, in place
+        const float below = threadIdx.x >= offset ? s_val[threadIdx.x - offset] : 0.f;
+        __syncthreads();
+        s_val[threadIdx.x] += below;
+        __syncthreads();
     }
-    out[r] = pick;
+    float running = threadIdx.x > 0 ? s_val[threadIdx.x - 1] : 0.f;
+    int mine = 0x7fffffff;
+    const float four[4] = {e.x, e.y, e.z, e.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        running += four[i];
+        if (mine == 0x7fffffff && first + i < vocab && running > target) mine = first + i;
+    }
+    if (mine != 0x7fffffff) atomicMin(&s_pick, mine);  // the first index whose running sum passes the target
+    __syncthreads();
+    if (threadIdx.x == 0) out[r] = s_pick;
 }
 
 // Greedy over a large vocabulary, stage 1: each workgroup scans one chunk of one row and leaves its
@@ -215,7 +269,7 @@ CIE_API int cie_argmax_static(void* stream, const float* logits, int* out, int r
 CIE_API int cie_sample(void* stream, const float* logits, const float* temperature,
                        const float* uniform, int* out, int rows, int vocab, int ld) {
     if (rows < 0 || vocab <= 0 || ld < vocab) return CIE_BAD_ARGUMENT;
-    if (temperature && !uniform) return CIE_BAD_ARGUMENT;
+    if (temperature && (!uniform || (vocab + kChunk - 1) / kChunk > kMaxChunks)) return CIE_BAD_ARGUMENT;
     if (rows == 0) return CIE_OK;
     sample_kernel<<<rows, kThreads, 0, static_cast<hipStream_t>(stream)>>>(logits, temperature, uniform,
                                                                            out, vocab, ld);

@@ -13,6 +13,7 @@ a library (src/cloud_engine/model.py:89-137), with the small kernels around it.
 
 from __future__ import annotations
 
+import weakref
 from dataclasses import dataclass
 from typing import Any, Optional, Union
 
@@ -41,10 +42,22 @@ FUSED_SMALL_WEIGHT = 6 << 20
 # float32 logits of more rows than this go to the library (the hand-written kernel streams the weight once per
 # 64 rows; up to 64 rows it is one pass either way)
 FUSED_LOGIT_ROWS = 64
-# An ``into=`` product with fewer than this many 16-column tiles and K of at least 2 * PART_K cuts K
-# into parts of about PART_K for more workgroups (partial products, summed by the next norm kernel).
+# An ``into=`` product with fewer than this many 16-column tiles and a K of at least ``PART_MIN_K`` cuts K
+# into parts for more workgroups (partial products, summed by the next norm kernel).
 PART_BELOW_TILES = 512
-PART_K = 2752
+PART_MIN_K = 4096
+PART_WORKGROUPS = 512   # column tiles x parts that a cut aims for at least
+PART_K = 4096           # ... and the longest stretch of K a part takes
+
+
+def plan_k_parts(tiles: int, k: int) -> int:
+    """Into how many parts the K of an ``into=`` product with ``tiles`` column tiles is cut: enough for
+    ``PART_WORKGROUPS`` workgroups, and no part longer than ``PART_K``.  Measured at 8 rows with the weight
+    coming from memory (down products; microseconds for 2 / 4 / 8 parts): 128 tiles, K 11,008: 12.7 / 11.8 /
+    11.9 (here 4); 224 tiles, K 18,944: 32.7 / 31.1 / 29.3 (here 5); 320 tiles, K 13,824: 33.4 / 29.7 / 29.8
+    (here 4).  More parts cost the norm kernel that adds them as much as they gain the product."""
+    parts = max(-(-PART_WORKGROUPS // max(tiles, 1)), -(-k // PART_K))
+    return max(1, min(parts, 16, -(-k // 128)))  # (the kernel cuts K in steps of 128)
 
 
 @dataclass
@@ -89,6 +102,20 @@ class PartialSum:
     parts: torch.Tensor
 
 
+_WIDENED: dict[int, tuple["weakref.ref", torch.Tensor]] = {}
+
+
+def _widened(weight: torch.Tensor) -> torch.Tensor:
+    """``weight`` in float32, made at its first use (an output head of 150,000 rows is not copied every step)."""
+    key = id(weight)
+    kept = _WIDENED.get(key)
+    if kept is not None and kept[0]() is weight:
+        return kept[1]
+    wide = weight.float()
+    _WIDENED[key] = (weakref.ref(weight, lambda _gone, key=key: _WIDENED.pop(key, None)), wide)
+    return wide
+
+
 def _fusable(rows: int, k: int, row_stride: int, weight: torch.Tensor) -> bool:
     return weight.dtype == torch.bfloat16 and rows >= 1 and k % 8 == 0 and row_stride % 8 == 0
 
@@ -126,9 +153,9 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     if rows == 0 and into is None:  # nothing to multiply: no kernel, and no widened copy of the weight
         return torch.empty((0, n // 2 if silu else n), dtype=torch.float32 if wants_f32 else x.dtype, device=x.device)
     fusable = _fusable(rows, k, x.stride(0) if rows > 1 else k, weight)
-    cut_k = into is not None and -(-n // 16) < PART_BELOW_TILES and k >= 2 * PART_K
+    cut_k = into is not None and -(-n // 16) < PART_BELOW_TILES and k >= PART_MIN_K
     if fusable and cut_k and rows <= (FUSED_PARTS_ROWS_NARROW if -(-n // 16) < PARTS_NARROW_TILES else FUSED_PARTS_ROWS):
-        return PartialSum(ops.gemm_fused(weight, ops.EPI_PARTIAL, x, bias=bias, k_parts=-(-k // PART_K)))
+        return PartialSum(ops.gemm_fused(weight, ops.EPI_PARTIAL, x, bias=bias, k_parts=plan_k_parts(-(-n // 16), k)))
     if fusable and wants_f32 and rows > FUSED_LOGIT_ROWS and into is None and not silu and bias is None:
         out = ops.gemm_library(x, weight, out_dtype=torch.float32)  # logits of many rows: one pass over the weight
         if out is not None:
@@ -149,8 +176,9 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     if weight.dtype == torch.float32:
         out = ops.gemm_f32(x, weight, bias)
     elif wants_f32:
-        # a shape the kernel refuses: widen the operands, exact products, float32 sums
-        out = x.float() @ weight.float().t()
+        # a shape the kernel refuses (a width that is no multiple of 8): widened operands, exact products,
+        # float32 sums; the widened weight is made once and kept for as long as the weight lives
+        out = x.float() @ _widened(weight).t()
         out = out if bias is None else out + bias.float()
     else:
         out = ops.gemm_library(x, weight, bias) if x.is_cuda and x.stride(1) == 1 else None

@@ -618,6 +618,30 @@ def test_sample_greedy_and_temperature(ops):
         assert lo - 1e-5 <= u <= cdf[got[r]].item() + 1e-5, (r, got[r], lo, u, cdf[got[r]].item())
 
 
+@pytest.mark.parametrize("vocab", [1024, 4099, 151936])
+def test_sample_over_many_chunks(ops, vocab):
+    """A vocabulary of many chunks of the kernel's walk (and one that ends inside a chunk, with rows that are
+    not 16-byte aligned): the token is the one whose share of [0, 1) holds the row's number, for numbers
+    at the very start, inside and at the very end, and for a row whose weight sits in its last tokens."""
+    g = torch.Generator().manual_seed(62)
+    rows = 7
+    logits = (torch.randn((rows, vocab), generator=g) * 2).cuda()
+    logits[5, vocab - 3:] += 30.0       # nearly all weight in the last three tokens
+    logits[6, : vocab - 1] -= 60.0      # all of it in the last one
+    temperature = torch.tensor([0.7, 1.0, 1.5, 0.3, 1.0, 1.0, 1.0]).cuda()
+    uniform = torch.tensor([0.0, 0.37, 0.999999, 0.5, 0.123456, 0.9, 0.4]).cuda()
+    got = ops.sample(logits, temperature, uniform).tolist()
+    for r in range(rows):
+        p = torch.softmax(logits[r].double() / temperature[r].double(), dim=-1).cpu()
+        cdf = torch.cumsum(p, dim=0)
+        u = float(uniform[r])
+        lo = cdf[got[r] - 1].item() if got[r] > 0 else 0.0
+        assert 0 <= got[r] < vocab and lo - 2e-5 <= u <= cdf[got[r]].item() + 2e-5, (r, got[r], lo, u, cdf[got[r]].item())
+    assert got[5] >= vocab - 3 and got[6] == vocab - 1
+    # the same draw whatever else is in the batch: row 1 alone
+    assert ops.sample(logits[1:2], temperature[1:2], uniform[1:2]).tolist() == [got[1]]
+
+
 def test_sample_frequencies(ops):
     """Empirical frequencies on a four-token vocabulary follow softmax(l / T)."""
     logits = torch.tensor([[0.0, 1.0, 2.0, -1.0]]).repeat(4000, 1).cuda()

@@ -186,6 +186,7 @@ def test_block_part(dtype, rows, part_k, monkeypatch):
         from cie_amd.parts import linear
 
         monkeypatch.setattr(linear, "PART_K", part_k)
+        monkeypatch.setattr(linear, "PART_MIN_K", 2 * part_k)
     from cie_amd.config import Qwen2Config
     from cie_amd.parts.block import PreNormBlock
 

@@ -389,6 +389,7 @@ def test_products_cut_along_k_match_plain(tiny_folders, plain, monkeypatch, grap
     from cie_amd.parts import linear
 
     monkeypatch.setattr(linear, "PART_K", 128)  # Tiny-B's down product has K = 328: three parts
+    monkeypatch.setattr(linear, "PART_MIN_K", 256)
     folder, raw, _ = tiny_folders["B"]
     requests, expected = plain["B"]
     steps = replay_util.mixed(requests, live=4, decode_tail=30, seed=6)

@@ -59,3 +59,31 @@ def test_the_fallback_build_folder_must_be_this_users_own(tmp_path, monkeypatch)
     folder.rmdir()
     folder.symlink_to(tmp_path)  # a link is no folder of ours, wherever it points
     assert folder not in library._build_dirs()
+
+
+def test_k_parts_follow_tiles_and_k():
+    """The cut of a long K: enough parts for 512 workgroups, no part longer than 4,096, never more parts than
+    K has slices of 128; the shapes that were measured keep their measured choice."""
+    from cie_amd.parts.linear import plan_k_parts
+
+    assert plan_k_parts(128, 11008) == 4      # the 3B down product
+    assert plan_k_parts(224, 18944) == 5      # 7B
+    assert plan_k_parts(320, 13824) == 4      # 14B
+    assert plan_k_parts(6, 328) == 3 and plan_k_parts(3, 88) == 1
+    assert plan_k_parts(500, 4096) == 2 and plan_k_parts(1, 1 << 20) == 16
+
+
+def test_a_widened_head_is_made_once_and_let_go_with_its_weight():
+    import gc
+
+    import torch
+
+    from cie_amd.parts import linear
+
+    weight = torch.ones((5, 3), dtype=torch.bfloat16)
+    first = linear._widened(weight)
+    assert first.dtype == torch.float32 and linear._widened(weight) is first
+    key = id(weight)
+    del weight
+    gc.collect()
+    assert key not in linear._WIDENED
