@@ -46,6 +46,10 @@ class EngineConfig:
     # request admitted before it (the reference admits without a look at the pool, src/cloud_engine/scheduler.py:
     # 438-458, and long prompts then evict each other and are computed twice); False: as the reference
     admit_within_pool: bool = True
+    # the matrix products of a step that fills the token budget (and of one request's full portion) time every
+    # algorithm the vendor library has for their shapes at their first call, a few seconds each, instead of
+    # the handful its heuristic proposes; False: the heuristic's candidates only
+    search_library_algorithms: bool = True
     seed: int = 0
 
     def validated(self) -> "EngineConfig":

@@ -1,8 +1,11 @@
 // Matrix products with many rows go to the vendor library (hipBLASLt), as the reference leaves its
 // products to a library.  This is the thin host side of that: one handle, and for every shape the
-// descriptors and the algorithm (the library's heuristic pick, or the fastest of its candidates), kept
-// after the first call, so that a
-// step's few hundred products cost a table lookup and one launch each instead of a heuristic query.
+// descriptors and the algorithm, kept after the first call, so that a step's few hundred products cost a
+// table lookup and one launch each instead of a heuristic query.  The algorithm is the library's heuristic
+// pick, the fastest of the heuristic's candidates, or the fastest of every algorithm the library has for
+// the shape (a few hundred to two thousand for bf16, by the version of the library that the process has
+// loaded; with 2,048 rows and a wide result the best of them is 14 to 18 % faster than the best the
+// heuristic proposes, for up to a few seconds at the shape's first call).
 //
 //   C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]),  bf16 operands and bias, float32 sums, bf16 result
 //   (or, without bias, a float32 result: the logits)
@@ -10,10 +13,15 @@
 // In the library's column-major terms: D (N x M, ld N) = W^T (W stored K x N, ld K, transposed) *
 // A (K x M, ld lda); the bias is added along D's rows (the N dimension).
 #include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 #include "common.h"
 
@@ -43,18 +51,21 @@ void destroy(Plan& plan) {
 }
 
 constexpr int kCandidates = 16;
+using Found = std::vector<hipblasLtMatmulHeuristicResult_t>;
 
-// Descriptors for a shape and the algorithms the library's heuristic proposes, best guess first;
-// returns how many fit the workspace (0: the library has none).
-int make_plan(Plan& plan, hipblasLtMatmulHeuristicResult_t (&found)[kCandidates], int M, int N, int K, int lda,
-              bool has_bias, bool f32_out, size_t workspace_limit) {
+// Descriptors for a shape and the algorithms to choose from: those the library's heuristic proposes, best
+// guess first, and after them, if `every`, all others the library says it can run on this shape.  Returns
+// how many of the heuristic's fit the workspace (0: the library has none; `found` may then hold nothing).
+int make_plan(Plan& plan, Found& found, int M, int N, int K, int lda, bool has_bias, bool f32_out,
+              size_t workspace_limit, bool every) {
     const hipblasOperation_t transposed = HIPBLAS_OP_T, plain = HIPBLAS_OP_N;
+    const hipDataType result_type = f32_out ? HIP_R_32F : HIP_R_16BF;
     bool good = ok(hipblasLtMatmulDescCreate(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F)) &&
                 ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &transposed, sizeof(transposed))) &&
                 ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain))) &&
                 ok(hipblasLtMatrixLayoutCreate(&plan.w, HIP_R_16BF, K, N, K)) &&
                 ok(hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, K, M, lda)) &&
-                ok(hipblasLtMatrixLayoutCreate(&plan.d, f32_out ? HIP_R_32F : HIP_R_16BF, N, M, N));
+                ok(hipblasLtMatrixLayoutCreate(&plan.d, result_type, N, M, N));
     if (good && has_bias) {
         const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
         const hipDataType bias_type = HIP_R_16BF;
@@ -66,14 +77,31 @@ int make_plan(Plan& plan, hipblasLtMatmulHeuristicResult_t (&found)[kCandidates]
     if (!ok(hipblasLtMatmulPreferenceCreate(&preference))) return 0;
     const uint64_t limit = workspace_limit;
     int count = 0;
+    hipblasLtMatmulHeuristicResult_t proposed[kCandidates];
     good = ok(hipblasLtMatmulPreferenceSetAttribute(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit))) &&
            ok(hipblasLtMatmulAlgoGetHeuristic(g_handle, plan.desc, plan.w, plan.a, plan.d, plan.d, preference, kCandidates,
-                                              found, &count));
+                                              proposed, &count));
     hipblasLtMatmulPreferenceDestroy(preference);
     if (!good) return 0;
-    int kept = 0;
+    found.clear();
     for (int i = 0; i < count; ++i)
-        if (ok(found[i].state) && found[i].workspaceSize <= workspace_limit) found[kept++] = found[i];
+        if (ok(proposed[i].state) && proposed[i].workspaceSize <= workspace_limit) found.push_back(proposed[i]);
+    const int kept = static_cast<int>(found.size());
+    if (kept == 0 || !every) return kept;
+    Found all;
+    if (!ok(hipblaslt_ext::getAllAlgos(g_handle, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, transposed, plain, HIP_R_16BF,
+                                       HIP_R_16BF, result_type, result_type, HIPBLAS_COMPUTE_32F, all)))
+        return kept;
+    const float one = 1.f, zero = 0.f;
+    for (auto& candidate : all) {
+        size_t needs = 0;
+        if (!ok(hipblaslt_ext::matmulIsAlgoSupported(g_handle, plan.desc, &one, plan.w, plan.a, &zero, plan.d, plan.d,
+                                                     candidate.algo, needs)) ||
+            needs > workspace_limit)
+            continue;
+        candidate.workspaceSize = needs;
+        found.push_back(candidate);
+    }
     return kept;
 }
 
@@ -83,14 +111,34 @@ int make_plan(Plan& plan, hipblasLtMatmulHeuristicResult_t (&found)[kCandidates]
 // is 2.5 times slower than another once its weight has to be streamed.
 constexpr size_t kColdBytes = size_t(640) << 20;
 
+// Largest |x - y| and largest |x| of two results, as the bits of non-negative floats (which order as
+// unsigned integers do); a NaN on either side counts as an infinite difference.
+__device__ inline float as_float(float v) { return v; }
+__device__ inline float as_float(unsigned short bf16_bits) { return __uint_as_float(unsigned(bf16_bits) << 16); }
+
+template <typename T>
+__global__ void results_differ_kernel(const T* __restrict__ x, const T* __restrict__ y, size_t count,
+                                      unsigned* __restrict__ out) {
+    float diff = 0.f, size = 0.f;
+    for (size_t i = blockIdx.x * size_t(blockDim.x) + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) {
+        const float a = as_float(x[i]), b = as_float(y[i]);
+        const float d = fabsf(a - b);
+        diff = (d == d) ? fmaxf(diff, d) : __builtin_inff();
+        size = fmaxf(size, fabsf(a));
+    }
+    atomicMax(out, __float_as_uint(diff));
+    atomicMax(out + 1, __float_as_uint(size));
+}
+
 // Time the candidates on the call's own rows (the result is overwritten by the real call that follows)
 // and return the index of the fastest; 0 if timing is not possible.  A candidate's time is the shortest of
-// a few batches of runs; all candidates are timed once, then the four best again with more batches, so
-// that a candidate is not chosen or dropped for what else happened while it ran (clocks that had not come
-// up yet, a neighbour's work).
+// a few batches of runs; all candidates are timed once, then the best few again with more batches, taken in
+// turn, so that a candidate is not chosen or dropped for what else happened while it ran (clocks that had
+// not come up yet, a neighbour's work).  A winner that the heuristic did not propose is kept only if its
+// result agrees with that of the heuristic's first choice.
 struct Timing {
     const Plan& plan;
-    const hipblasLtMatmulHeuristicResult_t* found;
+    const Found& found;
     hipStream_t stream;
     const void* a;
     const char* w;
@@ -102,31 +150,72 @@ struct Timing {
     hipEvent_t begin, end;
     int turn = 0;
 
-    bool run(int i) {
+    bool run(int i, void* into = nullptr, bool first_copy = false) {
         const float one = 1.f, zero = 0.f;
-        const void* weight = cold ? cold + w_bytes * (turn++ % copies) : w;
-        return ok(hipblasLtMatmul(g_handle, plan.desc, &one, weight, plan.w, a, plan.a, &zero, c, plan.d, c, plan.d,
-                                  &found[i].algo, workspace, found[i].workspaceSize, stream));
+        const void* weight = cold && !first_copy ? cold + w_bytes * (turn++ % copies) : w;
+        void* result = into ? into : c;
+        return ok(hipblasLtMatmul(g_handle, plan.desc, &one, weight, plan.w, a, plan.a, &zero, result, plan.d, result,
+                                  plan.d, &found[i].algo, workspace, found[i].workspaceSize, stream));
     }
     // milliseconds of the fastest batch; negative if a call failed
-    float time(int i, int batches, int runs) {
+    float time(int i, int batches, int runs, bool warm = true) {
         float best = -1.f;
-        if (!run(i)) return -1.f;  // warm-up
+        if (warm && !run(i)) return -1.f;
         for (int b = 0; b < batches; ++b) {
             bool good = hipEventRecord(begin, stream) == hipSuccess;
             for (int r = 0; r < runs && good; ++r) good = run(i);
             float ms = 0.f;
             good = good && hipEventRecord(end, stream) == hipSuccess && hipEventSynchronize(end) == hipSuccess &&
                    hipEventElapsedTime(&ms, begin, end) == hipSuccess;
-            if (!good) return -1.f;
+            if (!good) {
+                (void)hipGetLastError();
+                return -1.f;
+            }
             if (best < 0.f || ms < best) best = ms;
         }
         return best;
     }
 };
 
-int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int count, hipStream_t stream,
-            const void* a, const void* w, size_t w_bytes, void* c, void* workspace, bool many_rows) {
+// Does candidate `i` give what candidate 0 gives (to the rounding of the result type and of another order
+// of sums)?  False also if that cannot be found out.
+bool agrees_with_first(Timing& timing, int i, size_t elements, bool f32_out) {
+    const size_t bytes = elements * (f32_out ? 4 : 2);
+    char* other = nullptr;
+    if (hipMalloc(reinterpret_cast<void**>(&other), bytes + 256) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    unsigned* verdict = reinterpret_cast<unsigned*>(other + (bytes + 7) / 8 * 8);
+    bool good = hipMemsetAsync(verdict, 0, 8, timing.stream) == hipSuccess && timing.run(0, nullptr, true) &&
+                timing.run(i, other, true);
+    if (good) {
+        const int blocks = 1024, threads = 256;
+        if (f32_out)
+            results_differ_kernel<float><<<blocks, threads, 0, timing.stream>>>(
+                static_cast<const float*>(timing.c), reinterpret_cast<const float*>(other), elements, verdict);
+        else
+            results_differ_kernel<unsigned short><<<blocks, threads, 0, timing.stream>>>(
+                static_cast<const unsigned short*>(timing.c), reinterpret_cast<const unsigned short*>(other), elements, verdict);
+        good = hipGetLastError() == hipSuccess;
+    }
+    unsigned bits[2] = {0, 0};
+    good = good && hipMemcpyAsync(bits, verdict, 8, hipMemcpyDeviceToHost, timing.stream) == hipSuccess &&
+           hipStreamSynchronize(timing.stream) == hipSuccess;
+    hipStreamSynchronize(timing.stream);
+    hipFree(other);
+    if (!good) {
+        (void)hipGetLastError();
+        return false;
+    }
+    float diff, size;
+    memcpy(&diff, &bits[0], 4);
+    memcpy(&size, &bits[1], 4);
+    return diff <= size * (1.f / 64.f);
+}
+
+int fastest(const Plan& plan, const Found& found, int proposed, hipStream_t stream, const void* a, const void* w,
+            size_t w_bytes, void* c, void* workspace, bool many_rows, size_t elements, bool f32_out) {
     hipEvent_t begin = nullptr, end = nullptr;
     if (hipEventCreate(&begin) != hipSuccess || hipEventCreate(&end) != hipSuccess) return 0;
     int copies = static_cast<int>((kColdBytes + w_bytes - 1) / w_bytes);
@@ -146,14 +235,19 @@ int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int
     Timing timing{plan, found, stream, a, static_cast<const char*>(w), cold, w_bytes, copies, c, workspace, begin, end};
     // short products scatter more: more runs in a batch
     const int runs = many_rows ? 2 : 6;
-    constexpr int kFinalists = 4;
-    int finalist[kCandidates];
-    float finalist_ms[kCandidates];
+    const int count = static_cast<int>(found.size());
+    const bool every = count > proposed;
+    // three rounds: everything once; the best 32 of a long list twice more, in turn; the best few five times
+    constexpr int kMost = 32;
+    const int wanted = every ? kMost : 4;
+    int finalist[kMost + 1];
+    float finalist_ms[kMost + 1];
     int finalists = 0;
-    for (int i = 0; i < count && i < kCandidates; ++i) {
-        const float ms = timing.time(i, 2, runs);
+    for (int i = 0; i < count; ++i) {
+        const float ms = timing.time(i, i < proposed ? 2 : 1, runs);
         if (ms < 0.f) continue;
-        int at = finalists++;
+        if (finalists == wanted && ms >= finalist_ms[finalists - 1]) continue;
+        int at = finalists < wanted ? finalists++ : finalists - 1;
         for (; at > 0 && finalist_ms[at - 1] > ms; --at) {  // kept in order of time
             finalist[at] = finalist[at - 1];
             finalist_ms[at] = finalist_ms[at - 1];
@@ -161,15 +255,41 @@ int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int
         finalist[at] = i;
         finalist_ms[at] = ms;
     }
-    if (finalists > kFinalists) finalists = kFinalists;
-    int best = finalists ? finalist[0] : 0;
-    float best_ms = -1.f;
-    for (int f = 0; f < finalists; ++f) {
-        const float ms = timing.time(finalist[f], 5, runs);
-        if (ms >= 0.f && (best_ms < 0.f || ms < best_ms)) {
-            best_ms = ms;
-            best = finalist[f];
+    auto again = [&](int rounds) {
+        for (int f = 0; f < finalists; ++f) finalist_ms[f] = -1.f;
+        for (int round = 0; round < rounds; ++round)
+            for (int f = 0; f < finalists; ++f) {
+                const float ms = timing.time(finalist[f], 1, runs, round == 0);
+                if (ms >= 0.f && (finalist_ms[f] < 0.f || ms < finalist_ms[f])) finalist_ms[f] = ms;
+            }
+        for (int f = 1; f < finalists; ++f) {  // in order of time again; failed ones last
+            const int index = finalist[f];
+            const float ms = finalist_ms[f];
+            int at = f;
+            for (; at > 0 && (finalist_ms[at - 1] < 0.f || (ms >= 0.f && finalist_ms[at - 1] > ms)); --at) {
+                finalist[at] = finalist[at - 1];
+                finalist_ms[at] = finalist_ms[at - 1];
+            }
+            finalist[at] = index;
+            finalist_ms[at] = ms;
         }
+    };
+    if (finalists > 8) {
+        again(2);
+        finalists = 8;
+    }
+    again(5);
+    int best = 0;
+    for (;;) {
+        int at = -1;
+        for (int f = 0; f < finalists; ++f)
+            if (finalist_ms[f] >= 0.f && (at < 0 || finalist_ms[f] < finalist_ms[at])) at = f;
+        if (at < 0) break;  // none left: the heuristic's first choice
+        if (finalist[at] < proposed || agrees_with_first(timing, finalist[at], elements, f32_out)) {
+            best = finalist[at];
+            break;
+        }
+        finalist_ms[at] = -1.f;
     }
     hipEventDestroy(begin);
     hipEventDestroy(end);
@@ -182,9 +302,10 @@ int fastest(const Plan& plan, const hipblasLtMatmulHeuristicResult_t* found, int
 
 }  // namespace
 
-// With `tune`, a shape's first call (outside graph capture) times the heuristic's candidates on the call's
-// own rows and on copies of its weight (device memory of its own, freed again) and keeps the fastest;
-// otherwise the heuristic's first choice is kept.
+// With `tune` 1, a shape's first call (outside graph capture) times the heuristic's candidates on the call's
+// own rows and on copies of its weight (device memory of its own, freed again) and keeps the fastest; with
+// `tune` 2 it times every algorithm the library can run on the shape (a few seconds); with 0 the heuristic's
+// first choice is kept.
 // Returns CIE_BAD_ARGUMENT for a shape the library has no algorithm for (the caller then takes another
 // route) and CIE_LAUNCH_FAILED if the library's call itself fails.  `workspace` is device memory of
 // `workspace_bytes` that stays valid while the product runs; calls on one stream may share it.
@@ -199,23 +320,28 @@ CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w
         auto it = g_plans.find(key);
         if (it == g_plans.end()) {
             Plan fresh;
-            hipblasLtMatmulHeuristicResult_t found[kCandidates];
-            const int count = make_plan(fresh, found, M, N, K, lda, bias != nullptr, f32_out != 0, workspace ? workspace_bytes : 0);
-            if (count == 0) {
+            Found found;
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            const bool may_time = tune && hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) == hipSuccess &&
+                                  capturing == hipStreamCaptureStatusNone;
+            const int proposed = make_plan(fresh, found, M, N, K, lda, bias != nullptr, f32_out != 0,
+                                           workspace ? workspace_bytes : 0, may_time && tune >= 2);
+            if (proposed == 0) {
                 destroy(fresh);
                 return CIE_BAD_ARGUMENT;
             }
             int chosen = 0;
-            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-            if (tune && count > 1 && hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) == hipSuccess &&
-                capturing == hipStreamCaptureStatusNone) {
+            if (may_time && found.size() > 1) {
                 if (bias) hipblasLtMatmulDescSetAttribute(fresh.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
                 // short products are timed over more runs: their times scatter more
-                chosen = fastest(fresh, found, count, static_cast<hipStream_t>(stream), a, w, size_t(N) * K * 2, c, workspace,
-                                 M >= 512);
+                chosen = fastest(fresh, found, proposed, static_cast<hipStream_t>(stream), a, w, size_t(N) * K * 2, c,
+                                 workspace, M >= 512, size_t(M) * N, f32_out != 0);
             }
             fresh.algo = found[chosen].algo;
             fresh.workspace = found[chosen].workspaceSize;
+            if (getenv("CIE_LIBRARY_REPORT"))  // which algorithm a shape got, for whoever reads a profile
+                fprintf(stderr, "[cie_amd library] %d x %d x %d: candidate %d of %zu (%d proposed): %s\n", M, N, K, chosen,
+                        found.size(), proposed, hipblaslt_ext::getKernelNameFromAlgo(g_handle, fresh.algo).c_str());
             it = g_plans.emplace(key, fresh).first;
         }
         plan = &it->second;

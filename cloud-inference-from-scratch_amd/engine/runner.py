@@ -21,6 +21,7 @@ import torch
 
 from ..cache.manager import CacheManager, PagedKV
 from ..config.engine_config import EngineConfig
+from ..kernels import ops
 from ..profiling import trace_range
 from ..sampling.sampler import Sampler
 from .batch import StepBatch, to_device_staging
@@ -81,6 +82,8 @@ class Runner:
                              if self.graphs is not None and config.graph_mixed_steps > 0 else None)
         self._staging = [None, None]
         self._staging_turn = 0
+        if config.search_library_algorithms:
+            ops.LIBRARY_SEARCH_ROWS.update({config.token_budget, min(config.prefill_chunk, config.token_budget)})
 
     def _tokens_from_bytes(self, needs: list[Any]) -> int:
         element = torch.tensor([], dtype=self.dtype).element_size()

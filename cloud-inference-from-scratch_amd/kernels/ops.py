@@ -525,6 +525,17 @@ LIBRARY_WORKSPACE_BYTES = 64 << 20
 # from 32 on (the buckets of captured decode steps) are the shapes that recur: they time the library's
 # candidate algorithms at their first call and keep the fastest; others take its first choice.
 LIBRARY_TUNE_ROWS = 512
+# Row counts whose products time every algorithm the library has, not only the heuristic's candidates (a few
+# seconds for each shape, once in a process): an engine names the sizes of its full prompt portions here.
+LIBRARY_SEARCH_ROWS: set[int] = set()
+
+
+def _tune_level(rows: int) -> int:
+    if rows >= LIBRARY_TUNE_ROWS and rows in LIBRARY_SEARCH_ROWS:
+        return 2
+    if (rows >= LIBRARY_TUNE_ROWS and rows % 256 == 0) or (rows >= 32 and rows & (rows - 1) == 0):
+        return 1
+    return 0
 
 
 def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -556,7 +567,7 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     code = load_library().cie_gemm_library(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k),
         _i(1 if out_dtype == torch.float32 else 0), _ptr(workspace), workspace.numel(),
-        _i(1 if (m >= LIBRARY_TUNE_ROWS and m % 256 == 0) or (m >= 32 and m & (m - 1) == 0) else 0))
+        _i(_tune_level(m)))
     if code == 1:
         return None
     _run("cie_gemm_library", code)

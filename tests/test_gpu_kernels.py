@@ -846,3 +846,23 @@ def test_gemm_library_matches_float64(ops, shape):
         wide[:, :k] = a
         torch.testing.assert_close(ops.gemm_library(wide[:, :k], w, b).double(), expect + b.double(), rtol=1e-2,
                                    atol=1e-2 * math.sqrt(k))
+
+
+def test_gemm_library_with_every_algorithm_timed(ops, monkeypatch):
+    """A row count that an engine has named has every algorithm of the library timed at a shape's first
+    call, and the one kept is still the product: shapes that no other test uses, so that their first call is here."""
+    monkeypatch.setattr(ops, "LIBRARY_SEARCH_ROWS", {768})
+    assert ops._tune_level(768) == 2 and ops._tune_level(1024) == 1 and ops._tune_level(700) == 0
+    for n, k in ((1040, 520), (264, 1288)):
+        a, w, b = rand((768, k), torch.bfloat16, 30), rand((n, k), torch.bfloat16, 31), rand((n,), torch.bfloat16, 32)
+        expect = a.double() @ w.double().t()
+        for _ in range(2):
+            out = ops.gemm_library(a, w)
+            if out is None:
+                pytest.skip("the library has no algorithm for this shape")
+            torch.testing.assert_close(out.double(), expect, rtol=1e-2, atol=1e-2 * math.sqrt(k))
+            torch.testing.assert_close(ops.gemm_library(a, w, b).double(), expect + b.double(), rtol=1e-2,
+                                       atol=1e-2 * math.sqrt(k))
+            exact = ops.gemm_library(a, w, out_dtype=torch.float32)
+            if exact is not None:
+                torch.testing.assert_close(exact.double(), expect, rtol=1e-4, atol=1e-4 * math.sqrt(k))
