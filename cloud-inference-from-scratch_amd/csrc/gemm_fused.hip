@@ -28,12 +28,15 @@
 // (the order of k inside a product is free as long as both operands agree).
 // No workgroup ever waits for another: a device-wide fence between workgroups costs more on
 // this GPU than the whole product.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes as one value (a struct is copied as memory)
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4, EPI_ROPE = 5 };
 
@@ -596,6 +599,220 @@ int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, int k_part
     return CIE_BAD_ARGUMENT;
 }
 
+// ---------------------------------------------------------------------------------------------
+// 17 to 128 rows: waves that own columns and share the rows of A.
+//
+// With more than 16 rows the kernel above spends more of the memory pipeline on the rows of A (which
+// every wave fetches for its own slices of K) than on W.  Here the four waves of a workgroup take the
+// same slice of 128 k values together: the workgroup's 256 threads fetch the slice of A once (whole
+// 256-byte row segments) into LDS, every wave streams its own NT tiles of 16 columns of W over all of
+// K (or a grid.z part of it) and reads the rows of A from LDS in the MFMA layout.  A wave's loads run
+// DIST slices ahead of its products, in a ring of DIST + 1 sets of registers that the unrolled loop
+// addresses by constants (a copy from a set whose load is still under way would wait for it).
+template <int EPI, int MT, int NT, int DIST, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs a) {
+    static_assert(EPI == EPI_SILU || EPI == EPI_PARTIAL || EPI == EPI_BF16, "epilogues of this form");
+    static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
+    constexpr int kWaves = WAVES;
+    constexpr int kThreads = WAVES * 64;
+    constexpr int kRing = DIST + 1;
+    constexpr int kRows = MT * 16;
+    constexpr int kStageBytesA = kRows * kStageRow;
+    constexpr int kStagesA = MT <= 4 ? 2 : 1;  // (two stages of 128 rows would pass the 64 KB of static LDS)
+    __shared__ __attribute__((aligned(16))) char shared[kStagesA * kStageBytesA + kWaves * kStageTile + kRows * sizeof(float)];
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    char* stage_w = shared + kStagesA * kStageBytesA + wave * kStageTile;
+    float* scale_lds = reinterpret_cast<float*>(shared + kStagesA * kStageBytesA + kWaves * kStageTile);
+    const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
+    // SILU: the wave's gate tile and its up tile; else NT adjacent tiles
+    const int tile_first = (EPI == EPI_SILU) ? blockIdx.x * kWaves + wave : (blockIdx.x * kWaves + wave) * NT;
+
+    const int load_row = lane >> 4;        // of the four rows of a load of W
+    const int load_col = (lane & 15) * 8;  // k offset inside the 128
+    const bf16_t* w_rows[NT][4];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = i * 4 + load_row;
+            const int n = (EPI == EPI_SILU) ? min(tile_first * 16 + row, cols - 1) + t * a.up_offset
+                                            : min((tile_first + t) * 16 + row, cols - 1);
+            w_rows[t][i] = a.w + static_cast<size_t>(n) * a.K;
+        }
+    // the slice of A: thread t takes the piece (t % 16) of rows t / 16 + (threads / 16) i (a row past the
+    // last one computes a copy that is not stored; past the last row tile, a thread repeats the last row)
+    constexpr int kRowsPerPass = kThreads / 16;
+    constexpr int kPasses = (kRows + kRowsPerPass - 1) / kRowsPerPass;
+    const int a_row = threadIdx.x >> 4;
+    const bf16_t* a_rows[kPasses];
+    int a_stage_row[kPasses];
+#pragma unroll
+    for (int i = 0; i < kPasses; ++i) {
+        a_stage_row[i] = min(i * kRowsPerPass + a_row, kRows - 1);
+        a_rows[i] = a.a + static_cast<size_t>(min(a_stage_row[i], a.M - 1)) * a.lda;
+    }
+    const int k_begin = blockIdx.z * a.k_per_part;
+    const int k_end = min(a.K, k_begin + a.k_per_part);
+    const int slices = (k_end - k_begin + 127) / 128;
+
+    // Every load is unconditional and stands in straight-line code, so that the compiler can wait for a
+    // slice by counting the loads behind it (after a load under a condition it waits for all): a piece
+    // past the end of the part reads the part's last piece again, and the piece of A is zeroed when used.
+    struct Slot {
+        u32x4 w[NT][4];
+        u32x4 a[kPasses];
+    };
+    Slot ring0, ring1, ring2;  // (the third only with DIST 2)
+    auto fetch = [&](Slot& into, int slice) __attribute__((always_inline)) {
+        const int k = min(k_begin + slice * 128 + load_col, k_end - 8);
+#pragma unroll
+        for (int i = 0; i < kPasses; ++i) into.a[i] = *reinterpret_cast<const u32x4*>(a_rows[i] + k);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) into.w[t][i] = *reinterpret_cast<const u32x4*>(w_rows[t][i] + k);
+    };
+
+    floatx4 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const int row_tiles_used = (a.M + 15) / 16;  // (row tiles past the last row are not multiplied)
+
+    auto step = [&](const Slot& now, Slot& ahead, int slice) __attribute__((always_inline)) {
+        char* stage_a = shared + (kStagesA == 2 ? (slice & 1) * kStageBytesA : 0);
+        if (kStagesA == 1) __syncthreads();  // every wave has read the slice before
+        const bool inside = k_begin + slice * 128 + load_col < k_end;
+#pragma unroll
+        for (int i = 0; i < kPasses; ++i)
+            *reinterpret_cast<u32x4*>(stage_a + a_stage_row[i] * kStageRow + load_col * 2) =
+                inside ? now.a[i] : u32x4{0u, 0u, 0u, 0u};
+        fetch(ahead, slice + DIST);
+        u32x4 bt[NT][4];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {  // through the wave's staging area (its LDS operations keep their order)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<u32x4*>(stage_w + (i * 4 + load_row) * kStageRow + load_col * 2) = now.w[t][i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bt[t][j] = *reinterpret_cast<const u32x4*>(stage_w + r * kStageRow + j * 64 + g * 16);
+        }
+        __syncthreads();  // the slice of A is in LDS
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (mt >= row_tiles_used) break;  // uniform
+            u32x4 av[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                av[j] = *reinterpret_cast<const u32x4*>(stage_a + (mt * 16 + r) * kStageRow + j * 64 + g * 16);
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, av[j]), __builtin_bit_cast(bf16x8, bt[t][j]), acc[mt][t], 0, 0, 0);
+        }
+    };
+
+    // Rows that still lack their 1/rms: a few lanes sum a row's partial sums.  Their loads are issued
+    // before the first loads of the product and summed behind them, so that the wait is for them alone
+    // (a loop of load and add here would stand a row's whole latency chain before the first slice).
+    const bool scaled_rows = EPI == EPI_SILU && a.row_sumsq != nullptr;
+    constexpr int kPerRowAny = kThreads / kRows;
+    constexpr int kPerRow = kPerRowAny >= 8 ? 8 : kPerRowAny >= 4 ? 4 : kPerRowAny >= 2 ? 2 : 1;  // lanes per row
+    constexpr int kHeld = 16;  // float4 loads a lane has under way at once
+    const int scale_row = threadIdx.x / kPerRow, scale_sub = threadIdx.x % kPerRow;
+    const bool scale_lane = scaled_rows && scale_row < kRows;
+    const bool scale_by_four = scaled_rows && a.sumsq_parts % 4 == 0 && a.sumsq_parts >= 4;
+    const float* scale_from = scaled_rows ? a.row_sumsq + static_cast<size_t>(min(scale_row, a.M - 1)) * a.sumsq_parts : nullptr;
+    float4 held[kHeld];
+    if (scale_by_four) {
+#pragma unroll
+        for (int i = 0; i < kHeld; ++i)  // (past the end: the last four again, not added below)
+            held[i] = *reinterpret_cast<const float4*>(scale_from + min((scale_sub + i * kPerRow) * 4, a.sumsq_parts - 4));
+    }
+    fetch(ring0, 0);
+    if (DIST > 1) fetch(ring1, 1);
+    if (scaled_rows) {
+        float sq = 0.f;
+        if (scale_by_four) {
+#pragma unroll
+            for (int i = 0; i < kHeld; ++i)
+                if ((scale_sub + i * kPerRow) * 4 < a.sumsq_parts) sq += (held[i].x + held[i].y) + (held[i].z + held[i].w);
+            for (int p = (scale_sub + kHeld * kPerRow) * 4; p < a.sumsq_parts; p += kPerRow * 4) {  // (a very wide model)
+                const float4 v = *reinterpret_cast<const float4*>(scale_from + p);
+                sq += (v.x + v.y) + (v.z + v.w);
+            }
+        } else {
+            for (int p = scale_sub; p < a.sumsq_parts; p += kPerRow) sq += scale_from[p];
+        }
+#pragma unroll
+        for (int offset = kPerRow / 2; offset > 0; offset >>= 1) sq += __shfl_xor(sq, offset, kWave);
+        if (scale_lane && scale_sub == 0) scale_lds[scale_row] = 1.0f / sqrtf(sq / static_cast<float>(a.K) + a.eps);
+    }
+    // (whole turns of the ring: a step past the last slice multiplies zeros)
+#pragma unroll 1
+    for (int base = 0; base < slices; base += kRing) {
+        if constexpr (DIST == 1) {
+            step(ring0, ring1, base);
+            step(ring1, ring0, base + 1);
+        } else {
+            step(ring0, ring2, base);
+            step(ring1, ring0, base + 1);
+            step(ring2, ring1, base + 2);
+        }
+    }
+    if (scaled_rows && slices == 0) __syncthreads();  // (the scales, if no step stood between)
+
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        if (mt >= row_tiles_used) break;
+        if (EPI == EPI_SILU) {
+            float row_scale[4] = {1.f, 1.f, 1.f, 1.f};
+            if (scaled_rows) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) row_scale[i] = scale_lds[mt * 16 + g * 4 + i];
+            }
+            if (tile_first * 16 < cols)  // wave-uniform
+                store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], mt * 16, tile_first * 16 + r, tile_first, lane, row_scale);
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                if ((tile_first + t) * 16 < cols)  // wave-uniform
+                    store_tile<EPI>(a, acc[mt][t], acc[mt][t], mt * 16, (tile_first + t) * 16 + r, tile_first + t, lane);
+        }
+    }
+}
+
+template <int EPI, int NT, int DIST, int WAVES>
+int launch_shared_rows_waves(hipStream_t s, int k_parts, const FusedArgs& a) {
+    const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
+    const int tiles = (cols + 15) / 16;
+    const int per_workgroup = WAVES * ((EPI == EPI_SILU) ? 1 : NT);
+    const dim3 grid((tiles + per_workgroup - 1) / per_workgroup, 1, k_parts);
+    if (a.M <= 32)
+        gemm_shared_rows_kernel<EPI, 2, NT, DIST, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
+    else if (a.M <= 64)
+        gemm_shared_rows_kernel<EPI, 4, NT, DIST, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
+    else
+        gemm_shared_rows_kernel<EPI, 8, NT, DIST, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
+    return cie_after_launch();
+}
+
+template <int EPI, int NT, int DIST>
+int launch_shared_rows(hipStream_t s, int waves, int k_parts, const FusedArgs& a) {
+    switch (waves) {
+        case 2: return launch_shared_rows_waves<EPI, NT, DIST, 2>(s, k_parts, a);
+        case 3: return launch_shared_rows_waves<EPI, NT, DIST, 3>(s, k_parts, a);
+        case 4: return launch_shared_rows_waves<EPI, NT, DIST, 4>(s, k_parts, a);
+    }
+    return CIE_BAD_ARGUMENT;
+}
+
 }  // namespace
 
 // epilogue: 0 bf16, 1 float32, 2 SiLU-gate (W = [gate rows; up rows], N = 2 * outputs), 3 residual
@@ -698,4 +915,54 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
     if (M <= 16) return launch_waves<EPI_ROPE, 1, 2>(s, waves, grid, f);
     if (M <= 32) return launch_waves<EPI_ROPE, 2, 2>(s, waves, grid, f);
     return launch_waves<EPI_ROPE, 4, 2>(s, waves, grid, f);
+}
+
+// The form for 17 to 128 rows in which a workgroup's four waves own columns and share the rows of A
+// through LDS (one workgroup row: M <= 128).  epilogue 0 (bf16, + bias), 2 (SiLU-gate; row_sumsq as in
+// cie_gemm_fused, for any number of rows here) or 4 (k_parts partial products).  column_tiles 1 or 2 tiles of
+// 16 columns per wave (SiLU: the gate tile and its up tile), 2 to 4 waves per workgroup; distance 1 or 2
+// slices of 128 k that a wave's loads run ahead.
+CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const void* w, const void* bias, void* c, int M,
+                                 int N, int K, int epilogue, int column_tiles, int waves, int k_parts, int distance,
+                                 const float* row_sumsq, int sumsq_parts, float eps) {
+    if (M <= 0 || M > 128 || N <= 0 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
+    if (epilogue != EPI_BF16 && epilogue != EPI_SILU && epilogue != EPI_PARTIAL) return CIE_BAD_ARGUMENT;
+    if (epilogue == EPI_SILU && (N % 2 || bias || column_tiles != 2)) return CIE_BAD_ARGUMENT;
+    if (column_tiles != 1 && column_tiles != 2) return CIE_BAD_ARGUMENT;
+    if (distance != 1 && distance != 2) return CIE_BAD_ARGUMENT;
+    if (k_parts < 1 || k_parts > 64 || (k_parts > 1 && epilogue != EPI_PARTIAL)) return CIE_BAD_ARGUMENT;
+    if (row_sumsq && (epilogue != EPI_SILU || sumsq_parts < 1 || !(eps > 0.f))) return CIE_BAD_ARGUMENT;
+    FusedArgs f;
+    f.a = static_cast<const bf16_t*>(a);
+    f.lda = lda;
+    f.w = static_cast<const bf16_t*>(w);
+    f.bias = static_cast<const bf16_t*>(bias);
+    f.c = c;
+    f.residual = nullptr;
+    f.sumsq = nullptr;
+    f.M = M;
+    f.N = N;
+    f.K = K;
+    f.up_offset = (epilogue == EPI_SILU) ? N / 2 : 0;
+    f.k_per_part = ((K + k_parts - 1) / k_parts + 127) / 128 * 128;
+    f.norm_weight = nullptr;
+    f.scaled_out = nullptr;
+    f.row_sumsq = row_sumsq;
+    f.sumsq_parts = sumsq_parts;
+    f.eps = eps;
+    f.rope = RopeArgs{};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool far = distance == 2;
+    switch (epilogue) {
+        case EPI_SILU:
+            return far ? launch_shared_rows<EPI_SILU, 2, 2>(s, waves, 1, f) : launch_shared_rows<EPI_SILU, 2, 1>(s, waves, 1, f);
+        case EPI_BF16:
+            if (column_tiles == 2) return far ? launch_shared_rows<EPI_BF16, 2, 2>(s, waves, 1, f) : launch_shared_rows<EPI_BF16, 2, 1>(s, waves, 1, f);
+            return far ? launch_shared_rows<EPI_BF16, 1, 2>(s, waves, 1, f) : launch_shared_rows<EPI_BF16, 1, 1>(s, waves, 1, f);
+        case EPI_PARTIAL:
+            if (column_tiles == 2)
+                return far ? launch_shared_rows<EPI_PARTIAL, 2, 2>(s, waves, k_parts, f) : launch_shared_rows<EPI_PARTIAL, 2, 1>(s, waves, k_parts, f);
+            return far ? launch_shared_rows<EPI_PARTIAL, 1, 2>(s, waves, k_parts, f) : launch_shared_rows<EPI_PARTIAL, 1, 1>(s, waves, k_parts, f);
+    }
+    return CIE_BAD_ARGUMENT;
 }

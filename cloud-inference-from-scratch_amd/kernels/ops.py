@@ -519,6 +519,61 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
     return out
 
 
+SHARED_ROWS_MAX = 128  # rows of the form whose waves share the rows of A
+
+
+def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                     column_tiles: int = 2, waves: int = 4, k_parts: int = 1, distance: int = 1,
+                     row_sumsq: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+    """``a @ weight.T`` for 17 to 128 rows (it takes fewer too) in the form whose four waves per
+    workgroup own columns and share each slice of ``a`` through LDS: ``EPI_BF16`` (+ bias),
+    ``EPI_SILU`` (weight = gate rows over up rows; with ``row_sumsq`` and ``eps`` the rows of ``a``
+    lack their ``rsqrt(mean square + eps)``, as in :func:`gemm_fused`) or ``EPI_PARTIAL``
+    (``k_parts`` float32 partial products [k_parts, M, N], bias in part 0).  ``column_tiles``
+    tiles of 16 columns per wave, loads ``distance`` slices of 128 k ahead."""
+    _gpu("weight", weight, torch.bfloat16, 2)
+    n, k = weight.shape
+    if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
+        raise ValueError("a must be a bf16 GPU matrix with unit inner stride")
+    m = a.shape[0]
+    if not (1 <= m <= SHARED_ROWS_MAX and a.shape[1] == k):
+        raise ValueError(f"a {tuple(a.shape)} vs K={k} and at most {SHARED_ROWS_MAX} rows")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    if not (k % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
+        raise ValueError(f"K and the row stride must be multiples of 8 (are {k}, {lda}) and the operands 16-byte aligned")
+    if epilogue not in (EPI_BF16, EPI_SILU, EPI_PARTIAL):
+        raise ValueError(f"epilogue {epilogue} is not one this form has")
+    if not (1 <= k_parts <= 64 and (k_parts == 1 or epilogue == EPI_PARTIAL)):
+        raise ValueError(f"k_parts {k_parts} does not fit the epilogue")
+    if epilogue == EPI_SILU:
+        column_tiles = 2
+        if n % 2 or bias is not None:
+            raise ValueError("the SiLU epilogue needs an even N and no bias")
+    if column_tiles not in (1, 2) or distance not in (1, 2) or waves not in (2, 3, 4):
+        raise ValueError(f"column_tiles {column_tiles} / distance {distance} not in (1, 2), or waves {waves} not in (2, 3, 4)")
+    if bias is not None:
+        _gpu("bias", bias, torch.bfloat16, 1)
+        if bias.shape[0] != n:
+            raise ValueError(f"bias must be [{n}]")
+    parts_in = 0
+    if row_sumsq is not None:
+        _gpu("row_sumsq", row_sumsq, torch.float32, 2)
+        if not (epilogue == EPI_SILU and row_sumsq.shape[0] >= m and eps > 0):
+            raise ValueError("rows that lack their scale go to the SiLU epilogue, with a positive eps")
+        parts_in = row_sumsq.shape[1]
+    device = weight.device
+    if epilogue == EPI_BF16:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    elif epilogue == EPI_SILU:
+        out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=device)
+    else:
+        out = torch.empty((k_parts, m, n), dtype=torch.float32, device=device)
+    _run("cie_gemm_shared_rows", load_library().cie_gemm_shared_rows(
+        _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k), _i(epilogue),
+        _i(column_tiles), _i(waves), _i(k_parts), _i(distance), _ptr(row_sumsq), _i(parts_in), _f(eps)))
+    return out
+
+
 _WORKSPACES: dict[torch.device, torch.Tensor] = {}
 LIBRARY_WORKSPACE_BYTES = 64 << 20
 # Products of at least this many rows, in steps of 256 (full prompt portions), and of a power of two of rows

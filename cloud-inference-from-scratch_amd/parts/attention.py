@@ -118,6 +118,7 @@ SPLIT_MIN_KEYS = 32  # the fewest keys of a one-wave part
 SPLIT_DECODE_KEYS = 192  # contexts from which the keys of decode rows are cut into parts at all
 JOINED_DECODE_ROWS = 32  # up to this many single-token sequences beside prompt portions ride in the prompt form's launch
 PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's keys are cut
+PROMPT_TARGET_WORKGROUPS = 256  # workgroups that cutting a prompt form's keys aims at
 # Tiles of 128 rows x kv heads from which prompt portions take the form of eight waves: enough to give most
 # compute units a workgroup without cutting the keys (whose parts, 64 KB of sums per tile and kv head, cost that
 # form more than they gain it: 512 tokens behind 1,536 keys, 7B heads, 60 us in two parts against 40 us in the form
@@ -256,7 +257,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     if n_tiles:
         # few tiles and many keys: parts of the keys, about as many workgroups as compute units
         n_splits, per_split, part_o, part_ml = 1, 0, None, None
-        wanted = min(cuts, int(256 / (n_tiles * num_kv_heads) + 0.5))
+        wanted = min(cuts, int(PROMPT_TARGET_WORKGROUPS / (n_tiles * num_kv_heads) + 0.5))
         if wanted > 1:
             per_split = -(-(-(-max_keys // wanted)) // 128) * 128
             n_splits = -(-max_keys // per_split)

@@ -3,9 +3,12 @@
 float32: the hand-written true-float32 kernel, always.  bfloat16 with up to
 ``FUSED_ROWS`` rows (decode steps, the output head), and up to 64 or 128 rows where
 it is the faster one (a small weight, a long K): the hand-written
-matrix-core kernel that streams the weight once and takes over its neighbours'
+matrix-core kernels that stream the weight once and take over their neighbours'
 work: a SiLU-gate behind (``epilogue="silu"``), the add into the float32
-residual stream (``into=residual``), or float32 results for the logits.
+residual stream (``into=residual``), or float32 results for the logits.  They
+come in two forms: waves that share K and own all rows (few rows; the q/k/v,
+o_proj and head products), and waves that own columns and share the rows through
+LDS (the SiLU-gate product up to 64 rows and every product whose K is cut).
 bfloat16 with more rows: the vendor library's product (hipBLASLt through a
 thin cached interface of this package), as the reference leaves its products to
 a library (src/cloud_engine/model.py:89-137), with the small kernels around it.
@@ -43,21 +46,46 @@ FUSED_SMALL_WEIGHT = 6 << 20
 # 64 rows; up to 64 rows it is one pass either way)
 FUSED_LOGIT_ROWS = 64
 # An ``into=`` product with fewer than this many 16-column tiles and a K of at least ``PART_MIN_K`` cuts K
-# into parts for more workgroups (partial products, summed by the next norm kernel).
+# into parts for more workgroups (partial products, summed by the next norm kernel; ``plan_shared_parts``).
 PART_BELOW_TILES = 512
 PART_MIN_K = 4096
-PART_WORKGROUPS = 512   # column tiles x parts that a cut aims for at least
-PART_K = 4096           # ... and the longest stretch of K a part takes
+PART_K = 1024           # the shortest stretch of K a part takes
 
 
-def plan_k_parts(tiles: int, k: int) -> int:
-    """Into how many parts the K of an ``into=`` product with ``tiles`` column tiles is cut: enough for
-    ``PART_WORKGROUPS`` workgroups, and no part longer than ``PART_K``.  Measured at 8 rows with the weight
-    coming from memory (down products; microseconds for 2 / 4 / 8 parts): 128 tiles, K 11,008: 12.7 / 11.8 /
-    11.9 (here 4); 224 tiles, K 18,944: 32.7 / 31.1 / 29.3 (here 5); 320 tiles, K 13,824: 33.4 / 29.7 / 29.8
-    (here 4).  More parts cost the norm kernel that adds them as much as they gain the product."""
-    parts = max(-(-PART_WORKGROUPS // max(tiles, 1)), -(-k // PART_K))
-    return max(1, min(parts, 16, -(-k // 128)))  # (the kernel cuts K in steps of 128)
+# SiLU-gate products of up to this many rows take the form whose waves own columns and share the rows of A
+# through LDS (gate/up of the 3B shape at 32 / 64 rows: 21 / 24 us against the library's 26 / 27 us and 5 us
+# for the SiLU kernel behind it; 14B: 50 / 56 against 55 / 62 + 6; 7B: level); from 65 rows on the library is
+# level or ahead (3B at 128 rows: 34 against 30 + 5 us).
+SHARED_SILU_ROWS = 64
+COMPUTE_UNITS = 256
+
+
+def plan_shared_silu(pairs: int) -> tuple[int, bool]:
+    """Waves per workgroup (each wave takes one gate tile and its up tile) for the shared-rows SiLU product,
+    and whether every workgroup then has a compute unit of its own.  A compute unit streams at most some
+    30 GB/s however many loads it has under way, so what counts is the most pairs that meet on one unit:
+    workgroups of four waves, or of three where that needs fewer turns (688 pairs of the 3B shape: 172
+    workgroups of four or 230 of three, one turn each; 1,184 of the 7B shape: two turns of four waves or
+    two of three, 70 against 61 us at 64 rows; 864 of the 14B shape: one turn of four, 56 against 81 us)."""
+    best = None
+    for waves in (4, 3, 2):
+        turns = -(-(-(-pairs // waves)) // COMPUTE_UNITS)
+        if best is None or turns * waves < best[0]:
+            best = (turns * waves, waves, turns == 1)
+    return best[1], best[2]
+
+
+def plan_shared_parts(tiles: int, k: int) -> tuple[int, int, int]:
+    """(column tiles per wave, waves, parts of K) of a cut product in the shared-rows form: workgroups of four
+    waves, one tile of 16 columns per wave (two for a wide result), and as many parts as give about one
+    workgroup per compute unit.  Measured at 8 / 64 rows (us; the form of waves that share K, at its best
+    cut, beside it): 128 tiles, K 11,008: 8 parts 11.0 / 14.8 (13.2 / 17.7); 224 tiles, K 18,944: 4 parts
+    26.1 / 35.3 (29.7 / 43.8); 320 tiles, K 13,824, two tiles per wave: 4 parts 28.6 / 38.7 (30.0 / 44.0)."""
+    column_tiles = 1 if tiles <= COMPUTE_UNITS else 2
+    waves = 4
+    blocks = -(-tiles // (column_tiles * waves))
+    parts = max(1, min(COMPUTE_UNITS // blocks, 16, k // PART_K))
+    return column_tiles, waves, parts
 
 
 @dataclass
@@ -139,8 +167,12 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     if isinstance(x, ScaledRows):
         rows, k = x.rows.shape
         if epilogue == "silu" and weight.shape[0] % 2 == 0 and bias is None and weight.dtype == torch.bfloat16:
-            if rows <= FUSED_ROWS and _fusable(rows, k, x.rows.stride(0) if rows > 1 else k, weight):
-                return ops.gemm_fused(weight, ops.EPI_SILU, x.rows, row_sumsq=x.sumsq, eps=x.eps)
+            if _fusable(rows, k, x.rows.stride(0) if rows > 1 else k, weight):
+                waves, own_unit = plan_shared_silu(-(-weight.shape[0] // 32))
+                if FUSED_ROWS < rows <= SHARED_SILU_ROWS or (rows <= FUSED_ROWS and own_unit):
+                    return ops.gemm_shared_rows(weight, ops.EPI_SILU, x.rows, waves=waves, row_sumsq=x.sumsq, eps=x.eps)
+                if rows <= FUSED_ROWS:
+                    return ops.gemm_fused(weight, ops.EPI_SILU, x.rows, row_sumsq=x.sumsq, eps=x.eps)
             # more rows: the library's product of the rows as they are, the scale in the SiLU kernel behind it
             out = ops.gemm_library(x.rows, weight) if x.rows.stride(1) == 1 else None
             if out is not None:
@@ -155,7 +187,13 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     fusable = _fusable(rows, k, x.stride(0) if rows > 1 else k, weight)
     cut_k = into is not None and -(-n // 16) < PART_BELOW_TILES and k >= PART_MIN_K
     if fusable and cut_k and rows <= (FUSED_PARTS_ROWS_NARROW if -(-n // 16) < PARTS_NARROW_TILES else FUSED_PARTS_ROWS):
-        return PartialSum(ops.gemm_fused(weight, ops.EPI_PARTIAL, x, bias=bias, k_parts=plan_k_parts(-(-n // 16), k)))
+        column_tiles, waves, parts = plan_shared_parts(-(-n // 16), k)
+        return PartialSum(ops.gemm_shared_rows(weight, ops.EPI_PARTIAL, x, bias=bias, column_tiles=column_tiles,
+                                               waves=waves, k_parts=parts))
+    if fusable and silu and n % 2 == 0 and bias is None and into is None and not wants_f32 and rows <= SHARED_SILU_ROWS:
+        waves, own_unit = plan_shared_silu(-(-n // 32))
+        if rows > FUSED_ROWS or own_unit:
+            return ops.gemm_shared_rows(weight, ops.EPI_SILU, x, waves=waves)
     if fusable and wants_f32 and rows > FUSED_LOGIT_ROWS and into is None and not silu and bias is None:
         out = ops.gemm_library(x, weight, out_dtype=torch.float32)  # logits of many rows: one pass over the weight
         if out is not None:

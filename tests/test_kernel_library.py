@@ -61,16 +61,21 @@ def test_the_fallback_build_folder_must_be_this_users_own(tmp_path, monkeypatch)
     assert folder not in library._build_dirs()
 
 
-def test_k_parts_follow_tiles_and_k():
-    """The cut of a long K: enough parts for 512 workgroups, no part longer than 4,096, never more parts than
-    K has slices of 128; the shapes that were measured keep their measured choice."""
-    from cie_amd.parts.linear import plan_k_parts
+def test_cut_products_and_silu_products_plan_by_compute_units():
+    """The cut of a long K: workgroups of four waves, about one for each compute unit, no part shorter than
+    ``PART_K``; the SiLU product: the fewest pairs of tiles that meet on one compute unit.  The shapes that were
+    measured keep their measured choice."""
+    from cie_amd.parts.linear import plan_shared_parts, plan_shared_silu
 
-    assert plan_k_parts(128, 11008) == 4      # the 3B down product
-    assert plan_k_parts(224, 18944) == 5      # 7B
-    assert plan_k_parts(320, 13824) == 4      # 14B
-    assert plan_k_parts(6, 328) == 3 and plan_k_parts(3, 88) == 1
-    assert plan_k_parts(500, 4096) == 2 and plan_k_parts(1, 1 << 20) == 16
+    assert plan_shared_parts(128, 11008) == (1, 4, 8)     # the 3B down product
+    assert plan_shared_parts(224, 18944) == (1, 4, 4)     # 7B
+    assert plan_shared_parts(320, 13824) == (2, 4, 6)     # 14B
+    assert plan_shared_parts(6, 328) == (1, 4, 1) and plan_shared_parts(3, 4096) == (1, 4, 4)
+    assert plan_shared_parts(500, 1 << 20) == (2, 4, 4) and plan_shared_parts(1, 1 << 20) == (1, 4, 16)
+    assert plan_shared_silu(688) == (3, True)      # 3B: 230 workgroups of three waves
+    assert plan_shared_silu(1184) == (3, False)    # 7B: two turns either way, three waves are less per turn
+    assert plan_shared_silu(864) == (4, True)      # 14B: 216 workgroups of four
+    assert plan_shared_silu(1) == (2, True)        # a narrow one: no idle waves
 
 
 def test_a_widened_head_is_made_once_and_let_go_with_its_weight():
