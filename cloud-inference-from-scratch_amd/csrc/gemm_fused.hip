@@ -611,7 +611,7 @@ int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, int k_part
 // addresses by constants (a copy from a set whose load is still under way would wait for it).
 template <int EPI, int MT, int NT, int DIST, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs a) {
-    static_assert(EPI == EPI_SILU || EPI == EPI_PARTIAL || EPI == EPI_BF16, "epilogues of this form");
+    static_assert(EPI == EPI_SILU || EPI == EPI_PARTIAL || EPI == EPI_BF16 || EPI == EPI_F32, "epilogues of this form");
     static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
     constexpr int kWaves = WAVES;
     constexpr int kThreads = WAVES * 64;
@@ -918,7 +918,8 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
 }
 
 // The form for 17 to 128 rows in which a workgroup's four waves own columns and share the rows of A
-// through LDS (one workgroup row: M <= 128).  epilogue 0 (bf16, + bias), 2 (SiLU-gate; row_sumsq as in
+// through LDS (one workgroup row: M <= 128).  epilogue 0 (bf16, + bias), 1 (float32, + bias; two tiles a wave,
+// distance 1), 2 (SiLU-gate; row_sumsq as in
 // cie_gemm_fused, for any number of rows here) or 4 (k_parts partial products).  column_tiles 1 or 2 tiles of
 // 16 columns per wave (SiLU: the gate tile and its up tile), 2 to 4 waves per workgroup; distance 1 or 2
 // slices of 128 k that a wave's loads run ahead.
@@ -926,7 +927,7 @@ CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const voi
                                  int N, int K, int epilogue, int column_tiles, int waves, int k_parts, int distance,
                                  const float* row_sumsq, int sumsq_parts, float eps) {
     if (M <= 0 || M > 128 || N <= 0 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
-    if (epilogue != EPI_BF16 && epilogue != EPI_SILU && epilogue != EPI_PARTIAL) return CIE_BAD_ARGUMENT;
+    if (epilogue != EPI_BF16 && epilogue != EPI_F32 && epilogue != EPI_SILU && epilogue != EPI_PARTIAL) return CIE_BAD_ARGUMENT;
     if (epilogue == EPI_SILU && (N % 2 || bias || column_tiles != 2)) return CIE_BAD_ARGUMENT;
     if (column_tiles != 1 && column_tiles != 2) return CIE_BAD_ARGUMENT;
     if (distance != 1 && distance != 2) return CIE_BAD_ARGUMENT;
@@ -959,6 +960,9 @@ CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const voi
         case EPI_BF16:
             if (column_tiles == 2) return far ? launch_shared_rows<EPI_BF16, 2, 2>(s, waves, 1, f) : launch_shared_rows<EPI_BF16, 2, 1>(s, waves, 1, f);
             return far ? launch_shared_rows<EPI_BF16, 1, 2>(s, waves, 1, f) : launch_shared_rows<EPI_BF16, 1, 1>(s, waves, 1, f);
+        case EPI_F32:  // (the logits: two tiles a wave, loads one slice ahead)
+            if (column_tiles != 2 || far) return CIE_BAD_ARGUMENT;
+            return launch_shared_rows<EPI_F32, 2, 1>(s, waves, 1, f);
         case EPI_PARTIAL:
             if (column_tiles == 2)
                 return far ? launch_shared_rows<EPI_PARTIAL, 2, 2>(s, waves, k_parts, f) : launch_shared_rows<EPI_PARTIAL, 2, 1>(s, waves, k_parts, f);

@@ -526,7 +526,7 @@ def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias:
                      column_tiles: int = 2, waves: int = 4, k_parts: int = 1, distance: int = 1,
                      row_sumsq: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
     """``a @ weight.T`` for 17 to 128 rows (it takes fewer too) in the form whose four waves per
-    workgroup own columns and share each slice of ``a`` through LDS: ``EPI_BF16`` (+ bias),
+    workgroup own columns and share each slice of ``a`` through LDS: ``EPI_BF16`` or ``EPI_F32`` (+ bias),
     ``EPI_SILU`` (weight = gate rows over up rows; with ``row_sumsq`` and ``eps`` the rows of ``a``
     lack their ``rsqrt(mean square + eps)``, as in :func:`gemm_fused`) or ``EPI_PARTIAL``
     (``k_parts`` float32 partial products [k_parts, M, N], bias in part 0).  ``column_tiles``
@@ -541,8 +541,10 @@ def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias:
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
     if not (k % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         raise ValueError(f"K and the row stride must be multiples of 8 (are {k}, {lda}) and the operands 16-byte aligned")
-    if epilogue not in (EPI_BF16, EPI_SILU, EPI_PARTIAL):
+    if epilogue not in (EPI_BF16, EPI_F32, EPI_SILU, EPI_PARTIAL):
         raise ValueError(f"epilogue {epilogue} is not one this form has")
+    if epilogue == EPI_F32:
+        column_tiles, distance = 2, 1
     if not (1 <= k_parts <= 64 and (k_parts == 1 or epilogue == EPI_PARTIAL)):
         raise ValueError(f"k_parts {k_parts} does not fit the epilogue")
     if epilogue == EPI_SILU:
@@ -564,6 +566,8 @@ def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias:
     device = weight.device
     if epilogue == EPI_BF16:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
+    elif epilogue == EPI_F32:
+        out = torch.empty((m, n), dtype=torch.float32, device=device)
     elif epilogue == EPI_SILU:
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=device)
     else:

@@ -194,6 +194,9 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
         waves, own_unit = plan_shared_silu(-(-n // 32))
         if rows > FUSED_ROWS or own_unit:
             return ops.gemm_shared_rows(weight, ops.EPI_SILU, x, waves=waves)
+    if fusable and wants_f32 and FUSED_ROWS < rows <= ops.SHARED_ROWS_MAX and into is None and not silu:
+        # logits of 17 to 128 rows: the shared-rows form (the 3B head at 64 rows: 170 -> ? us)
+        return ops.gemm_shared_rows(weight, ops.EPI_F32, x, bias=bias, waves=4)
     if fusable and wants_f32 and rows > FUSED_LOGIT_ROWS and into is None and not silu and bias is None:
         out = ops.gemm_library(x, weight, out_dtype=torch.float32)  # logits of many rows: one pass over the weight
         if out is not None:

@@ -865,6 +865,9 @@ def test_gemm_shared_rows_matches_float64(ops, shape, waves):
         for tiles in (1, 2):
             out = ops.gemm_shared_rows(w, ops.EPI_BF16, a, bias=b, column_tiles=tiles, waves=waves, distance=distance)
             torch.testing.assert_close(out.double(), expect + b.double(), **tol)
+            out = ops.gemm_shared_rows(w, ops.EPI_F32, a, bias=b, waves=waves)  # as for logits
+            assert out.dtype == torch.float32
+            torch.testing.assert_close(out.double(), expect + b.double(), rtol=1e-4, atol=1e-4 * math.sqrt(k))
             for parts in (1, 3, 7):
                 rows = wide[:, :k] if parts == 3 else a
                 out = ops.gemm_shared_rows(w, ops.EPI_PARTIAL, rows, bias=b, column_tiles=tiles, waves=waves,
