@@ -84,6 +84,14 @@ class Attention(Part):
         linear(blank(self.hidden_size), self.w_qkv, self.b_qkv)
         linear(blank(self.num_heads * self.head_dim), self.w_o, self.b_o)
 
+    def shape_projection(self, qkv: torch.Tensor, batch) -> torch.Tensor:
+        """The seam between projection and rotation: what a variant of this mixer does to the projected
+        rows ``[tokens, (query heads + 2 key heads) * head_dim]`` (bias added; queries first, then keys,
+        then values) before they are rotated and the keys and values go to the cache, such as a norm over
+        each query and key head.  The default does nothing, and only a mixer that leaves it so lets the
+        projection's own kernel rotate and write the cache."""
+        return qkv
+
     def forward(self, x, batch, view, writes: bool = True, residual: Optional[torch.Tensor] = None,
                 next_norm=None):
         if batch.max_context > self.position.max_position and self.position.rotates:
@@ -92,7 +100,8 @@ class Attention(Part):
             )
         rows = x.shape[0]
         few = rows <= FUSED_ROWS or (rows <= FUSED_SMALL_ROWS and self.w_qkv.numel() <= FUSED_SMALL_WEIGHT)
-        if (x.dtype == torch.bfloat16 and few and self.head_dim % 32 == 0
+        untouched = type(self).shape_projection is Attention.shape_projection
+        if (x.dtype == torch.bfloat16 and few and untouched and self.head_dim % 32 == 0
                 and x.shape[1] % 8 == 0 and (rows == 1 or x.stride(0) % 8 == 0)):
             # few rows (where the hand-written product is the faster one): its epilogue rotates and writes the cache
             qkv = ops.gemm_qkv_rope(self.w_qkv, x, self.b_qkv, self.cos, self.sin, batch.positions,
@@ -100,7 +109,7 @@ class Attention(Part):
                                     self.num_heads, self.num_kv_heads, self.head_dim,
                                     rotate=self.position.rotates, write_kv=writes)
         else:
-            qkv = linear(x, self.w_qkv, self.b_qkv)
+            qkv = self.shape_projection(linear(x, self.w_qkv, self.b_qkv), batch)
             ops.rope_kv_write(qkv, self.cos, self.sin, batch.positions, batch.seq_of_token, batch.seq_slot,
                               view.block_table, view.k_pool, view.v_pool, self.num_heads, self.num_kv_heads,
                               self.head_dim, rotate=self.position.rotates, write_kv=writes)

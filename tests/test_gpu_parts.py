@@ -176,6 +176,54 @@ def test_attention_part_whole_and_in_portions(dtype, rotary):
     check(torch.cat([first, second, third, fourth]).float().cpu(), expected[1], dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_mixer_that_norms_its_heads_between_projection_and_rotation(dtype):
+    """The seam between projection and rotation: a variant of the attention mixer, defined here, that
+    divides every query and key head by its root mean square before the rotation overrides one method and
+    reuses the rest (with the projection's own rotation switched off for it).  Expected: the plain
+    functions composed with that norm, whole; the part runs a portion and then single tokens, 32-wide
+    heads (which the fused projection would otherwise take)."""
+    from cie_amd.config import PartSpec
+    from cie_amd.parts.attention import Attention
+
+    hidden, heads, kv_heads, head_dim, eps = 64, 4, 2, 32, 1e-5
+
+    def normed(rows_of_heads):
+        wide = rows_of_heads.float()
+        return wide * torch.rsqrt(wide.pow(2).mean(-1, keepdim=True) + eps)
+
+    class NormedHeads(Attention):
+        def shape_projection(self, qkv, batch):
+            rows = qkv.shape[0]
+            shaped = qkv.view(rows, heads + 2 * kv_heads, head_dim)
+            out = shaped.clone()
+            out[:, : heads + kv_heads] = normed(shaped[:, : heads + kv_heads]).to(qkv.dtype)
+            return out.view(rows, -1)
+
+    position = PartSpec.of("rotary_half", head_dim=head_dim, theta=1e4, max_position=128)
+    mixer = NormedHeads(hidden, heads, kv_heads, head_dim, qkv_bias=True, out_bias=False, position=position)
+    w = bound(mixer, "a.", dtype, 8, scale=0.3)
+    length = 27
+    manager, device_cache = harness([mixer.cache_need()], [length],
+                                    dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    x = torch.randn((length, hidden), generator=torch.Generator().manual_seed(9)).to(mixer.dtype)
+    cos, sin = plain.rope_tables(head_dim, length, 1e4)
+    positions = torch.arange(length)
+    proj = lambda name: plain.linear(x.float(), w[f"a.{name}.weight"], w[f"a.{name}.bias"]).view(length, -1, head_dim)
+    q = plain.apply_rope(normed(proj("q_proj")), cos, sin, positions)
+    k = plain.apply_rope(normed(proj("k_proj")), cos, sin, positions)
+    context = plain.causal_attention(q, k, proj("v_proj"), 1.0 / math.sqrt(head_dim))
+    expected = plain.linear(context, w["a.o_proj.weight"])
+    view = device_cache.view(0)
+    first = mixer.forward(x[:12].cuda(), batch_of(manager, [(0, 0, 12)]), view)
+    manager.commit_lengths({"r0": 12})
+    rest = []
+    for at in range(12, length):
+        rest.append(mixer.forward(x[at:at + 1].cuda(), batch_of(manager, [(0, at, 1)]), view))
+        manager.commit_lengths({"r0": at + 1})
+    check(torch.cat([first, *rest]).float().cpu(), expected, dtype)
+
+
 @pytest.mark.parametrize("part_k", [None, 32])
 @pytest.mark.parametrize("rows", [13, 40, 72, 100])
 @pytest.mark.parametrize("dtype", DTYPES)
