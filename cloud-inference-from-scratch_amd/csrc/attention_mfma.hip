@@ -67,6 +67,14 @@ __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs 
         }
         range_begin += split * per_split;
         range_end = min(hi, range_begin + per_split);
+        if (range_begin >= range_end) {  // no keys in this share: its statistics say so, its sums are never read
+            float* pml = a.part_ml + ((static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + split) * ROWS * 2;
+            if (lane < ROWS) {
+                pml[lane * 2] = -INFINITY;
+                pml[lane * 2 + 1] = 0.f;
+            }
+            return;
+        }
     }
 
     // Q fragments (B operand) and each lane's row facts
@@ -220,6 +228,7 @@ __global__ void __launch_bounds__(64) paged_attention_mfma_kernel(AttentionArgs 
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int row = rt * 16 + g * 4 + i;
+                if (row >= n_rows) continue;  // (the merge reads the tile's own rows only)
 #pragma unroll
                 for (int dt = 0; dt < ND; ++dt) po[static_cast<size_t>(row) * D + dt * 16 + r] = o[rt][dt][i];
             }
@@ -289,6 +298,7 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
     const int start = a.seq_start[seq];
     const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
     const int n_rows = n_tok * group;
+    const int rt_used = (n_rows + 15) / 16;  // row tiles that hold a row at all (a single token beside portions: one)
     const int first_row_token = a.q_start_loc[seq] + q0;
     const int page_mask = (1 << a.page_shift) - 1;
     const int* table = a.block_table + static_cast<size_t>(a.seq_slot[seq]) * a.table_width;
@@ -306,6 +316,14 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
         }
         range_begin += blockIdx.y * per_split;
         range_end = min(hi, range_begin + per_split);
+        if (range_begin >= range_end) {  // no keys in this share: its statistics say so, its sums are never read
+            float* pml = a.part_ml + ((static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + blockIdx.y) * ROWS * 2;
+            if (threadIdx.x < ROWS) {
+                pml[threadIdx.x * 2] = -INFINITY;
+                pml[threadIdx.x * 2 + 1] = 0.f;
+            }
+            return;  // (the whole workgroup: the range is the same for all its waves)
+        }
     }
     const int first_pos = start + q0;              // position of the tile's first token
     const int last_pos = start + q0 + n_tok - 1;   // and of its last
@@ -391,6 +409,7 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
+                if (rt >= rt_used) break;  // (the same for the whole workgroup)
                 floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int j = 0; j < NK; ++j)
@@ -409,6 +428,7 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
         bool moved = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
+            if (rt >= rt_used) break;
             if (edge) {
                 const int pos = row_pos[rt];
                 const int row_lo = (a.window > 0) ? pos + 1 - a.window : 0;
@@ -436,6 +456,7 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
             // the products that wrote these accumulators were issued a whole score phase ago
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
+                if (rt >= rt_used) break;
                 float alpha_o[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha[rt], g * 4 + i, kWave);
@@ -449,6 +470,7 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
         // ---- probabilities (one fused multiply-add and one exp2 each) and O += P . V, row tile by row tile
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
+            if (rt >= rt_used) break;
             float p_sum = 0.f;
             uint32_t pw[4];
 #pragma unroll
@@ -509,6 +531,7 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
     }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
+        if (rt >= rt_used) break;  // (no row of it exists: nothing to sum, nothing to store)
         const int owner = rt % WAVES;
         if (WAVES > 1) {
             float w_o[4];
@@ -549,6 +572,7 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int row = rt * 16 + g * 4 + i;
+                if (row >= n_rows) continue;  // (the merge reads the tile's own rows only)
 #pragma unroll
                 for (int dt = 0; dt < ND; ++dt) po[static_cast<size_t>(row) * D + dt * 16 + r] = o[rt][dt][i];
             }
@@ -626,10 +650,11 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
 #pragma unroll
         for (int u = 0; u < kEarly; ++u) {
             const int s = mine + u * groups;
-            if (s < a.n_splits) num += early[u] * weight[s];
+            if (s < a.n_splits && weight[s] != 0.f) num += early[u] * weight[s];  // (a share without keys wrote no sums)
         }
 #pragma unroll 4
-        for (int s = mine + kEarly * groups; s < a.n_splits; s += groups) num += po_row[s * stride] * weight[s];
+        for (int s = mine + kEarly * groups; s < a.n_splits; s += groups)
+            if (weight[s] != 0.f) num += po_row[s * stride] * weight[s];
     }
     group_sum[threadIdx.x] = num;
     __syncthreads();
