@@ -237,7 +237,8 @@ int fastest(const Plan& plan, const Found& found, int proposed, hipStream_t stre
     const int runs = many_rows ? 2 : 6;
     const int count = static_cast<int>(found.size());
     const bool every = count > proposed;
-    // three rounds: everything once; the best 32 of a long list twice more, in turn; the best few five times
+    // rounds: everything once; the best 32 of a long list twice more, in turn; the best eight five times; the
+    // best three twelve times
     constexpr int kMost = 32;
     const int wanted = every ? kMost : 4;
     int finalist[kMost + 1];
@@ -279,6 +280,10 @@ int fastest(const Plan& plan, const Found& found, int proposed, hipStream_t stre
         finalists = 8;
     }
     again(5);
+    if (finalists > 3) {  // the last few once more, longer: candidates within a few percent of each other change places
+        finalists = 3;
+        again(12);
+    }
     int best = 0;
     for (;;) {
         int at = -1;
