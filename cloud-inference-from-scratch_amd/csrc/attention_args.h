@@ -43,7 +43,14 @@ struct AttentionArgs {
     int xcds_per_head;  // prompt forms: > 0 if every kv head has that many of the kXcds XCDs (and their L2) to itself
     const int* max_context_dev;  // if set (a captured graph replays with other lengths): keys per split are
                                  // derived from this device value, the longest context of the step
+    int whole_in_first_share;    // with splits: a tile whose keys all lie in the first share writes its result
+                                 // itself and takes no part in the merge (the form of eight waves)
 };
+
+// Whether a tile that sees the keys [first_begin, hi) has them all in the first of its shares of per_split keys.
+__host__ __device__ inline bool all_in_first_share(int first_begin, int hi, int per_split) {
+    return hi <= first_begin + per_split;
+}
 
 // The prompt form of eight waves per 128-row tile (csrc/attention_prompt.hip); returns a CIE_* code.
 int launch_prompt_form(hipStream_t stream, const AttentionArgs& a, int head_dim);

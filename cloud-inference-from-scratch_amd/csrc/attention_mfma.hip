@@ -615,6 +615,17 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
     const int q0 = a.tile_seq ? a.tile_q0[tile] : 0;
     const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
     if (row >= n_tok * group) return;
+    if (a.whole_in_first_share) {  // a tile with all its keys in the first share has written its result itself
+        const int hi = a.seq_start[seq] + q0 + n_tok;
+        const int lo = (a.window > 0) ? max(0, a.seq_start[seq] + q0 + 1 - a.window) : 0;
+        int per_split = a.keys_per_split;
+        if (a.max_context_dev) {
+            int most = *a.max_context_dev;
+            if (a.window > 0) most = min(most, a.window + 2 * kKeysPerBlock);
+            per_split = ((most + a.n_splits - 1) / a.n_splits + kKeysPerBlock - 1) & ~(kKeysPerBlock - 1);
+        }
+        if (all_in_first_share(lo & ~(kKeysPerBlock - 1), hi, per_split)) return;
+    }
     const size_t unit0 = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits;
     const int per_row = head_dim / 4;            // threads that cover a row of sums
     const int groups = kMergeThreads / per_row;  // parts summed side by side
@@ -669,6 +680,77 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
     packed.x = from_float<bf16_t>(num[0] * inv).bits | (static_cast<uint32_t>(from_float<bf16_t>(num[1] * inv).bits) << 16);
     packed.y = from_float<bf16_t>(num[2] * inv).bits | (static_cast<uint32_t>(from_float<bf16_t>(num[3] * inv).bits) << 16);
     *reinterpret_cast<uint2*>(dst) = packed;
+}
+
+// The same merge for tiles of many rows and few shares (prompt portions whose keys are cut): a workgroup
+// takes 16 rows of a (tile, kv head), a thread four head dimensions at a time of one row; every thread
+// of a row makes the shares' weights for itself from the few statistics.  (With one workgroup for each row,
+// as above, a step of 2,048 tokens would start 32,768 workgroups.)
+constexpr int kMergeFewShares = 16;
+
+__global__ void __launch_bounds__(256)
+attention_merge_rows_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
+    const int tile = blockIdx.x;
+    const int kv_head = blockIdx.y;
+    const int row = blockIdx.z * 16 + threadIdx.x / 16;
+    const int lane16 = threadIdx.x % 16;
+    const int group = a.q_heads / a.kv_heads;
+    const int seq = a.tile_seq ? a.tile_seq[tile] : tile;
+    const int q0 = a.tile_seq ? a.tile_q0[tile] : 0;
+    const int n_tok = min(a.tokens_per_tile, a.seq_q_len[seq] - q0);
+    if (row >= n_tok * group) return;
+    if (a.whole_in_first_share) {  // a tile with all its keys in the first share has written its result itself
+        const int hi = a.seq_start[seq] + q0 + n_tok;
+        const int lo = (a.window > 0) ? max(0, a.seq_start[seq] + q0 + 1 - a.window) : 0;
+        int per_split = a.keys_per_split;
+        if (a.max_context_dev) {
+            int most = *a.max_context_dev;
+            if (a.window > 0) most = min(most, a.window + 2 * kKeysPerBlock);
+            per_split = ((most + a.n_splits - 1) / a.n_splits + kKeysPerBlock - 1) & ~(kKeysPerBlock - 1);
+        }
+        if (all_in_first_share(lo & ~(kKeysPerBlock - 1), hi, per_split)) return;
+    }
+    const size_t unit0 = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits;
+    float weight[kMergeFewShares];
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < kMergeFewShares; ++s) {
+        weight[s] = (s < a.n_splits) ? a.part_ml[((unit0 + s) * rows_per_tile + row) * 2] : -INFINITY;
+        m_all = fmaxf(m_all, weight[s]);
+    }
+    float den = 0.f;
+#pragma unroll
+    for (int s = 0; s < kMergeFewShares; ++s) {
+        const float w = (weight[s] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(weight[s] - m_all);  // maxima are kept in base 2
+        weight[s] = w;
+        if (s < a.n_splits) den += a.part_ml[((unit0 + s) * rows_per_tile + row) * 2 + 1] * w;
+    }
+    const float inv = 1.0f / den;
+    const int tok = row / group;
+    const int head = row - tok * group;
+    bf16_t* dst = a.out + static_cast<size_t>(a.q_start_loc[seq] + q0 + tok) * a.q_heads * head_dim +
+                  static_cast<size_t>(kv_head * group + head) * head_dim;
+    for (int d = lane16 * 4; d < head_dim; d += 64) {
+        floatx4 num = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < kMergeFewShares; ++s)
+            if (s < a.n_splits && weight[s] != 0.f)  // (a share without keys wrote no sums)
+                num += *reinterpret_cast<const floatx4*>(a.part_o + ((unit0 + s) * rows_per_tile + row) * head_dim + d) * weight[s];
+        uint2 packed;
+        packed.x = from_float<bf16_t>(num[0] * inv).bits | (static_cast<uint32_t>(from_float<bf16_t>(num[1] * inv).bits) << 16);
+        packed.y = from_float<bf16_t>(num[2] * inv).bits | (static_cast<uint32_t>(from_float<bf16_t>(num[3] * inv).bits) << 16);
+        *reinterpret_cast<uint2*>(dst + d) = packed;
+    }
+}
+
+// Which of the two merges a step's shape takes.
+int launch_merge(hipStream_t s, const AttentionArgs& a, int n_tiles, int head_dim, int rows_per_tile) {
+    const int rows = a.tokens_per_tile * (a.q_heads / a.kv_heads);
+    if (rows_per_tile >= kPromptTileRows && a.n_splits <= kMergeFewShares)  // (with fewer rows a tile the first is the faster one)
+        attention_merge_rows_kernel<<<dim3(n_tiles, a.kv_heads, (rows + 15) / 16), 256, 0, s>>>(a, head_dim, rows_per_tile);
+    else
+        attention_merge_kernel<<<dim3(n_tiles, a.kv_heads, rows), kMergeThreads, 0, s>>>(a, head_dim, rows_per_tile);
+    return cie_after_launch();
 }
 
 template <int D>
@@ -761,14 +843,14 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     a.keys_per_split = n_splits > 1 ? keys_per_split : 0;
     a.max_context_dev = n_splits > 1 ? max_context_dev : nullptr;
     a.n_tiles = n_tiles;
+    a.whole_in_first_share = (tile_waves == kPromptWaves && n_splits > 1) ? 1 : 0;
     a.xcds_per_head = (kv_heads <= kXcds && kXcds % kv_heads == 0) ? kXcds / kv_heads : 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;
     if (tile_waves == kPromptWaves) {
         rc = launch_prompt_form(s, a, head_dim);
         if (rc != CIE_OK || n_splits == 1) return rc;
-        attention_merge_kernel<<<dim3(n_tiles, kv_heads, tokens_per_tile * group), kMergeThreads, 0, s>>>(a, head_dim, kPromptTileRows);
-        return cie_after_launch();
+        return launch_merge(s, a, n_tiles, head_dim, kPromptTileRows);
     }
     switch (head_dim) {
         case 32: rc = launch_for_dim<32>(s, a, n_tiles, row_tiles, tile_waves); break;
@@ -779,6 +861,5 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
         default: return CIE_BAD_ARGUMENT;
     }
     if (rc != CIE_OK || n_splits == 1) return rc;
-    attention_merge_kernel<<<dim3(n_tiles, kv_heads, tokens_per_tile * group), kMergeThreads, 0, s>>>(a, head_dim, 16 * row_tiles);
-    return cie_after_launch();
+    return launch_merge(s, a, n_tiles, head_dim, 16 * row_tiles);
 }

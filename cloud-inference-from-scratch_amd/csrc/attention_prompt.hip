@@ -111,6 +111,7 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
     const int lo = (a.window > 0) ? max(0, start + q0 + 1 - a.window) : 0;
     int range_begin = lo & ~(kKeysPerBlock - 1);
     int range_end = hi;
+    bool whole = a.n_splits == 1;  // this workgroup sees all the tile's keys and writes its result itself
     if (a.n_splits > 1) {
         int per_split = a.keys_per_split;
         if (a.max_context_dev) {
@@ -118,8 +119,21 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
             if (a.window > 0) most = min(most, a.window + 2 * kKeysPerBlock);
             per_split = ((most + a.n_splits - 1) / a.n_splits + kKeysPerBlock - 1) & ~(kKeysPerBlock - 1);
         }
-        range_begin += blockIdx.y * per_split;
-        range_end = min(hi, range_begin + per_split);
+        if (a.whole_in_first_share && all_in_first_share(range_begin, hi, per_split)) {
+            if (blockIdx.y > 0) return;  // (the merge leaves such a tile alone too)
+            whole = true;
+        } else {
+            range_begin += blockIdx.y * per_split;
+            range_end = min(hi, range_begin + per_split);
+            if (range_begin >= range_end) {  // no keys in this share: its statistics say so, its sums are never read
+                float* pml = a.part_ml + ((static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + blockIdx.y) * kPromptTileRows * 2;
+                if (threadIdx.x < kPromptTileRows) {
+                    pml[threadIdx.x * 2] = -INFINITY;
+                    pml[threadIdx.x * 2 + 1] = 0.f;
+                }
+                return;
+            }
+        }
     }
     const int last_group = (hi - 1) & ~15;  // the last 16 keys that have a page
 
@@ -384,7 +398,7 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
             for (int i = 0; i < 4; ++i)
                 o[rt][dt][i] = o[rt][dt][i] * w_own_o[i] +
                                lds_o[(quarter * kMeetTile + dt * 4 + i) * kWave + lane] * w_other_o[i];
-        if (a.n_splits > 1) {  // this share's sums and statistics for the merge kernel
+        if (!whole) {  // this share's sums and statistics for the merge kernel
             const size_t unit = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + blockIdx.y;
             float* po = a.part_o + unit * kPromptTileRows * D;
             float* pml = a.part_ml + unit * kPromptTileRows * 2;
