@@ -17,6 +17,9 @@
 //               first half and the 16 they rotate with (half-split pairing), adds the bias, rounds
 //               to bf16 as the plain epilogue would, rotates q and k by the row's position and
 //               writes q to C[m, n], k and v into the paged cache (v transposed).
+//   ROPE8       the same with one tile per workgroup: 8 dimensions of a head's first half and the 8 they
+//               rotate with share the tile, so that a weight of few columns gives twice the workgroups
+//               (up to 16 rows).
 //
 // One kernel: a workgroup owns one or two tiles of 16 columns (SILU: a gate tile and its up tile)
 // and 16, 32 or 64 rows; its WAVES waves cut K into slices of 128 and take them round-robin.
@@ -38,7 +41,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes as one value (a struct is copied as memory)
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4, EPI_ROPE = 5 };
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4, EPI_ROPE = 5, EPI_ROPE8 = 6 };
 
 // What the ROPE epilogue needs beside the product: where each row's token sits, and the cache.
 struct RopeArgs {
@@ -271,6 +274,88 @@ __device__ __forceinline__ void store_rope(const FusedArgs& a, const floatx4& lo
     }
 }
 
+// The same epilogue where one tile holds both halves: lane (r, g) has dimension j*8 + (r & 7) of the first
+// half (r < 8) or of the second (r >= 8), and its partner sits eight lanes away.
+__device__ __forceinline__ RopeRows rope8_prefetch(const FusedArgs& a, int head, int j, int lane, int m_base) {
+    const RopeArgs& p = a.rope;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int d = j * 8 + (r & 7) + (r >> 3) * (p.head_dim / 2);
+    const bool is_query = head < p.q_heads;
+    RopeRows rows;
+    rows.bias_lo = a.bias ? to_float(a.bias[head * p.head_dim + d]) : 0.f;  // (the lane's own column)
+    rows.bias_hi = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m_base + g * 4 + i;
+        rows.pos[i] = -1;
+        rows.page[i] = -1;
+        rows.c[i] = 1.f;
+        rows.s[i] = 0.f;
+        if (m >= a.M) continue;
+        rows.pos[i] = p.positions[m];
+        if (!is_query && p.write_kv) rows.page[i] = p.seq_of_token[m];
+    }
+    return rows;
+}
+
+__device__ __forceinline__ void rope8_prefetch_rest(const FusedArgs& a, int head, int j, int lane, RopeRows& rows) {
+    const RopeArgs& p = a.rope;
+    const int half = p.head_dim / 2;
+    const int d = j * 8 + (lane & 7);  // the angle's index: the same for a dimension and its partner
+    const bool is_value = head >= p.q_heads + p.kv_heads;
+    int slot[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int pos = rows.pos[i];
+        if (pos >= 0 && !is_value && p.rotate) {
+            rows.c[i] = p.cos_table[static_cast<size_t>(pos) * half + d];
+            rows.s[i] = p.sin_table[static_cast<size_t>(pos) * half + d];
+        }
+        slot[i] = rows.page[i] >= 0 ? p.seq_slot[rows.page[i]] : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (slot[i] >= 0)
+            rows.page[i] = p.block_table[static_cast<size_t>(slot[i]) * p.table_width + rows.pos[i] / p.page_size];
+        if (rows.pos[i] < 0) rows.pos[i] = 0;
+    }
+}
+
+__device__ __forceinline__ void store_rope8(const FusedArgs& a, const floatx4& acc, int head, int j, int lane,
+                                            const RopeRows& rows, int m_base) {
+    const RopeArgs& p = a.rope;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int D = p.head_dim;
+    const bool second = r >= 8;
+    const int d = j * 8 + (r & 7) + (second ? D / 2 : 0);
+    const bool is_query = head < p.q_heads;
+    const bool is_value = head >= p.q_heads + p.kv_heads;
+    const int kv_head = is_query ? 0 : (head - p.q_heads) % p.kv_heads;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m_base + g * 4 + i;
+        const float x = to_float(from_float<bf16_t>(acc[i] + rows.bias_lo));
+        const float partner = __shfl_xor(x, 8, kWave);  // (every lane takes part, also those of rows that do not exist)
+        if (m >= a.M) continue;
+        // first half: x cos - partner sin; second half: x cos + partner sin (values, unrotated heads: c = 1, s = 0)
+        const bf16_t y = from_float<bf16_t>(second ? x * rows.c[i] + partner * rows.s[i] : x * rows.c[i] - partner * rows.s[i]);
+        if (is_query) {
+            static_cast<bf16_t*>(a.c)[static_cast<size_t>(m) * a.N + head * D + d] = y;
+            continue;
+        }
+        const int page = rows.page[i];
+        if (page < 0) continue;
+        const int in_page = rows.pos[i] % p.page_size;
+        const size_t head_base = (static_cast<size_t>(page) * p.kv_heads + kv_head) * p.page_size * D;
+        if (is_value)
+            p.v_pool[head_base + in_page + static_cast<size_t>(d) * p.page_size] = y;
+        else
+            p.k_pool[head_base + static_cast<size_t>(in_page) * D + d] = y;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // MT row tiles (M <= 16*MT per workgroup row; more rows: more workgroup rows) and NT column tiles
 // per workgroup: with SILU the gate tile and its up tile, else NT adjacent tiles.  Every weight
@@ -282,6 +367,7 @@ template <int WAVES, int EPI, int MT, int NT>
 __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
     static_assert(EPI != EPI_ROPE || NT == 2, "the ROPE epilogue pairs the two halves of a head");
+    static_assert(EPI != EPI_ROPE8 || (NT == 1 && MT == 1), "the one-tile ROPE epilogue: one tile, up to 16 rows");
     static_assert(MT <= WAVES || WAVES == 1, "a wave ends at most one row tile");
     // slices of 128 k values whose weight loads are in flight together
     constexpr int U = (MT == 1 && NT == 1) ? 4 : (MT == 4) ? 1 : 2;
@@ -302,7 +388,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
     const int tile_first = (EPI == EPI_SILU || EPI == EPI_ROPE) ? blockIdx.x : blockIdx.x * NT;
     // ROPE: workgroup b takes tile b % (D/32) of the first half of head b / (D/32), and its partner
-    const int rope_tiles = (EPI == EPI_ROPE) ? a.rope.head_dim / 32 : 1;
+    // (ROPE8: 8 dimensions b % (D/16) of the first half and their 8 partners)
+    const int rope_tiles = (EPI == EPI_ROPE) ? a.rope.head_dim / 32 : (EPI == EPI_ROPE8) ? a.rope.head_dim / 16 : 1;
     const int rope_head = blockIdx.x / rope_tiles;
     const int rope_tile = blockIdx.x - rope_head * rope_tiles;
 
@@ -321,7 +408,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         for (int i = 0; i < 4; ++i) {
             const int row = i * 4 + load_row;
             int n;
-            if (EPI == EPI_ROPE)
+            if (EPI == EPI_ROPE8)
+                n = rope_head * a.rope.head_dim + rope_tile * 8 + (row & 7) + (row >> 3) * (a.rope.head_dim / 2);
+            else if (EPI == EPI_ROPE)
                 n = rope_head * a.rope.head_dim + rope_tile * 16 + row + t * (a.rope.head_dim / 2);
             else if (EPI == EPI_SILU)
                 n = min(tile_first * 16 + row, cols - 1) + t * a.up_offset;
@@ -351,8 +440,10 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         for (int t = 0; t < NT; ++t) acc[mt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
     RopeRows rope_rows;
     // (the wave that will store row tile `wave`, below)
-    bool rope_pending = EPI == EPI_ROPE && wave < MT;
-    if (rope_pending) rope_rows = rope_prefetch(a, rope_head, rope_tile, lane, m0 + wave * 16);
+    bool rope_pending = (EPI == EPI_ROPE || EPI == EPI_ROPE8) && wave < MT;
+    if (rope_pending)
+        rope_rows = (EPI == EPI_ROPE8) ? rope8_prefetch(a, rope_head, rope_tile, lane, m0 + wave * 16)
+                                       : rope_prefetch(a, rope_head, rope_tile, lane, m0 + wave * 16);
     ResidRows resid_rows[NT];
     if (EPI == EPI_RESID && wave < MT) {
 #pragma unroll
@@ -402,7 +493,10 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
             scale_pending = false;
         }
         if (rope_pending) {  // likewise
-            rope_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
+            if (EPI == EPI_ROPE8)
+                rope8_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
+            else
+                rope_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
             rope_pending = false;
         }
 #pragma unroll
@@ -448,7 +542,12 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         }
     }
 
-    if (rope_pending) rope_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);  // (a K so short that this wave had no slice)
+    if (rope_pending) {  // (a K so short that this wave had no slice)
+        if (EPI == EPI_ROPE8)
+            rope8_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
+        else
+            rope_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
+    }
     if (scaled_rows) {
         if (scale_pending) sum_row_parts();  // (likewise)
 #pragma unroll
@@ -543,7 +642,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        if (EPI == EPI_ROPE) {
+        if (EPI == EPI_ROPE8) {
+            store_rope8(a, acc[mt][0], rope_head, rope_tile, lane, rope_rows, m0 + mt * 16);
+        } else if (EPI == EPI_ROPE) {
             store_rope(a, acc[mt][0], acc[mt][NT - 1], rope_head, rope_tile, lane, rope_rows, m0 + mt * 16);
         } else if (EPI == EPI_SILU) {
             store_tile<EPI>(a, acc[mt][0], acc[mt][NT - 1], m0 + mt * 16, tile_first * 16 + r, tile_first, lane, row_scale);
@@ -877,6 +978,10 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
 // `c` [M, N] receives the rotated queries (its key and value columns are left alone); rotated keys and
 // values go to the cache page of each row's position.  `waves` waves per workgroup share K (1, 2, 4, 8;
 // with more than 16 rows 4 or 8).
+// (Below this many pairs of tiles a product of up to 16 rows takes one tile a workgroup: the 3B shape's 80 pairs
+// leave two thirds of the compute units without a workgroup.)
+constexpr unsigned kSplitPairsBelow = 128;
+
 CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
                               int M, int N, int K, int waves, const float* cos_table, const float* sin_table,
                               const int* positions, const int* seq_of_token, const int* seq_slot,
@@ -912,6 +1017,10 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
                       page_size, rotate, write_kv};
     const dim3 grid((q_heads + 2 * kv_heads) * (head_dim / 32), M <= 64 ? 1 : (M + 63) / 64, 1);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (M <= 16 && grid.x < kSplitPairsBelow) {  // few columns: one tile a workgroup, twice the workgroups
+        const dim3 twice((q_heads + 2 * kv_heads) * (head_dim / 16), 1, 1);
+        return launch_waves<EPI_ROPE8, 1, 1>(s, waves, twice, f);
+    }
     if (M <= 16) return launch_waves<EPI_ROPE, 1, 2>(s, waves, grid, f);
     if (M <= 32) return launch_waves<EPI_ROPE, 2, 2>(s, waves, grid, f);
     return launch_waves<EPI_ROPE, 4, 2>(s, waves, grid, f);

@@ -633,6 +633,9 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     return out
 
 
+QKV_SPLIT_PAIRS_BELOW = 128  # (as in the kernel library: below this many pairs of tiles, one tile a workgroup)
+
+
 def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Tensor], cos: torch.Tensor,
                   sin: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, seq_slot: torch.Tensor,
                   block_table: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, q_heads: int,
@@ -679,6 +682,8 @@ def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Te
     page_size = _check_pools(k_pool, v_pool, torch.bfloat16, kv_heads, head_dim)
     if waves is None:
         _, waves, _ = plan_fused(m, n // 32, k)
+        if m <= 16 and n // 32 < QKV_SPLIT_PAIRS_BELOW:
+            waves = min(waves, 4)  # (the kernel then takes one tile a workgroup, twice the workgroups: 8.1 -> 7.2 us)
     if not (waves in ((1, 2, 4, 8) if m <= 16 else (4, 8))):
         raise ValueError(f"{waves} waves per workgroup with {m} rows is not a form the kernel has")
     out = torch.empty((m, n), dtype=torch.bfloat16, device=weight.device)
