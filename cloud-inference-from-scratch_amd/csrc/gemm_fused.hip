@@ -13,6 +13,7 @@
 //               RMSNorm that follows needs no reduction over the row
 //   PARTIAL     K is cut into grid.z parts; part p writes acc to C[p, m, n] (float32, bias in
 //               part 0).  The add + norm kernel sums the parts.  For few columns and long K.
+//               (Only in the second form, further down.)
 //   ROPE        W stacks the rows of q, k and v heads: a workgroup takes 16 dimensions of a head's
 //               first half and the 16 they rotate with (half-split pairing), adds the bias, rounds
 //               to bf16 as the plain epilogue would, rotates q and k by the row's position and
@@ -678,7 +679,7 @@ int launch_waves(hipStream_t s, int waves, dim3 grid, const FusedArgs& a) {
 }
 
 template <int EPI>
-int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, int k_parts, const FusedArgs& a) {
+int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, const FusedArgs& a) {
     const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
     const int tiles = (cols + 15) / 16;
     const int m_blocks = (a.M + 16 * row_tiles - 1) / (16 * row_tiles);
@@ -686,16 +687,16 @@ int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, int k_part
     constexpr int NT1 = (EPI == EPI_SILU) ? 2 : 1;  // the SiLU epilogue always pairs a gate tile with its up tile
     if (row_tiles == 1) {
         if (column_tiles != 1) return CIE_BAD_ARGUMENT;
-        return launch_waves<EPI, 1, NT1>(s, waves, dim3(tiles, m_blocks, k_parts), a);
+        return launch_waves<EPI, 1, NT1>(s, waves, dim3(tiles, m_blocks, 1), a);
     }
     if (EPI == EPI_SILU || column_tiles == 2) {
         const int groups = (EPI == EPI_SILU) ? tiles : (tiles + 1) / 2;
-        if (row_tiles == 2) return launch_waves<EPI, 2, 2>(s, waves, dim3(groups, m_blocks, k_parts), a);
-        if (row_tiles == 4) return launch_waves<EPI, 4, 2>(s, waves, dim3(groups, m_blocks, k_parts), a);
+        if (row_tiles == 2) return launch_waves<EPI, 2, 2>(s, waves, dim3(groups, m_blocks, 1), a);
+        if (row_tiles == 4) return launch_waves<EPI, 4, 2>(s, waves, dim3(groups, m_blocks, 1), a);
     } else if constexpr (EPI != EPI_SILU) {
         if (column_tiles != 1) return CIE_BAD_ARGUMENT;
-        if (row_tiles == 2) return launch_waves<EPI, 2, 1>(s, waves, dim3(tiles, m_blocks, k_parts), a);
-        if (row_tiles == 4) return launch_waves<EPI, 4, 1>(s, waves, dim3(tiles, m_blocks, k_parts), a);
+        if (row_tiles == 2) return launch_waves<EPI, 2, 1>(s, waves, dim3(tiles, m_blocks, 1), a);
+        if (row_tiles == 4) return launch_waves<EPI, 4, 1>(s, waves, dim3(tiles, m_blocks, 1), a);
     }
     return CIE_BAD_ARGUMENT;
 }
@@ -917,7 +918,7 @@ int launch_shared_rows(hipStream_t s, int waves, int k_parts, const FusedArgs& a
 }  // namespace
 
 // epilogue: 0 bf16, 1 float32, 2 SiLU-gate (W = [gate rows; up rows], N = 2 * outputs), 3 residual
-// accumulate (+ sums of squares), 4 partial products of k_parts parts of K to c[k_parts, M, N].
+// accumulate (+ sums of squares).  (Products whose K is cut into parts take the other form, below.)
 // row_tiles 1, 2, 4: 16, 32, 64 rows per workgroup (more rows: more workgroups, each streaming W again);
 // `waves` waves per workgroup share K (1, 2, 4, 8; with more than one row tile 4 or 8);
 // column_tiles 1 or 2 tiles of 16 columns per workgroup (2 only with more than one row tile: the rows of
@@ -928,7 +929,7 @@ int launch_shared_rows(hipStream_t s, int waves, int k_parts, const FusedArgs& a
 // rows of `a` lack the factor rsqrt(sum of the row's partial sums / K + eps), applied before the SiLU.
 CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
                            float* residual, float* sumsq, int M, int N, int K, int epilogue, int row_tiles,
-                           int waves, int column_tiles, int k_parts, const float* norm_weight, void* scaled_out,
+                           int waves, int column_tiles, const float* norm_weight, void* scaled_out,
                            const float* row_sumsq, int sumsq_parts, float eps) {
     if (M <= 0 || N <= 0 || K <= 0 || K % 8 || !a || !w || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
     if (row_tiles != 1 && row_tiles != 2 && row_tiles != 4) return CIE_BAD_ARGUMENT;
@@ -936,7 +937,6 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     if (epilogue == EPI_SILU && (N % 2 || bias)) return CIE_BAD_ARGUMENT;
     if (epilogue == EPI_RESID && (!residual || !sumsq)) return CIE_BAD_ARGUMENT;
     if (epilogue != EPI_RESID && !c) return CIE_BAD_ARGUMENT;
-    if (k_parts < 1 || k_parts > 64 || (k_parts > 1 && epilogue != EPI_PARTIAL)) return CIE_BAD_ARGUMENT;
     // the folded norm: a scaled copy needs the weight and the RESID epilogue; rows that lack their scale
     // are taken by the SILU epilogue of one row tile
     if ((scaled_out != nullptr) != (norm_weight != nullptr) || (scaled_out && epilogue != EPI_RESID)) return CIE_BAD_ARGUMENT;
@@ -954,7 +954,7 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     f.N = N;
     f.K = K;
     f.up_offset = (epilogue == EPI_SILU) ? N / 2 : 0;
-    f.k_per_part = ((K + k_parts - 1) / k_parts + 127) / 128 * 128;
+    f.k_per_part = (K + 127) / 128 * 128;
     f.norm_weight = norm_weight;
     f.scaled_out = static_cast<bf16_t*>(scaled_out);
     f.row_sumsq = row_sumsq;
@@ -963,11 +963,10 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     f.rope = RopeArgs{};
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (epilogue) {
-        case EPI_BF16: return launch<EPI_BF16>(s, row_tiles, waves, column_tiles, k_parts, f);
-        case EPI_F32: return launch<EPI_F32>(s, row_tiles, waves, column_tiles, k_parts, f);
-        case EPI_SILU: return launch<EPI_SILU>(s, row_tiles, waves, column_tiles, k_parts, f);
-        case EPI_RESID: return launch<EPI_RESID>(s, row_tiles, waves, column_tiles, k_parts, f);
-        case EPI_PARTIAL: return launch<EPI_PARTIAL>(s, row_tiles, waves, column_tiles, k_parts, f);
+        case EPI_BF16: return launch<EPI_BF16>(s, row_tiles, waves, column_tiles, f);
+        case EPI_F32: return launch<EPI_F32>(s, row_tiles, waves, column_tiles, f);
+        case EPI_SILU: return launch<EPI_SILU>(s, row_tiles, waves, column_tiles, f);
+        case EPI_RESID: return launch<EPI_RESID>(s, row_tiles, waves, column_tiles, f);
     }
     return CIE_BAD_ARGUMENT;
 }

@@ -410,17 +410,16 @@ FUSED_MAX_ROWS = 64  # rows one workgroup of ``gemm_fused`` takes; more rows run
 FUSED_PAIR_WORKGROUPS = 256  # workgroups that must remain when workgroups of many rows take two column tiles
 
 
-def plan_fused(rows: int, column_tiles: int, k: int, k_parts: int = 1) -> tuple[int, int, int]:
+def plan_fused(rows: int, column_tiles: int, k: int) -> tuple[int, int, int]:
     """(row tiles, waves per workgroup, column tiles per workgroup) of ``gemm_fused``
-    for ``rows`` rows, ``column_tiles`` tiles of 16 columns, ``k_parts`` parts of
-    K of ``k`` each.  16, 32 or 64 rows per workgroup (more rows: more workgroups,
+    for ``rows`` rows, ``column_tiles`` tiles of 16 columns and a K of ``k``.  16, 32 or 64 rows per workgroup (more rows: more workgroups,
     each streaming the weight again).  With more than 16 rows a workgroup takes
     two column tiles if that still leaves enough workgroups (each activation
     value a wave loads then meets two weight tiles).  As many waves share K as it
     takes to fill the GPU, each with at least one 128-wide slice."""
     row_tiles = 1 if rows <= 16 else 2 if rows <= 32 else 4
-    pair = row_tiles > 1 and column_tiles * k_parts >= 2 * FUSED_PAIR_WORKGROUPS
-    groups = (-(-column_tiles // 2) if pair else column_tiles) * k_parts * -(-rows // FUSED_MAX_ROWS)
+    pair = row_tiles > 1 and column_tiles >= 2 * FUSED_PAIR_WORKGROUPS
+    groups = (-(-column_tiles // 2) if pair else column_tiles) * -(-rows // FUSED_MAX_ROWS)
     waves = 1 if row_tiles == 1 else 4
     while waves < 8 and groups * waves < FUSED_TARGET_WAVES and waves * 2 * 128 <= k:
         waves *= 2
@@ -429,7 +428,7 @@ def plan_fused(rows: int, column_tiles: int, k: int, k_parts: int = 1) -> tuple[
 
 def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optional[torch.Tensor] = None,
                residual_out: Optional[torch.Tensor] = None, sumsq_out: Optional[torch.Tensor] = None,
-               plan: Optional[tuple[int, int, int]] = None, k_parts: int = 1,
+               plan: Optional[tuple[int, int, int]] = None,
                norm_weight: Optional[torch.Tensor] = None, scaled_out: Optional[torch.Tensor] = None,
                row_sumsq: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
     """Few-row matrix product ``a @ weight.T`` (bf16 operands, float32 sums) fused
@@ -437,9 +436,7 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
     ``a W^T + bias``; ``EPI_SILU`` (weight = gate rows over up rows) returns
     ``silu(gate) * up`` [M, N/2]; ``EPI_RESID`` adds the product
     into ``residual_out`` (float32 [M, N]) and returns the partial sums of
-    squares of its new rows [M, ceil(N/16)]; ``EPI_PARTIAL`` cuts K into
-    ``k_parts`` parts and returns their float32 partial products
-    [k_parts, M, N] (bias in part 0), to be summed by ``add_parts_rmsnorm``.
+    squares of its new rows [M, ceil(N/16)].  (Partial products of a cut K: :func:`gemm_shared_rows`.)
     An RMSNorm between an ``EPI_RESID`` product and an ``EPI_SILU`` product of up to 16
     rows can ride along: with ``norm_weight`` (float32 [N]) and ``scaled_out`` (bf16
     [M, N]) the former also writes the new residual times the weight, and the latter,
@@ -457,15 +454,13 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
         raise ValueError(f"K and the row stride must be multiples of 8, are {k} and {lda}")
     if not (a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         raise ValueError("operands must be 16-byte aligned")
-    if not (1 <= k_parts <= 64 and (k_parts == 1 or epilogue == EPI_PARTIAL)):
-        raise ValueError(f"k_parts {k_parts} does not fit the epilogue")
     device = weight.device
     if bias is not None:
         _gpu("bias", bias, torch.bfloat16, 1)
         if not (bias.shape[0] == n and epilogue != EPI_SILU):
             raise ValueError("bias does not fit")
     columns = n // 2 if epilogue == EPI_SILU else n
-    row_tiles, waves, column_tiles = plan or plan_fused(m, -(-columns // 16), -(-k // k_parts), k_parts)
+    row_tiles, waves, column_tiles = plan or plan_fused(m, -(-columns // 16), k)
     if epilogue == EPI_SILU:
         column_tiles = 1 if row_tiles == 1 else 2  # always a gate tile with its up tile
     if not (
@@ -478,8 +473,6 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
         out = torch.empty((m, n), dtype=torch.bfloat16, device=device)
     elif epilogue == EPI_F32:
         out = torch.empty((m, n), dtype=torch.float32, device=device)
-    elif epilogue == EPI_PARTIAL:
-        out = torch.empty((k_parts, m, n), dtype=torch.float32, device=device)
     elif epilogue == EPI_SILU:
         if not (n % 2 == 0):
             raise ValueError(f"the SiLU epilogue needs an even N, got {n}")
@@ -515,7 +508,7 @@ def gemm_fused(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optio
     _run("cie_gemm_fused", load_library().cie_gemm_fused(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(None if epilogue == EPI_RESID else out),
         _ptr(residual), _ptr(sumsq), _i(m), _i(n), _i(k), _i(epilogue), _i(row_tiles), _i(waves), _i(column_tiles),
-        _i(k_parts), _ptr(norm_weight), _ptr(scaled_out), _ptr(row_sumsq), _i(parts_in), _f(eps)))
+        _ptr(norm_weight), _ptr(scaled_out), _ptr(row_sumsq), _i(parts_in), _f(eps)))
     return out
 
 
