@@ -57,6 +57,10 @@ PART_K = 1024           # the shortest stretch of K a part takes
 # for the SiLU kernel behind it; 14B: 50 / 56 against 55 / 62 + 6; 7B: level); from 65 rows on the library is
 # level or ahead (3B at 128 rows: 34 against 30 + 5 us).
 SHARED_SILU_ROWS = 64
+# float32 logits take that form up to this many rows (the head of the 3B / 7B / 14B shape, us: 64 rows 156 against
+# 173 in the form whose waves share K; 72 rows 165 / 239 / 333 against the library's 174 / 249 / 349; 96 rows
+# 172 / 255 / 346 against 174 / 238 / 338)
+SHARED_LOGIT_ROWS = 80
 COMPUTE_UNITS = 256
 
 
@@ -194,8 +198,8 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
         waves, own_unit = plan_shared_silu(-(-n // 32))
         if rows > FUSED_ROWS or own_unit:
             return ops.gemm_shared_rows(weight, ops.EPI_SILU, x, waves=waves)
-    if fusable and wants_f32 and FUSED_ROWS < rows <= ops.SHARED_ROWS_MAX and into is None and not silu:
-        # logits of 17 to 128 rows: the shared-rows form (the 3B head at 64 rows: 170 -> ? us)
+    if fusable and wants_f32 and FUSED_ROWS < rows <= SHARED_LOGIT_ROWS and into is None and not silu:
+        # logits of 17 to 80 rows: the shared-rows form
         return ops.gemm_shared_rows(weight, ops.EPI_F32, x, bias=bias, waves=4)
     if fusable and wants_f32 and rows > FUSED_LOGIT_ROWS and into is None and not silu and bias is None:
         out = ops.gemm_library(x, weight, out_dtype=torch.float32)  # logits of many rows: one pass over the weight
