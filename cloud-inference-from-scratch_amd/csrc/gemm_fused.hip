@@ -709,15 +709,15 @@ int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, const Fuse
 // same slice of 128 k values together: the workgroup's 256 threads fetch the slice of A once (whole
 // 256-byte row segments) into LDS, every wave streams its own NT tiles of 16 columns of W over all of
 // K (or a grid.z part of it) and reads the rows of A from LDS in the MFMA layout.  A wave's loads run
-// DIST slices ahead of its products, in a ring of DIST + 1 sets of registers that the unrolled loop
-// addresses by constants (a copy from a set whose load is still under way would wait for it).
-template <int EPI, int MT, int NT, int DIST, int WAVES>
+// one slice ahead of its products, in two sets of registers that the loop, unrolled by two, addresses by
+// constants (a copy from a set whose load is still under way would wait for it; two slices ahead, with
+// three sets, were 1 to 3 us slower at every size).
+template <int EPI, int MT, int NT, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs a) {
     static_assert(EPI == EPI_SILU || EPI == EPI_PARTIAL || EPI == EPI_BF16 || EPI == EPI_F32, "epilogues of this form");
     static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
     constexpr int kWaves = WAVES;
     constexpr int kThreads = WAVES * 64;
-    constexpr int kRing = DIST + 1;
     constexpr int kRows = MT * 16;
     constexpr int kStageBytesA = kRows * kStageRow;
     constexpr int kStagesA = MT <= 4 ? 2 : 1;  // (two stages of 128 rows would pass the 64 KB of static LDS)
@@ -767,7 +767,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs 
         u32x4 w[NT][4];
         u32x4 a[kPasses];
     };
-    Slot ring0, ring1, ring2;  // (the third only with DIST 2)
+    Slot ring0, ring1;
     auto fetch = [&](Slot& into, int slice) __attribute__((always_inline)) {
         const int k = min(k_begin + slice * 128 + load_col, k_end - 8);
 #pragma unroll
@@ -793,7 +793,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs 
         for (int i = 0; i < kPasses; ++i)
             *reinterpret_cast<u32x4*>(stage_a + a_stage_row[i] * kStageRow + load_col * 2) =
                 inside ? now.a[i] : u32x4{0u, 0u, 0u, 0u};
-        fetch(ahead, slice + DIST);
+        fetch(ahead, slice + 1);
         u32x4 bt[NT][4];
 #pragma unroll
         for (int t = 0; t < NT; ++t) {  // through the wave's staging area (its LDS operations keep their order)
@@ -838,7 +838,6 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs 
             held[i] = *reinterpret_cast<const float4*>(scale_from + min((scale_sub + i * kPerRow) * 4, a.sumsq_parts - 4));
     }
     fetch(ring0, 0);
-    if (DIST > 1) fetch(ring1, 1);
     if (scaled_rows) {
         float sq = 0.f;
         if (scale_by_four) {
@@ -858,15 +857,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs 
     }
     // (whole turns of the ring: a step past the last slice multiplies zeros)
 #pragma unroll 1
-    for (int base = 0; base < slices; base += kRing) {
-        if constexpr (DIST == 1) {
-            step(ring0, ring1, base);
-            step(ring1, ring0, base + 1);
-        } else {
-            step(ring0, ring2, base);
-            step(ring1, ring0, base + 1);
-            step(ring2, ring1, base + 2);
-        }
+    for (int base = 0; base < slices; base += 2) {
+        step(ring0, ring1, base);
+        step(ring1, ring0, base + 1);
     }
     if (scaled_rows && slices == 0) __syncthreads();  // (the scales, if no step stood between)
 
@@ -890,27 +883,27 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs 
     }
 }
 
-template <int EPI, int NT, int DIST, int WAVES>
+template <int EPI, int NT, int WAVES>
 int launch_shared_rows_waves(hipStream_t s, int k_parts, const FusedArgs& a) {
     const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
     const int tiles = (cols + 15) / 16;
     const int per_workgroup = WAVES * ((EPI == EPI_SILU) ? 1 : NT);
     const dim3 grid((tiles + per_workgroup - 1) / per_workgroup, 1, k_parts);
     if (a.M <= 32)
-        gemm_shared_rows_kernel<EPI, 2, NT, DIST, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
+        gemm_shared_rows_kernel<EPI, 2, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
     else if (a.M <= 64)
-        gemm_shared_rows_kernel<EPI, 4, NT, DIST, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
+        gemm_shared_rows_kernel<EPI, 4, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
     else
-        gemm_shared_rows_kernel<EPI, 8, NT, DIST, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
+        gemm_shared_rows_kernel<EPI, 8, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
     return cie_after_launch();
 }
 
-template <int EPI, int NT, int DIST>
+template <int EPI, int NT>
 int launch_shared_rows(hipStream_t s, int waves, int k_parts, const FusedArgs& a) {
     switch (waves) {
-        case 2: return launch_shared_rows_waves<EPI, NT, DIST, 2>(s, k_parts, a);
-        case 3: return launch_shared_rows_waves<EPI, NT, DIST, 3>(s, k_parts, a);
-        case 4: return launch_shared_rows_waves<EPI, NT, DIST, 4>(s, k_parts, a);
+        case 2: return launch_shared_rows_waves<EPI, NT, 2>(s, k_parts, a);
+        case 3: return launch_shared_rows_waves<EPI, NT, 3>(s, k_parts, a);
+        case 4: return launch_shared_rows_waves<EPI, NT, 4>(s, k_parts, a);
     }
     return CIE_BAD_ARGUMENT;
 }
@@ -1026,19 +1019,17 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
 }
 
 // The form for 17 to 128 rows in which a workgroup's four waves own columns and share the rows of A
-// through LDS (one workgroup row: M <= 128).  epilogue 0 (bf16, + bias), 1 (float32, + bias; two tiles a wave,
-// distance 1), 2 (SiLU-gate; row_sumsq as in
+// through LDS (one workgroup row: M <= 128).  epilogue 0 (bf16, + bias), 1 (float32, + bias; two tiles a wave),
+// 2 (SiLU-gate; row_sumsq as in
 // cie_gemm_fused, for any number of rows here) or 4 (k_parts partial products).  column_tiles 1 or 2 tiles of
-// 16 columns per wave (SiLU: the gate tile and its up tile), 2 to 4 waves per workgroup; distance 1 or 2
-// slices of 128 k that a wave's loads run ahead.
+// 16 columns per wave (SiLU: the gate tile and its up tile), 2 to 4 waves per workgroup.
 CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const void* w, const void* bias, void* c, int M,
-                                 int N, int K, int epilogue, int column_tiles, int waves, int k_parts, int distance,
+                                 int N, int K, int epilogue, int column_tiles, int waves, int k_parts,
                                  const float* row_sumsq, int sumsq_parts, float eps) {
     if (M <= 0 || M > 128 || N <= 0 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
     if (epilogue != EPI_BF16 && epilogue != EPI_F32 && epilogue != EPI_SILU && epilogue != EPI_PARTIAL) return CIE_BAD_ARGUMENT;
     if (epilogue == EPI_SILU && (N % 2 || bias || column_tiles != 2)) return CIE_BAD_ARGUMENT;
     if (column_tiles != 1 && column_tiles != 2) return CIE_BAD_ARGUMENT;
-    if (distance != 1 && distance != 2) return CIE_BAD_ARGUMENT;
     if (k_parts < 1 || k_parts > 64 || (k_parts > 1 && epilogue != EPI_PARTIAL)) return CIE_BAD_ARGUMENT;
     if (row_sumsq && (epilogue != EPI_SILU || sumsq_parts < 1 || !(eps > 0.f))) return CIE_BAD_ARGUMENT;
     FusedArgs f;
@@ -1061,20 +1052,16 @@ CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const voi
     f.eps = eps;
     f.rope = RopeArgs{};
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool far = distance == 2;
     switch (epilogue) {
-        case EPI_SILU:
-            return far ? launch_shared_rows<EPI_SILU, 2, 2>(s, waves, 1, f) : launch_shared_rows<EPI_SILU, 2, 1>(s, waves, 1, f);
+        case EPI_SILU: return launch_shared_rows<EPI_SILU, 2>(s, waves, 1, f);
         case EPI_BF16:
-            if (column_tiles == 2) return far ? launch_shared_rows<EPI_BF16, 2, 2>(s, waves, 1, f) : launch_shared_rows<EPI_BF16, 2, 1>(s, waves, 1, f);
-            return far ? launch_shared_rows<EPI_BF16, 1, 2>(s, waves, 1, f) : launch_shared_rows<EPI_BF16, 1, 1>(s, waves, 1, f);
-        case EPI_F32:  // (the logits: two tiles a wave, loads one slice ahead)
-            if (column_tiles != 2 || far) return CIE_BAD_ARGUMENT;
-            return launch_shared_rows<EPI_F32, 2, 1>(s, waves, 1, f);
+            return column_tiles == 2 ? launch_shared_rows<EPI_BF16, 2>(s, waves, 1, f) : launch_shared_rows<EPI_BF16, 1>(s, waves, 1, f);
+        case EPI_F32:  // (the logits: two tiles a wave)
+            if (column_tiles != 2) return CIE_BAD_ARGUMENT;
+            return launch_shared_rows<EPI_F32, 2>(s, waves, 1, f);
         case EPI_PARTIAL:
-            if (column_tiles == 2)
-                return far ? launch_shared_rows<EPI_PARTIAL, 2, 2>(s, waves, k_parts, f) : launch_shared_rows<EPI_PARTIAL, 2, 1>(s, waves, k_parts, f);
-            return far ? launch_shared_rows<EPI_PARTIAL, 1, 2>(s, waves, k_parts, f) : launch_shared_rows<EPI_PARTIAL, 1, 1>(s, waves, k_parts, f);
+            return column_tiles == 2 ? launch_shared_rows<EPI_PARTIAL, 2>(s, waves, k_parts, f)
+                                     : launch_shared_rows<EPI_PARTIAL, 1>(s, waves, k_parts, f);
     }
     return CIE_BAD_ARGUMENT;
 }

@@ -516,14 +516,14 @@ SHARED_ROWS_MAX = 128  # rows of the form whose waves share the rows of A
 
 
 def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optional[torch.Tensor] = None,
-                     column_tiles: int = 2, waves: int = 4, k_parts: int = 1, distance: int = 1,
+                     column_tiles: int = 2, waves: int = 4, k_parts: int = 1,
                      row_sumsq: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
     """``a @ weight.T`` for 17 to 128 rows (it takes fewer too) in the form whose four waves per
     workgroup own columns and share each slice of ``a`` through LDS: ``EPI_BF16`` or ``EPI_F32`` (+ bias),
     ``EPI_SILU`` (weight = gate rows over up rows; with ``row_sumsq`` and ``eps`` the rows of ``a``
     lack their ``rsqrt(mean square + eps)``, as in :func:`gemm_fused`) or ``EPI_PARTIAL``
     (``k_parts`` float32 partial products [k_parts, M, N], bias in part 0).  ``column_tiles``
-    tiles of 16 columns per wave, loads ``distance`` slices of 128 k ahead."""
+    tiles of 16 columns per wave, ``waves`` waves per workgroup."""
     _gpu("weight", weight, torch.bfloat16, 2)
     n, k = weight.shape
     if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
@@ -537,15 +537,15 @@ def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias:
     if epilogue not in (EPI_BF16, EPI_F32, EPI_SILU, EPI_PARTIAL):
         raise ValueError(f"epilogue {epilogue} is not one this form has")
     if epilogue == EPI_F32:
-        column_tiles, distance = 2, 1
+        column_tiles = 2
     if not (1 <= k_parts <= 64 and (k_parts == 1 or epilogue == EPI_PARTIAL)):
         raise ValueError(f"k_parts {k_parts} does not fit the epilogue")
     if epilogue == EPI_SILU:
         column_tiles = 2
         if n % 2 or bias is not None:
             raise ValueError("the SiLU epilogue needs an even N and no bias")
-    if column_tiles not in (1, 2) or distance not in (1, 2) or waves not in (2, 3, 4):
-        raise ValueError(f"column_tiles {column_tiles} / distance {distance} not in (1, 2), or waves {waves} not in (2, 3, 4)")
+    if column_tiles not in (1, 2) or waves not in (2, 3, 4):
+        raise ValueError(f"column_tiles {column_tiles} not in (1, 2), or waves {waves} not in (2, 3, 4)")
     if bias is not None:
         _gpu("bias", bias, torch.bfloat16, 1)
         if bias.shape[0] != n:
@@ -567,7 +567,7 @@ def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias:
         out = torch.empty((k_parts, m, n), dtype=torch.float32, device=device)
     _run("cie_gemm_shared_rows", load_library().cie_gemm_shared_rows(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k), _i(epilogue),
-        _i(column_tiles), _i(waves), _i(k_parts), _i(distance), _ptr(row_sumsq), _i(parts_in), _f(eps)))
+        _i(column_tiles), _i(waves), _i(k_parts), _ptr(row_sumsq), _i(parts_in), _f(eps)))
     return out
 
 

@@ -854,34 +854,34 @@ def test_gemm_shared_rows_matches_float64(ops, shape, waves):
     """The form for 17 to 128 rows whose waves own columns and share the rows of A through LDS: plain with
     bias, SiLU-gate with and without rows that lack their 1/rms, and partial products of a cut K (parts that
     end inside a slice of 128, a part without any k, bias in the first part only); widths and row counts that
-    fill no tile, one and two tiles a wave, loads one and two slices ahead, rows given as a strided view."""
+    fill no tile, one and two tiles a wave, rows given as a strided view."""
     m, n, k = shape
     a, w, b = rand((m, k), torch.bfloat16, 40), rand((n, k), torch.bfloat16, 41, scale=0.1), rand((n,), torch.bfloat16, 42)
     wide = torch.zeros((m, k + 24), dtype=torch.bfloat16).cuda()
     wide[:, :k] = a
     expect = a.double() @ w.double().t()
     tol = dict(rtol=1e-2, atol=1e-2 * math.sqrt(k) * 0.1)
-    for distance in (1, 2):
-        for tiles in (1, 2):
-            out = ops.gemm_shared_rows(w, ops.EPI_BF16, a, bias=b, column_tiles=tiles, waves=waves, distance=distance)
-            torch.testing.assert_close(out.double(), expect + b.double(), **tol)
-            out = ops.gemm_shared_rows(w, ops.EPI_F32, a, bias=b, waves=waves)  # as for logits
-            assert out.dtype == torch.float32
-            torch.testing.assert_close(out.double(), expect + b.double(), rtol=1e-4, atol=1e-4 * math.sqrt(k))
-            for parts in (1, 3, 7):
-                rows = wide[:, :k] if parts == 3 else a
-                out = ops.gemm_shared_rows(w, ops.EPI_PARTIAL, rows, bias=b, column_tiles=tiles, waves=waves,
-                                           k_parts=parts, distance=distance)
-                assert out.shape == (parts, m, n) and out.dtype == torch.float32
-                torch.testing.assert_close(out.double().sum(0), expect + b.double(), rtol=1e-4, atol=1e-4 * math.sqrt(k))
-        gate, up = expect[:, : n // 2], expect[:, n // 2:]
-        out = ops.gemm_shared_rows(w, ops.EPI_SILU, a, waves=waves, distance=distance)
-        assert out.shape == (m, n // 2) and out.dtype == torch.bfloat16
-        torch.testing.assert_close(out.double(), torch.nn.functional.silu(gate) * up, rtol=2e-2, atol=2e-2)
-        # rows that lack their 1/rms: partial sums of squares of some other row vector stand for the norm's
-        sumsq = torch.rand((m + 3, 5), generator=torch.Generator().manual_seed(43)).cuda() * k
+    for tiles in (1, 2):
+        out = ops.gemm_shared_rows(w, ops.EPI_BF16, a, bias=b, column_tiles=tiles, waves=waves)
+        torch.testing.assert_close(out.double(), expect + b.double(), **tol)
+        for parts in (1, 3, 7):
+            rows = wide[:, :k] if parts == 3 else a
+            out = ops.gemm_shared_rows(w, ops.EPI_PARTIAL, rows, bias=b, column_tiles=tiles, waves=waves, k_parts=parts)
+            assert out.shape == (parts, m, n) and out.dtype == torch.float32
+            torch.testing.assert_close(out.double().sum(0), expect + b.double(), rtol=1e-4, atol=1e-4 * math.sqrt(k))
+    out = ops.gemm_shared_rows(w, ops.EPI_F32, a, bias=b, waves=waves)  # as for logits
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out.double(), expect + b.double(), rtol=1e-4, atol=1e-4 * math.sqrt(k))
+    gate, up = expect[:, : n // 2], expect[:, n // 2:]
+    out = ops.gemm_shared_rows(w, ops.EPI_SILU, a, waves=waves)
+    assert out.shape == (m, n // 2) and out.dtype == torch.bfloat16
+    torch.testing.assert_close(out.double(), torch.nn.functional.silu(gate) * up, rtol=2e-2, atol=2e-2)
+    # rows that lack their 1/rms: partial sums of squares of some other row vector stand for the norm's (a count
+    # that is no multiple of four, one that a lane holds at once, one that needs the loop behind it)
+    for sumsq_parts in (5, 8, 264):
+        sumsq = torch.rand((m + 3, sumsq_parts), generator=torch.Generator().manual_seed(43)).cuda() * k / sumsq_parts
         scale = torch.rsqrt(sumsq[:m].double().sum(1, keepdim=True) / k + 1e-5)
-        out = ops.gemm_shared_rows(w, ops.EPI_SILU, a, waves=waves, distance=distance, row_sumsq=sumsq, eps=1e-5)
+        out = ops.gemm_shared_rows(w, ops.EPI_SILU, a, waves=waves, row_sumsq=sumsq, eps=1e-5)
         torch.testing.assert_close(out.double(), torch.nn.functional.silu(gate * scale) * (up * scale), rtol=2e-2, atol=2e-2)
 
 
