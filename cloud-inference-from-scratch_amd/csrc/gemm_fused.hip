@@ -705,8 +705,8 @@ int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, const Fuse
 // 17 to 128 rows: waves that own columns and share the rows of A.
 //
 // With more than 16 rows the kernel above spends more of the memory pipeline on the rows of A (which
-// every wave fetches for its own slices of K) than on W.  Here the four waves of a workgroup take the
-// same slice of 128 k values together: the workgroup's 256 threads fetch the slice of A once (whole
+// every wave fetches for its own slices of K) than on W.  Here the two to four waves of a workgroup take the
+// same slice of 128 k values together: the workgroup's threads fetch the slice of A once (whole
 // 256-byte row segments) into LDS, every wave streams its own NT tiles of 16 columns of W over all of
 // K (or a grid.z part of it) and reads the rows of A from LDS in the MFMA layout.  A wave's loads run
 // one slice ahead of its products, in two sets of registers that the loop, unrolled by two, addresses by
