@@ -889,7 +889,9 @@ int launch_shared_rows_waves(hipStream_t s, int k_parts, const FusedArgs& a) {
     const int tiles = (cols + 15) / 16;
     const int per_workgroup = WAVES * ((EPI == EPI_SILU) ? 1 : NT);
     const dim3 grid((tiles + per_workgroup - 1) / per_workgroup, 1, k_parts);
-    if (a.M <= 32)
+    if (a.M <= 16)
+        gemm_shared_rows_kernel<EPI, 1, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
+    else if (a.M <= 32)
         gemm_shared_rows_kernel<EPI, 2, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
     else if (a.M <= 64)
         gemm_shared_rows_kernel<EPI, 4, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
