@@ -712,6 +712,16 @@ int launch(hipStream_t s, int row_tiles, int waves, int column_tiles, const Fuse
 // one slice ahead of its products, in two sets of registers that the loop, unrolled by two, addresses by
 // constants (a copy from a set whose load is still under way would wait for it; two slices ahead, with
 // three sets, were 1 to 3 us slower at every size).
+// Its LDS: one or two stages of the rows' slice, a staging area per wave, the rows' scales.  Two stages where
+// they fit the 160 KB of a workgroup (128 rows and four waves: 86 KB, more than a kernel gets without asking).
+template <int MT, int WAVES>
+struct SharedRowsLds {
+    static constexpr int kStageBytesA = MT * 16 * kStageRow;
+    static constexpr int kRest = WAVES * kStageTile + MT * 16 * static_cast<int>(sizeof(float));
+    static constexpr int kStagesA = 2 * kStageBytesA + kRest <= 160 * 1024 ? 2 : 1;
+    static constexpr int kBytes = kStagesA * kStageBytesA + kRest;
+};
+
 template <int EPI, int MT, int NT, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs a) {
     static_assert(EPI == EPI_SILU || EPI == EPI_PARTIAL || EPI == EPI_BF16 || EPI == EPI_F32, "epilogues of this form");
@@ -720,8 +730,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs 
     constexpr int kThreads = WAVES * 64;
     constexpr int kRows = MT * 16;
     constexpr int kStageBytesA = kRows * kStageRow;
-    constexpr int kStagesA = MT <= 4 ? 2 : 1;  // (two stages of 128 rows would pass the 64 KB of static LDS)
-    __shared__ __attribute__((aligned(16))) char shared[kStagesA * kStageBytesA + kWaves * kStageTile + kRows * sizeof(float)];
+    constexpr int kStagesA = SharedRowsLds<MT, WAVES>::kStagesA;
+    extern __shared__ __attribute__((aligned(16))) char shared[];  // SharedRowsLds<MT, WAVES>::kBytes of them
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
     const int r = lane & 15;
@@ -883,21 +893,34 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs 
     }
 }
 
+template <int EPI, int MT, int NT, int WAVES>
+int launch_shared_rows_tiles(hipStream_t s, dim3 grid, const FusedArgs& a) {
+    constexpr int kBytes = SharedRowsLds<MT, WAVES>::kBytes;
+    if (kBytes > 64 * 1024) {  // more than a kernel gets without asking: once per kernel (and again is harmless)
+        static bool asked = false;
+        if (!asked) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_shared_rows_kernel<EPI, MT, NT, WAVES>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, kBytes) != hipSuccess) {
+                (void)hipGetLastError();
+                return CIE_LAUNCH_FAILED;
+            }
+            asked = true;
+        }
+    }
+    gemm_shared_rows_kernel<EPI, MT, NT, WAVES><<<grid, WAVES * 64, kBytes, s>>>(a);
+    return cie_after_launch();
+}
+
 template <int EPI, int NT, int WAVES>
 int launch_shared_rows_waves(hipStream_t s, int k_parts, const FusedArgs& a) {
     const int cols = (EPI == EPI_SILU) ? a.up_offset : a.N;
     const int tiles = (cols + 15) / 16;
     const int per_workgroup = WAVES * ((EPI == EPI_SILU) ? 1 : NT);
     const dim3 grid((tiles + per_workgroup - 1) / per_workgroup, 1, k_parts);
-    if (a.M <= 16)
-        gemm_shared_rows_kernel<EPI, 1, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
-    else if (a.M <= 32)
-        gemm_shared_rows_kernel<EPI, 2, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
-    else if (a.M <= 64)
-        gemm_shared_rows_kernel<EPI, 4, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
-    else
-        gemm_shared_rows_kernel<EPI, 8, NT, WAVES><<<grid, WAVES * 64, 0, s>>>(a);
-    return cie_after_launch();
+    if (a.M <= 16) return launch_shared_rows_tiles<EPI, 1, NT, WAVES>(s, grid, a);
+    if (a.M <= 32) return launch_shared_rows_tiles<EPI, 2, NT, WAVES>(s, grid, a);
+    if (a.M <= 64) return launch_shared_rows_tiles<EPI, 4, NT, WAVES>(s, grid, a);
+    return launch_shared_rows_tiles<EPI, 8, NT, WAVES>(s, grid, a);
 }
 
 template <int EPI, int NT>
@@ -1020,7 +1043,7 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
     return launch_waves<EPI_ROPE, 4, 2>(s, waves, grid, f);
 }
 
-// The form for 17 to 128 rows in which a workgroup's four waves own columns and share the rows of A
+// The form for 17 to 128 rows in which a workgroup's waves own columns and share the rows of A
 // through LDS (one workgroup row: M <= 128).  epilogue 0 (bf16, + bias), 1 (float32, + bias; two tiles a wave),
 // 2 (SiLU-gate; row_sumsq as in
 // cie_gemm_fused, for any number of rows here) or 4 (k_parts partial products).  column_tiles 1 or 2 tiles of
