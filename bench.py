@@ -3,7 +3,7 @@
 (default: the 3B one) with random weights, plus prefill and roofline figures.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
-                    [--shape 3b|7b|14b] [--layers N] [--long-contexts 16384,32768]
+                    [--shape 3b|7b|14b|32b|72b] [--layers N] [--long-contexts 16384,32768]
 
 A "step" is one decode step of the whole engine (scheduler iteration: plan,
 step function, sampling, token hand-over).  Protocol after the reference's
@@ -26,6 +26,7 @@ ONE JSON line is printed.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import statistics
 import sys
@@ -175,7 +176,7 @@ def main(argv=None) -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=4096)
-    parser.add_argument("--shape", default="3b", choices=["3b", "7b", "14b"])
+    parser.add_argument("--shape", default="3b", choices=["3b", "7b", "14b", "32b", "72b"])
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
     parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     parser.add_argument("--prefill-tokens", type=int, default=2048)
@@ -200,13 +201,22 @@ def main(argv=None) -> int:
     elem = 2 if args.dtype == "bf16" else 4
     steps, warmup = args.steps, max(args.warmup, 1)
 
+    def release() -> None:
+        # (an engine's memory has to be back before the next engine is built: the large shapes fit once)
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    def say(text: str) -> None:
+        print(f"[bench] {text}", file=sys.stderr, flush=True)
+
     def point(batch: int, context: int):
         """(tokens/s of each measured window, the median window's ms per step and roofline share)."""
         context = min(context, config.max_position_embeddings - SLACK)  # (the last positions are the slack's)
+        say(f"decode, batch {batch}, context {context}")
         engine = make_engine(config, args.dtype, batch, context, args.prefill_tokens)
         measured = decode_windows(engine, config, batch, context, steps, warmup, seed=batch)
         del engine
-        torch.cuda.empty_cache()
+        release()
         rates = [batch * steps / seconds for seconds, _ in measured]
         seconds, mean_context = sorted(measured)[len(measured) // 2]
         achieved = decode_bytes(config, layers, batch, mean_context, elem) / (seconds / steps) / 1e9
@@ -244,10 +254,11 @@ def main(argv=None) -> int:
                      "frac": round(achieved / HBM_GBPS, 4)},
     }
     if not args.no_range and args.context > args.prefill_tokens + 1:
+        say(f"decode over the range {args.prefill_tokens} to {args.context}")
         engine = make_engine(config, args.dtype, args.batch, args.context, args.prefill_tokens)
         runs = decode_range(engine, config, args.batch, args.prefill_tokens, args.context, seed=7)
         del engine
-        torch.cuda.empty_cache()
+        release()
         range_rates = [args.batch * n / seconds for seconds, n in runs]
         seconds, n = sorted(runs)[len(runs) // 2]
         mean_context = (args.prefill_tokens + args.context) / 2.0
@@ -258,10 +269,11 @@ def main(argv=None) -> int:
             "ms_per_step": round(seconds / n * 1e3, 4), "frac": round(through / HBM_GBPS, 4),
         }
     if not args.no_prefill:
+        say(f"prefill of {args.prefill_tokens} tokens")
         engine = make_engine(config, args.dtype, 1, args.prefill_tokens + 1, args.prefill_tokens)
         seconds = time_prefill(engine, config, args.prefill_tokens, seed=99)
         del engine
-        torch.cuda.empty_cache()
+        release()
         median = statistics.median(seconds)
         flops = prefill_flops(config, layers, args.prefill_tokens)
         line["prefill"] = {

@@ -85,7 +85,10 @@ class DecoderModel:
             {self.spec.head_name: self.spec.embedding_name, "model." + self.spec.head_name: self.spec.embedding_name}
             if self.spec.tie_word_embeddings else {}
         )
-        tensors = source.load(expected, dtype, device, tied_optional=tied_optional)
+        # (a source that can hand out tensors one by one is asked to: the model then needs its own size of
+        # device memory and one layer's tensors, not twice its size)
+        take = getattr(source, "open", None) or source.load
+        tensors = take(expected, dtype, device, tied_optional=tied_optional)
         self.embedding = tensors[self.spec.embedding_name].contiguous()
         self.head = self.embedding if self.spec.tie_word_embeddings else tensors[self.spec.head_name].contiguous()
         self.final_norm.bind(tensors, self.spec.final_norm_name + ".", self.dtype, device)

@@ -84,9 +84,11 @@ class SafetensorsSource:
                     index[key] = (path, tuple(handle.get_slice(key).get_shape()))
         return index
 
-    def load(self, expected: Mapping[str, TensorSpec], dtype: str, device: str | torch.device,
-             tied_optional: Mapping[str, str] | None = None) -> dict[str, torch.Tensor]:
-        """``tied_optional`` maps a tensor name that may be present although the
+    def open(self, expected: Mapping[str, TensorSpec], dtype: str, device: str | torch.device,
+             tied_optional: Mapping[str, str] | None = None) -> "TensorsOnDemand":
+        """Check names and shapes of the whole folder against ``expected`` (one
+        :class:`WeightError` for all faults), then hand out tensors as they are asked
+        for.  ``tied_optional`` maps a tensor name that may be present although the
         model does not use it (a tied head) to the tensor it must equal."""
         import safetensors
 
@@ -103,31 +105,57 @@ class SafetensorsSource:
             raise WeightError(missing, unexpected, wrong)
 
         target = torch_dtype(dtype)
-        present_twins = {twin for name, twin in tied_optional.items() if name in index}
-        by_path: dict[Path, list[str]] = {}
-        for name in list(expected) + [n for n in tied_optional if n in index]:
-            by_path.setdefault(index[name][0], []).append(name)
-        out: dict[str, torch.Tensor] = {}
-        stored: dict[str, torch.Tensor] = {}  # raw copies needed for the tied-head check only
-        for path, names in by_path.items():
-            with safetensors.safe_open(str(path), framework="pt", device="cpu") as handle:
-                for name in names:
-                    tensor = handle.get_tensor(name)
-                    if name in expected:
-                        spec = expected[name]
-                        out[name] = tensor.to(_target_dtype(spec, tensor.dtype, target)).to(device)
-                    if name in tied_optional or name in present_twins:
-                        stored[name] = tensor
-        problems = [
-            f"{name} is present in a tied model but differs from {twin}"
-            for name, twin in tied_optional.items()
-            if name in stored
-            and (twin not in stored or stored[twin].shape != stored[name].shape
-                 or not torch.equal(stored[twin], stored[name]))
-        ]
+        handles: dict[Path, Any] = {}
+
+        def stored(name: str) -> torch.Tensor:
+            path = index[name][0]
+            if path not in handles:
+                handles[path] = safetensors.safe_open(str(path), framework="pt", device="cpu")
+            return handles[path].get_tensor(name)
+
+        problems = []
+        for name, twin in tied_optional.items():
+            if name in index and (twin not in index or index[twin][1] != index[name][1]
+                                  or not torch.equal(stored(twin), stored(name))):
+                problems.append(f"{name} is present in a tied model but differs from {twin}")
         if problems:
             raise WeightError([], [], [], problems)
-        return out
+
+        def make(name: str) -> torch.Tensor:
+            tensor = stored(name)
+            return tensor.to(_target_dtype(expected[name], tensor.dtype, target)).to(device)
+
+        return TensorsOnDemand(expected, make)
+
+    def load(self, expected: Mapping[str, TensorSpec], dtype: str, device: str | torch.device,
+             tied_optional: Mapping[str, str] | None = None) -> dict[str, torch.Tensor]:
+        """All tensors of :meth:`open` at once, as a dictionary."""
+        return dict(self.open(expected, dtype, device, tied_optional).items())
+
+
+class TensorsOnDemand(Mapping):
+    """Name → tensor on the target device, made when it is asked for and not kept.
+
+    A model binds its tensors one after the other and keeps its own forms of some
+    (q/k/v as one matrix, gate and up as one); with every tensor made at its turn the
+    checkpoint's tensors and the model's never lie side by side in device memory in
+    full, so a model may take more than half of it."""
+
+    def __init__(self, names, make) -> None:
+        self._names = tuple(names)
+        self._known = frozenset(self._names)
+        self._make = make
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        if name not in self._known:
+            raise KeyError(name)
+        return self._make(name)
+
+    def __iter__(self):
+        return iter(self._names)
+
+    def __len__(self) -> int:
+        return len(self._names)
 
 
 class RandomSource:
@@ -157,14 +185,22 @@ class RandomSource:
             raise ValueError(f"unknown init {spec.init!r}")
         return values
 
+    def open(self, expected: Mapping[str, TensorSpec], dtype: str, device: str | torch.device,
+             tied_optional: Mapping[str, str] | None = None) -> TensorsOnDemand:
+        """Tensors drawn as they are asked for (each from its own seed, so the order of asking does not matter)."""
+        target = torch_dtype(dtype)
+        place = {name: index for index, name in enumerate(expected)}
+
+        def make(name: str) -> torch.Tensor:
+            spec = expected[name]
+            return self.draw(place[name], spec).to(_target_dtype(spec, torch.bfloat16, target)).to(device)
+
+        return TensorsOnDemand(expected, make)
+
     def load(self, expected: Mapping[str, TensorSpec], dtype: str, device: str | torch.device,
              tied_optional: Mapping[str, str] | None = None) -> dict[str, torch.Tensor]:
-        target = torch_dtype(dtype)
-        out = {}
-        for index, (name, spec) in enumerate(expected.items()):
-            tensor = self.draw(index, spec)
-            out[name] = tensor.to(_target_dtype(spec, torch.bfloat16, target)).to(device)
-        return out
+        """All tensors of :meth:`open` at once, as a dictionary."""
+        return dict(self.open(expected, dtype, device, tied_optional).items())
 
 
 def write_model_folder(model_dir: str | Path, config: Any, seed: int,

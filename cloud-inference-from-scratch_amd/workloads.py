@@ -33,6 +33,11 @@ SHAPES: dict[str, dict[str, Any]] = {
                intermediate_size=18944, vocab_size=152064, rms_norm_eps=1e-6, tie_word_embeddings=False),
     "14b": dict(_COMMON, hidden_size=5120, num_hidden_layers=48, num_attention_heads=40, num_key_value_heads=8,
                 intermediate_size=13824, vocab_size=152064, rms_norm_eps=1e-5, tie_word_embeddings=False),
+    # the family's two largest: 65 and 145 GB of bf16 weights, for one GPU's 288 GB
+    "32b": dict(_COMMON, hidden_size=5120, num_hidden_layers=64, num_attention_heads=40, num_key_value_heads=8,
+                intermediate_size=27648, vocab_size=152064, rms_norm_eps=1e-5, tie_word_embeddings=False),
+    "72b": dict(_COMMON, hidden_size=8192, num_hidden_layers=80, num_attention_heads=64, num_key_value_heads=8,
+                intermediate_size=29568, vocab_size=152064, rms_norm_eps=1e-5, tie_word_embeddings=False),
 }
 
 

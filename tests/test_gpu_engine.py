@@ -350,3 +350,29 @@ def test_command_line_generates(tiny_folders, tmp_path):
         capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stderr[-2000:]
     assert '"completed_total": 1' in done.stdout
+
+
+@pytest.mark.parametrize("from_folder", [False, True])
+def test_loading_needs_the_models_own_size_of_device_memory_not_twice(tmp_path, from_folder):
+    """A model's tensors are made one by one while it binds them (its own forms of some are copies: q/k/v as one
+    matrix, gate and up as one), so loading peaks at the model's size plus a layer's tensors."""
+    from cie_amd.config import config_from_dict
+    from cie_amd.engine.loading import load_model, random_model
+    from cie_amd.weights import write_model_folder
+
+    raw = dict(TINY["A"], hidden_size=512, intermediate_size=2048, num_attention_heads=8, num_key_value_heads=2,
+               head_dim=64, num_hidden_layers=12, vocab_size=1024)
+    config = config_from_dict(raw)
+    if from_folder:
+        write_model_folder(tmp_path, config, seed=2)
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    before = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    model = load_model(tmp_path, "bfloat16")[0] if from_folder else random_model(config, 2, draw_device="cuda")
+    held = torch.cuda.memory_allocated() - before
+    peak = torch.cuda.max_memory_allocated() - before
+    per_layer = held / raw["num_hidden_layers"]
+    assert held > 80e6  # (about 90 MB: the check below is about something)
+    assert peak < held + 4 * per_layer, (held, peak)
+    del model

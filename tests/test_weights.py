@@ -123,3 +123,25 @@ def test_tensor_stored_in_32_bit_stays_so(tmp_path):
     assert torch.equal(loaded["model.norm.weight"], tensors["model.norm.weight"])
     assert loaded["model.layers.0.input_layernorm.weight"].dtype == torch.bfloat16
     assert loaded["model.embed_tokens.weight"].dtype == torch.bfloat16
+
+
+def test_open_hands_out_tensors_one_by_one_and_checks_the_folder_first(tmp_path):
+    config = config_from_dict(TINY_B)
+    write_model_folder(tmp_path, config, seed=5)
+    expected = expected_of(TINY_B)
+    for source in (SafetensorsSource(tmp_path), RandomSource(5)):
+        whole = source.load(expected, "bfloat16", "cpu")
+        lazy = source.open(expected, "bfloat16", "cpu")
+        assert list(lazy) == list(expected) and len(lazy) == len(expected)
+        name = "model.layers.1.mlp.down_proj.weight"
+        first, second = lazy[name], lazy[name]
+        assert torch.equal(first, whole[name]) and first is not second  # made anew each time, not kept
+        assert all(torch.equal(lazy[n], whole[n]) for n in reversed(list(expected)))  # in any order
+        with pytest.raises(KeyError):
+            lazy["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    # the folder's faults are reported when it is opened, before a tensor is asked for
+    tensors = RandomSource(5).load(expected, "bfloat16", "cpu")
+    del tensors["model.norm.weight"]
+    write_tensors(tmp_path / "short", TINY_B, tensors)
+    with pytest.raises(WeightError, match="missing tensors"):
+        SafetensorsSource(tmp_path / "short").open(expected, "bfloat16", "cpu")
