@@ -1,13 +1,15 @@
 // True float32 matrix product for the 32-bit path: C = A * W^T (+ bias).
 //   A [M, K] row-major (row stride lda), W [N, K] row-major (a Linear's weight), C [M, N].
 // Plain fused multiply-adds in float32, no matrix-core reduced-precision mode.
-// Every output element is one sequential sum over k, so a row's result does not
-// depend on how many other rows are in the batch.
+// Every output element is a sum over k in one fixed order (blocks of 256 k summed one after the other, the
+// blocks' sums added in turn: the rounding error grows with 256 + K/256 terms, not with K), so a row's result
+// does not depend on how many other rows are in the batch.
 // 64x64 output tile per workgroup, 16-deep k slices through LDS, 4x4 per thread.
 #include "common.h"
 
 namespace {
 constexpr int BM = 64, BN = 64, BK = 16;
+constexpr int kSlicesPerBlock = 16;  // 256 k: a block's sum joins the total
 }
 
 __global__ void __launch_bounds__(256)
@@ -20,7 +22,8 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
     const int n0 = blockIdx.x * BN;
     const int tx = threadIdx.x % 16;
     const int ty = threadIdx.x / 16;
-    float acc[4][4] = {};
+    float acc[4][4] = {}, total[4][4] = {};
+    int slice = 0;
     for (int k0 = 0; k0 < K; k0 += BK) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -46,6 +49,16 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
         }
+        if (++slice == kSlicesPerBlock) {
+            slice = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    total[i][j] += acc[i][j];
+                    acc[i][j] = 0.f;
+                }
+        }
         __syncthreads();
     }
 #pragma unroll
@@ -55,7 +68,7 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W,
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int n = n0 + tx * 4 + j;
-            if (n < N) C[static_cast<size_t>(m) * ldc + n] = acc[i][j] + (bias ? bias[n] : 0.f);
+            if (n < N) C[static_cast<size_t>(m) * ldc + n] = (total[i][j] + acc[i][j]) + (bias ? bias[n] : 0.f);
         }
     }
 }
