@@ -69,7 +69,24 @@ class EngineConfig:
         return config
 
 
+# The reference's names (src/cloud_engine/config.py:25-48) of the options that this engine has under a name of
+# its own: both are taken, with the same meaning.
+REFERENCE_NAMES = {
+    "max_active_sequences": "max_running",
+    "max_batched_tokens": "token_budget",
+    "prefill_chunk_size": "prefill_chunk",
+    "block_size": "page_size",
+    "prefix_cache_max_blocks": "prefix_cache_pages",
+    "cuda_graph_decode": "graph_decode",
+}
+
+
 def build_engine_config(base: EngineConfig | None = None, **overrides: Any) -> EngineConfig:
+    for theirs, ours in REFERENCE_NAMES.items():
+        if theirs in overrides:
+            if ours in overrides:
+                raise ValueError(f"{theirs} and {ours} name the same option: give one")
+            overrides[ours] = overrides.pop(theirs)
     known = {item.name for item in fields(EngineConfig)}
     unknown = set(overrides) - known
     if unknown:

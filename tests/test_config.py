@@ -103,6 +103,19 @@ def test_engine_options():
         build_engine_config(token_budget=0)
 
 
+def test_engine_options_under_the_references_names():
+    """src/cloud_engine/config.py:25-48 names six of the options otherwise; both names mean the same."""
+    theirs = build_engine_config(max_active_sequences=5, max_batched_tokens=96, prefill_chunk_size=24, block_size=8,
+                                 prefix_cache_max_blocks=7, cuda_graph_decode=False, kv_cache_bytes=1 << 20)
+    ours = build_engine_config(max_running=5, token_budget=96, prefill_chunk=24, page_size=8, prefix_cache_pages=7,
+                               graph_decode=False, kv_cache_bytes=1 << 20)
+    assert theirs == ours
+    with pytest.raises(ValueError, match="block_size and page_size name the same option"):
+        build_engine_config(block_size=8, page_size=16)
+    with pytest.raises(ValueError, match="max_batched_tokens|token_budget"):
+        build_engine_config(max_batched_tokens=0)
+
+
 def test_another_architecture_registers_without_touching_the_package():
     class ToyConfig(Qwen2Config):
         architecture = "ToyForCausalLM"
