@@ -535,7 +535,7 @@ def test_trace_run_takes_many_short_requests_and_names_a_step_that_does_not_fit(
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape,layers,vocab", [("0.5b", 2, None), ("3b", 1, None), ("7b", 1, 20011), ("72b", 1, 8209)])
+@pytest.mark.parametrize("shape,layers,vocab", [("0.5b", 2, None), ("3b", 1, None), ("7b", 1, 20011), ("14b", 1, 20011), ("72b", 1, 8209)])
 def test_replay_at_the_sizes_of_real_models(tmp_path_factory, shape, layers, vocab, dtype):
     """The widths, head counts and vocabulary of models of the family (few layers,
     random weights; the largest with a short vocabulary, to keep its files small): the
