@@ -632,3 +632,56 @@ def test_replay_with_the_keys_of_prompt_portions_cut(tiny_folders, monkeypatch):
     replay_util.compare(rows, expected, **TOL["bfloat16"])
     assert any(per_tile > 1 and splits > 1 for per_tile, splits in seen), seen
     assert runner.cache.stats().pages_used == 0
+
+
+@pytest.fixture(scope="module")
+def long_context_case(tmp_path_factory):
+    """(folder, raw, requests, plain float32 logits, plain bfloat16 logits) of the 6,040-token case, made once."""
+    from conftest import make_folder
+
+    raw = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_size=256, num_hidden_layers=2,
+               num_attention_heads=4, num_key_value_heads=1, head_dim=128, intermediate_size=520, vocab_size=1003,
+               rms_norm_eps=1e-6, rope_theta=1e6, max_position_embeddings=8192, tie_word_embeddings=True,
+               attention_bias=True, use_sliding_window=False, eos_token_id=1002)
+    folder, tensors = make_folder(tmp_path_factory.mktemp("long_context"), raw, seed=41, factor=6.0)
+    requests = {"long": random_tokens(6040, raw["vocab_size"], seed=17), "short": random_tokens(90, raw["vocab_size"], seed=18)}
+    weights = {k: v.float() for k, v in tensors.items()}
+    expected = {rid: plain_qwen2.forward(raw, weights, tokens) for rid, tokens in requests.items()}
+    rough = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
+    return folder, raw, requests, expected, rough
+
+
+@pytest.mark.parametrize("dtype,graphs", [("float32", False), ("bfloat16", False), ("bfloat16", True)])
+def test_replay_of_a_context_of_six_thousand_tokens(long_context_case, dtype, graphs):
+    """Thousands of keys behind a token, through the engine and not only through the attention kernel: a prompt of
+    6,000 tokens in portions of up to 2,048 (the later ones behind thousands of keys, their keys cut into parts), its
+    last tokens one by one beside another request's portion and single tokens (keys of a single token cut into
+    parts by the longest context of the step).  Heads of 128 as in the family's models, queries and keys scaled so
+    that a token attends to a few keys anywhere in its context: a lost or misplaced block of far keys moves the logits.
+    Once more with the steps of single tokens replayed from a captured graph."""
+    folder, raw, requests, expected, rough = long_context_case
+    long, short = requests["long"], requests["short"]
+    steps = []
+
+    def step(entries, end=()):
+        steps.append({"step": len(steps), "end": list(end),
+                      "entries": [{"id": rid, "tokens": tokens, "want": want} for rid, tokens, want in entries]})
+
+    step([("long", long[:2048], [0, 1000, 2047])])
+    step([("long", long[2048:4096], [0, 2047])])
+    step([("long", long[4096:5990], [3, 1893])])
+    step([("long", long[5990:6000], list(range(10))), ("short", short[:50], [49])])  # a short portion behind 5,990 keys
+    for i in range(40):
+        step([("long", [long[6000 + i]], [0]), ("short", [short[50 + i]], [0])], end=["long", "short"] if i == 39 else [])
+    runner = make_runner(folder, dtype, replay_util.max_live_tokens(steps, page=16), 16, graph_decode=graphs)
+    rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+    assert len(rows["long"]) == 3 + 2 + 2 + 10 + 40 and len(rows["short"]) == 41
+    if graphs:
+        assert runner.graph_captures == 1 and runner.graph_replays >= 39, (runner.graph_captures, runner.graph_replays)
+    if dtype == "float32":
+        worst = replay_util.compare(rows, expected, every_position=False, **F32_TOL)
+        print(f"6,040 tokens float32: worst |diff| {worst:.3e}", flush=True)
+    else:
+        print("6,040 tokens bfloat16: rms %.3e worst %.3e, plain in bfloat16 %.3e %.3e"
+              % replay_util.closer_than_plain_bfloat16(rows, expected, rough), flush=True)
+    assert runner.cache.stats().pages_used == 0
