@@ -38,13 +38,6 @@ using Key = std::tuple<int, int, int, int, int, int>;  // M, N, K, lda, has bias
 
 hipblasLtHandle_t g_handle = nullptr;
 std::map<Key, Plan> g_plans;
-// Row counts that share a timing: the algorithm that won for the first row count of a group (the library's index
-// of it) serves the group's other row counts, so that a server whose steps bring every row count between two
-// sizes times a few dozen shapes and not a few thousand.  A group holds a few winners: an algorithm that loads
-// two rows at a time does not run on an odd row count, which then times for itself and for the odd ones after it.
-using GroupKey = std::tuple<int, int, int, int, int>;  // group's rows, N, K, has bias, float32 result
-constexpr size_t kGroupWinners = 4;
-std::map<GroupKey, std::vector<hipblasLtMatmulAlgo_t>> g_group_choices;
 std::mutex g_mutex;
 
 bool ok(hipblasStatus_t status) { return status == HIPBLAS_STATUS_SUCCESS; }
@@ -78,7 +71,8 @@ int make_plan(Plan& plan, Found& found, int M, int N, int K, int lda, const void
         const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
         const hipDataType bias_type = HIP_R_16BF;
         // (the pointer too: asked whether it can run an algorithm on a product with a bias and no pointer to it, the
-        // library answers "invalid value"; every call sets its own pointer again)
+        // library answers "invalid value", and a search over all its algorithms finds none; every call sets its
+        // own pointer again)
         good = ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue))) &&
                ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type))) &&
                ok(hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)));
@@ -316,37 +310,17 @@ int fastest(const Plan& plan, const Found& found, int proposed, hipStream_t stre
     return best;
 }
 
-// A copy of `winner` (an algorithm that another row count of the same product chose) fitted to the plan's
-// shape, if the library can run it there within the workspace.
-bool fitted(const Plan& plan, const hipblasLtMatmulAlgo_t& winner, size_t workspace_limit,
-            hipblasLtMatmulHeuristicResult_t& out) {
-    out = hipblasLtMatmulHeuristicResult_t{};
-    out.algo = winner;
-    const float one = 1.f, zero = 0.f;
-    size_t needs = 0;
-    if (!ok(hipblaslt_ext::matmulIsAlgoSupported(g_handle, plan.desc, &one, plan.w, plan.a, &zero, plan.d, plan.d, out.algo,
-                                                 needs)) ||
-        needs > workspace_limit)
-        return false;
-    out.workspaceSize = needs;
-    out.state = HIPBLAS_STATUS_SUCCESS;
-    return true;
-}
-
 }  // namespace
 
 // With `tune` 1, a shape's first call (outside graph capture) times the heuristic's candidates on the call's
 // own rows and on copies of its weight (device memory of its own, freed again) and keeps the fastest; with
 // `tune` 2 it times every algorithm the library can run on the shape (a few seconds); with 0 the heuristic's
-// first choice is kept.  `group_rows` > 0 names a group of row counts that share one timing: the first of
-// them to come is timed as `tune` says; the others time its winner (if the library can run it on their shape)
-// against the heuristic's first choice for theirs, and nothing else.
+// first choice is kept.
 // Returns CIE_BAD_ARGUMENT for a shape the library has no algorithm for (the caller then takes another
 // route) and CIE_LAUNCH_FAILED if the library's call itself fails.  `workspace` is device memory of
 // `workspace_bytes` that stays valid while the product runs; calls on one stream may share it.
 CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w, const void* bias, void* c, int M,
-                             int N, int K, int f32_out, void* workspace, size_t workspace_bytes, int tune,
-                             int group_rows) {
+                             int N, int K, int f32_out, void* workspace, size_t workspace_bytes, int tune) {
     if (M <= 0 || N <= 0 || K <= 0 || lda < K || !a || !w || !c || (f32_out && bias)) return CIE_BAD_ARGUMENT;
     Plan* plan = nullptr;
     {
@@ -367,43 +341,16 @@ CIE_API int cie_gemm_library(void* stream, const void* a, int lda, const void* w
                 return CIE_BAD_ARGUMENT;
             }
             int chosen = 0;
-            const GroupKey group{group_rows, N, K, bias ? 1 : 0, f32_out ? 1 : 0};
-            // the heuristic's first choice and the group's winners that run on this shape
-            Found few;
-            bool from_group = false;
-            if (group_rows > 0 && may_time) {
-                few.push_back(found[0]);
-                for (const hipblasLtMatmulAlgo_t& winner : g_group_choices[group]) {
-                    hipblasLtMatmulHeuristicResult_t shared;
-                    if (!fitted(fresh, winner, workspace ? workspace_bytes : 0, shared)) continue;
-                    from_group = true;
-                    bool twice = false;
-                    for (auto& have : few) twice = twice || hipblaslt_ext::getIndexFromAlgo(have.algo) == hipblaslt_ext::getIndexFromAlgo(shared.algo);
-                    if (!twice) few.push_back(shared);
-                }
-            }
-            const hipStream_t on = static_cast<hipStream_t>(stream);
-            if (from_group) {
-                // What won at one row count of a group can lose at another (a tile more, a last tile nearly empty):
-                // the winners are timed against the heuristic's first choice, a few candidates instead of all.
-                found = few;
-                if (found.size() > 1)
-                    chosen = fastest(fresh, found, static_cast<int>(found.size()), on, a, w, size_t(N) * K * 2, c, workspace,
-                                     M >= 512, size_t(M) * N, f32_out != 0);
-            } else if (may_time && found.size() > 1) {
+            if (may_time && found.size() > 1) {
                 // short products are timed over more runs: their times scatter more
-                chosen = fastest(fresh, found, proposed, on, a, w, size_t(N) * K * 2, c, workspace, M >= 512, size_t(M) * N,
-                                 f32_out != 0);
-                if (group_rows > 0 && g_group_choices[group].size() < kGroupWinners)
-                    g_group_choices[group].push_back(found[chosen].algo);
+                chosen = fastest(fresh, found, proposed, static_cast<hipStream_t>(stream), a, w, size_t(N) * K * 2, c,
+                                 workspace, M >= 512, size_t(M) * N, f32_out != 0);
             }
             fresh.algo = found[chosen].algo;
             fresh.workspace = found[chosen].workspaceSize;
             if (getenv("CIE_LIBRARY_REPORT"))  // which algorithm a shape got, for whoever reads a profile
-                fprintf(stderr, "[cie_amd library] %d x %d x %d: candidate %d of %zu (%d proposed%s), index %d: %s\n", M, N, K,
-                        chosen, found.size(), proposed, from_group ? ": the heuristic's first and its group's" : "",
-                        hipblaslt_ext::getIndexFromAlgo(fresh.algo),
-                        hipblaslt_ext::getKernelNameFromAlgo(g_handle, fresh.algo).c_str());
+                fprintf(stderr, "[cie_amd library] %d x %d x %d: candidate %d of %zu (%d proposed): %s\n", M, N, K, chosen,
+                        found.size(), proposed, hipblaslt_ext::getKernelNameFromAlgo(g_handle, fresh.algo).c_str());
             it = g_plans.emplace(key, fresh).first;
         }
         plan = &it->second;

@@ -580,24 +580,14 @@ LIBRARY_TUNE_ROWS = 512
 # Row counts whose products time every algorithm the library has, not only the heuristic's candidates (a few
 # seconds for each shape, once in a process): an engine names the sizes of its full prompt portions here.
 LIBRARY_SEARCH_ROWS: set[int] = set()
-# Other row counts above the hand-written kernels' 128 share a timing in groups of this many (129..192, 193..256,
-# ...): the first of a group to come times the heuristic's candidates (a few hundredths of a second for a
-# shape), the others take its winner.  Steps that bring a prompt portion beside a changing number of single
-# tokens meet every row count; the heuristic's first choice is 5 to 15 % behind the timed one at many of them.
-LIBRARY_GROUP_ROWS = 64
 
 
-def _tune_level(rows: int) -> tuple[int, int]:
-    """(how the library's algorithm for products of ``rows`` rows is chosen at their first call: 0 its
-    heuristic's first, 1 the fastest of the heuristic's candidates, 2 the fastest of all it has; the group of
-    row counts that share the choice, named by its largest, or 0: the row count alone)."""
+def _tune_level(rows: int) -> int:
     if rows >= LIBRARY_TUNE_ROWS and rows in LIBRARY_SEARCH_ROWS:
-        return 2, 0
+        return 2
     if (rows >= LIBRARY_TUNE_ROWS and rows % 256 == 0) or (rows >= 32 and rows & (rows - 1) == 0):
-        return 1, 0
-    if rows > 128:
-        return 1, -(-rows // LIBRARY_GROUP_ROWS) * LIBRARY_GROUP_ROWS
-    return 0, 0
+        return 1
+    return 0
 
 
 def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -626,10 +616,10 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
         # cleared once: algorithms that meet through flags in the workspace leave them cleared after each call
         workspace = _WORKSPACES[device] = torch.zeros(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
     out = torch.empty((m, n), dtype=out_dtype, device=device)
-    tune, group = _tune_level(m)
     code = load_library().cie_gemm_library(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k),
-        _i(1 if out_dtype == torch.float32 else 0), _ptr(workspace), workspace.numel(), _i(tune), _i(group))
+        _i(1 if out_dtype == torch.float32 else 0), _ptr(workspace), workspace.numel(),
+        _i(_tune_level(m)))
     if code == 1:
         return None
     _run("cie_gemm_library", code)

@@ -186,6 +186,8 @@ def main(argv: list[str] | None = None) -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--requests", type=int, default=None, help="another number of requests than the profile's")
+    parser.add_argument("--prefill-chunk", type=int, default=None, help="another portion size than the profile's")
+    parser.add_argument("--token-budget", type=int, default=None, help="another token budget than the profile's")
     parser.add_argument("--verify", type=int, default=0, metavar="N",
                         help="afterwards run the first N requests alone and compare their tokens "
                              "(float32: must be equal; bfloat16: reported)")
@@ -195,6 +197,12 @@ def main(argv: list[str] | None = None) -> int:
         if args.requests < 1:
             parser.error("--requests must be positive")
         profile = replace(profile, requests=args.requests, lead_requests=min(profile.lead_requests, args.requests))
+    for option in ("prefill_chunk", "token_budget"):
+        value = getattr(args, option)
+        if value is not None:
+            if value < 1:
+                parser.error(f"--{option.replace('_', '-')} must be positive")
+            profile = replace(profile, **{option: value})
     record = run_profile(profile, layers=args.layers, dtype=args.dtype, seed=args.seed, shape=args.shape,
                          verify=args.verify)
     print(json.dumps(record))
