@@ -29,12 +29,14 @@ def _engine_options(parser: argparse.ArgumentParser) -> None:
                         help="instead of --model: a config.json to run with seeded random weights")
     parser.add_argument("--seed", type=int, default=0, help="seed of random weights and of sampling")
     parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32", "bfloat16", "float32"])
-    parser.add_argument("--page-size", type=int, default=16)
+    # (engine options that are not given keep the engine's defaults)
+    parser.add_argument("--page-size", type=int, default=None, help="tokens per cache page (a power of two)")
     parser.add_argument("--kv-tokens", type=int, default=None, help="cache pool size in tokens")
-    parser.add_argument("--token-budget", type=int, default=2048)
-    parser.add_argument("--prefill-chunk", type=int, default=256)
-    parser.add_argument("--max-running", type=int, default=16)
-    parser.add_argument("--max-model-len", type=int, default=4096)
+    parser.add_argument("--kv-pages", type=int, default=None, help="cache pool size in pages, instead of --kv-tokens")
+    parser.add_argument("--token-budget", type=int, default=None, help="most tokens in a step")
+    parser.add_argument("--prefill-chunk", type=int, default=None, help="most tokens of one prompt in a step")
+    parser.add_argument("--max-running", type=int, default=None, help="most requests that hold cache at a time")
+    parser.add_argument("--max-model-len", type=int, default=None)
 
 
 def parser() -> argparse.ArgumentParser:
@@ -74,9 +76,16 @@ def _make_engine(args: argparse.Namespace):
     from .config import config_from_dict
     from .engine import Engine
 
-    options = dict(dtype=args.dtype, page_size=args.page_size, kv_tokens=args.kv_tokens,
-                   token_budget=args.token_budget, prefill_chunk=args.prefill_chunk,
-                   max_running=args.max_running, max_model_len=args.max_model_len, seed=args.seed)
+    from .config.engine_config import EngineConfig
+
+    if args.kv_pages is not None and args.kv_tokens is not None:
+        raise SystemExit("cie: --kv-pages and --kv-tokens both size the cache pool: give one")
+    options = dict(dtype=args.dtype, seed=args.seed)
+    for name in ("page_size", "kv_tokens", "token_budget", "prefill_chunk", "max_running", "max_model_len"):
+        if getattr(args, name) is not None:
+            options[name] = getattr(args, name)
+    if args.kv_pages is not None:
+        options["kv_tokens"] = args.kv_pages * options.get("page_size", EngineConfig.page_size)
     if args.random_weights:
         with open(args.random_weights, encoding="utf-8") as handle:
             config = config_from_dict(json.load(handle))

@@ -346,10 +346,14 @@ def test_command_line_generates(tiny_folders, tmp_path):
     assert done.returncode == 0 and (out_dir / "model.safetensors").is_file() and (out_dir / "config.json").is_file()
     done = subprocess.run(
         [sys.executable, str(ROOT / "bin" / "cie"), "generate", "--token-ids", "1,2,3", "--model", str(out_dir),
-         "--max-output-tokens", "4", "--temperature", "0.8", "--seed", "3", "--metrics", "--max-model-len", "64"],
+         "--max-output-tokens", "4", "--temperature", "0.8", "--seed", "3", "--metrics", "--max-model-len", "64",
+         "--kv-pages", "12", "--page-size", "8"],
         capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stderr[-2000:]
-    assert '"completed_total": 1' in done.stdout
+    assert '"completed_total": 1' in done.stdout and '"pages_total": 12' in done.stdout
+    done = subprocess.run([sys.executable, str(ROOT / "bin" / "cie"), "generate", "--token-ids", "1", "--model", str(out_dir),
+                           "--kv-pages", "12", "--kv-tokens", "96"], capture_output=True, text=True, timeout=300)
+    assert done.returncode != 0 and "give one" in done.stderr
 
 
 @pytest.mark.parametrize("from_folder", [False, True])
