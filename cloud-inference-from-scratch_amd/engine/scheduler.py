@@ -88,6 +88,10 @@ class Scheduler:
                              and self._launch is not None and self._launchable is not None)
         self._flying: _InFlight | None = None
         self._collecting = False
+        # a step has just failed for want of pages and one request has given way: nobody is let in until
+        # those that stayed have run a step (else the one that gave way comes straight back, the step fails
+        # again, and so on for ever if the guard at admission errs on the side of room)
+        self._gave_way = False
 
     # ---------------------------------------------------------------- callers
     def submit(self, prompt: Sequence[int], gen: GenerationConfig, label: str = "",
@@ -151,17 +155,20 @@ class Scheduler:
         requests have taken what is known of them (plus the token each is about to sample)."""
         if self._free is None:
             return True
+        # (a request takes whole pages: one more token can cost a page)
+        page = max(1, int(getattr(self.config, "page_size", 1)))
+        whole_pages = lambda tokens: -(-tokens // page) * page
         spoken_for = 0
         for other in self.active:
             if other.is_final:
                 continue
             held = self._resident(other) if self._resident is not None else 0
-            spoken_for += max(0, other.known + 1 - held)
-        return self._free() - spoken_for >= request.known + 1
+            spoken_for += max(0, whole_pages(other.known + 1) - held)
+        return self._free() - spoken_for >= whole_pages(request.known + 1)
 
     def _admit(self) -> bool:
         moved = False
-        while self.waiting and len(self.active) < self.config.max_running:
+        while self.waiting and len(self.active) < self.config.max_running and not (self._gave_way and self.active):
             head = self.waiting[0]
             # A preempted request that came back the moment its own pages were free would take them from
             # the same requests again, for ever.  A newcomer that does not fit would push someone out or
@@ -208,6 +215,7 @@ class Scheduler:
             if not (_is_shortage(error) and self._make_room(error)):
                 self._fail_plan(plan, error)
             return
+        self._gave_way = False
         self._account(plan, sampled)
 
     def _start(self, plan: StepPlan) -> None:
@@ -221,6 +229,7 @@ class Scheduler:
             if not (_is_shortage(error) and self._make_room(error)):
                 self._fail_plan(plan, error)
             return
+        self._gave_way = False
         self._flying = _InFlight(plan, handle)
 
     def _fail_plan(self, plan: StepPlan, error: Exception) -> None:
@@ -339,6 +348,7 @@ class Scheduler:
         victim.state = RequestState.WAITING
         self.waiting.appendleft(victim)
         self.metrics.totals.preempted += 1
+        self._gave_way = True
         return True
 
     def _give_back(self, request: Request, preempted: bool = False) -> None:

@@ -62,7 +62,8 @@ class FakeRunner:
 
 
 def make(runner, **overrides):
-    options = dict(max_model_len=128, max_running=4, max_queue_size=8, token_budget=16, prefill_chunk=4)
+    # (the fake runners count tokens, not pages: a page of one token)
+    options = dict(max_model_len=128, max_running=4, max_queue_size=8, token_budget=16, prefill_chunk=4, page_size=1)
     options.update(overrides)
     return Scheduler(build_engine_config(**options), runner, Metrics())
 
@@ -505,7 +506,7 @@ def test_pages_that_only_the_prefix_index_holds_do_not_block_admission():
     manager = CacheManager([PagedKV(1, 8)], page_size=4, kv_tokens=64, max_running=8, max_model_len=64,
                            prefix_cache_pages=12)
     runner = ManagerRunner(manager)
-    scheduler = make(runner, max_model_len=64, max_running=8, token_budget=64, prefill_chunk=16)
+    scheduler = make(runner, max_model_len=64, max_running=8, token_budget=64, prefill_chunk=16, page_size=4)
     for i in range(3):  # three prompts of 17 tokens leave four full pages each
         scheduler.submit([i + 1] * 17, GenerationConfig(max_output_tokens=1))
     scheduler.run_until_done(50)
@@ -529,3 +530,51 @@ def test_a_cache_without_pages_admits_side_by_side():
     assert len(scheduler.active) == 4
     scheduler.run_until_done(50)
     assert runner.most_side_by_side == 4 and all(r.output == [100, 101, 102, 103] for r in requests)
+
+
+@pytest.mark.parametrize("seed", [3, 12, 21, 30])
+def test_pools_of_whole_pages_drain_under_random_loads(seed):
+    """Random prompts (half of them behind a common prefix), output lengths and arrivals through the real cache
+    manager with a pool of a few pages, a prefix index and both ways of admission.  A request takes whole pages, so
+    the room that admission reckons with has to be reckoned in pages, and a request that has just given way must
+    not come back before the others have run: else it is let in, the step fails for want of a page, it gives way
+    again, and nothing ever runs (seed 12 did exactly that, 1,883 times over, before this was seen to)."""
+    import random
+
+    from cie_amd.cache.manager import CacheManager, PagedKV
+
+    rng = random.Random(seed)
+    limit, vocab = 128, 256
+    prefix = [rng.randrange(vocab) for _ in range(40)]
+    requests = []
+    for _ in range(60):
+        n = rng.randint(1, limit // 2)
+        prompt = prefix[: rng.randint(0, min(40, n - 1))] if rng.random() < 0.5 and n > 1 else []
+        prompt = prompt + [rng.randrange(vocab) for _ in range(n - len(prompt))]
+        out = rng.randint(1, min(40, limit - n - 1))
+        rng.choice([0.0, 0.0, 0.7, 1.3])
+        requests.append((prompt, GenerationConfig(max_output_tokens=out, eos_token_id=rng.choice([None, None, rng.randrange(vocab)]))))
+        rng.randrange(1000)
+    page, running = rng.choice([4, 8, 16]), rng.choice([4, 8, 16])
+    budget, chunk, within = rng.choice([32, 64, 256]), rng.choice([7, 16, 64]), rng.random() < 0.5
+    manager = CacheManager([PagedKV(2, 16)], page_size=page, kv_tokens=3 * limit, max_running=running, max_model_len=limit,
+                           prefix_cache_pages=16)
+    runner = ManagerRunner(manager)
+    runner.publish_prefix = lambda request: manager.publish_prefix(request.request_id, request.prompt)
+    scheduler = make(runner, page_size=page, kv_tokens=3 * limit, max_running=running, max_queue_size=100, max_model_len=limit,
+                     max_output_tokens=64, token_budget=budget, prefill_chunk=chunk, prefix_cache_pages=16,
+                     admit_within_pool=within)
+    handles, pending, steps = [], list(requests), 0
+    while pending or scheduler.has_work():
+        for _ in range(rng.randint(0, 3)):
+            if pending:
+                prompt, gen = pending.pop(0)
+                handles.append(scheduler.submit(prompt, gen))
+        scheduler.step()
+        steps += 1
+        assert steps < 2000, ("the scheduler does not drain", page, running, budget, chunk, within,
+                              [(r.state.value, r.cached, r.preemptions) for r in scheduler.active])
+    assert all(h.state is RequestState.COMPLETED for h in handles)
+    assert all(len(h.output) == h.gen.max_output_tokens or h.finish_reason == "eos_token_reached" for h in handles)
+    manager.assert_invariants()
+    assert manager.stats().pages_used == manager.stats().prefix_pages_used
