@@ -112,6 +112,36 @@ def fixed_portions(requests: dict[str, list[int]], portion: int = 8, live: int =
     return steps
 
 
+def random_trace(rng, lengths: list[int], vocab: int, page: int, live_most: int = 4) -> tuple[dict[str, list[int]], list[dict]]:
+    """Requests of the given lengths with random tokens, and steps that feed them in random cuts: up to
+    ``live_most`` live at a time, some left out of a step, portions of one token, two tokens, up to a page's
+    edge, one past it, or anything; logits wanted at random places.  ``rng`` is a ``random.Random``."""
+    requests = {f"r{i}": [rng.randrange(vocab) for _ in range(n)] for i, n in enumerate(lengths)}
+    waiting, live, steps = list(requests), {}, []
+    while waiting or live:
+        while waiting and len(live) < live_most and (not live or rng.random() < 0.5):
+            live[waiting.pop(0)] = 0
+        entries, end = [], []
+        for rid in [rid for rid in live if rng.random() < 0.8] or [next(iter(live))]:
+            left = len(requests[rid]) - live[rid]
+            to_edge = page - live[rid] % page
+            kind = rng.random()
+            size = (1 if kind < 0.35 else 2 if kind < 0.55 else to_edge if kind < 0.7 else to_edge + 1 if kind < 0.8
+                    else rng.randint(1, left))
+            size = max(1, min(size, left))
+            want = set(rng.sample(range(size), k=min(size, rng.choice([0, 1, 1, 2, size]))))
+            if rng.random() < 0.5:
+                want.add(size - 1)
+            entries.append({"id": rid, "tokens": requests[rid][live[rid]: live[rid] + size], "want": sorted(want)})
+            live[rid] += size
+            if live[rid] == len(requests[rid]):
+                end.append(rid)
+        for rid in end:
+            del live[rid]
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+    return requests, steps
+
+
 def max_live_tokens(steps: list[dict], page: int = 64) -> int:
     """Most tokens live requests hold at any time, each rounded up to ``page``."""
     held: dict[str, int] = {}

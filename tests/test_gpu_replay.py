@@ -685,3 +685,37 @@ def test_replay_of_a_context_of_six_thousand_tokens(long_context_case, dtype, gr
         print("6,040 tokens bfloat16: rms %.3e worst %.3e, plain in bfloat16 %.3e %.3e"
               % replay_util.closer_than_plain_bfloat16(rows, expected, rough), flush=True)
     assert runner.cache.stats().pages_used == 0
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_traces_match_plain(tiny_folders, seed):
+    """Requests of random lengths fed in random cuts (single tokens, pairs, up to a page's edge, one past it,
+    anything), up to four live, some left out of a step, logits wanted at random places, in a pool of exactly the
+    live requests' pages, eager or from captured graphs: float32 within the tolerance of the fixed schedules;
+    bfloat16, row by row, no further from the float32 logits than 1.5 times what the plain implementation run in
+    bfloat16 is at that row (or the fixed tolerance, where that is larger)."""
+    import random
+
+    rng = random.Random(1000 + seed)
+    name = "ABC"[seed % 3]
+    folder, raw, tensors = tiny_folders[name]
+    page = rng.choice([16, 64]) if name == "A" else rng.choice([8, 16, 64])
+    lengths = [rng.randint(1, raw["max_position_embeddings"]) for _ in range(rng.randint(2, 7))]
+    requests, steps = replay_util.random_trace(rng, lengths, raw["vocab_size"], page)
+    weights = {k: v.float() for k, v in tensors.items()}
+    expected = {rid: plain_qwen2.forward(raw, weights, tokens) for rid, tokens in requests.items()}
+    rough = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
+    for dtype in ("float32", "bfloat16"):
+        graphs = rng.random() < 0.5
+        print(f"case {name} page {page} {dtype} graphs {graphs}: lengths {lengths}, {len(steps)} steps", flush=True)
+        runner = make_runner(folder, dtype, replay_util.max_live_tokens(steps, page=page), page, graph_decode=graphs)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        if dtype == "float32":
+            replay_util.compare(rows, {rid: expected[rid] for rid in rows}, every_position=False, **F32_TOL)
+        else:
+            for rid, by_position in rows.items():
+                for position, row in by_position.items():
+                    off = float((torch.from_numpy(row) - expected[rid][position]).abs().max())
+                    plain_off = float((rough[rid][position].float() - expected[rid][position]).abs().max())
+                    assert off <= max(BF16_TOL["atol"], 1.5 * plain_off), (rid, position, off, plain_off)
+        assert runner.cache.stats().pages_used == 0
