@@ -719,3 +719,38 @@ def test_random_traces_match_plain(tiny_folders, seed):
                     plain_off = float((rough[rid][position].float() - expected[rid][position]).abs().max())
                     assert off <= max(BF16_TOL["atol"], 1.5 * plain_off), (rid, position, off, plain_off)
         assert runner.cache.stats().pages_used == 0
+
+
+@pytest.mark.parametrize("shape,seed", [("0.5b", 49), ("3b", 54), ("7b", 48), ("14b", 50)])
+def test_random_traces_at_the_sizes_of_real_models(tmp_path_factory, shape, seed):
+    """Random cuts at the widths and heads that serving meets (one layer, a short vocabulary): steps of one row to
+    several hundred meet the hand-written products of few rows, those whose waves share the rows, the library's,
+    and both attention forms.  Float32 against float64 layers within four times the plain float32 implementation's
+    own distance; bfloat16 closer to the float32 logits than the plain implementation run in bfloat16."""
+    import random
+
+    from conftest import make_folder
+    from cie_amd.workloads import SHAPES
+
+    raw = dict(SHAPES[shape], architectures=["Qwen2ForCausalLM"], num_hidden_layers=2 if shape == "0.5b" else 1,
+               vocab_size=4099, eos_token_id=4098)
+    folder, tensors = make_folder(tmp_path_factory.mktemp(f"random_{shape}"), raw, seed=31, factor=1.5)
+    rng = random.Random(seed)
+    page = rng.choice([16, 64])
+    lengths = [rng.choice([rng.randint(1, 40), rng.randint(1, 200), rng.randint(100, 700)]) for _ in range(rng.randint(3, 5))]
+    requests, steps = replay_util.random_trace(rng, lengths, raw["vocab_size"], page)
+    print(f"{shape}: lengths {lengths}, {len(steps)} steps, most rows in a step "
+          f"{max(sum(len(e['tokens']) for e in step['entries']) for step in steps)}", flush=True)
+    weights = {k: v.float() for k, v in tensors.items()}
+    expected = {rid: plain_qwen2.forward(raw, weights, tokens) for rid, tokens in requests.items()}
+    exact = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.float64) for rid, tokens in requests.items()}
+    rough = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
+    plain_error = max(float((expected[rid] - exact[rid]).abs().max()) for rid in requests)
+    for dtype in ("float32", "bfloat16"):
+        runner = make_runner(folder, dtype, replay_util.max_live_tokens(steps, page=page), page, graph_decode=dtype == "bfloat16")
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        if dtype == "float32":
+            replay_util.compare(rows, {rid: exact[rid] for rid in rows}, every_position=False, rtol=0.0, atol=4 * plain_error + 1e-6)
+        else:
+            replay_util.closer_than_plain_bfloat16(rows, expected, rough)
+        assert runner.cache.stats().pages_used == 0
