@@ -754,3 +754,46 @@ def test_random_traces_at_the_sizes_of_real_models(tmp_path_factory, shape, seed
         else:
             replay_util.closer_than_plain_bfloat16(rows, expected, rough)
         assert runner.cache.stats().pages_used == 0
+
+
+@pytest.mark.parametrize("seed", [22, 32, 56, 94, 125, 142, 200, 201, 202, 203])
+def test_random_configurations_and_traces(tmp_path_factory, seed):
+    """A configuration drawn at random (head sizes from 16 to 256 in steps of 16, one to four key heads with one to
+    eight query heads each, widths that are multiples of 2, 4 or 8 only, any vocabulary, one to three layers, bias
+    or none, tied head or not, the norms' eps, the rotation's base) under a trace drawn at random: float32 against
+    float64 layers within four times the plain float32 implementation's own distance, bfloat16 closer to the float32
+    logits than the plain implementation run in bfloat16."""
+    import random
+
+    from conftest import make_folder
+
+    rng = random.Random(seed)
+    head_dim = rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 128, 160, 192, 256])
+    kv_heads = rng.choice([1, 1, 2, 3, 4])
+    q_heads = kv_heads * rng.choice([1, 2, 3, 4, 5, 7, 8])
+    raw = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_size=rng.choice([2, 4, 8, 8]) * rng.randint(6, 60),
+               num_hidden_layers=rng.randint(1, 3), num_attention_heads=q_heads, num_key_value_heads=kv_heads,
+               head_dim=head_dim, intermediate_size=rng.choice([2, 8, 16]) * rng.randint(5, 60),
+               vocab_size=rng.randint(40, 2500), rms_norm_eps=rng.choice([1e-6, 1e-5, 1e-3]),
+               rope_theta=rng.choice([1e4, 1e6, 5e5]), max_position_embeddings=rng.randint(48, 400),
+               tie_word_embeddings=rng.random() < 0.5, attention_bias=rng.random() < 0.7, use_sliding_window=False,
+               eos_token_id=1)
+    print({k: raw[k] for k in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim", "intermediate_size",
+                               "vocab_size", "num_hidden_layers")}, flush=True)
+    folder, tensors = make_folder(tmp_path_factory.mktemp(f"drawn_{seed}"), raw, seed=seed, factor=rng.choice([1.5, 4.0, 8.0]))
+    page = rng.choice([4, 8, 16, 64])
+    lengths = [rng.randint(1, raw["max_position_embeddings"]) for _ in range(rng.randint(2, 5))]
+    requests, steps = replay_util.random_trace(rng, lengths, raw["vocab_size"], page)
+    weights = {k: v.float() for k, v in tensors.items()}
+    expected = {rid: plain_qwen2.forward(raw, weights, tokens) for rid, tokens in requests.items()}
+    exact = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.float64) for rid, tokens in requests.items()}
+    rough = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
+    plain_error = max(float((expected[rid] - exact[rid]).abs().max()) for rid in requests)
+    for dtype in ("float32", "bfloat16"):
+        runner = make_runner(folder, dtype, replay_util.max_live_tokens(steps, page=page), page, graph_decode=rng.random() < 0.5)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        if rows and dtype == "float32":
+            replay_util.compare(rows, {rid: exact[rid] for rid in rows}, every_position=False, rtol=0.0, atol=4 * plain_error + 1e-6)
+        elif rows:
+            replay_util.closer_than_plain_bfloat16(rows, expected, rough)
+        assert runner.cache.stats().pages_used == 0
