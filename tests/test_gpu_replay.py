@@ -797,3 +797,40 @@ def test_random_configurations_and_traces(tmp_path_factory, seed):
         elif rows:
             replay_util.closer_than_plain_bfloat16(rows, expected, rough)
         assert runner.cache.stats().pages_used == 0
+
+
+@pytest.mark.parametrize("seed", [21, 22, 23])
+def test_random_traces_behind_thousands_of_keys(tmp_path_factory, seed):
+    """One request of several thousand tokens (up to 14,000) and a few short ones under a trace drawn at random:
+    portions of any length behind contexts of any length, single tokens whose keys are cut into parts, heads of 64
+    and 128 with one to eight query heads a key head, queries and keys scaled so that far keys matter."""
+    import random
+
+    from conftest import make_folder
+
+    rng = random.Random(seed)
+    head_dim = rng.choice([64, 128, 128])
+    kv_heads = rng.choice([1, 2])
+    q_heads = kv_heads * rng.choice([1, 2, 4, 5, 8])
+    longest = rng.choice([3000, 6000, 9000, 14000])
+    raw = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_size=128, num_hidden_layers=rng.randint(1, 2),
+               num_attention_heads=q_heads, num_key_value_heads=kv_heads, head_dim=head_dim, intermediate_size=256,
+               vocab_size=503, rms_norm_eps=1e-6, rope_theta=1e6, max_position_embeddings=longest + 64,
+               tie_word_embeddings=True, attention_bias=True, use_sliding_window=False, eos_token_id=1)
+    folder, tensors = make_folder(tmp_path_factory.mktemp(f"long_{seed}"), raw, seed=seed, factor=rng.choice([4.0, 6.0]))
+    page = rng.choice([16, 16, 64])
+    lengths = [rng.randint(longest // 2, longest)] + [rng.randint(1, 300) for _ in range(rng.randint(1, 3))]
+    rng.shuffle(lengths)
+    requests, steps = replay_util.random_trace(rng, lengths, raw["vocab_size"], page)
+    print(f"heads {q_heads}/{kv_heads} x {head_dim}, lengths {lengths}, {len(steps)} steps", flush=True)
+    weights = {k: v.float() for k, v in tensors.items()}
+    expected = {rid: plain_qwen2.forward(raw, weights, tokens) for rid, tokens in requests.items()}
+    rough = {rid: plain_qwen2.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
+    for dtype in ("float32", "bfloat16"):
+        runner = make_runner(folder, dtype, replay_util.max_live_tokens(steps, page=page), page, graph_decode=rng.random() < 0.5)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        if dtype == "float32":
+            replay_util.compare(rows, {rid: expected[rid] for rid in rows}, every_position=False, rtol=1e-4, atol=5e-5)
+        else:
+            replay_util.closer_than_plain_bfloat16(rows, expected, rough)
+        assert runner.cache.stats().pages_used == 0
