@@ -405,6 +405,12 @@ class CacheManager:
                 self._prefix[key] = node
                 if parent is not None:
                     parent.children += 1
+            elif node.page != table[i]:
+                # The index has these tokens on another page: a request that came after this one was admitted
+                # stored them first, and this one computed a copy of its own.  What lies below is not stored
+                # under that page: whoever holds a page of the index must hold all above it, or the pages
+                # above could not be evicted while the request lives although only the index holds them.
+                break
             else:
                 self._prefix.move_to_end(key)
             parent = node
@@ -493,5 +499,11 @@ class CacheManager:
             listed = {page for table in group.tables.values() for page in table if page >= 0}
             indexed = {node.page for node in self._prefix.values()} if group is self.groups[0] else set()
             assert listed | indexed == set(group.allocator._holders), "a used page is in no table"
+        if self.groups:
+            holders_of = self.groups[0].allocator.holders_of
+            for node in self._prefix.values():
+                if node.parent is not None:
+                    missing = set(holders_of(node.page)) - set(holders_of(node.parent.page))
+                    assert not missing, f"{sorted(missing)} hold page {node.page} of the index but not the page above it"
         assert len(self._slots) + len(self._free_slots) == self.max_running, "request slot lost"
         assert len(set(self._slots.values())) == len(self._slots), "two requests share a slot"

@@ -416,3 +416,30 @@ def test_free_tokens_count_what_the_index_would_give_back():
     m.assert_invariants()
     only_state = manager(unit_specs=[FixedState((3,))])
     assert only_state.free_tokens() > 1 << 40, "a cache without pages never limits admission"
+
+
+def test_a_copy_of_indexed_tokens_is_not_stored_below_the_page_the_index_has():
+    """Two requests with the same first tokens are admitted before either has stored anything: each computes
+    pages of its own.  The one that publishes second finds its tokens in the index on the other's pages; what it
+    has below them must not be hung under those pages, which it does not hold: they would then be held by the index
+    alone and yet not be evictable while it lives (two such pages once left a lone request without the one page
+    it still needed, in a pool that had room for it)."""
+    m = manager(kv_tokens=40, prefix_cache_pages=8)  # pages of 4 tokens, 10 pages
+    common = list(range(8))
+    first, second = common + [90, 91, 92], common + [70, 71, 72, 73, 74, 75]
+    assert m.admit("first", first) == 0 and m.admit("second", second) == 0
+    m.ensure_capacity_batch({"first": 11, "second": 14})
+    m.commit_lengths({"first": 11, "second": 14})
+    assert m.publish_prefix("first", first) == 8       # two pages of common tokens
+    assert m.publish_prefix("second", second) == 0     # the same tokens on pages of its own: nothing stored under them
+    m.assert_invariants()
+    m.release("first", first)
+    # what the index holds alone can be evicted, and free_tokens counts no more than that
+    assert m.stats().prefix_pages_used == 2 and m.free_tokens() == (10 - 4) * 4
+    m.ensure_capacity_batch({"second": 14 + 6 * 4})    # the second one grows into everything that is left
+    assert m.stats().prefix_pages_used == 0
+    m.assert_invariants()
+    m.release("second", second)
+    assert m.stats().pages_used == m.stats().prefix_pages_used == 3  # its own three full prompt pages, stored at its end
+    m.clear_prefix_index()
+    assert m.stats().pages_used == 0
