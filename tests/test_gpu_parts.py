@@ -621,3 +621,48 @@ def test_toy_routed_feed_forward_own_position_encoding_and_window_layer(tmp_path
     assert held(full) == 15 and held(windowed) <= -(-config_class.WINDOW // 8) + 1
     runner.cache.release("long")
     runner.cache.assert_invariants()
+
+
+@pytest.mark.parametrize("seed", [201, 202, 203, 204])
+def test_toy_window_layer_under_random_traces(tmp_path, seed):
+    """The toy model with a windowed layer (a cache group of its own whose pages come back as the window passes),
+    routed experts and its own position encoding under traces drawn at random, in float32: windows from 5 to 64
+    keys against pages of 4 to 16, cuts anywhere, a pool of exactly the live requests' pages."""
+    import random
+
+    from cie_amd.config import build_engine_config, load_config
+    from cie_amd.engine import Runner, load_model
+    from cie_amd.parts.model import expected_tensors
+    from cie_amd.weights import RandomSource, write_tensors
+
+    rng = random.Random(seed)
+    config_class = register_routed_toy()
+    config_class.EXPERTS = 3
+    config_class.WINDOW = rng.choice([5, 8, 16, 20, 33, 64])
+    kv_heads = rng.choice([1, 2])
+    raw = dict(architectures=["ToyRoutedWindowForCausalLM"], model_type="qwen2", hidden_size=64, num_hidden_layers=2,
+               num_attention_heads=kv_heads * rng.choice([1, 2, 4]), num_key_value_heads=kv_heads,
+               head_dim=rng.choice([16, 32, 64]), intermediate_size=72, vocab_size=80, rms_norm_eps=1e-5, rope_theta=1e4,
+               max_position_embeddings=rng.choice([96, 160, 300]), tie_word_embeddings=True)
+    try:
+        write_tensors(tmp_path, raw, {})
+        tensors = RandomSource(seed, std=0.15).load(expected_tensors(load_config(tmp_path).model_spec()), "float32", "cpu")
+        write_tensors(tmp_path, raw, tensors)
+        model, _ = load_model(tmp_path, "float32")
+        page = rng.choice([4, 8, 16])
+        lengths = [rng.randint(1, raw["max_position_embeddings"]) for _ in range(rng.randint(2, 5))]
+        requests, steps = replay_util.random_trace(rng, lengths, raw["vocab_size"], page)
+        print(f"window {config_class.WINDOW}, page {page}, lengths {lengths}, {len(steps)} steps", flush=True)
+        longest_portion = max(len(entry["tokens"]) for step in steps for entry in step["entries"])
+        engine_config = build_engine_config(
+            dtype="float32", page_size=page, kv_tokens=replay_util.max_live_tokens(steps, page=page), max_running=4,
+            max_model_len=raw["max_position_embeddings"], prefix_cache_pages=0, graph_decode=rng.random() < 0.5,
+            prefill_chunk=longest_portion)
+        runner = Runner(model, engine_config)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        weights = {k: v.float() for k, v in tensors.items()}
+        expected = {rid: routed_toy_plain(raw, weights, requests[rid], config_class) for rid in rows}
+        replay_util.compare(rows, expected, every_position=False, rtol=1e-4, atol=5e-5)
+        assert runner.cache.stats().pages_used == 0
+    finally:
+        config_class.WINDOW = 20
