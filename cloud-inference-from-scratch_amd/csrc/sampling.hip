@@ -108,6 +108,69 @@ __device__ __forceinline__ float fixed_block_sum(float v, float* s_val) {
     return total;
 }
 
+// The first index in [begin, end) of `row` whose running sum of exp((l - best) * inv_t), counted from `begin`,
+// passes the target; the target is `fraction` of the span's whole sum if `of_whole`, else `fraction` itself.
+// Every thread of the workgroup calls it and gets the result (it contains barriers).  s_chunk holds the sums of
+// the span's chunks of kChunk numbers: the span has at most kMaxChunks of them.
+__device__ int pick_in_span(const float* row, int begin, int end, float best, float inv_t, float fraction, bool of_whole,
+                            float* s_val, int* s_idx, float* s_chunk, float* s_target, int* s_pick) {
+    const int chunks = (end - begin + kChunk - 1) / kChunk;
+    for (int c = 0; c < chunks; ++c) {
+        const float4 e = exp_of_four(row, begin + c * kChunk + threadIdx.x * 4, end, best, inv_t);
+        const float sum = fixed_block_sum((e.x + e.y) + (e.z + e.w), s_val);
+        if (threadIdx.x == 0) s_chunk[c] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float target = fraction;
+        if (of_whole) {
+            float total = 0.f;
+            for (int c = 0; c < chunks; ++c) total += s_chunk[c];
+            target = fraction * total;
+        }
+        float running = 0.f;
+        int owner = chunks - 1;  // if rounding leaves the target unreached: the last chunk (and its last token)
+        for (int c = 0; c < chunks; ++c) {
+            if (running + s_chunk[c] > target) {
+                owner = c;
+                break;
+            }
+            running += s_chunk[c];
+        }
+        *s_target = target - running;  // what is left to reach inside the chunk
+        s_idx[0] = owner;
+        *s_pick = min(end, begin + (owner + 1) * kChunk) - 1;
+    }
+    __syncthreads();
+    const int owner = s_idx[0];
+    const float target = *s_target;
+    __syncthreads();
+    // inside the chunk: the sums of the threads before this one (in index order), then the thread's own four
+    const int first = begin + owner * kChunk + threadIdx.x * 4;
+    const float4 e = exp_of_four(row, first, end, best, inv_t);
+    s_val[threadIdx.x] = (e.x + e.y) + (e.z + e.w);
+    __syncthreads();
+    for (int offset = 1; offset < kThreads; offset <<= 1) {  // running sums over the threads, in place
+        const float below = threadIdx.x >= offset ? s_val[threadIdx.x - offset] : 0.f;
+        __syncthreads();
+        s_val[threadIdx.x] += below;
+        __syncthreads();
+    }
+    float running = threadIdx.x > 0 ? s_val[threadIdx.x - 1] : 0.f;
+    int mine = 0x7fffffff;
+    const float four[4] = {e.x, e.y, e.z, e.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        running += four[i];
+        if (mine == 0x7fffffff && first + i < end && running > target) mine = first + i;
+    }
+    if (mine != 0x7fffffff) atomicMin(s_pick, mine);  // the first index whose running sum passes the target
+    __syncthreads();
+    const int picked = *s_pick;
+    __syncthreads();
+    return picked;
+}
+
 __global__ void __launch_bounds__(kThreads)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
               const float* __restrict__ uniform, int* __restrict__ out, int vocab, int ld) {
@@ -126,57 +189,117 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
         if (threadIdx.x == 0) out[r] = best_idx;
         return;
     }
-    const float inv_t = 1.0f / temp;
-    const int chunks = (vocab + kChunk - 1) / kChunk;
-    for (int c = 0; c < chunks; ++c) {
-        const float4 e = exp_of_four(row, c * kChunk + threadIdx.x * 4, vocab, best, inv_t);
-        const float sum = fixed_block_sum((e.x + e.y) + (e.z + e.w), s_val);
-        if (threadIdx.x == 0) s_chunk[c] = sum;
+    const int picked = pick_in_span(row, 0, vocab, best, 1.0f / temp, uniform[r], true, s_val, s_idx, s_chunk, &s_target,
+                                    &s_pick);
+    if (threadIdx.x == 0) out[r] = picked;
+}
+
+// Over a large vocabulary a row is taken by many workgroups.  Stage 1: each scans one part of one row and leaves
+// the part's largest logit, its first index and, where the row has a temperature, the part's sum of
+// exp((l - the part's largest) / T), summed in a fixed order.  Stage 2 (one workgroup per row): the row's
+// largest logit (greedy rows are done), the parts' sums brought to that scale and added in index order, the part
+// in which the running sum passes u times the whole, and the index inside that part as above.
+constexpr int kMaxParts = 1024;
+
+__global__ void __launch_bounds__(kThreads)
+sample_parts_kernel(const float* __restrict__ logits, const float* __restrict__ temperature, float* __restrict__ part_val,
+                    int* __restrict__ part_idx, float* __restrict__ part_sum, int vocab, int ld, int part) {
+    __shared__ float s_val[kThreads];
+    __shared__ int s_idx[kThreads];
+    const int r = blockIdx.y;
+    const int begin = blockIdx.x * part;
+    const int end = min(vocab, begin + part);
+    const float* row = logits + static_cast<size_t>(r) * ld;
+    float best;
+    int best_idx;
+    argmax_block(row + begin, end - begin, s_val, s_idx, best, best_idx);
+    const float temp = temperature[r];
+    float sum = 0.f;
+    if (temp > 0.f) {
+        const float inv_t = 1.0f / temp;
+        for (int first = begin; first < end; first += kChunk) {  // chunk by chunk, each by the fixed tree
+            const float4 e = exp_of_four(row, first + threadIdx.x * 4, end, best, inv_t);
+            sum += fixed_block_sum((e.x + e.y) + (e.z + e.w), s_val);
+        }
     }
+    if (threadIdx.x == 0) {
+        part_val[r * gridDim.x + blockIdx.x] = best;
+        part_idx[r * gridDim.x + blockIdx.x] = begin + best_idx;
+        part_sum[r * gridDim.x + blockIdx.x] = sum;
+    }
+}
+
+__global__ void __launch_bounds__(kThreads)
+sample_final_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                    const float* __restrict__ uniform, const float* __restrict__ part_val,
+                    const int* __restrict__ part_idx, const float* __restrict__ part_sum, int* __restrict__ out, int vocab,
+                    int ld, int part, int parts) {
+    __shared__ float s_val[kThreads];
+    __shared__ int s_idx[kThreads];
+    __shared__ float s_chunk[kMaxParts];
+    __shared__ float s_target;
+    __shared__ int s_pick;
+    const int r = blockIdx.x;
+    float best = -INFINITY;
+    int best_idx = 0x7fffffff;
+    for (int c = threadIdx.x; c < parts; c += kThreads) {  // parts are in index order: ties keep the lower index
+        const float v = part_val[r * parts + c];
+        const int i = part_idx[r * parts + c];
+        if (v > best || (v == best && i < best_idx)) {
+            best = v;
+            best_idx = i;
+        }
+    }
+    s_val[threadIdx.x] = best;
+    s_idx[threadIdx.x] = best_idx;
+    __syncthreads();
+    for (int stride = kThreads / 2; stride > 0; stride >>= 1) {
+        if (threadIdx.x < stride) {
+            const float v = s_val[threadIdx.x + stride];
+            const int i = s_idx[threadIdx.x + stride];
+            if (v > s_val[threadIdx.x] || (v == s_val[threadIdx.x] && i < s_idx[threadIdx.x])) {
+                s_val[threadIdx.x] = v;
+                s_idx[threadIdx.x] = i;
+            }
+        }
+        __syncthreads();
+    }
+    best = s_val[0];
+    best_idx = s_idx[0] == 0x7fffffff ? 0 : s_idx[0];
+    __syncthreads();
+    const float temp = temperature[r];
+    if (!(temp > 0.f)) {
+        if (threadIdx.x == 0) out[r] = best_idx;
+        return;
+    }
+    const float inv_t = 1.0f / temp;
+    for (int c = threadIdx.x; c < parts; c += kThreads)
+        s_chunk[c] = part_sum[r * parts + c] * expf((part_val[r * parts + c] - best) * inv_t);
     __syncthreads();
     if (threadIdx.x == 0) {
         float total = 0.f;
-        for (int c = 0; c < chunks; ++c) total += s_chunk[c];
+        for (int c = 0; c < parts; ++c) total += s_chunk[c];
         const float target = uniform[r] * total;
         float running = 0.f;
-        int owner = chunks - 1;  // if rounding leaves the target unreached: the last chunk (and its last token)
-        for (int c = 0; c < chunks; ++c) {
+        int owner = parts - 1;
+        for (int c = 0; c < parts; ++c) {
             if (running + s_chunk[c] > target) {
                 owner = c;
                 break;
             }
             running += s_chunk[c];
         }
-        s_target = target - running;  // what is left to reach inside the chunk
+        s_target = target - running;
         s_idx[0] = owner;
-        s_pick = min(vocab, (owner + 1) * kChunk) - 1;
     }
     __syncthreads();
     const int owner = s_idx[0];
-    const float target = s_target;
+    const float left = s_target;
     __syncthreads();
-    // inside the chunk: the sums of the threads before this one (in index order), then the thread's own four
-    const int first = owner * kChunk + threadIdx.x * 4;
-    const float4 e = exp_of_four(row, first, vocab, best, inv_t);
-    s_val[threadIdx.x] = (e.x + e.y) + (e.z + e.w);
-    __syncthreads();
-    for (int offset = 1; offset < kThreads; offset <<= 1) {  // running sums over the threads, in place
-        const float below = threadIdx.x >= offset ? s_val[threadIdx.x - offset] : 0.f;
-        __syncthreads();
-        s_val[threadIdx.x] += below;
-        __syncthreads();
-    }
-    float running = threadIdx.x > 0 ? s_val[threadIdx.x - 1] : 0.f;
-    int mine = 0x7fffffff;
-    const float four[4] = {e.x, e.y, e.z, e.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        running += four[i];
-        if (mine == 0x7fffffff && first + i < vocab && running > target) mine = first + i;
-    }
-    if (mine != 0x7fffffff) atomicMin(&s_pick, mine);  // the first index whose running sum passes the target
-    __syncthreads();
-    if (threadIdx.x == 0) out[r] = s_pick;
+    const float* row = logits + static_cast<size_t>(r) * ld;
+    const int picked = pick_in_span(row, owner * part, min(vocab, (owner + 1) * part), best, inv_t, left, false, s_val, s_idx,
+                                    s_chunk, &s_target, &s_pick);
+    if (threadIdx.x == 0) out[r] = picked;
 }
 
 // Greedy over a large vocabulary, stage 1: each workgroup scans one chunk of one row and leaves its
@@ -263,6 +386,26 @@ CIE_API int cie_argmax_static(void* stream, const float* logits, int* out, int r
                                                                                       vocab, ld, chunk);
     if (cie_after_launch() != CIE_OK) return CIE_LAUNCH_FAILED;
     argmax_final_kernel<<<rows, kThreads, 0, s>>>(chunk_val, chunk_idx, out, static_cast<int>(chunks));
+    return cie_after_launch();
+}
+
+// Temperature sampling (and greedy where a row's temperature is 0) over a large vocabulary in two stages;
+// part_val / part_idx / part_sum hold rows * parts entries, parts = ceil(vocab / part), part a multiple of 1,024.
+CIE_API int cie_sample_parts(void* stream, const float* logits, const float* temperature, const float* uniform,
+                             float* part_val, int* part_idx, float* part_sum, int* out, int rows, int vocab, int ld,
+                             int part) {
+    if (rows < 0 || vocab <= 0 || ld < vocab || part <= 0 || part % kChunk || part / kChunk > kMaxParts || rows > 65535 ||
+        !temperature || !uniform || !part_val || !part_idx || !part_sum)
+        return CIE_BAD_ARGUMENT;
+    const int parts = (vocab + part - 1) / part;
+    if (parts > kMaxParts) return CIE_BAD_ARGUMENT;
+    if (rows == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    sample_parts_kernel<<<dim3(parts, rows), kThreads, 0, s>>>(logits, temperature, part_val, part_idx, part_sum, vocab, ld,
+                                                              part);
+    if (cie_after_launch() != CIE_OK) return CIE_LAUNCH_FAILED;
+    sample_final_kernel<<<rows, kThreads, 0, s>>>(logits, temperature, uniform, part_val, part_idx, part_sum, out, vocab, ld,
+                                                  part, parts);
     return cie_after_launch();
 }
 

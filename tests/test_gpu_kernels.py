@@ -618,11 +618,12 @@ def test_sample_greedy_and_temperature(ops):
         assert lo - 1e-5 <= u <= cdf[got[r]].item() + 1e-5, (r, got[r], lo, u, cdf[got[r]].item())
 
 
-@pytest.mark.parametrize("vocab", [1024, 4099, 151936])
+@pytest.mark.parametrize("vocab", [1024, 4099, 8192, 9001, 151936])
 def test_sample_over_many_chunks(ops, vocab):
     """A vocabulary of many chunks of the kernel's walk (and one that ends inside a chunk, with rows that are
-    not 16-byte aligned): the token is the one whose share of [0, 1) holds the row's number, for numbers
-    at the very start, inside and at the very end, and for a row whose weight sits in its last tokens."""
+    not 16-byte aligned), and from 8,192 tokens on rows that many workgroups take in parts and a second kernel
+    finishes: the token is the one whose share of [0, 1) holds the row's number, for numbers at the very start,
+    inside and at the very end, and for a row whose weight sits in its last tokens."""
     g = torch.Generator().manual_seed(62)
     rows = 7
     logits = (torch.randn((rows, vocab), generator=g) * 2).cuda()
@@ -640,6 +641,12 @@ def test_sample_over_many_chunks(ops, vocab):
     assert got[5] >= vocab - 3 and got[6] == vocab - 1
     # the same draw whatever else is in the batch: row 1 alone
     assert ops.sample(logits[1:2], temperature[1:2], uniform[1:2]).tolist() == [got[1]]
+    # rows without a temperature among the others: the first index of the largest logit
+    logits[3, vocab - 1] = logits[3, 5] = logits[3].max() + 1
+    mixed = temperature.clone()
+    mixed[3] = mixed[0] = 0.0
+    again = ops.sample(logits, mixed, uniform).tolist()
+    assert again[3] == 5 and again[0] == int(torch.argmax(logits[0])) and again[1] == got[1] and again[6] == got[6]
 
 
 def test_sample_frequencies(ops):
