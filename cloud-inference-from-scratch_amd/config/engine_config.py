@@ -35,7 +35,11 @@ class EngineConfig:
     prefill_chunk: int = 2048
     page_size: int = 16  # reference: block_size, fixed at 16 there
     kv_tokens: int | None = None  # pool size in tokens; None: from kv_cache_bytes
-    kv_cache_bytes: int = 4 << 30
+    # the pool in bytes (the reference's knob, 4 GiB there); None: kv_cache_fraction of the device memory that is
+    # free once the weights are loaded.  Either way the pool is no larger than what max_running requests of
+    # max_model_len tokens and the prefix index can use.
+    kv_cache_bytes: int | None = None
+    kv_cache_fraction: float = 0.9
     prefix_cache_pages: int = 256  # reference: prefix_cache_max_blocks
     graph_decode: bool = True  # reference: cuda_graph_decode
     # steps of up to 128 rows that bring prompt portions are captured too, from the second time a shape comes
@@ -69,6 +73,10 @@ class EngineConfig:
             raise ValueError("graph_mixed_steps must be non-negative")
         if config.kv_tokens is not None and config.kv_tokens < config.page_size:
             raise ValueError("kv_tokens too small for even one page")
+        if config.kv_cache_bytes is not None and config.kv_cache_bytes < 1:
+            raise ValueError("kv_cache_bytes must be positive")
+        if not 0.0 < config.kv_cache_fraction <= 1.0:
+            raise ValueError("kv_cache_fraction must lie in (0, 1]")
         return config
 
 

@@ -91,7 +91,11 @@ class Runner:
         if per_token == 0:
             return self.config.page_size
         page = self.config.page_size
-        tokens = self.config.kv_cache_bytes // per_token
+        budget = self.config.kv_cache_bytes
+        if budget is None:
+            free, _total = torch.cuda.mem_get_info(self.device)
+            budget = int(free * self.config.kv_cache_fraction)
+        tokens = budget // per_token
         # more than every slot full plus the prefix index can never be used
         useful = (self.config.max_running * -(-self.config.max_model_len // page) + self.config.prefix_cache_pages) * page
         return max(page, min(tokens, useful) // page * page)

@@ -101,6 +101,11 @@ def test_engine_options():
         build_engine_config(dtype="float16")
     with pytest.raises(ValueError, match="token_budget"):
         build_engine_config(token_budget=0)
+    with pytest.raises(ValueError, match="kv_cache_fraction"):
+        build_engine_config(kv_cache_fraction=0.0)
+    with pytest.raises(ValueError, match="kv_cache_bytes"):
+        build_engine_config(kv_cache_bytes=0)
+    assert build_engine_config().kv_cache_bytes is None and build_engine_config().kv_cache_fraction == 0.9
 
 
 def test_engine_options_under_the_references_names():

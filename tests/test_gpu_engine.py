@@ -380,3 +380,18 @@ def test_loading_needs_the_models_own_size_of_device_memory_not_twice(tmp_path, 
     assert held > 80e6  # (about 90 MB: the check below is about something)
     assert peak < held + 4 * per_layer, (held, peak)
     del model
+
+
+def test_the_pool_is_sized_by_what_the_requests_can_use_or_by_the_memory_that_is_free(tiny_folders):
+    """Without a size the pool takes a fraction of the free device memory, but never more pages than max_running
+    requests of max_model_len tokens and the prefix index can use; a size in bytes or tokens is taken as given."""
+    from cie_amd import Engine
+
+    folder, raw, _ = tiny_folders["A"]
+    engine = Engine(folder, dtype="bfloat16", max_running=3, max_model_len=100, page_size=16, prefix_cache_pages=5)
+    assert engine.runner.cache.stats().pages_total == 3 * 7 + 5  # 7 pages a request: 100 tokens
+    per_token = 2 * raw["num_hidden_layers"] * raw["num_key_value_heads"] * 16 * 2  # keys and values, bfloat16
+    engine = Engine(folder, dtype="bfloat16", max_running=3, max_model_len=100, page_size=16, kv_cache_bytes=40 * per_token)
+    assert engine.runner.cache.stats().pages_total == 2  # 40 tokens' worth: two whole pages
+    engine = Engine(folder, dtype="bfloat16", max_running=3, max_model_len=100, page_size=16, kv_tokens=64)
+    assert engine.runner.cache.stats().pages_total == 4
