@@ -3,7 +3,7 @@
 (default: the 3B one) with random weights, plus prefill and roofline figures.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
-                    [--shape 3b|7b|14b|32b|72b] [--layers N] [--long-contexts 16384,32768]
+                    [--shape 0.5b|3b|7b|14b|32b|72b] [--layers N] [--long-contexts 16384,32768]
 
 A "step" is one decode step of the whole engine (scheduler iteration: plan,
 step function, sampling, token hand-over).  Protocol after the reference's
@@ -176,7 +176,7 @@ def main(argv=None) -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=4096)
-    parser.add_argument("--shape", default="3b", choices=["3b", "7b", "14b", "32b", "72b"])
+    parser.add_argument("--shape", default="3b", choices=["0.5b", "3b", "7b", "14b", "32b", "72b"])
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in config)")
     parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     parser.add_argument("--prefill-tokens", type=int, default=2048)
