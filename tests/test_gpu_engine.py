@@ -395,3 +395,33 @@ def test_the_pool_is_sized_by_what_the_requests_can_use_or_by_the_memory_that_is
     assert engine.runner.cache.stats().pages_total == 2  # 40 tokens' worth: two whole pages
     engine = Engine(folder, dtype="bfloat16", max_running=3, max_model_len=100, page_size=16, kv_tokens=64)
     assert engine.runner.cache.stats().pages_total == 4
+
+
+def test_a_serving_workload_runs_and_its_tokens_do_not_depend_on_the_batch():
+    """``cie workload`` on a profile made small (one layer of the smallest shape, six requests, float32): the record's
+    fields, and the first requests run once more, alone, give the same tokens (``run_profile`` raises if not)."""
+    from dataclasses import replace
+
+    from cie_amd.workloads import PROFILES, run_profile
+
+    profile = replace(PROFILES["mixed"], requests=6)
+    record = run_profile(profile, layers=1, dtype="float32", shape="0.5b", verify=3)
+    assert record["verified"] == {"requests": 3, "same_tokens_alone": 3}
+    assert (record["workload"], record["shape"], record["layers"], record["layers_full"], record["requests"]) == \
+        ("mixed", "0.5b", 1, 24, 6)
+    assert record["output_tokens"] > 0 and record["input_tokens"] > 0 and record["elapsed_s"] > 0
+    assert record["output_tokens_per_s"] == pytest.approx(record["output_tokens"] / record["elapsed_s"], rel=0.01)
+    for key in ("ttft_ms", "itl_ms", "e2e_ms"):
+        assert record[key]["p50"] <= record[key]["p95"]
+    assert record["preempted"] == 0 and "synthetic" in record["data"]
+
+
+def test_ceilings_reports_what_the_gpu_reaches():
+    done = subprocess.run([sys.executable, str(ROOT / "bin" / "cie"), "ceilings"], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    record = json.loads(done.stdout.strip().splitlines()[-1])
+    for key in ("copy_1GiB_GBps", "read_1GiB_library_mv_GBps", "read_1GiB_few_row_product_GBps",
+                "read_45MB_few_row_product_GBps"):
+        assert 1000 < record[key] < 8000, (key, record[key])  # between a tenth of the published bandwidth and all of it
+    for key in ("bf16_8192_cubed_library_TFLOPs", "bf16_8192_cubed_library_tuned_TFLOPs"):
+        assert 300 < record[key] < 2500, (key, record[key])
