@@ -136,3 +136,25 @@ def test_another_architecture_registers_without_touching_the_package():
 def test_part_spec_is_hashable_and_sorted():
     a = PartSpec.of("rms_norm", size=8, eps=1e-6)
     assert a == PartSpec.of("rms_norm", eps=1e-6, size=8) and hash(a) == hash(PartSpec.of("rms_norm", eps=1e-6, size=8))
+
+
+def test_command_line_without_a_gpu(tmp_path):
+    """What of ``cie`` needs no GPU: the registry's names, a model folder with random weights, the benchmark's refusal
+    of more than one GPU handed through."""
+    import json
+    import subprocess
+    import sys
+
+    from conftest import ROOT, TINY_B
+
+    cie = [sys.executable, str(ROOT / "bin" / "cie")]
+    done = subprocess.run(cie + ["models"], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0 and "Qwen2ForCausalLM" in json.loads(done.stdout)["architectures"]
+    (tmp_path / "config.json").write_text(json.dumps(TINY_B))
+    done = subprocess.run(cie + ["init-model", "--config", str(tmp_path / "config.json"), "--out", str(tmp_path / "model"),
+                                 "--seed", "3"], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert (tmp_path / "model" / "model.safetensors").is_file()
+    assert json.loads((tmp_path / "model" / "config.json").read_text())["hidden_size"] == TINY_B["hidden_size"]
+    done = subprocess.run(cie + ["bench", "--gpus", "4"], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 2 and "one GPU" in done.stdout

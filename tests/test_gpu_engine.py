@@ -425,3 +425,48 @@ def test_ceilings_reports_what_the_gpu_reaches():
         assert 1000 < record[key] < 8000, (key, record[key])  # between a tenth of the published bandwidth and all of it
     for key in ("bf16_8192_cubed_library_TFLOPs", "bf16_8192_cubed_library_tuned_TFLOPs"):
         assert 300 < record[key] < 2500, (key, record[key])
+
+
+def test_text_prompts_go_through_the_folders_tokenizer(tiny_folders, tmp_path):
+    """A prompt given as text is cut by the ``tokenizer.json`` of the model folder and the result comes back as text
+    too (a word-level tokenizer made here, over the tiny model's 256 ids); without that file text is refused with
+    a message and token ids still work."""
+    import shutil
+
+    from tokenizers import Tokenizer, decoders, models, pre_tokenizers
+
+    from cie_amd import Engine, GenerationConfig
+
+    folder, raw, tensors = tiny_folders["A"]
+    with_words = tmp_path / "with_tokenizer"
+    shutil.copytree(folder, with_words)
+    tokenizer = Tokenizer(models.WordLevel({f"w{i}": i for i in range(raw["vocab_size"])}, unk_token="w0"))
+    tokenizer.pre_tokenizer = pre_tokenizers.Whitespace()
+    tokenizer.decoder = decoders.WordPiece(prefix="##")
+    tokenizer.save(str(with_words / "tokenizer.json"))
+    prompt = [7, 8, 9, 10, 11]
+    expected = plain.generate_greedy(raw, float_weights(tensors), prompt, 5)
+    engine = make_engine(with_words)
+    gen = GenerationConfig(max_output_tokens=5, eos_token_id=None)
+    result = engine.generate(["w7 w8 w9 w10 w11"], gen)[0]
+    assert result.token_ids == expected and result.text == " ".join(f"w{t}" for t in expected)
+    done = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "cie"), "generate", "w7 w8 w9 w10 w11", "--model", str(with_words),
+         "--max-output-tokens", "5", "--dtype", "fp32", "--no-stream", "--ignore-eos", "--max-model-len", "64"],
+        capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert done.stdout.split() == [f"w{t}" for t in expected]
+    bare = make_engine(folder)
+    with pytest.raises(ValueError, match="tokenizer.json"):
+        bare.generate(["w7 w8"], gen)
+    assert bare.generate([prompt], gen)[0].token_ids == expected
+
+
+def test_command_line_metrics_prints_the_counters_of_a_run(tiny_folders):
+    folder, _, _ = tiny_folders["B"]
+    done = subprocess.run([sys.executable, str(ROOT / "bin" / "cie"), "metrics", "--model", str(folder), "--token-ids", "3 4 5",
+                           "--max-output-tokens", "6", "--max-model-len", "64"], capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-2000:]
+    counters = json.loads(done.stdout)
+    assert counters["requests"]["completed_total"] == 1 and counters["tokens"]["output_total"] <= 6
+    assert counters["kv_cache"]["pages_used"] == counters["kv_cache"]["prefix_pages_used"]
