@@ -470,3 +470,23 @@ def test_command_line_metrics_prints_the_counters_of_a_run(tiny_folders):
     counters = json.loads(done.stdout)
     assert counters["requests"]["completed_total"] == 1 and counters["tokens"]["output_total"] <= 6
     assert counters["kv_cache"]["pages_used"] == counters["kv_cache"]["prefix_pages_used"]
+
+
+def test_generation_with_profiler_ranges_switched_on(tiny_folders):
+    """``ENGINE_NVTX=1`` puts named ranges around the phases of every iteration (torch emits them as roctx ranges):
+    the same tokens come out."""
+    import os
+
+    folder, raw, tensors = tiny_folders["A"]
+    prompt = [7, 8, 9, 10, 11]
+    expected = plain.generate_greedy(raw, float_weights(tensors), prompt, 5)
+    code = ("import sys; sys.path.insert(0, %r); import cie_amd\n"
+            "from cie_amd import Engine, GenerationConfig, profiling\n"
+            "assert profiling.trace_range('a') is not profiling.trace_range('b'), 'ranges are off'\n"
+            "engine = Engine(%r, dtype='float32', kv_tokens=256, max_model_len=64)\n"
+            "print(engine.generate([%r], GenerationConfig(max_output_tokens=5, eos_token_id=None))[0].token_ids)\n"
+            ) % (str(ROOT), str(folder), prompt)
+    done = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300,
+                          env={**os.environ, "ENGINE_NVTX": "1"})
+    assert done.returncode == 0, done.stderr[-2000:]
+    assert done.stdout.strip().splitlines()[-1] == str(expected)
