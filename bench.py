@@ -4,6 +4,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
                     [--shape 0.5b|3b|7b|14b|32b|72b] [--layers N] [--long-contexts 16384,32768]
+                    [--mixed-portions 16,64,248]
 
 A "step" is one decode step of the whole engine (scheduler iteration: plan,
 step function, sampling, token hand-over).  Protocol after the reference's
@@ -20,6 +21,8 @@ states ("2,048-token prefill, then decode to 4,096").  The whole range is
 measured beside it (``range``): prompts of ``--prefill-tokens``, then every
 decode step up to ``--context``, one warm-up run and three measured ones.
 ``prefill`` is one prompt of ``--prefill-tokens`` run to its first token.
+``--mixed-portions`` adds the time of the steps that chunked serving meets: the
+batch's decode tokens beside one portion of a further prompt (``mixed``).
 ONE JSON line is printed.
 """
 
@@ -149,6 +152,49 @@ def decode_range(engine, config, batch: int, first: int, last: int, seed: int, w
     return out
 
 
+def mixed_steps(engine, config, batch: int, context: int, portions: list[int], seed: int, steps: int = 24):
+    """``batch`` requests decoding near ``context`` tokens; for each portion size, steps that carry
+    their tokens and one portion of a long prompt.  Returns {portion: median seconds per step}."""
+    import dataclasses
+
+    import torch
+
+    from cie_amd import GenerationConfig
+    from cie_amd.engine import RequestState
+
+    settle = 4
+    decoded = (len(portions) + 1) * (steps + 2 * settle + 4) + SLACK
+    gen = GenerationConfig(max_output_tokens=decoded, eos_token_id=None)
+    requests = [engine.submit(prompt, gen) for prompt in random_prompts(config, batch, context - decoded, seed)]
+    while any(r.state is not RequestState.DECODING for r in requests):
+        engine.step()
+    base = engine.scheduler.config
+    out = {}
+    for portion in portions:
+        # the scheduler cuts the long prompt into portions of this size beside the decode tokens
+        engine.scheduler.config = dataclasses.replace(base, token_budget=batch + portion, prefill_chunk=portion)
+        prompt = random_prompts(config, 1, portion * (steps + settle + 2), seed + portion)[0]
+        long = engine.submit(prompt, GenerationConfig(max_output_tokens=1, eos_token_id=None))
+        for _ in range(settle):  # (a shape is captured the second time it comes)
+            engine.step()
+        seconds = []
+        for _ in range(steps):
+            torch.cuda.synchronize()
+            start = time.perf_counter()
+            engine.step()
+            torch.cuda.synchronize()
+            seconds.append(time.perf_counter() - start)
+        assert not long.is_final and all(r.state is RequestState.DECODING for r in requests)
+        out[portion] = statistics.median(seconds)
+        while not long.is_final:
+            engine.step()
+    engine.scheduler.config = base
+    for r in requests:
+        assert not r.is_final
+        engine.scheduler.cancel(r)
+    return out
+
+
 def time_prefill(engine, config, tokens: int, seed: int) -> list[float]:
     """Seconds of each measured run: one prompt from submission to its first token."""
     import torch
@@ -184,6 +230,8 @@ def main(argv=None) -> int:
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--no-range", action="store_true", help="skip the run over the whole range of contexts")
     parser.add_argument("--long-contexts", default="", help="further decode points of the main batch, e.g. 16384,32768")
+    parser.add_argument("--mixed-portions", default="",
+                        help="also time steps of the batch's decode tokens beside a prompt portion of these sizes, e.g. 16,64,248")
     args = parser.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not run (this engine is single-GPU)")
@@ -294,6 +342,16 @@ def main(argv=None) -> int:
         points[key] = round(statistics.median(rates), 2)
         fractions[key] = round(achieved / HBM_GBPS, 4)
         all_runs[key] = [round(r, 2) for r in rates]
+    portions = [int(c) for c in args.mixed_portions.split(",") if c]
+    if portions:
+        say(f"steps of {args.batch} decode tokens beside a prompt portion of {portions}")
+        longest = max(portions)
+        engine = make_engine(config, args.dtype, args.batch + 1, max(args.context, 64 * longest), args.prefill_tokens)
+        took = mixed_steps(engine, config, args.batch, args.context, portions, seed=5)
+        del engine
+        release()
+        line["mixed"] = {"decoding": args.batch, "context": args.context,
+                         "ms_per_step": {str(portion): round(s * 1e3, 4) for portion, s in took.items()}}
     if points:
         line["points"] = points
         line["points_frac"] = fractions

@@ -23,7 +23,7 @@ def test_more_than_one_gpu_is_said_and_refused():
 def test_one_json_line_with_the_agreed_fields():
     """A short run of one layer of the default shape: the line's fields, and that its figures follow from one another."""
     command = [sys.executable, str(ROOT / "bench.py"), "--gpus", "1", "--steps", "4", "--warmup", "1", "--layers", "1",
-               "--context", "256", "--prefill-tokens", "64"]
+               "--context", "256", "--prefill-tokens", "64", "--mixed-portions", "6,20"]
     done = subprocess.run(command, capture_output=True, text=True, timeout=600)
     assert done.returncode == 0, done.stderr[-3000:]
     lines = done.stdout.strip().splitlines()
@@ -47,3 +47,7 @@ def test_one_json_line_with_the_agreed_fields():
     assert prefill["tokens"] == 64 and prefill["value"] == pytest.approx(64 / (prefill["ms"] / 1e3), rel=0.02)
     assert 0 < prefill["frac"] < 1 and 0 < roofline["frac"] < 1
     assert set(line["points"]) == {"decode_b1", "decode_b64"} and all(v > 0 for v in line["points"].values())
+    # the steps that carry a prompt portion beside the decode tokens
+    mixed = line["mixed"]
+    assert (mixed["decoding"], mixed["context"]) == (8, 256)
+    assert set(mixed["ms_per_step"]) == {"6", "20"} and all(v > 0 for v in mixed["ms_per_step"].values())
