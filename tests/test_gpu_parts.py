@@ -666,3 +666,100 @@ def test_toy_window_layer_under_random_traces(tmp_path, seed):
         assert runner.cache.stats().pages_used == 0
     finally:
         config_class.WINDOW = 20
+
+
+# ----------------------------------------------------------------------------------------------------
+# The run order is data: a layer may read the cache that another layer writes.  Again a toy,
+# registered from here: three attention layers, the middle one without keys and values of its own.
+def register_shared_cache_toy():
+    from cie_amd.config import register_architecture
+    from cie_amd.config.qwen2 import Qwen2Config
+    from cie_amd.config.specs import LayerCall, ModelSpec
+
+    class SharedCacheConfig(Qwen2Config):
+        architecture = "ToySharedCacheForCausalLM"
+
+        def model_spec(self) -> ModelSpec:
+            base = super().model_spec()
+            # layer 1 attends, with its own queries, to the keys and values that layer 0 wrote
+            order = (LayerCall(0, 0), LayerCall(1, 0, writes=False), LayerCall(2, 1))
+            return ModelSpec(
+                architecture=self.architecture, vocab_size=self.vocab_size, hidden_size=self.hidden_size,
+                layers=base.layers, order=order, final_norm=base.final_norm,
+                tie_word_embeddings=self.tie_word_embeddings, max_position=self.max_position_embeddings)
+
+    register_architecture("ToySharedCacheForCausalLM", SharedCacheConfig)
+    return SharedCacheConfig
+
+
+def shared_cache_plain(raw, weights, tokens):
+    """Whole-sequence reference from the plain parts: layer 1 uses layer 0's rotated keys and its values."""
+    eps, d = raw["rms_norm_eps"], plain.head_dim_of(raw)
+    t = len(tokens)
+    positions = torch.arange(t)
+    cos, sin = plain.rope_tables(d, t, raw["rope_theta"])
+    h = weights["model.embed_tokens.weight"][torch.tensor(tokens)]
+    kept = None
+    for layer in range(3):
+        p = f"model.layers.{layer}."
+        x = plain.rms_norm(h, weights[p + "input_layernorm.weight"], eps)
+
+        def proj(name):
+            return plain.linear(x, weights[f"{p}self_attn.{name}.weight"], weights[f"{p}self_attn.{name}.bias"]).view(t, -1, d)
+
+        q = plain.apply_rope(proj("q_proj"), cos, sin, positions)
+        if layer == 1:
+            k, v = kept
+        else:
+            k, v = plain.apply_rope(proj("k_proj"), cos, sin, positions), proj("v_proj")
+        if layer == 0:
+            kept = (k, v)
+        context = plain.causal_attention(q, k, v, 1.0 / math.sqrt(d), past_len=0)
+        h = h + plain.linear(context, weights[p + "self_attn.o_proj.weight"])
+        h = h + plain.swiglu(plain.rms_norm(h, weights[p + "post_attention_layernorm.weight"], eps),
+                             weights[p + "mlp.gate_proj.weight"], weights[p + "mlp.up_proj.weight"],
+                             weights[p + "mlp.down_proj.weight"])
+    h = plain.rms_norm(h, weights["model.norm.weight"], eps)
+    return h @ weights["lm_head.weight"].t()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_that_reads_the_cache_another_layer_writes(tmp_path, dtype):
+    """Three layers on two cache units: the middle layer writes nothing and reads the first layer's pages.
+    Whole, in portions and mixed with pages used again, with captured decode steps, against the plain model."""
+    from cie_amd.config import build_engine_config, load_config
+    from cie_amd.engine import Runner, load_model
+    from cie_amd.parts.model import expected_tensors
+    from cie_amd.weights import RandomSource, write_tensors
+
+    register_shared_cache_toy()
+    raw = dict(architectures=["ToySharedCacheForCausalLM"], model_type="qwen2", hidden_size=80, num_hidden_layers=3,
+               num_attention_heads=5, num_key_value_heads=1, head_dim=32, intermediate_size=104, vocab_size=91,
+               rms_norm_eps=1e-5, rope_theta=1e4, max_position_embeddings=200, tie_word_embeddings=False)
+    write_tensors(tmp_path, raw, {})
+    spec = load_config(tmp_path).model_spec()
+    assert spec.cache_units == 2
+    tensors = RandomSource(12, std=0.12).load(expected_tensors(spec), "float32", "cpu")
+    # the middle layer's own key and value projections are loaded and never used: garbage there must not show
+    for name in ("k_proj", "v_proj"):
+        tensors[f"model.layers.1.self_attn.{name}.weight"] = tensors[f"model.layers.1.self_attn.{name}.weight"] * 50.0
+    if dtype == "bfloat16":  # the plain model runs the weights the engine holds
+        tensors = {k: (v.to(torch.bfloat16).float() if v.is_floating_point() else v) for k, v in tensors.items()}
+    write_tensors(tmp_path, raw, tensors)
+    model, _ = load_model(tmp_path, dtype)
+    requests = {f"s{i}": random_tokens(n, 91, 300 + i) for i, n in enumerate([150, 37, 64, 9, 101])}
+    reference = {rid: shared_cache_plain(raw, tensors, tokens) for rid, tokens in requests.items()}
+    magnitude = max(1.0, max(float(r.abs().max()) for r in reference.values()))
+    tolerance = dict(rtol=1e-4, atol=5e-5) if dtype == "float32" else dict(rtol=2e-2, atol=2e-2 * magnitude)
+    for graphs in (False, True):
+        mixed_steps = replay_util.mixed(requests, live=3)
+        engine_config = build_engine_config(
+            dtype=dtype, page_size=8, kv_tokens=replay_util.max_live_tokens(mixed_steps, page=8), max_running=4,
+            max_model_len=200, prefix_cache_pages=0, graph_decode=graphs)
+        runner = Runner(model, engine_config)
+        assert len(runner.cache.groups) == 1 and sorted(runner.cache.unit_group) == [0, 1]
+        for steps in (replay_util.whole(requests), replay_util.tail_one_by_one(requests, tail=32),
+                      replay_util.portions(requests), mixed_steps):
+            rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+            replay_util.compare(rows, reference, **tolerance)
+            assert runner.cache.stats().pages_used == 0
