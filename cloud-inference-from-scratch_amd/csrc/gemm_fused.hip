@@ -79,6 +79,15 @@ struct FusedArgs {
     const float* row_sumsq;    // SILU: [M, sumsq_parts] or null
     int sumsq_parts;
     float eps;
+    // ROPE with the norm in front of it folded in (a few rows): the rows of A are not read but made here, as
+    // bf16((fold_residual + the sum of fold_parts) * fold_weight), and the product is multiplied by each row's
+    // 1/rms; the first workgroup writes the summed stream to fold_residual_out (another buffer than
+    // fold_residual, which the other workgroups are still reading).
+    const float* fold_residual;  // [M, K] float32 or null
+    const float* fold_parts;     // [fold_n_parts, M, K] float32
+    int fold_n_parts;
+    const float* fold_weight;    // [K] float32
+    float* fold_residual_out;    // [M, K] float32
     RopeArgs rope;         // ROPE only
 };
 
@@ -364,8 +373,12 @@ __device__ __forceinline__ void store_rope8(const FusedArgs& a, const floatx4& a
 constexpr int kStageRow = 256 + 16;           // bytes of a row in a staging area: the padding spreads the rows over the banks
 constexpr int kStageTile = 16 * kStageRow;    // a wave's staging area
 
-template <int WAVES, int EPI, int MT, int NT>
+constexpr int kFoldRows = 4;       // the most rows whose norm the q/k/v product makes itself
+constexpr int kFoldElems = 8192;   // rows x K it keeps in LDS for that (16 KB)
+
+template <int WAVES, int EPI, int MT, int NT, bool FOLD = false>
 __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
+    static_assert(!FOLD || (MT == 1 && (EPI == EPI_ROPE || EPI == EPI_ROPE8)), "the folded norm: q/k/v of one row tile");
     static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
     static_assert(EPI != EPI_ROPE || NT == 2, "the ROPE epilogue pairs the two halves of a head");
     static_assert(EPI != EPI_ROPE8 || (NT == 1 && MT == 1), "the one-tile ROPE epilogue: one tile, up to 16 rows");
@@ -380,6 +393,9 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     __shared__ __attribute__((aligned(16))) char shared[kSharedBytes + 16 * sizeof(float)];  // + the rows' scales
     float* reduce = reinterpret_cast<float*>(shared);
     char* stage = shared + (threadIdx.x / kWave) * kStageTile;
+    __shared__ __attribute__((aligned(16))) bf16_t fold_rows[FOLD ? kFoldElems : 8];  // [M][K]: the rows of A made here
+    __shared__ float fold_sq[FOLD ? WAVES * kFoldRows : 1];
+    __shared__ float fold_scale[FOLD ? kFoldRows : 1];
 
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
@@ -431,7 +447,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         for (int i = 0; i < 4; ++i) {
             const int m = m0 + mt * 16 + (kStageA ? i * 4 + load_row : r);
             row_ok[mt][i] = m < a.M;
-            a_rows[mt][i] = a.a + static_cast<size_t>(min(m, a.M - 1)) * a.lda + (kStageA ? load_col : i * 32 + g * 8);
+            a_rows[mt][i] = FOLD ? nullptr
+                                 : a.a + static_cast<size_t>(min(m, a.M - 1)) * a.lda + (kStageA ? load_col : i * 32 + g * 8);
         }
 
     floatx4 acc[MT][NT];
@@ -477,6 +494,119 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
 
     const int k_begin = blockIdx.z * a.k_per_part;
     const int k_end = min(a.K, k_begin + a.k_per_part);
+    if constexpr (FOLD) {
+        // The wave's first pieces of W are asked for, then the rows of A are made while they travel: the
+        // stream plus its pending partial sums, times the norm's weight, as bf16 into LDS (the rows' 1/rms
+        // multiplies the sums at the end: the product is linear in its rows).
+        uint4 b[U][NT][4];
+        auto load_w = [&](int kbase) __attribute__((always_inline)) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int k0 = kbase + u * WAVES * 128;
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        b[u][t][i] = (k0 + load_col < k_end) ? *reinterpret_cast<const uint4*>(w_rows[t][i] + k0) : uint4{0, 0, 0, 0};
+            }
+        };
+        int kbase = k_begin + wave * 128;
+        if (kbase < k_end) load_w(kbase);
+        if (rope_pending) {  // behind the wave's first loads of W
+            if (EPI == EPI_ROPE8)
+                rope8_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
+            else
+                rope_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
+            rope_pending = false;
+        }
+        const bool writer = blockIdx.x == 0;
+        float sq[kFoldRows] = {0.f, 0.f, 0.f, 0.f};
+        for (int c = threadIdx.x * 8; c < a.K; c += WAVES * kWave * 8) {
+            const float4 w0 = *reinterpret_cast<const float4*>(a.fold_weight + c);
+            const float4 w1 = *reinterpret_cast<const float4*>(a.fold_weight + c + 4);
+#pragma unroll
+            for (int m = 0; m < kFoldRows; ++m) {
+                if (m >= a.M) break;  // (uniform)
+                const size_t at = static_cast<size_t>(m) * a.K + c;
+                float4 x0 = *reinterpret_cast<const float4*>(a.fold_residual + at);
+                float4 x1 = *reinterpret_cast<const float4*>(a.fold_residual + at + 4);
+                // eight parts at a time, their loads all under way before the first is added (a part past the
+                // last reads the last again and is not added)
+                for (int p0 = 0; p0 < a.fold_n_parts; p0 += 8) {
+                    float4 v[8][2];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int part = min(p0 + j, a.fold_n_parts - 1);
+                        const float* src = a.fold_parts + (static_cast<size_t>(part) * a.M + m) * a.K + c;
+                        v[j][0] = *reinterpret_cast<const float4*>(src);
+                        v[j][1] = *reinterpret_cast<const float4*>(src + 4);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        if (p0 + j >= a.fold_n_parts) break;
+                        x0.x += v[j][0].x; x0.y += v[j][0].y; x0.z += v[j][0].z; x0.w += v[j][0].w;
+                        x1.x += v[j][1].x; x1.y += v[j][1].y; x1.z += v[j][1].z; x1.w += v[j][1].w;
+                    }
+                }
+                sq[m] += (x0.x * x0.x + x0.y * x0.y) + (x0.z * x0.z + x0.w * x0.w) + (x1.x * x1.x + x1.y * x1.y) +
+                         (x1.z * x1.z + x1.w * x1.w);
+                if (writer) {
+                    *reinterpret_cast<float4*>(a.fold_residual_out + at) = x0;
+                    *reinterpret_cast<float4*>(a.fold_residual_out + at + 4) = x1;
+                }
+                uint4 packed;
+                packed.x = pack_bf16(x0.x * w0.x, x0.y * w0.y);
+                packed.y = pack_bf16(x0.z * w0.z, x0.w * w0.w);
+                packed.z = pack_bf16(x1.x * w1.x, x1.y * w1.y);
+                packed.w = pack_bf16(x1.z * w1.z, x1.w * w1.w);
+                *reinterpret_cast<uint4*>(fold_rows + at) = packed;
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < kFoldRows; ++m) {
+            float v = sq[m];
+#pragma unroll
+            for (int offset = kWave / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+            if (lane == 0) fold_sq[wave * kFoldRows + m] = v;
+        }
+        __syncthreads();  // the rows and the waves' sums of squares are in LDS
+        if (threadIdx.x < kFoldRows) {
+            float total = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) total += fold_sq[w * kFoldRows + threadIdx.x];
+            fold_scale[threadIdx.x] = 1.0f / sqrtf(total / static_cast<float>(a.K) + a.eps);
+        }
+#pragma unroll 1
+        while (kbase < k_end) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ka = kbase + u * WAVES * 128;
+                uint4 av[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int k_lane = ka + i * 32 + g * 8;
+                    av[i] = (r < a.M && k_lane < k_end)
+                                ? *reinterpret_cast<const uint4*>(fold_rows + static_cast<size_t>(r) * a.K + k_lane)
+                                : uint4{0, 0, 0, 0};
+                }
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        *reinterpret_cast<uint4*>(stage + (i * 4 + load_row) * kStageRow + load_col * 2) = b[u][t][i];
+                    uint4 bt[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) bt[j] = *reinterpret_cast<const uint4*>(stage + r * kStageRow + j * 64 + g * 16);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8, av[j]), __builtin_bit_cast(bf16x8, bt[j]), acc[0][t], 0, 0, 0);
+                }
+            }
+            kbase += U * WAVES * 128;
+            if (kbase < k_end) load_w(kbase);
+        }
+    } else {
 #pragma unroll 1
     for (int kbase = k_begin + wave * 128; kbase < k_end; kbase += U * WAVES * 128) {
         uint4 b[U][NT][4];
@@ -541,6 +671,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
                             __builtin_bit_cast(bf16x8, av[mt][j]), __builtin_bit_cast(bf16x8, bt[j]), acc[mt][t], 0, 0, 0);
             }
         }
+    }
     }
 
     if (rope_pending) {  // (a K so short that this wave had no slice)
@@ -641,6 +772,14 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
                 store_resid(a, acc[0][t], resid_rows[t], m0, (tile_first + t) * 16 + r, tile_first + t, lane);
         return;
     }
+    if constexpr (FOLD) {  // the rows' 1/rms, which the rows of A were made without
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float scale = fold_scale[min(g * 4 + i, kFoldRows - 1)];  // (rows past the last are not stored)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[0][t][i] *= scale;
+        }
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         if (EPI == EPI_ROPE8) {
@@ -658,14 +797,14 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     }
 }
 
-template <int EPI, int MT, int NT>
+template <int EPI, int MT, int NT, bool FOLD = false>
 int launch_waves(hipStream_t s, int waves, dim3 grid, const FusedArgs& a) {
     if constexpr (MT == 1) {
         switch (waves) {
-            case 1: gemm_rows_kernel<1, EPI, MT, NT><<<grid, 64, 0, s>>>(a); break;
-            case 2: gemm_rows_kernel<2, EPI, MT, NT><<<grid, 128, 0, s>>>(a); break;
-            case 4: gemm_rows_kernel<4, EPI, MT, NT><<<grid, 256, 0, s>>>(a); break;
-            case 8: gemm_rows_kernel<8, EPI, MT, NT><<<grid, 512, 0, s>>>(a); break;
+            case 1: gemm_rows_kernel<1, EPI, MT, NT, FOLD><<<grid, 64, 0, s>>>(a); break;
+            case 2: gemm_rows_kernel<2, EPI, MT, NT, FOLD><<<grid, 128, 0, s>>>(a); break;
+            case 4: gemm_rows_kernel<4, EPI, MT, NT, FOLD><<<grid, 256, 0, s>>>(a); break;
+            case 8: gemm_rows_kernel<8, EPI, MT, NT, FOLD><<<grid, 512, 0, s>>>(a); break;
             default: return CIE_BAD_ARGUMENT;
         }
     } else {  // more row tiles: four or eight waves (waves that find no slice of K add zeros)
@@ -978,6 +1117,11 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     f.row_sumsq = row_sumsq;
     f.sumsq_parts = sumsq_parts;
     f.eps = eps;
+    f.fold_residual = nullptr;
+    f.fold_parts = nullptr;
+    f.fold_n_parts = 0;
+    f.fold_weight = nullptr;
+    f.fold_residual_out = nullptr;
     f.rope = RopeArgs{};
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (epilogue) {
@@ -999,12 +1143,32 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
 // leave two thirds of the compute units without a workgroup.)
 constexpr unsigned kSplitPairsBelow = 128;
 
-CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
-                              int M, int N, int K, int waves, const float* cos_table, const float* sin_table,
-                              const int* positions, const int* seq_of_token, const int* seq_slot,
-                              const int* block_table, int table_width, void* k_pool, void* v_pool, int q_heads,
-                              int kv_heads, int head_dim, int page_size, int rotate, int write_kv) {
-    if (M <= 0 || (M + 63) / 64 > 65535 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
+namespace {
+struct FoldedNorm {  // the norm in front of the q/k/v product, made by the product itself (see FusedArgs)
+    const float* residual = nullptr;
+    const float* parts = nullptr;
+    int n_parts = 0;
+    const float* weight = nullptr;
+    float eps = 0.f;
+    float* residual_out = nullptr;
+};
+
+int qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
+             int M, int N, int K, int waves, const float* cos_table, const float* sin_table,
+             const int* positions, const int* seq_of_token, const int* seq_slot,
+             const int* block_table, int table_width, void* k_pool, void* v_pool, int q_heads,
+             int kv_heads, int head_dim, int page_size, int rotate, int write_kv, const FoldedNorm* fold) {
+    if (fold) {
+        if (M <= 0 || M > kFoldRows || K <= 0 || K % 8 || static_cast<long long>(M) * K > kFoldElems || !w || !c)
+            return CIE_BAD_ARGUMENT;
+        if (!fold->residual || !fold->parts || fold->n_parts < 1 || fold->n_parts > 64 || !fold->weight ||
+            !(fold->eps > 0.f) || !fold->residual_out || fold->residual_out == fold->residual)
+            return CIE_BAD_ARGUMENT;
+        a = nullptr;
+        lda = K;
+    } else if (M <= 0 || (M + 63) / 64 > 65535 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) {
+        return CIE_BAD_ARGUMENT;
+    }
     if (q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 32 || page_size <= 0 || table_width <= 0 ||
         N != (q_heads + 2 * kv_heads) * head_dim)
         return CIE_BAD_ARGUMENT;
@@ -1029,18 +1193,65 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
     f.row_sumsq = nullptr;
     f.sumsq_parts = 0;
     f.eps = 0.f;
+    f.fold_residual = nullptr;
+    f.fold_parts = nullptr;
+    f.fold_n_parts = 0;
+    f.fold_weight = nullptr;
+    f.fold_residual_out = nullptr;
     f.rope = RopeArgs{cos_table, sin_table, positions, seq_of_token, seq_slot, block_table, table_width,
                       static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads, head_dim,
                       page_size, rotate, write_kv};
     const dim3 grid((q_heads + 2 * kv_heads) * (head_dim / 32), M <= 64 ? 1 : (M + 63) / 64, 1);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (M <= 16 && grid.x < kSplitPairsBelow) {  // few columns: one tile a workgroup, twice the workgroups
-        const dim3 twice((q_heads + 2 * kv_heads) * (head_dim / 16), 1, 1);
-        return launch_waves<EPI_ROPE8, 1, 1>(s, waves, twice, f);
+    const dim3 twice((q_heads + 2 * kv_heads) * (head_dim / 16), 1, 1);
+    const bool one_tile = M <= 16 && grid.x < kSplitPairsBelow;  // few columns: one tile a workgroup, twice the workgroups
+    if (fold) {
+        f.fold_residual = fold->residual;
+        f.fold_parts = fold->parts;
+        f.fold_n_parts = fold->n_parts;
+        f.fold_weight = fold->weight;
+        f.eps = fold->eps;
+        f.fold_residual_out = fold->residual_out;
+        if (one_tile) return launch_waves<EPI_ROPE8, 1, 1, true>(s, waves, twice, f);
+        return launch_waves<EPI_ROPE, 1, 2, true>(s, waves, grid, f);
     }
+    if (one_tile) return launch_waves<EPI_ROPE8, 1, 1>(s, waves, twice, f);
     if (M <= 16) return launch_waves<EPI_ROPE, 1, 2>(s, waves, grid, f);
     if (M <= 32) return launch_waves<EPI_ROPE, 2, 2>(s, waves, grid, f);
     return launch_waves<EPI_ROPE, 4, 2>(s, waves, grid, f);
+}
+}  // namespace
+
+CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
+                              int M, int N, int K, int waves, const float* cos_table, const float* sin_table,
+                              const int* positions, const int* seq_of_token, const int* seq_slot,
+                              const int* block_table, int table_width, void* k_pool, void* v_pool, int q_heads,
+                              int kv_heads, int head_dim, int page_size, int rotate, int write_kv) {
+    return qkv_rope(stream, a, lda, w, bias, c, M, N, K, waves, cos_table, sin_table, positions, seq_of_token, seq_slot,
+                    block_table, table_width, k_pool, v_pool, q_heads, kv_heads, head_dim, page_size, rotate, write_kv,
+                    nullptr);
+}
+
+// The same for up to 4 rows (rows x K <= 8,192) whose RMSNorm the product makes itself: the rows are
+// (residual + the n_parts partial sums `parts` [n_parts, M, K]) * norm_weight * 1/rms, and the summed stream goes
+// to residual_out [M, K] (another buffer than residual).  A decode step of a few sequences saves the norm's kernel.
+CIE_API int cie_gemm_qkv_rope_folded_norm(void* stream, const float* residual, const float* parts, int n_parts,
+                                          const float* norm_weight, float eps, float* residual_out, const void* w,
+                                          const void* bias, void* c, int M, int N, int K, int waves,
+                                          const float* cos_table, const float* sin_table, const int* positions,
+                                          const int* seq_of_token, const int* seq_slot, const int* block_table,
+                                          int table_width, void* k_pool, void* v_pool, int q_heads, int kv_heads,
+                                          int head_dim, int page_size, int rotate, int write_kv) {
+    FoldedNorm fold;
+    fold.residual = residual;
+    fold.parts = parts;
+    fold.n_parts = n_parts;
+    fold.weight = norm_weight;
+    fold.eps = eps;
+    fold.residual_out = residual_out;
+    return qkv_rope(stream, nullptr, K, w, bias, c, M, N, K, waves, cos_table, sin_table, positions, seq_of_token,
+                    seq_slot, block_table, table_width, k_pool, v_pool, q_heads, kv_heads, head_dim, page_size, rotate,
+                    write_kv, &fold);
 }
 
 // The form for 17 to 128 rows in which a workgroup's waves own columns and share the rows of A
@@ -1075,6 +1286,11 @@ CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const voi
     f.row_sumsq = row_sumsq;
     f.sumsq_parts = sumsq_parts;
     f.eps = eps;
+    f.fold_residual = nullptr;
+    f.fold_parts = nullptr;
+    f.fold_n_parts = 0;
+    f.fold_weight = nullptr;
+    f.fold_residual_out = nullptr;
     f.rope = RopeArgs{};
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (epilogue) {

@@ -629,28 +629,61 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
 QKV_SPLIT_PAIRS_BELOW = 128  # (as in the kernel library: below this many pairs of tiles, one tile a workgroup)
 
 
-def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Tensor], cos: torch.Tensor,
+FOLDED_NORM_ROWS = 4      # the most rows whose norm the q/k/v product makes itself ...
+FOLDED_NORM_VALUES = 8192  # ... and the most values (rows x K) it keeps for that
+
+
+def folds_norm(rows: int, k: int) -> bool:
+    """Whether ``gemm_qkv_rope`` takes ``unsummed=`` for this many rows of ``k`` values."""
+    return 1 <= rows <= FOLDED_NORM_ROWS and rows * k <= FOLDED_NORM_VALUES and k % 8 == 0
+
+
+def gemm_qkv_rope(weight: torch.Tensor, a: Optional[torch.Tensor], bias: Optional[torch.Tensor], cos: torch.Tensor,
                   sin: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, seq_slot: torch.Tensor,
                   block_table: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, q_heads: int,
                   kv_heads: int, head_dim: int, rotate: bool = True, write_kv: bool = True,
-                  waves: Optional[int] = None) -> torch.Tensor:
+                  waves: Optional[int] = None, unsummed: Optional[tuple] = None):
     """The q/k/v product of a few rows (64 per workgroup) fused with what ``rope_kv_write`` does:
     ``a @ weight.T + bias`` for weight [(Hq+2Hkv)*D, K], queries and keys rotated
     by each row's position, keys and values written into the cache.  Returns the
     buffer [M, (Hq+2Hkv)*D] whose query columns hold the rotated queries (its key
     and value columns are not written).  Same results as ``gemm_fused`` followed
-    by ``rope_kv_write``.  Head sizes in steps of 32."""
+    by ``rope_kv_write``.  Head sizes in steps of 32.
+
+    ``unsummed=(residual, parts, norm_weight, eps)`` instead of ``a`` (``folds_norm`` says for which sizes):
+    the rows are the RMSNorm of ``residual + parts.sum(0)`` (float32 [M, K] and [P, M, K], float32 weight),
+    made inside the product; returns ``(buffer, summed)`` with the summed stream in a tensor of its own."""
     _gpu("weight", weight, torch.bfloat16, 2)
     n, k = weight.shape
-    if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
-        raise ValueError("a must be a bf16 GPU matrix with unit inner stride")
-    m = a.shape[0]
-    if not (m >= 1 and a.shape[1] == k):
-        raise ValueError(f"a {tuple(a.shape)}: rows of K={k}")
-    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    if unsummed is not None:
+        residual, parts, norm_weight, eps = unsummed
+        _gpu("residual", residual, torch.float32, 2)
+        _gpu("parts", parts, torch.float32, 3)
+        _gpu("norm_weight", norm_weight, torch.float32, 1)
+        m = residual.shape[0]
+        if a is not None or not folds_norm(m, k):
+            raise ValueError(f"the product makes the norm of up to {FOLDED_NORM_ROWS} rows and {FOLDED_NORM_VALUES} "
+                             f"values itself, not of {m} rows of {k}; and then takes no rows")
+        if not (residual.shape == (m, k) and parts.shape[1:] == (m, k) and 1 <= parts.shape[0] <= 64
+                and norm_weight.shape == (k,) and eps > 0):
+            raise ValueError(f"residual {tuple(residual.shape)}, parts {tuple(parts.shape)}, weight "
+                             f"{tuple(norm_weight.shape)} do not fit rows of K={k}")
+        if not (residual.is_contiguous() and parts.is_contiguous() and norm_weight.is_contiguous()
+                and residual.data_ptr() % 16 == 0 and parts.data_ptr() % 16 == 0 and norm_weight.data_ptr() % 16 == 0):
+            raise ValueError("residual, parts and weight must be contiguous and 16-byte aligned")
+        lda = k
+    else:
+        if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
+            raise ValueError("a must be a bf16 GPU matrix with unit inner stride")
+        m = a.shape[0]
+        if not (m >= 1 and a.shape[1] == k):
+            raise ValueError(f"a {tuple(a.shape)}: rows of K={k}")
+        lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+        if not (a.data_ptr() % 16 == 0):
+            raise ValueError("operands must be 16-byte aligned")
     if not (k % 8 == 0 and lda % 8 == 0):
         raise ValueError(f"K and the row stride must be multiples of 8, are {k} and {lda}")
-    if not (a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
+    if not (weight.data_ptr() % 16 == 0):
         raise ValueError("operands must be 16-byte aligned")
     if not (head_dim % 32 == 0):
         raise ValueError(f"the fused rotation takes head sizes in steps of 32, not {head_dim}")
@@ -680,6 +713,14 @@ def gemm_qkv_rope(weight: torch.Tensor, a: torch.Tensor, bias: Optional[torch.Te
     if not (waves in ((1, 2, 4, 8) if m <= 16 else (4, 8))):
         raise ValueError(f"{waves} waves per workgroup with {m} rows is not a form the kernel has")
     out = torch.empty((m, n), dtype=torch.bfloat16, device=weight.device)
+    if unsummed is not None:
+        summed = torch.empty_like(residual)
+        _run("cie_gemm_qkv_rope_folded_norm", load_library().cie_gemm_qkv_rope_folded_norm(
+            _stream(), _ptr(residual), _ptr(parts), _i(parts.shape[0]), _ptr(norm_weight), _f(eps), _ptr(summed),
+            _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k), _i(waves), _ptr(cos), _ptr(sin), _ptr(positions),
+            _ptr(seq_of_token), _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]), _ptr(k_pool), _ptr(v_pool),
+            _i(q_heads), _i(kv_heads), _i(head_dim), _i(page_size), _i(1 if rotate else 0), _i(1 if write_kv else 0)))
+        return out, summed
     _run("cie_gemm_qkv_rope", load_library().cie_gemm_qkv_rope(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k), _i(waves), _ptr(cos),
         _ptr(sin), _ptr(positions), _ptr(seq_of_token), _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]),

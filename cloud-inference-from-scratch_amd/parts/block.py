@@ -18,7 +18,7 @@ import torch
 from ..config.specs import LayerSpec
 from ..weights.tensors import TensorSpec
 from .base import build_part, register_part
-from .linear import PartialSum, RowSumsq
+from .linear import PartialSum, RowSumsq, UnsummedRows
 
 
 class PreNormBlock:
@@ -59,12 +59,19 @@ class PreNormBlock:
 
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], batch, view,
                 writes: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
-        x = normalise(self.norm1, residual, pending, self.dtype)
+        if (isinstance(pending, PartialSum) and getattr(self.mixer, "takes_unsummed_rows", False)
+                and getattr(self.norm1, "folds_into_products", False) and UnsummedRows.fits(residual, self.dtype)):
+            # a few rows: the mixer's first product sums the parts and makes the norm itself (a kernel less)
+            x = UnsummedRows(residual, pending.parts, self.norm1, self.dtype)
+        else:
+            x = normalise(self.norm1, residual, pending, self.dtype)
         extra = {"residual": residual} if getattr(self.mixer, "adds_to_residual", False) else {}
         if (extra and getattr(self.mixer, "folds_next_norm", False) and getattr(self.norm2, "folds_into_products", False)
                 and getattr(self.feed_forward, "takes_scaled_rows", False)):
             extra["next_norm"] = self.norm2  # the norm between the two rides along with their products
         mixed = self.mixer.forward(x, batch, view, writes, **extra)
+        if isinstance(x, UnsummedRows):
+            residual = x.residual  # the summed stream, where the mixer left it (and added its own output)
         x = normalise(self.norm2, residual, mixed, self.dtype)
         extra = {"residual": residual} if getattr(self.feed_forward, "adds_to_residual", False) else {}
         return residual, self.feed_forward.forward(x, **extra)

@@ -134,6 +134,40 @@ class PartialSum:
     parts: torch.Tensor
 
 
+# Rows up to which the q/k/v product sums the stream's pending parts and makes the norm itself.  Every workgroup
+# of the product then reads the whole row and all its parts (3B shape, 8 parts: 72 KB through each compute unit's
+# cache), which costs it 1.5 to 3 us where the norm's own kernel takes 4.6: decode of one sequence 434 -> 444
+# tokens/s (3B), 1,019 -> 1,062 (0.5B), 160 -> 161 (14B); with two rows 863 -> 848 (3B) and 1,996 -> 2,014 (0.5B),
+# with four 1,684 -> 1,548 and 3,798 -> 3,634: one row it is.
+UNSUMMED_ROWS = 1
+
+
+@dataclass
+class UnsummedRows:
+    """Stands where an RMSNorm's output would, before anything was computed: the rows are the norm ``norm``
+    of ``residual + parts.sum(0)``.  Only a mixer that says ``takes_unsummed_rows`` is shown it.  Whoever
+    sums the parts leaves the summed stream in ``residual`` (the same tensor, summed in place, or another
+    one): the block reads it there afterwards."""
+
+    residual: torch.Tensor
+    parts: torch.Tensor
+    norm: Any
+    dtype: torch.dtype = torch.bfloat16
+
+    @staticmethod
+    def fits(residual: torch.Tensor, dtype: torch.dtype) -> bool:
+        rows, width = residual.shape
+        return dtype == torch.bfloat16 and residual.is_cuda and rows <= UNSUMMED_ROWS and ops.folds_norm(rows, width)
+
+    @property
+    def shape(self):
+        return self.residual.shape
+
+    def complete(self) -> torch.Tensor:
+        """The norm's output after all (the parts are added into the stream in place)."""
+        return ops.add_parts_rmsnorm(self.residual, self.parts, self.norm.weight, self.norm.eps)
+
+
 _WIDENED: dict[int, tuple["weakref.ref", torch.Tensor]] = {}
 
 

@@ -580,6 +580,61 @@ def test_gemm_qkv_rope_equals_product_then_rotation(ops, geometry, rows, waves):
                           k_pool[..., :16].contiguous(), v_pool[:, :, :16].contiguous(), 1, 1, 16)
 
 
+@pytest.mark.parametrize("geometry", [(16, 2, 128, 16, 2048), (4, 2, 32, 8, 96), (3, 1, 64, 4, 328), (28, 4, 128, 16, 3584),
+                                      (5, 5, 96, 32, 200), (64, 8, 128, 16, 8192)])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4])
+@pytest.mark.parametrize("waves", [None, 1, 8])
+@pytest.mark.parametrize("n_parts", [1, 8, 11])
+def test_gemm_qkv_rope_that_sums_the_stream_and_makes_the_norm_itself(ops, geometry, rows, waves, n_parts):
+    """The q/k/v product of a few rows that is given the residual stream and its pending partial sums instead
+    of normalised rows: the summed stream, the rotated queries and the cache against float64 arithmetic on
+    the kernel's own operand rounding (rows are bf16(x * weight), their 1/rms multiplies the sums)."""
+    q_heads, kv_heads, head_dim, page_size, hidden = geometry
+    if not ops.folds_norm(rows, hidden):
+        with pytest.raises(ValueError, match="makes the norm of up to"):
+            ops.gemm_qkv_rope(rand(((q_heads + 2 * kv_heads) * head_dim, hidden), torch.bfloat16, 1), None, None,
+                              *([torch.zeros(1, device="cuda")] * 8), q_heads, kv_heads, head_dim,
+                              unsummed=(torch.zeros((rows, hidden), device="cuda"), torch.zeros((1, rows, hidden), device="cuda"),
+                                        torch.ones(hidden, device="cuda"), 1e-6))
+        return
+    n = (q_heads + 2 * kv_heads) * head_dim
+    eps = 1e-5
+    lengths = [40, 35, 100, 33][:rows]
+    k_pool, v_pool, table, slots, _ = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=61)
+    k_two, v_two = k_pool.clone(), v_pool.clone()
+    positions = [length - 1 for length in lengths]
+    residual = rand((rows, hidden), torch.float32, 62, 2.0)
+    parts = rand((n_parts, rows, hidden), torch.float32, 63, 0.7)
+    norm_weight = (1.0 + rand((hidden,), torch.float32, 64, 0.3)).contiguous()
+    w, b = rand((n, hidden), torch.bfloat16, 65, 0.05), rand((n,), torch.bfloat16, 66)
+    cos, sin = plain_qwen2.rope_tables(head_dim, 512, 1e6)
+    half = head_dim // 2
+    cos, sin = cos[:, :half].contiguous().cuda(), sin[:, :half].contiguous().cuda()
+    meta = (torch.tensor(positions, dtype=torch.int32).cuda(), torch.arange(rows, dtype=torch.int32).cuda(),
+            torch.tensor(slots, dtype=torch.int32).cuda(), table)
+    before = residual.clone()
+    fused, summed = ops.gemm_qkv_rope(w, None, b, cos, sin, *meta, k_pool, v_pool, q_heads, kv_heads, head_dim,
+                                      waves=waves, unsummed=(residual, parts, norm_weight, eps))
+    assert torch.equal(residual, before) and summed.data_ptr() != residual.data_ptr()  # the stream it read is left alone
+    want_sum = residual.double() + parts.double().sum(0)
+    torch.testing.assert_close(summed.double(), want_sum, rtol=1e-6, atol=1e-5)
+    scale = torch.rsqrt(want_sum.pow(2).mean(-1, keepdim=True) + eps)
+    operand = (summed * norm_weight).to(torch.bfloat16).double()  # the rows as the kernel rounds them
+    unrotated = ((operand @ w.double().t()) * scale + b.double()).to(torch.bfloat16)
+    ops.rope_kv_write(unrotated, cos, sin, *meta, k_two, v_two, q_heads, kv_heads, head_dim)
+    q_cols = q_heads * head_dim
+    # a bf16 step in a value before its rotation moves the rotated pair by that much of the larger of the two
+    step = dict(rtol=2 ** -6, atol=2 ** -7 * float(unrotated.float().abs().max()))
+    torch.testing.assert_close(fused[:, :q_cols].float(), unrotated[:, :q_cols].float(), **step)
+    torch.testing.assert_close(k_pool.float(), k_two.float(), **step)
+    torch.testing.assert_close(v_pool.float(), v_two.float(), **step)
+    # ... and it agrees with the two kernels it replaces to the rounding of their different order
+    normed = ops.add_parts_rmsnorm(residual.clone(), parts, norm_weight, eps)
+    two = ops.gemm_qkv_rope(w, normed, b, cos, sin, *meta, k_two, v_two, q_heads, kv_heads, head_dim)
+    torch.testing.assert_close(fused[:, :q_cols].float(), two[:, :q_cols].float(), rtol=2 ** -5,
+                               atol=2 ** -6 * float(unrotated.float().abs().max()))
+
+
 def test_rope_shift_invariance():
     """Scores of rotated q and k depend on the distance of their positions only
     (pins sign and pairing of the rotation in the plain implementation)."""

@@ -267,6 +267,50 @@ def test_block_part(dtype, rows, part_k, monkeypatch):
         check(pending.float().cpu(), branch, dtype)
 
 
+def test_block_whose_first_product_sums_the_pending_parts_of_one_row():
+    """A decode row whose stream still lacks the partial products of the layer before: in bfloat16 the block
+    hands both to its mixer, whose q/k/v product sums them and makes the norm itself.  The stream that comes
+    back is another tensor (the one that went in is left as it was), and everything agrees with the plain
+    block on the summed stream."""
+    from cie_amd.config import Qwen2Config
+    from cie_amd.parts.block import PreNormBlock
+    from cie_amd.parts.linear import PartialSum, RowSumsq
+
+    raw = dict(model_type="qwen2", hidden_size=96, num_hidden_layers=1, num_attention_heads=3,
+               num_key_value_heads=1, intermediate_size=88, vocab_size=32, rms_norm_eps=1e-5, rope_theta=1e4,
+               max_position_embeddings=128)
+    block = PreNormBlock(Qwen2Config.from_hf_config(raw).model_spec().layers[0])
+    w = bound(block, "model.layers.0.", "bfloat16", 15, scale=0.3)
+    prompt = 12
+    manager, device_cache = harness([block.cache_need()], [prompt + 1], dtype=block.dtype)
+    g = torch.Generator().manual_seed(16)
+    h = torch.randn((prompt + 1, 96), generator=g)
+    parts = torch.randn((5, 1, 96), generator=g) * 0.4
+    view = device_cache.view(0)
+    block.forward(h[:prompt].clone().cuda(), None, batch_of(manager, [(0, 0, prompt)]), view)
+    manager.commit_lengths({"r0": prompt})
+    last = h[prompt:].clone().cuda()
+    kept = last.clone()
+    out_residual, pending = block.forward(last, PartialSum(parts.cuda()), batch_of(manager, [(0, prompt, 1)]), view)
+    assert out_residual.data_ptr() != last.data_ptr() and torch.equal(last, kept)
+    summed = h.clone()
+    summed[prompt] += parts.sum(0)[0]
+    p = "model.layers.0."
+    cos, sin = plain.rope_tables(32, prompt + 1, 1e4)
+    a = plain.rms_norm(summed, w[p + "input_layernorm.weight"], 1e-5)
+    mid = summed + plain.attention_layer(a, w, p + "self_attn.", raw, cos, sin, torch.arange(prompt + 1))
+    m = plain.rms_norm(mid, w[p + "post_attention_layernorm.weight"], 1e-5)
+    branch = plain.swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    if isinstance(pending, PartialSum):
+        check(out_residual.cpu(), mid[prompt:], "bfloat16")
+        check(pending.parts.sum(0).cpu(), branch[prompt:], "bfloat16")
+    elif isinstance(pending, RowSumsq):
+        check(out_residual.cpu(), (mid + branch)[prompt:], "bfloat16")
+    else:
+        check(out_residual.cpu(), mid[prompt:], "bfloat16")
+        check(pending.float().cpu(), branch[prompt:], "bfloat16")
+
+
 # -- a toy mixer with state of its own -----------------------------------------------------
 def register_toy():
     """A decaying running sum per request: s_t = decay * s_{t-1} + W x_t, y_t = s_t.
