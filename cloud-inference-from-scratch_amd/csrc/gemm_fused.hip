@@ -520,46 +520,72 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
             rope_pending = false;
         }
         const bool writer = blockIdx.x == 0;
+        constexpr int kTogether = WAVES <= 4 ? 2 : 1;  // rows whose loads travel together
         float sq[kFoldRows] = {0.f, 0.f, 0.f, 0.f};
         for (int c = threadIdx.x * 8; c < a.K; c += WAVES * kWave * 8) {
             const float4 w0 = *reinterpret_cast<const float4*>(a.fold_weight + c);
             const float4 w1 = *reinterpret_cast<const float4*>(a.fold_weight + c + 4);
 #pragma unroll
-            for (int m = 0; m < kFoldRows; ++m) {
-                if (m >= a.M) break;  // (uniform)
-                const size_t at = static_cast<size_t>(m) * a.K + c;
-                float4 x0 = *reinterpret_cast<const float4*>(a.fold_residual + at);
-                float4 x1 = *reinterpret_cast<const float4*>(a.fold_residual + at + 4);
+            for (int m2 = 0; m2 < kFoldRows; m2 += kTogether) {
+                if (m2 >= a.M) break;  // (uniform)
+                // two rows at a time where the registers allow it (up to four waves: 512 each), so that the loads
+                // of both are under way together (a second row past the last reads the last again; nothing of
+                // it is kept)
+                float4 x0[kTogether], x1[kTogether];
+                size_t at[kTogether];
+#pragma unroll
+                for (int h = 0; h < kTogether; ++h) {
+                    at[h] = static_cast<size_t>(min(m2 + h, a.M - 1)) * a.K + c;
+                    x0[h] = *reinterpret_cast<const float4*>(a.fold_residual + at[h]);
+                    x1[h] = *reinterpret_cast<const float4*>(a.fold_residual + at[h] + 4);
+                }
                 // eight parts at a time, their loads all under way before the first is added (a part past the
                 // last reads the last again and is not added)
                 for (int p0 = 0; p0 < a.fold_n_parts; p0 += 8) {
-                    float4 v[8][2];
+                    float4 v[kTogether][8][2];
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const int part = min(p0 + j, a.fold_n_parts - 1);
-                        const float* src = a.fold_parts + (static_cast<size_t>(part) * a.M + m) * a.K + c;
-                        v[j][0] = *reinterpret_cast<const float4*>(src);
-                        v[j][1] = *reinterpret_cast<const float4*>(src + 4);
+                    for (int h = 0; h < kTogether; ++h) {
+                        if (h > 0 && m2 + h >= a.M) {  // (uniform: a single row asks for nothing twice)
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) v[h][j][0] = v[h][j][1] = float4{0.f, 0.f, 0.f, 0.f};
+                            continue;
+                        }
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const int part = min(p0 + j, a.fold_n_parts - 1);
+                            const float* src = a.fold_parts + static_cast<size_t>(part) * a.M * a.K + at[h];
+                            v[h][j][0] = *reinterpret_cast<const float4*>(src);
+                            v[h][j][1] = *reinterpret_cast<const float4*>(src + 4);
+                        }
                     }
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        if (p0 + j >= a.fold_n_parts) break;
-                        x0.x += v[j][0].x; x0.y += v[j][0].y; x0.z += v[j][0].z; x0.w += v[j][0].w;
-                        x1.x += v[j][1].x; x1.y += v[j][1].y; x1.z += v[j][1].z; x1.w += v[j][1].w;
+                    for (int h = 0; h < kTogether; ++h)
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            // (a select, not a branch: behind a branch the compiler waits for each part's loads in turn)
+                            const bool real = p0 + j < a.fold_n_parts;
+                            x0[h].x += real ? v[h][j][0].x : 0.f; x0[h].y += real ? v[h][j][0].y : 0.f;
+                            x0[h].z += real ? v[h][j][0].z : 0.f; x0[h].w += real ? v[h][j][0].w : 0.f;
+                            x1[h].x += real ? v[h][j][1].x : 0.f; x1[h].y += real ? v[h][j][1].y : 0.f;
+                            x1[h].z += real ? v[h][j][1].z : 0.f; x1[h].w += real ? v[h][j][1].w : 0.f;
+                        }
+                }
+#pragma unroll
+                for (int h = 0; h < kTogether; ++h) {
+                    if (m2 + h >= a.M) break;  // (uniform)
+                    sq[m2 + h] += (x0[h].x * x0[h].x + x0[h].y * x0[h].y) + (x0[h].z * x0[h].z + x0[h].w * x0[h].w) +
+                                  (x1[h].x * x1[h].x + x1[h].y * x1[h].y) + (x1[h].z * x1[h].z + x1[h].w * x1[h].w);
+                    if (writer) {
+                        *reinterpret_cast<float4*>(a.fold_residual_out + at[h]) = x0[h];
+                        *reinterpret_cast<float4*>(a.fold_residual_out + at[h] + 4) = x1[h];
                     }
+                    uint4 packed;
+                    packed.x = pack_bf16(x0[h].x * w0.x, x0[h].y * w0.y);
+                    packed.y = pack_bf16(x0[h].z * w0.z, x0[h].w * w0.w);
+                    packed.z = pack_bf16(x1[h].x * w1.x, x1[h].y * w1.y);
+                    packed.w = pack_bf16(x1[h].z * w1.z, x1[h].w * w1.w);
+                    *reinterpret_cast<uint4*>(fold_rows + at[h]) = packed;
                 }
-                sq[m] += (x0.x * x0.x + x0.y * x0.y) + (x0.z * x0.z + x0.w * x0.w) + (x1.x * x1.x + x1.y * x1.y) +
-                         (x1.z * x1.z + x1.w * x1.w);
-                if (writer) {
-                    *reinterpret_cast<float4*>(a.fold_residual_out + at) = x0;
-                    *reinterpret_cast<float4*>(a.fold_residual_out + at + 4) = x1;
-                }
-                uint4 packed;
-                packed.x = pack_bf16(x0.x * w0.x, x0.y * w0.y);
-                packed.y = pack_bf16(x0.z * w0.z, x0.w * w0.w);
-                packed.z = pack_bf16(x1.x * w1.x, x1.y * w1.y);
-                packed.w = pack_bf16(x1.z * w1.z, x1.w * w1.w);
-                *reinterpret_cast<uint4*>(fold_rows + at) = packed;
             }
         }
 #pragma unroll

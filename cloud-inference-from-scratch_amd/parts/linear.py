@@ -135,11 +135,13 @@ class PartialSum:
 
 
 # Rows up to which the q/k/v product sums the stream's pending parts and makes the norm itself.  Every workgroup
-# of the product then reads the whole row and all its parts (3B shape, 8 parts: 72 KB through each compute unit's
-# cache), which costs it 1.5 to 3 us where the norm's own kernel takes 4.6: decode of one sequence 434 -> 444
-# tokens/s (3B), 1,019 -> 1,062 (0.5B), 160 -> 161 (14B); with two rows 863 -> 848 (3B) and 1,996 -> 2,014 (0.5B),
-# with four 1,684 -> 1,548 and 3,798 -> 3,634: one row it is.
-UNSUMMED_ROWS = 1
+# of the product then reads the rows and all their parts (3B shape, 8 parts: 72 KB a row through each compute
+# unit's cache) while its first weight loads travel, which costs it some 2 us where the norm's own kernel takes
+# 4.6.  Decode tokens/s without and with, at 1 / 2 / 4 sequences: 3B 435 -> 451, 860 -> 886, 1,665 -> 1,687;
+# 0.5B 1,013 -> 1,066, 1,994 -> 2,071, 3,792 -> 3,839; 7B 304 -> 308, 602 -> 605 (four rows of its width are
+# more than the kernel keeps).  (The parts' loads must not stand behind a branch: with one, the compiler waited
+# for each part in turn and the trade was even at two rows and lost 8 % at four.)
+UNSUMMED_ROWS = 4
 
 
 @dataclass
