@@ -644,14 +644,24 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
         const int s = mine + u * groups;
         early[u] = (active && s < a.n_splits) ? po_row[s * stride] : floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    float m_local = -INFINITY;
-    for (int s = threadIdx.x; s < a.n_splits; s += blockDim.x)
+    // (a thread's first share: its maximum and its sum come together and are kept for the second pass)
+    const bool has_first = threadIdx.x < a.n_splits;
+    const float2 first_ml = has_first ? *reinterpret_cast<const float2*>(
+                                            a.part_ml + ((unit0 + threadIdx.x) * rows_per_tile + row) * 2)
+                                      : float2{-INFINITY, 0.f};
+    float m_local = first_ml.x;
+    for (int s = threadIdx.x + blockDim.x; s < a.n_splits; s += blockDim.x)
         m_local = fmaxf(m_local, a.part_ml[((unit0 + s) * rows_per_tile + row) * 2]);
     const float m_all = block_max(m_local, scratch);
     float den_local = 0.f;
-    for (int s = threadIdx.x; s < a.n_splits; s += blockDim.x) {
+    if (has_first) {
+        const float w = (first_ml.x == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(first_ml.x - m_all);  // maxima are kept in base 2
+        weight[threadIdx.x] = w;
+        den_local = first_ml.y * w;
+    }
+    for (int s = threadIdx.x + blockDim.x; s < a.n_splits; s += blockDim.x) {
         const float* ml = a.part_ml + ((unit0 + s) * rows_per_tile + row) * 2;
-        const float w = (ml[0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m_all);  // maxima are kept in base 2
+        const float w = (ml[0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ml[0] - m_all);
         weight[s] = w;
         den_local += ml[1] * w;
     }
@@ -663,9 +673,23 @@ attention_merge_kernel(AttentionArgs a, int head_dim, int rows_per_tile) {
             const int s = mine + u * groups;
             if (s < a.n_splits && weight[s] != 0.f) num += early[u] * weight[s];  // (a share without keys wrote no sums)
         }
-#pragma unroll 4
-        for (int s = mine + kEarly * groups; s < a.n_splits; s += groups)
-            if (weight[s] != 0.f) num += po_row[s * stride] * weight[s];
+        // the rest eight at a time, their loads all under way before the first is used: no branch stands between
+        // them (behind one the compiler waits for each load in turn; a sequence over 4,096 keys in 128 shares
+        // has twelve of them per thread).  A share past the last reads the last again, and what a share without
+        // keys left in its place is read too: a select drops both.
+        for (int s0 = mine + kEarly * groups; s0 < a.n_splits; s0 += 8 * groups) {
+            floatx4 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = po_row[min(s0 + j * groups, a.n_splits - 1) * stride];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int s = s0 + j * groups;
+                const float w = weight[min(s, a.n_splits - 1)];
+                const bool real = s < a.n_splits && w != 0.f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) num[i] += real ? v[j][i] * w : 0.f;
+            }
+        }
     }
     group_sum[threadIdx.x] = num;
     __syncthreads();

@@ -79,23 +79,43 @@ __global__ void add_parts_rmsnorm_vec4_kernel(float* __restrict__ residual, cons
     const size_t part_stride = static_cast<size_t>(rows_total) * hidden;
     const float* part0 = parts + static_cast<size_t>(row) * hidden;
     float sum_sq = 0.f;
-    for (int h = threadIdx.x * 4; h < hidden; h += blockDim.x * 4) {
+    // One pass: the stream's four values and those of all parts, eight parts at a time with all their loads
+    // under way before the first is added.  No branch stands between the loads (behind one the compiler waits
+    // for each in turn): a part past the last reads the last again and is dropped by a select.
+    auto pass = [&](int h) __attribute__((always_inline)) {
         float4 x = *reinterpret_cast<const float4*>(res + h);
-#pragma unroll 4
-        for (int p = 0; p < n_parts; ++p) {
-            const float4 v = *reinterpret_cast<const float4*>(part0 + p * part_stride + h);
-            x.x += v.x; x.y += v.y; x.z += v.z; x.w += v.w;
+        for (int p0 = 0; p0 < n_parts; p0 += 8) {
+            float4 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                v[j] = *reinterpret_cast<const float4*>(part0 + min(p0 + j, n_parts - 1) * part_stride + h);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const bool real = p0 + j < n_parts;
+                x.x += real ? v[j].x : 0.f; x.y += real ? v[j].y : 0.f;
+                x.z += real ? v[j].z : 0.f; x.w += real ? v[j].w : 0.f;
+            }
         }
         if (write_residual) *reinterpret_cast<float4*>(res + h) = x;
         *reinterpret_cast<float4*>(staged + h) = x;
         sum_sq += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+    };
+    // The first pass (the only one of a row of up to 4,096 values on 1,024 threads) stands outside the loop (at a
+    // loop's head the compiler waits for every load that is under way), and the weight of its values is asked for
+    // with its other loads.
+    const int h_first = threadIdx.x * 4;
+    uint2 raw_first = uint2{0u, 0u};
+    if (h_first < hidden) {
+        raw_first = *reinterpret_cast<const uint2*>(weight + h_first);
+        pass(h_first);
     }
+    for (int h = h_first + blockDim.x * 4; h < hidden; h += blockDim.x * 4) pass(h);
     const float total = block_sum(sum_sq, scratch);
     const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
     bf16_t* dst = out + static_cast<size_t>(out_row) * hidden;
     for (int h = threadIdx.x * 4; h < hidden; h += blockDim.x * 4) {
         const float4 x = *reinterpret_cast<const float4*>(staged + h);
-        const uint2 raw = *reinterpret_cast<const uint2*>(weight + h);
+        const uint2 raw = h == h_first ? raw_first : *reinterpret_cast<const uint2*>(weight + h);
         uint2 packed;
         packed.x = pack_bf16((x.x * inv) * __uint_as_float(raw.x << 16), (x.y * inv) * __uint_as_float(raw.x & 0xffff0000u));
         packed.y = pack_bf16((x.z * inv) * __uint_as_float(raw.y << 16), (x.w * inv) * __uint_as_float(raw.y & 0xffff0000u));
