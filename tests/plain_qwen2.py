@@ -91,10 +91,13 @@ def head_dim_of(config: dict) -> int:
 
 
 def attention_layer(x: torch.Tensor, weights: dict, prefix: str, config: dict, cos, sin,
-                    positions: torch.Tensor) -> torch.Tensor:
+                    positions: torch.Tensor, query_chunk: int | None = None) -> torch.Tensor:
     """reference src/cloud_engine/model.py:132-137, 214-217: q/k/v projections
     (+ bias when ``attention_bias``, default true for qwen2, model.py:80), view as
-    heads, rotate q and k, attend, o_proj without bias."""
+    heads, rotate q and k, attend, o_proj without bias.  ``query_chunk``: the queries
+    are attended a chunk at a time behind the keys before them (``past_len`` of
+    attention.py:88-112), so that a sequence of tens of thousands of tokens needs no
+    score matrix of its whole square."""
     d = head_dim_of(config)
     bias = config.get("attention_bias", True)
     t = x.shape[0]
@@ -106,14 +109,22 @@ def attention_layer(x: torch.Tensor, weights: dict, prefix: str, config: dict, c
     q, k, v = proj("q_proj"), proj("k_proj"), proj("v_proj")
     q = apply_rope(q, cos, sin, positions)
     k = apply_rope(k, cos, sin, positions)
-    context = causal_attention(q, k, v, 1.0 / math.sqrt(d), past_len=0)
+    if query_chunk is None or t <= query_chunk:
+        context = causal_attention(q, k, v, 1.0 / math.sqrt(d), past_len=0)
+    else:
+        context = torch.cat([
+            causal_attention(q[start:start + query_chunk], k[:start + query_chunk], v[:start + query_chunk],
+                             1.0 / math.sqrt(d), past_len=start)
+            for start in range(0, t, query_chunk)])
     return linear(context, weights[f"{prefix}o_proj.weight"])
 
 
-def forward(config: dict, weights: dict, token_ids: list[int], dtype: torch.dtype = torch.float32) -> torch.Tensor:
+def forward(config: dict, weights: dict, token_ids: list[int], dtype: torch.dtype = torch.float32,
+            query_chunk: int | None = None, rows: list[int] | None = None) -> torch.Tensor:
     """reference src/cloud_engine/model.py:194-228: embedding, per layer
     h += attn(norm(h)); h += mlp(norm(h)), final norm, float32 head (tied to the
-    embedding when ``tie_word_embeddings``).  Returns float32 logits [T, vocab]."""
+    embedding when ``tie_word_embeddings``).  Returns float32 logits [T, vocab], or
+    those of the positions ``rows`` only (model.py:222-225 selects rows before the head)."""
     w = {name: (t.to(dtype) if t.is_floating_point() else t) for name, t in weights.items()}
     eps = config["rms_norm_eps"]
     ids = torch.tensor(token_ids, dtype=torch.long)
@@ -123,10 +134,12 @@ def forward(config: dict, weights: dict, token_ids: list[int], dtype: torch.dtyp
     for i in range(config["num_hidden_layers"]):
         p = f"model.layers.{i}."
         a = rms_norm(h, w[p + "input_layernorm.weight"], eps)
-        h = h + attention_layer(a, w, p + "self_attn.", config, cos, sin, positions)
+        h = h + attention_layer(a, w, p + "self_attn.", config, cos, sin, positions, query_chunk)
         m = rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
         h = h + swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
     h = rms_norm(h, w["model.norm.weight"], eps)
+    if rows is not None:
+        h = h[torch.tensor(rows, dtype=torch.long)]
     head = w["model.embed_tokens.weight"] if config.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return h.to(torch.float32) @ head.to(torch.float32).t()
 

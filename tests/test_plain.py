@@ -157,6 +157,20 @@ def test_forward_is_causal_and_uses_the_right_head():
     assert plain.forward(TINY_A, tied, [5]).shape == (1, 256) and final.shape == (1, 64)
 
 
+def test_queries_in_chunks_and_selected_rows_change_nothing():
+    """Long sequences are attended a chunk of queries at a time, and only the wanted rows pass the head:
+    the same logits as the whole square, at a chunk that divides the length and one that does not."""
+    for raw in (TINY_A, TINY_B):
+        weights = tiny_weights(raw)
+        tokens = random_tokens(60, raw["vocab_size"], 8)
+        whole = plain.forward(raw, weights, tokens)
+        for chunk in (20, 7, 1):
+            torch.testing.assert_close(plain.forward(raw, weights, tokens, query_chunk=chunk), whole, rtol=1e-5, atol=1e-6)
+        rows = [0, 13, 59]
+        torch.testing.assert_close(plain.forward(raw, weights, tokens, query_chunk=16, rows=rows), whole[rows],
+                                   rtol=1e-5, atol=1e-6)
+
+
 def test_forward_bias_matters_and_softmax_weights_sum_to_one():
     weights = tiny_weights(TINY_A)
     tokens = random_tokens(12, 256, 7)
