@@ -12,6 +12,9 @@ Beyond the reference:
   writes a cache).  Units with the same need form a *group* with pages, an
   allocator and block tables of its own: ``PagedKV(window=None)`` keeps all
   keys, ``PagedKV(window=w)`` gives pages back once the window has passed them.
+* A unit may hold several things at once (a mixer whose ``cache_need`` is a tuple: two states of different
+  shape, or pages and a state beside them): each is a *cell* with a number of its own, and everything below
+  (groups, states, the device side) is kept per cell; ``unit_cells`` says which cells a unit has.
 * ``FixedState`` units get no pages; every request owns one *slot* (a row index
   below ``max_running``) from admission to release, which addresses both the
   fixed-size state rows and the request's row of the device block tables.
@@ -125,9 +128,11 @@ class CacheStats:
 
 
 class _Group:
-    def __init__(self, spec: PagedKV, units: list[int], num_pages: int, page_size: int) -> None:
+    def __init__(self, spec: PagedKV, units: list[int], num_pages: int, page_size: int,
+                 most_per_request: int | None = None) -> None:
         self.spec = spec
         self.units = units
+        self.most_per_request = most_per_request  # pages a request ever holds at once (a window group); None: no bound
         self.allocator = PageAllocator(num_pages, page_size)
         self.tables: dict[str, list[int]] = {}  # logical page index -> physical page, -1 once released
 
@@ -166,7 +171,17 @@ class CacheManager:
         self.max_model_len = max_model_len
         self.element_bytes = element_bytes  # of one cached number; only the byte statistics use it
         self.table_width = -(-max_model_len // page_size)
-        self.unit_specs = tuple(unit_specs)
+        # a unit's need may be a tuple of needs: every need becomes a cell; a unit with one need is its own cell
+        cells: list[PagedKV | FixedState | None] = []
+        self.unit_cells: list[int | tuple[int, ...]] = []
+        for spec in unit_specs:
+            if isinstance(spec, (tuple, list)):
+                self.unit_cells.append(tuple(range(len(cells), len(cells) + len(spec))))
+                cells.extend(spec)
+            else:
+                self.unit_cells.append(len(cells))
+                cells.append(spec)
+        self.unit_specs = tuple(cells)
         self.groups: list[_Group] = []
         self.unit_group: dict[int, int] = {}
         self.state_units: dict[int, FixedState] = {}
@@ -177,12 +192,12 @@ class CacheManager:
         for unit, spec in enumerate(self.unit_specs):
             if isinstance(spec, PagedKV):
                 if spec not in by_spec:
-                    pages = full_pages
+                    pages, per_request = full_pages, None
                     if spec.window is not None:
                         per_request = -(-(spec.window + prefill_chunk) // page_size) + 1
                         pages = min(full_pages, max_running * per_request)
                     by_spec[spec] = len(self.groups)
-                    self.groups.append(_Group(spec, [], pages, page_size))
+                    self.groups.append(_Group(spec, [], pages, page_size, per_request))
                 index = by_spec[spec]
                 self.groups[index].units.append(unit)
                 self.unit_group[unit] = index
@@ -240,6 +255,19 @@ class CacheManager:
                             if group.allocator.holders_of(node.page) == (PREFIX_HOLDER,))
             pages.append(free)
         return min(pages) * self.page_size
+
+    def tokens_missing(self, request_id: str, upto: int) -> int:
+        """What ``request_id`` (admitted or not) would still take of :meth:`free_tokens` to hold ``upto``
+        tokens: the pages it lacks in the group where it lacks most, times the page size.  A group that
+        keeps a window never holds more than the window and one step's portion."""
+        most = 0
+        for group in self.groups:
+            pages = group.allocator.pages_for(upto)
+            if group.most_per_request is not None:
+                pages = min(pages, group.most_per_request)
+            table = group.tables.get(request_id, ())
+            most = max(most, pages - sum(1 for page in table if page >= 0))
+        return max(0, most) * self.page_size
 
     def take_dirty_rows(self) -> list[tuple[int, int, list[int]]]:
         """(group, slot, table) of every block-table row that changed since the last call."""

@@ -1,7 +1,6 @@
 // The one entry point of this library that allocates nothing.
 //
-// It has no counterpart in the reference (whose greedy step is torch's argmax,
-// src/cloud_engine/engine.py:486-487).  It is for callers that cannot call
+// It has no counterpart in the reference.  It is for callers that cannot call
 // hipMalloc: code that runs under HIP graph capture, tight serving loops that
 // must never stall on the allocator, and harnesses that forbid allocation.
 //

@@ -1,13 +1,14 @@
-// Fused rotary position encoding (half-split pairing: element i rotates with
-// element i + D/2) of q and k, and the write of rotated k and of v into the
-// paged cache.
+// Fused rotary position encoding of q and k, and the write of rotated k and of v
+// into the paged cache.  The first R = rotary_dim dimensions of a head rotate
+// (half-split pairing: element i rotates with element i + R/2, i < R/2); those
+// from R on pass through unchanged.  R = D is the reference's rotation.
 //
 //   qkv  [tokens, (Hq + 2*Hkv) * D]   q rotated in place
 //   keys   [pages, Hkv, page_size, D]
 //   values [pages, Hkv, D, page_size]  (transposed, as the attention kernels read them)
 //   slot of token t: page = block_table[seq_slot[seq_of_token[t]], pos / P], row = pos % P
 //
-// Angles come from a float32 cos/sin table [max_position, D/2]; the rotation is
+// Angles come from a float32 cos/sin table [max_position, R/2]; the rotation is
 // computed in float32 and rounded once.  One workgroup per (token, head).
 #include "common.h"
 
@@ -19,11 +20,11 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
                                      const int* __restrict__ seq_slot,
                                      const int* __restrict__ block_table, int table_width,
                                      T* __restrict__ k_pool, T* __restrict__ v_pool, int q_heads,
-                                     int kv_heads, int head_dim, int page_size, int rotate,
+                                     int kv_heads, int head_dim, int rotary_dim, int page_size, int rotate,
                                      int write_kv) {
     const int token = blockIdx.x;
     const int head = blockIdx.y;  // [0,Hq): q   [Hq,Hq+Hkv): k   [Hq+Hkv,Hq+2Hkv): v
-    const int half = head_dim / 2;
+    const int half = rotary_dim / 2;
     const int pos = positions[token];
     T* src = qkv + (static_cast<size_t>(token) * (q_heads + 2 * kv_heads) + head) * head_dim;
 
@@ -59,19 +60,21 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, const float* __restric
         target[i] = from_float<T>(x1 * c - x2 * s);
         target[i + half] = from_float<T>(x2 * c + x1 * s);
     }
+    if (dst)  // what does not rotate goes to the cache as it is
+        for (int i = rotary_dim + threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
 }
 
-// bf16, head_dim a multiple of 16: one workgroup per token; a thread takes 8 rotation pairs (or 8
-// value elements) at a time with 16-byte accesses.
+// bf16, head_dim a multiple of 8 and rotary_dim of 16: one workgroup per token; a thread takes 8 rotation
+// pairs (or 8 elements that pass through, or 8 value elements) at a time with 16-byte accesses.
 __global__ void __launch_bounds__(256)
 rope_kv_write_vec8_kernel(bf16_t* __restrict__ qkv, const float* __restrict__ cos_table,
                           const float* __restrict__ sin_table, const int* __restrict__ positions,
                           const int* __restrict__ seq_of_token, const int* __restrict__ seq_slot,
                           const int* __restrict__ block_table, int table_width, bf16_t* __restrict__ k_pool,
-                          bf16_t* __restrict__ v_pool, int q_heads, int kv_heads, int head_dim, int page_size,
-                          int rotate, int write_kv) {
+                          bf16_t* __restrict__ v_pool, int q_heads, int kv_heads, int head_dim, int rotary_dim,
+                          int page_size, int rotate, int write_kv) {
     const int token = blockIdx.x;
-    const int half = head_dim / 2;
+    const int half = rotary_dim / 2;
     const int chunks = half / 8;  // 8-pair chunks per head
     const int pos = positions[token];
     bf16_t* row = qkv + static_cast<size_t>(token) * (q_heads + 2 * kv_heads) * head_dim;
@@ -117,6 +120,15 @@ rope_kv_write_vec8_kernel(bf16_t* __restrict__ qkv, const float* __restrict__ co
         *reinterpret_cast<uint4*>(dst + i + half) = uint4{out_hi[0], out_hi[1], out_hi[2], out_hi[3]};
     }
     if (page < 0) return;
+    // key dimensions that do not rotate go to the cache as they are
+    const int passing = (head_dim - rotary_dim) / 8;
+    for (int item = threadIdx.x; item < kv_heads * passing; item += blockDim.x) {
+        const int head = item / passing;
+        const int d = rotary_dim + (item - head * passing) * 8;
+        bf16_t* dst = k_pool + ((static_cast<size_t>(page) * kv_heads + head) * page_size + in_page) * head_dim;
+        *reinterpret_cast<uint4*>(dst + d) =
+            *reinterpret_cast<const uint4*>(row + static_cast<size_t>(q_heads + head) * head_dim + d);
+    }
     // values: element d of the token goes to [d, pos % page_size] of the transposed page
     const int value_items = kv_heads * (head_dim / 8);
     for (int item = threadIdx.x; item < value_items; item += blockDim.x) {
@@ -137,17 +149,18 @@ CIE_API int cie_rope_kv_write(void* stream, int dtype, void* qkv, const float* c
                               const float* sin_table, const int* positions, const int* seq_of_token,
                               const int* seq_slot, const int* block_table, int table_width,
                               void* k_pool, void* v_pool, int tokens, int q_heads, int kv_heads,
-                              int head_dim, int page_size, int rotate, int write_kv) {
-    if (tokens < 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 2 || page_size <= 0 ||
-        table_width <= 0)
+                              int head_dim, int rotary_dim, int page_size, int rotate, int write_kv) {
+    if (tokens < 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || page_size <= 0 || table_width <= 0 ||
+        rotary_dim < 0 || rotary_dim % 2 || rotary_dim > head_dim)
         return CIE_BAD_ARGUMENT;
+    if (!rotate) rotary_dim = 0;
     if (tokens == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dtype == CIE_BF16 && head_dim % 16 == 0) {
+    if (dtype == CIE_BF16 && head_dim % 8 == 0 && rotary_dim % 16 == 0) {
         rope_kv_write_vec8_kernel<<<tokens, 256, 0, s>>>(
             static_cast<bf16_t*>(qkv), cos_table, sin_table, positions, seq_of_token, seq_slot, block_table, table_width,
-            static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads, head_dim, page_size, rotate,
-            write_kv);
+            static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads, head_dim, rotary_dim, page_size,
+            rotate, write_kv);
         return cie_after_launch();
     }
     dim3 grid(tokens, q_heads + 2 * kv_heads);
@@ -155,12 +168,12 @@ CIE_API int cie_rope_kv_write(void* stream, int dtype, void* qkv, const float* c
         rope_kv_write_kernel<float><<<grid, 64, 0, s>>>(
             static_cast<float*>(qkv), cos_table, sin_table, positions, seq_of_token, seq_slot, block_table,
             table_width, static_cast<float*>(k_pool), static_cast<float*>(v_pool), q_heads, kv_heads,
-            head_dim, page_size, rotate, write_kv);
+            head_dim, rotary_dim, page_size, rotate, write_kv);
     else if (dtype == CIE_BF16)
         rope_kv_write_kernel<bf16_t><<<grid, 64, 0, s>>>(
             static_cast<bf16_t*>(qkv), cos_table, sin_table, positions, seq_of_token, seq_slot, block_table,
             table_width, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads,
-            head_dim, page_size, rotate, write_kv);
+            head_dim, rotary_dim, page_size, rotate, write_kv);
     else
         return CIE_BAD_ARGUMENT;
     return cie_after_launch();

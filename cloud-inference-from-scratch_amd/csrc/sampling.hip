@@ -128,18 +128,27 @@ __device__ int pick_in_span(const float* row, int begin, int end, float best, fl
             for (int c = 0; c < chunks; ++c) total += s_chunk[c];
             target = fraction * total;
         }
-        float running = 0.f;
-        int owner = chunks - 1;  // if rounding leaves the target unreached: the last chunk (and its last token)
+        // If rounding leaves the target unreached (the sums here and the running sums below are made in
+        // different orders), the token is the last one that has any probability at all: the last chunk whose
+        // sum is not zero, and in it the last index whose own term is not zero.
+        float running = 0.f, before_owner = 0.f;
+        int owner = chunks - 1;
         for (int c = 0; c < chunks; ++c) {
             if (running + s_chunk[c] > target) {
                 owner = c;
+                before_owner = running;
                 break;
+            }
+            if (s_chunk[c] > 0.f) {
+                owner = c;
+                before_owner = running;
             }
             running += s_chunk[c];
         }
-        *s_target = target - running;  // what is left to reach inside the chunk
+        *s_target = target - before_owner;  // what is left to reach inside the chunk
         s_idx[0] = owner;
-        *s_pick = min(end, begin + (owner + 1) * kChunk) - 1;
+        s_idx[1] = -1;  // the last index of the chunk whose own term is not zero
+        *s_pick = 0x7fffffff;
     }
     __syncthreads();
     const int owner = s_idx[0];
@@ -159,14 +168,21 @@ __device__ int pick_in_span(const float* row, int begin, int end, float best, fl
     float running = threadIdx.x > 0 ? s_val[threadIdx.x - 1] : 0.f;
     int mine = 0x7fffffff;
     const float four[4] = {e.x, e.y, e.z, e.w};
+    int last = -1;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         running += four[i];
-        if (mine == 0x7fffffff && first + i < end && running > target) mine = first + i;
+        // (a token whose own term is zero is never the one: the sums of the threads before are made in
+        // another order than this running sum and may pass the target a hair earlier or later)
+        if (mine == 0x7fffffff && first + i < end && four[i] > 0.f && running > target) mine = first + i;
+        if (first + i < end && four[i] > 0.f) last = first + i;
     }
     if (mine != 0x7fffffff) atomicMin(s_pick, mine);  // the first index whose running sum passes the target
+    if (last >= 0) atomicMax(&s_idx[1], last);
     __syncthreads();
-    const int picked = *s_pick;
+    int picked = *s_pick;
+    if (picked == 0x7fffffff)  // unreached: the last token with a probability, or (none has one) the span's last
+        picked = s_idx[1] >= 0 ? s_idx[1] : min(end, begin + (owner + 1) * kChunk) - 1;
     __syncthreads();
     return picked;
 }
@@ -280,16 +296,22 @@ sample_final_kernel(const float* __restrict__ logits, const float* __restrict__ 
         float total = 0.f;
         for (int c = 0; c < parts; ++c) total += s_chunk[c];
         const float target = uniform[r] * total;
-        float running = 0.f;
+        // (unreached through rounding: the last part that has any probability, as inside a part)
+        float running = 0.f, before_owner = 0.f;
         int owner = parts - 1;
         for (int c = 0; c < parts; ++c) {
             if (running + s_chunk[c] > target) {
                 owner = c;
+                before_owner = running;
                 break;
+            }
+            if (s_chunk[c] > 0.f) {
+                owner = c;
+                before_owner = running;
             }
             running += s_chunk[c];
         }
-        s_target = target - running;
+        s_target = target - before_owner;
         s_idx[0] = owner;
     }
     __syncthreads();

@@ -71,7 +71,12 @@ class DeviceCache:
                 self._views[unit] = None
 
     def view(self, unit: int) -> Any:
-        return self._views[unit]
+        """What the mixer of cache unit ``unit`` is handed: a ``PagedView``, a ``StateView``, nothing, or,
+        for a mixer whose need is a tuple, the tuple of its views in the same order."""
+        cells = self.manager.unit_cells[unit]
+        if isinstance(cells, tuple):
+            return tuple(self._views[cell] for cell in cells)
+        return self._views[cells]
 
     def bytes(self) -> int:
         pools = self.key_pools + [p for p in self.value_pools if p is not None]

@@ -209,8 +209,8 @@ class MixedGraphs:
     replayed; with a 64-token portion 4.4 and 4.2 ms; with 256 tokens the GPU is the slower one either way).  A capture costs as
     much as ten such steps, so only shapes that come again are captured: a step's shape is (bucket of its
     single-token rows, the lengths of its portions); one that comes a second time (the portions of one
-    long prompt beside the same decoding requests do) is captured from that very step, with its real
-    tokens, slots and pages, and replayed from then on.  As in captured decode steps, the parts of the
+    long prompt beside the same decoding requests do) is captured, on rows of padding, and replayed from
+    then on.  As in captured decode steps, the parts of the
     keys are sized on the device from the step's longest context.  The least recently used shapes beyond
     ``limit`` are dropped.  The reference captures decode steps only (src/cloud_engine/engine.py:316-437)."""
 
@@ -321,15 +321,30 @@ class MixedGraphs:
         host[o["max_context"]] = max(e.start_pos + len(e.tokens) for e in list(single) + list(portions))
         step.dev.copy_(to_device_staging(host, self.runner.device), non_blocking=True)
 
+    def _fill_padding(self, step: _CapturedStep) -> None:
+        """Every row padding: token 0 on the pad slot, the portions at positions 0, 1, ... of it (its block
+        table names the pad page at every place)."""
+        o, host = step.offsets, step.host
+        positions = [0] * step.decode_rows + [p for count in step.portions for p in range(count)]
+        sequences = step.decode_rows + len(step.portions)
+        host[o["token_ids"]: o["token_ids"] + len(positions)] = 0
+        host[o["positions"]: o["positions"] + len(positions)] = torch.tensor(positions, dtype=torch.int32)
+        host[o["seq_slot"]: o["seq_slot"] + sequences] = self.runner.device_cache.pad_slot
+        host[o["seq_start"]: o["seq_start"] + sequences] = 0
+        host[o["max_context"]] = max(step.portions)
+        step.dev.copy_(to_device_staging(host, self.runner.device), non_blocking=True)
+
     def _capture(self, step: _CapturedStep) -> None:
-        """Capture from the buffer as it is filled: the step's own tokens, slots and pages (the cache has
-        room for them already), so that the run before the capture and the first replay write what the
-        step has to write anyway."""
+        """Capture on rows of padding, as the decode steps are: the run before the capture (libraries set
+        themselves up, tile lists are made) and the capture itself touch the pad slot and the pad page only,
+        so that a part which keeps a state per request (and would advance it at every run) sees each of the
+        step's tokens once, at the replay."""
         runner = self.runner
+        self._fill_padding(step)
         torch.cuda.synchronize()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):  # outside capture: libraries set themselves up, tile lists are made
+        with torch.cuda.stream(side):
             runner.model.forward(step.batch, runner.device_cache)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
@@ -347,12 +362,10 @@ class MixedGraphs:
         single = [e for e in entries if len(e.tokens) == 1]
         portions = [e for e in entries if len(e.tokens) > 1]
         step = self.steps.pop(shape, None)
-        fresh = step is None
-        if fresh:
+        if step is None:
             step = self._layout(shape)
-        self._fill(step, single, portions)
-        if fresh:
             self._capture(step)  # (a capture that fails leaves no half-made entry behind)
+        self._fill(step, single, portions)
         self.steps[shape] = step  # last in the order of use
         while len(self.steps) > self.limit:
             del self.steps[next(iter(self.steps))]

@@ -54,6 +54,50 @@ class PendingTokens:
         return dict(zip(self.request_ids, self.host.tolist()))
 
 
+# What a running engine needs of the device memory beside weights and cache, set aside before the cache takes
+# its share of what is free: the vendor library's workspace, the copies of a weight its timing runs stream
+# through (gemm_library.hip keeps up to 640 MB of them while a shape's candidates are timed), and a full step's
+# activations (per token and number of the model's width: the float32 stream, the 16-bit rows of the norms,
+# projections and feed-forward, and partial sums, some 64 bytes) and float32 logits.
+LIBRARY_TIMING_BYTES = 640 << 20
+ACTIVATION_BYTES_PER_NUMBER = 64
+
+
+def flat_needs(needs: Sequence[Any]) -> list[Any]:
+    """The needs of a model's cache units, a unit of several needs spread out."""
+    out: list[Any] = []
+    for need in needs:
+        out.extend(need) if isinstance(need, (tuple, list)) else out.append(need)
+    return out
+
+
+def reserve_bytes(config: EngineConfig, hidden_size: int, vocab_size: int) -> int:
+    """Device memory kept out of the cache's reach (see above)."""
+    reserve = ops.LIBRARY_WORKSPACE_BYTES
+    if config.search_library_algorithms:
+        reserve += LIBRARY_TIMING_BYTES
+    reserve += config.token_budget * hidden_size * ACTIVATION_BYTES_PER_NUMBER
+    reserve += 2 * config.max_running * vocab_size * 4
+    return reserve
+
+
+def tokens_from_bytes(config: EngineConfig, needs: Sequence[Any], element_bytes: int, free_bytes: int,
+                      hidden_size: int, vocab_size: int) -> int:
+    """The pool's size in tokens where none is given: ``kv_cache_bytes``, or ``kv_cache_fraction`` of the
+    ``free_bytes`` that are left once :func:`reserve_bytes` is set aside; never more than every slot full and
+    the prefix index can use, never less than one page."""
+    per_token = sum(n.numbers_per_token * element_bytes for n in flat_needs(needs) if isinstance(n, PagedKV))
+    page = config.page_size
+    if per_token == 0:
+        return page
+    budget = config.kv_cache_bytes
+    if budget is None:
+        budget = int(max(0, free_bytes - reserve_bytes(config, hidden_size, vocab_size)) * config.kv_cache_fraction)
+    tokens = budget // per_token
+    useful = (config.max_running * -(-config.max_model_len // page) + config.prefix_cache_pages) * page
+    return max(page, min(tokens, useful) // page * page)
+
+
 class Runner:
     def __init__(self, model: Any, config: EngineConfig, device: str | torch.device = "cuda:0") -> None:
         if not torch.cuda.is_available():
@@ -82,23 +126,17 @@ class Runner:
                              if self.graphs is not None and config.graph_mixed_steps > 0 else None)
         self._staging = [None, None]
         self._staging_turn = 0
-        if config.search_library_algorithms:
-            ops.LIBRARY_SEARCH_ROWS.update({config.token_budget, min(config.prefill_chunk, config.token_budget)})
+        # the row counts whose products time every algorithm of the vendor library: this engine's full steps
+        self.search_rows = (frozenset({config.token_budget, min(config.prefill_chunk, config.token_budget)})
+                            if config.search_library_algorithms else frozenset())
 
     def _tokens_from_bytes(self, needs: list[Any]) -> int:
-        element = torch.tensor([], dtype=self.dtype).element_size()
-        per_token = sum(n.numbers_per_token * element for n in needs if isinstance(n, PagedKV))
-        if per_token == 0:
-            return self.config.page_size
-        page = self.config.page_size
-        budget = self.config.kv_cache_bytes
-        if budget is None:
+        free = 0
+        if self.config.kv_cache_bytes is None:
             free, _total = torch.cuda.mem_get_info(self.device)
-            budget = int(free * self.config.kv_cache_fraction)
-        tokens = budget // per_token
-        # more than every slot full plus the prefix index can never be used
-        useful = (self.config.max_running * -(-self.config.max_model_len // page) + self.config.prefix_cache_pages) * page
-        return max(page, min(tokens, useful) // page * page)
+        spec = self.model.spec
+        return tokens_from_bytes(self.config, needs, torch.tensor([], dtype=self.dtype).element_size(), free,
+                                 spec.hidden_size, spec.vocab_size)
 
     # -- what the scheduler calls ------------------------------------------------
     def admit(self, request: Any) -> None:
@@ -112,12 +150,13 @@ class Runner:
         all bucket sizes, and let the products of full prompt portions (one request's portion, and the
         sizes up to the token budget that time the library's candidates) set themselves up.  Returns
         the number of graphs captured."""
-        captured = self.graphs.capture_all() if self.graphs is not None else 0
-        budget, chunk = self.config.token_budget, min(self.config.prefill_chunk, self.config.token_budget)
-        rows = {chunk} | {n for n in range(512, budget + 1, 256)}
-        warm = getattr(self.model, "warm_up", None)
-        if warm is not None:
-            warm(sorted(rows))
+        with ops.library_search(self.search_rows):
+            captured = self.graphs.capture_all() if self.graphs is not None else 0
+            budget, chunk = self.config.token_budget, min(self.config.prefill_chunk, self.config.token_budget)
+            rows = {chunk} | {n for n in range(512, budget + 1, 256)}
+            warm = getattr(self.model, "warm_up", None)
+            if warm is not None:
+                warm(sorted(rows))
         return captured
 
     def publish_prefix(self, request: Any) -> None:
@@ -147,6 +186,12 @@ class Runner:
     def free_tokens(self) -> int:
         """Tokens the pool could take now (see :meth:`CacheManager.free_tokens`)."""
         return self.cache.free_tokens()
+
+    def tokens_needed(self, request: Any, upto: int) -> int:
+        """What the request would still take of :meth:`free_tokens` to hold ``upto`` tokens: whole pages, in
+        the group that is shortest of them; a group that keeps a window only never asks for more than the
+        window's pages; a cache without pages asks for nothing."""
+        return self.cache.tokens_missing(request.request_id, upto)
 
     def execute_batch(self, plan: Any) -> dict[str, int]:
         """Run a scheduler's plan and sample where it asks to (the reference's
@@ -297,7 +342,8 @@ class Runner:
         )
         decode = all(len(e.tokens) == 1 for e in entries)
         tokens = sum(len(e.tokens) for e in entries)
-        with trace_range(f"ragged.forward.{'decode' if decode else 'mixed'}.requests_{len(entries)}.tokens_{tokens}"):
+        with trace_range(f"ragged.forward.{'decode' if decode else 'mixed'}.requests_{len(entries)}.tokens_{tokens}"), \
+                ops.library_search(self.search_rows):
             shape = None
             if not decode and feed is None and self.mixed_graphs is not None:
                 shape = self.mixed_graphs.wants(entries)

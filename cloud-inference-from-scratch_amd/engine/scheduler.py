@@ -81,6 +81,7 @@ class Scheduler:
         self._release_knows_preemption = "preempted" in inspect.signature(runner.release).parameters
         self._resident = getattr(runner, "allocated_tokens", None)
         self._free = getattr(runner, "free_tokens", None)
+        self._needed = getattr(runner, "tokens_needed", None)
         self._publish = getattr(runner, "publish_prefix", None)
         self._launch = getattr(runner, "launch_decode", None)
         self._launchable = getattr(runner, "can_launch_decode", None)
@@ -155,16 +156,15 @@ class Scheduler:
         requests have taken what is known of them (plus the token each is about to sample)."""
         if self._free is None:
             return True
-        # (a request takes whole pages: one more token can cost a page)
-        page = max(1, int(getattr(self.config, "page_size", 1)))
-        whole_pages = lambda tokens: -(-tokens // page) * page
-        spoken_for = 0
-        for other in self.active:
-            if other.is_final:
-                continue
-            held = self._resident(other) if self._resident is not None else 0
-            spoken_for += max(0, whole_pages(other.known + 1) - held)
-        return self._free() - spoken_for >= whole_pages(request.known + 1)
+        needed = self._needed
+        if needed is None:
+            # a runner that does not say what a request costs it: whole pages of ``page_size`` per token
+            # (one more token can cost a page), less what the request holds
+            page = max(1, int(getattr(self.config, "page_size", 1)))
+            resident = self._resident if self._resident is not None else (lambda _request: 0)
+            needed = lambda r, upto: max(0, -(-upto // page) * page - resident(r))
+        spoken_for = sum(needed(other, other.known + 1) for other in self.active if not other.is_final)
+        return self._free() - spoken_for >= needed(request, request.known + 1)
 
     def _admit(self) -> bool:
         moved = False

@@ -8,6 +8,8 @@ on operands it was not written for.  Kernels run on torch's current stream.
 
 from __future__ import annotations
 
+import contextlib
+
 from typing import Optional
 
 import torch
@@ -22,6 +24,21 @@ _ERRORS = {1: "bad argument (a size or option the kernel does not take)", 2: "ke
 
 class KernelError(RuntimeError):
     pass
+
+
+_COMPUTE_UNITS: dict[int, int] = {}
+
+
+def compute_units(device: "torch.device | int | None" = None) -> int:
+    """Compute units of the GPU the kernels run on, asked of the device once (the plans that spread
+    workgroups over the units are made from it); 256, an MI355X's, where no GPU is visible."""
+    if not torch.cuda.is_available():
+        return 256
+    index = torch.cuda.current_device() if device is None else torch.device(device).index if not isinstance(device, int) else device
+    index = torch.cuda.current_device() if index is None else index
+    if index not in _COMPUTE_UNITS:
+        _COMPUTE_UNITS[index] = torch.cuda.get_device_properties(index).multi_processor_count
+    return _COMPUTE_UNITS[index]
 
 
 def _code(dtype: torch.dtype) -> int:
@@ -190,22 +207,24 @@ def rmsnorm_from_sumsq(residual: torch.Tensor, sumsq: torch.Tensor, weight: torc
 def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
                   seq_of_token: torch.Tensor, seq_slot: torch.Tensor, block_table: torch.Tensor,
                   k_pool: torch.Tensor, v_pool: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int,
-                  rotate: bool = True, write_kv: bool = True) -> None:
+                  rotate: bool = True, write_kv: bool = True, rotary_dim: Optional[int] = None) -> None:
     """Rotate q (in place) and k, write k and v of every token into its cache slot.
 
-    qkv [T, (Hq+2Hkv)*D]; cos/sin float32 [max_position, D/2]; key pool
-    [pages, Hkv, page_size, D] and value pool [pages, Hkv, D, page_size] in qkv's
-    dtype; block_table int32 [slots, width]."""
+    qkv [T, (Hq+2Hkv)*D]; the first ``rotary_dim`` dimensions of every head rotate (all of them if
+    ``None``), dimension i with i + rotary_dim/2, the rest pass through; cos/sin float32
+    [max_position, rotary_dim/2]; key pool [pages, Hkv, page_size, D] and value pool
+    [pages, Hkv, D, page_size] in qkv's dtype; block_table int32 [slots, width]."""
     _gpu("qkv", qkv, dims=2)
     tokens = qkv.shape[0]
     if not (qkv.shape[1] == (q_heads + 2 * kv_heads) * head_dim):
         raise ValueError(f"qkv row is {qkv.shape[1]}, heads say {(q_heads + 2 * kv_heads) * head_dim}")
-    if not (head_dim % 2 == 0):
-        raise ValueError(f"head_dim must be even, is {head_dim}")
+    rotary_dim = head_dim if rotary_dim is None else rotary_dim
+    if rotate and not (0 < rotary_dim <= head_dim and rotary_dim % 2 == 0):
+        raise ValueError(f"rotary_dim must be even and at most the head size {head_dim}, is {rotary_dim}")
     for name, table in (("cos", cos), ("sin", sin)):
         _gpu(name, table, torch.float32, 2)
-        if not (table.shape[1] == head_dim // 2):
-            raise ValueError(f"{name} must be [max_position, {head_dim // 2}]")
+        if rotate and not (table.shape[1] == rotary_dim // 2):
+            raise ValueError(f"{name} must be [max_position, {rotary_dim // 2}]")
     if not (cos.shape == sin.shape):
         raise ValueError("cos and sin tables differ in shape")
     for name, meta in (("positions", positions), ("seq_of_token", seq_of_token)):
@@ -218,7 +237,8 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
     _run("cie_rope_kv_write", load_library().cie_rope_kv_write(
         _stream(), _i(_code(qkv.dtype)), _ptr(qkv), _ptr(cos), _ptr(sin), _ptr(positions), _ptr(seq_of_token),
         _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]), _ptr(k_pool), _ptr(v_pool), _i(tokens),
-        _i(q_heads), _i(kv_heads), _i(head_dim), _i(page_size), _i(1 if rotate else 0), _i(1 if write_kv else 0)))
+        _i(q_heads), _i(kv_heads), _i(head_dim), _i(rotary_dim if rotate else 0), _i(page_size),
+        _i(1 if rotate else 0), _i(1 if write_kv else 0)))
 
 
 def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None, row_sumsq: Optional[torch.Tensor] = None,
@@ -578,12 +598,25 @@ LIBRARY_WORKSPACE_BYTES = 64 << 20
 # candidate algorithms at their first call and keep the fastest; others take its first choice.
 LIBRARY_TUNE_ROWS = 512
 # Row counts whose products time every algorithm the library has, not only the heuristic's candidates (a few
-# seconds for each shape, once in a process): an engine names the sizes of its full prompt portions here.
-LIBRARY_SEARCH_ROWS: set[int] = set()
+# seconds for each shape, once in a process).  An engine names the sizes of its full prompt portions around its
+# own steps (:func:`library_search`); outside of that nothing is searched, so one engine's choice does not
+# reach another's steps.
+_search_rows: frozenset = frozenset()
+
+
+@contextlib.contextmanager
+def library_search(rows):
+    """While the block runs, library products of these row counts time every algorithm at a shape's first call."""
+    global _search_rows
+    previous, _search_rows = _search_rows, frozenset(rows)
+    try:
+        yield
+    finally:
+        _search_rows = previous
 
 
 def _tune_level(rows: int) -> int:
-    if rows >= LIBRARY_TUNE_ROWS and rows in LIBRARY_SEARCH_ROWS:
+    if rows >= LIBRARY_TUNE_ROWS and rows in _search_rows:
         return 2
     if (rows >= LIBRARY_TUNE_ROWS and rows % 256 == 0) or (rows >= 32 and rows & (rows - 1) == 0):
         return 1

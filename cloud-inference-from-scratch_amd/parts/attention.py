@@ -101,7 +101,10 @@ class Attention(Part):
             )
         rows = x.shape[0]
         few = rows <= FUSED_ROWS or (rows <= FUSED_SMALL_ROWS and self.w_qkv.numel() <= FUSED_SMALL_WEIGHT)
-        untouched = type(self).shape_projection is Attention.shape_projection
+        # the projection's own kernel rotates whole heads only, and only an untouched projection
+        rotary_dim = getattr(self.position, "rotary_dim", self.head_dim) if self.position.rotates else None
+        untouched = (type(self).shape_projection is Attention.shape_projection
+                     and rotary_dim in (None, self.head_dim))
         if isinstance(x, UnsummedRows):
             if untouched and self.head_dim % 32 == 0 and self.w_qkv.dtype == torch.bfloat16:
                 # the product sums the stream's pending parts and makes the norm of its rows itself
@@ -126,14 +129,14 @@ class Attention(Part):
             qkv = self.shape_projection(linear(x, self.w_qkv, self.b_qkv), batch)
             ops.rope_kv_write(qkv, self.cos, self.sin, batch.positions, batch.seq_of_token, batch.seq_slot,
                               view.block_table, view.k_pool, view.v_pool, self.num_heads, self.num_kv_heads,
-                              self.head_dim, rotate=self.position.rotates, write_kv=writes)
+                              self.head_dim, rotate=self.position.rotates, write_kv=writes, rotary_dim=rotary_dim)
         context = attend(qkv, batch, view, self.num_heads, self.num_kv_heads, self.head_dim,
                          self.window, self.scale)
         return linear(context, self.w_o, self.b_o, into=residual, then_norm=next_norm)
 
 
 WIDE_DECODE_KEYS = 2048  # contexts from which decode rows go to the four-wave form
-WIDE_TARGET_WORKGROUPS = 256  # workgroups the four-wave form cuts long contexts for
+# (the four-wave form cuts long contexts for as many workgroups as the GPU has compute units)
 FEW_DECODE_UNITS = 8  # (sequence, kv head) pairs below which they do not: parts of one wave fill the GPU better
 MANY_DECODE_UNITS = 96  # (sequence, kv head) pairs from which decode rows take the four-wave form at any context
 SHARED_DECODE_KEYS = 96  # contexts from which four waves share a decode row's keys without cutting them
@@ -141,14 +144,14 @@ SPLIT_MIN_KEYS = 32  # the fewest keys of a one-wave part
 SPLIT_DECODE_KEYS = 192  # contexts from which the keys of decode rows are cut into parts at all
 JOINED_DECODE_ROWS = 32  # up to this many single-token sequences beside prompt portions ride in the prompt form's launch
 PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's keys are cut
-PROMPT_TARGET_WORKGROUPS = 256  # workgroups that cutting a prompt form's keys aims at
+# (cutting a prompt form's keys aims at as many workgroups as the GPU has compute units)
 # Tiles of 128 rows x kv heads from which prompt portions take the form of eight waves: enough to give most
 # compute units a workgroup without cutting the keys (whose parts, 64 KB of sums per tile and kv head, cost that
 # form more than they gain it: 512 tokens behind 1,536 keys, 7B heads, 60 us in two parts against 40 us in the form
 # of four waves).  Measured at head size 128 (us, four waves -> eight): 2,048 tokens of one prompt 55.7 -> 51.4
 # (3B heads), 101 -> 58 (7B), 144 -> 84 (14B); behind 2,048 keys 108 -> 91, 195 -> 135, 284 -> 201; beside 8 single
 # tokens 108 -> 64, 138 -> 75, 182 -> 111.
-EIGHT_WAVE_TILES = 192
+EIGHT_WAVE_TILES = 0.75  # of the compute units
 
 
 def plan_splits(units: int, max_keys: int, target_waves: int = 1024, min_keys: int = 128) -> tuple[int, int]:
@@ -174,6 +177,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     generic kernel."""
     group = num_heads // num_kv_heads
     page_size = view.page_size
+    cus = ops.compute_units()  # compute units of the GPU
     if (qkv.dtype != torch.bfloat16 or head_dim not in ops.MFMA_HEAD_DIMS or group > 16 or page_size < 4
             or page_size & (page_size - 1)):
         return ops.paged_attention_generic(
@@ -192,7 +196,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     big_tiles = -(-prompt_tokens * group // 128) * num_kv_heads
     # (heads of 128 dimensions: with 64 the form of four waves is the faster one, 2,048 tokens behind 6,144
     # keys 114 against 140 us, since the softmax arithmetic per key is the same and the products are half)
-    eight = wide and head_dim == 128 and group <= 128 and big_tiles >= EIGHT_WAVE_TILES
+    eight = wide and head_dim == 128 and group <= 128 and big_tiles >= max(1, EIGHT_WAVE_TILES * cus)
 
     def decode_form(bound: int, units: int) -> tuple[int, dict]:
         # Decode rows, `units` (sequence, kv head) pairs over up to `bound` keys.  Long contexts: four waves
@@ -201,19 +205,19 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         # one-wave form below, whose parts are smaller (one sequence of the 3B shape over 32,000 keys: 333 -> 363
         # tokens/s; from four sequences on the forms are level).
         if wide and bound >= WIDE_DECODE_KEYS and units >= FEW_DECODE_UNITS:
-            return ops.TILE_WAVES, dict(target_waves=WIDE_TARGET_WORKGROUPS, min_keys=32 * ops.TILE_WAVES)
+            return ops.TILE_WAVES, dict(target_waves=cus, min_keys=32 * ops.TILE_WAVES)
         # Many pairs fill the GPU by themselves: the same form with the keys whole or in large parts
         # (64 sequences x 2 heads x 256 keys: 9.2 us against 11.1 us with one wave per part)
         if wide and units >= MANY_DECODE_UNITS and bound >= SHARED_DECODE_KEYS:
-            return ops.TILE_WAVES, dict(target_waves=1024 // ops.TILE_WAVES, min_keys=512)
+            return ops.TILE_WAVES, dict(target_waves=4 * cus // ops.TILE_WAVES, min_keys=512)
         # Otherwise one wave per part, parts down to one block of 32 keys (8 x 256 keys: 7.3 us in 8 parts,
         # 10.2 us in 2; 8 x 512 keys: 8.1 us in 16 parts, 10.6 us in 4) ...
         if bound >= SPLIT_DECODE_KEYS:
-            return 1, dict(target_waves=1024, min_keys=SPLIT_MIN_KEYS)
+            return 1, dict(target_waves=4 * cus, min_keys=SPLIT_MIN_KEYS)
         # ... and below some 200 keys, where the merge costs more than it saves, four waves that share a
         # sequence's few blocks inside one workgroup instead of one wave that takes them in turn
         # (8 x 128 keys: 6.5 against 6.9 us, 8 x 160: 7 against 11)
-        return (ops.TILE_WAVES if wide and bound >= SHARED_DECODE_KEYS else 1), dict(target_waves=1024, min_keys=bound + 1)
+        return (ops.TILE_WAVES if wide and bound >= SHARED_DECODE_KEYS else 1), dict(target_waves=4 * cus, min_keys=bound + 1)
 
     plan = batch.static_plan
     longest_dev = None
@@ -264,14 +268,14 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         else:
             tile_waves = ops.TILE_WAVES
             row_tiles = 4 if head_dim <= 128 else 1
-            while row_tiles > 1 and -(-prompt_tokens * group // (16 * row_tiles)) * num_kv_heads * cuts < 192:
+            while row_tiles > 1 and -(-prompt_tokens * group // (16 * row_tiles)) * num_kv_heads * cuts < 0.75 * cus:
                 row_tiles //= 2
     else:
         # one wave per tile; fewer rows where that would leave SIMDs without a wave (about a thousand
         # waves fill the GPU) or where the accumulators of a wide head would spill
         tile_waves = 1
         row_tiles = 2 if head_dim > 128 else 4
-        while row_tiles > 1 and (prompt_tokens * group // (16 * row_tiles)) * num_kv_heads < 1024:
+        while row_tiles > 1 and (prompt_tokens * group // (16 * row_tiles)) * num_kv_heads < 4 * cus:
             row_tiles //= 2
     while 16 * row_tiles < group:
         row_tiles *= 2
@@ -280,7 +284,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     if n_tiles:
         # few tiles and many keys: parts of the keys, about as many workgroups as compute units
         n_splits, per_split, part_o, part_ml = 1, 0, None, None
-        wanted = min(cuts, int(PROMPT_TARGET_WORKGROUPS / (n_tiles * num_kv_heads) + 0.5))
+        wanted = min(cuts, int(cus / (n_tiles * num_kv_heads) + 0.5))
         if wanted > 1:
             per_split = -(-(-(-max_keys // wanted)) // 128) * 128
             n_splits = -(-max_keys // per_split)

@@ -61,7 +61,6 @@ SHARED_SILU_ROWS = 64
 # 173 in the form whose waves share K; 72 rows 165 / 239 / 333 against the library's 174 / 249 / 349; 96 rows
 # 172 / 255 / 346 against 174 / 238 / 338)
 SHARED_LOGIT_ROWS = 80
-COMPUTE_UNITS = 256
 
 
 def plan_shared_silu(pairs: int) -> tuple[int, bool]:
@@ -72,8 +71,9 @@ def plan_shared_silu(pairs: int) -> tuple[int, bool]:
     workgroups of four or 230 of three, one turn each; 1,184 of the 7B shape: two turns of four waves or
     two of three, 70 against 61 us at 64 rows; 864 of the 14B shape: one turn of four, 56 against 81 us)."""
     best = None
+    units = ops.compute_units()
     for waves in (4, 3, 2):
-        turns = -(-(-(-pairs // waves)) // COMPUTE_UNITS)
+        turns = -(-(-(-pairs // waves)) // units)
         if best is None or turns * waves < best[0]:
             best = (turns * waves, waves, turns == 1)
     return best[1], best[2]
@@ -85,10 +85,11 @@ def plan_shared_parts(tiles: int, k: int) -> tuple[int, int, int]:
     workgroup per compute unit.  Measured at 8 / 64 rows (us; the form of waves that share K, at its best
     cut, beside it): 128 tiles, K 11,008: 8 parts 11.0 / 14.8 (13.2 / 17.7); 224 tiles, K 18,944: 4 parts
     26.1 / 35.3 (29.7 / 43.8); 320 tiles, K 13,824, two tiles per wave: 4 parts 28.6 / 38.7 (30.0 / 44.0)."""
-    column_tiles = 1 if tiles <= COMPUTE_UNITS else 2
+    units = ops.compute_units()
+    column_tiles = 1 if tiles <= units else 2
     waves = 4
     blocks = -(-tiles // (column_tiles * waves))
-    parts = max(1, min(COMPUTE_UNITS // blocks, 16, k // PART_K))
+    parts = max(1, min(units // blocks, 16, k // PART_K))
     return column_tiles, waves, parts
 
 

@@ -443,3 +443,50 @@ def test_a_copy_of_indexed_tokens_is_not_stored_below_the_page_the_index_has():
     assert m.stats().pages_used == m.stats().prefix_pages_used == 3  # its own three full prompt pages, stored at its end
     m.clear_prefix_index()
     assert m.stats().pages_used == 0
+
+
+def test_a_unit_of_several_needs_is_kept_cell_by_cell():
+    """A mixer may need several things at once (``cache_need`` a tuple): pages and a state beside them, or two
+    states.  Each is a cell; cells with equal paged needs share a group whichever unit they belong to."""
+    from cie_amd.cache.manager import CacheManager, FixedState, PagedKV
+
+    keys = PagedKV(2, 16)
+    manager = CacheManager([keys, (keys, FixedState((3,), "int32")), None, (FixedState((2, 8)), FixedState((1,)))],
+                           page_size=4, kv_tokens=32, max_running=2, max_model_len=16)
+    assert manager.unit_cells == [0, (1, 2), 3, (4, 5)]
+    assert manager.unit_group == {0: 0, 1: 0} and manager.groups[0].units == [0, 1]
+    assert set(manager.state_units) == {2, 4, 5} and manager.unit_specs[3] is None
+    manager.admit("a")
+    manager.ensure_capacity_batch({"a": 9})
+    manager.commit_lengths({"a": 9})
+    assert manager.allocated_tokens("a") == 12 and manager.tokens_missing("a", 13) == 4
+    manager.release("a")
+    manager.assert_invariants()
+
+
+def test_pool_size_from_free_memory_keeps_a_reserve():
+    """Where no pool size is given the cache takes a share of the device memory that is free after the weights,
+    less what a running engine needs beside it: the library's workspace and timing copies, a full step's
+    activations and logits."""
+    from cie_amd.cache.manager import FixedState, PagedKV
+    from cie_amd.config import build_engine_config
+    from cie_amd.engine.runner import reserve_bytes, tokens_from_bytes
+
+    needs = [PagedKV(2, 128)] * 4 + [(PagedKV(2, 128), FixedState((8,)))]
+    per_token = 5 * 2 * 256 * 2
+    config = build_engine_config(max_model_len=1 << 15, max_running=1024, token_budget=2048, page_size=16,
+                                 prefix_cache_pages=0)
+    reserve = reserve_bytes(config, hidden_size=2048, vocab_size=150_000)
+    assert reserve >= (64 << 20) + (640 << 20) + 2048 * 2048 * 64 + 2 * 1024 * 150_000 * 4
+    free = 8 << 30
+    tokens = tokens_from_bytes(config, needs, 2, free, 2048, 150_000)
+    assert tokens == int((free - reserve) * 0.9) // per_token // 16 * 16
+    assert reserve_bytes(build_engine_config(search_library_algorithms=False), 2048, 150_000) < reserve - (600 << 20)
+    # less free memory than the reserve: one page, not a negative pool
+    assert tokens_from_bytes(config, needs, 2, reserve // 2, 2048, 150_000) == 16
+    # bytes given: taken as they are; never more than every slot full can use
+    given = build_engine_config(base=config, kv_cache_bytes=per_token * 1000)
+    assert tokens_from_bytes(given, needs, 2, 0, 2048, 150_000) == 992
+    small = build_engine_config(max_model_len=64, max_running=2, page_size=16, prefix_cache_pages=3)
+    assert tokens_from_bytes(small, needs, 2, free, 2048, 150_000) == (2 * 4 + 3) * 16
+    assert tokens_from_bytes(config, [FixedState((4,))], 2, free, 64, 100) == 16  # nothing is paged

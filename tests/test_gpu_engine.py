@@ -420,11 +420,15 @@ def test_ceilings_reports_what_the_gpu_reaches():
     done = subprocess.run([sys.executable, str(ROOT / "bin" / "cie"), "ceilings"], capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stderr[-2000:]
     record = json.loads(done.stdout.strip().splitlines()[-1])
-    for key in ("copy_1GiB_GBps", "read_1GiB_library_mv_GBps", "read_1GiB_few_row_product_GBps",
-                "read_45MB_few_row_product_GBps"):
-        assert 1000 < record[key] < 8000, (key, record[key])  # between a tenth of the published bandwidth and all of it
-    for key in ("bf16_8192_cubed_library_TFLOPs", "bf16_8192_cubed_library_tuned_TFLOPs"):
-        assert 300 < record[key] < 2500, (key, record[key])
+    # what this kind of box has reached before (one MI355X, the record under profiles/), give or take 30 %: a
+    # figure outside of that is a measurement gone wrong (a timer around the wrong thing, a product that is
+    # not the one named), or a box in another state than any seen so far
+    seen_before = {"copy_1GiB_GBps": 5159.4, "read_1GiB_library_mv_GBps": 5402.1, "read_1GiB_few_row_product_GBps": 5549.7,
+                   "read_45MB_few_row_product_GBps": 4277.2, "bf16_8192_cubed_library_TFLOPs": 1420.6,
+                   "bf16_8192_cubed_library_tuned_TFLOPs": 1578.3}
+    for key, before in seen_before.items():
+        assert 0.7 * before <= record[key] <= 1.3 * before, (key, record[key], before)
+    assert record["bf16_8192_cubed_library_tuned_TFLOPs"] >= 0.97 * record["bf16_8192_cubed_library_TFLOPs"]
 
 
 def test_text_prompts_go_through_the_folders_tokenizer(tiny_folders, tmp_path):

@@ -177,6 +177,53 @@ def test_attention_part_whole_and_in_portions(dtype, rotary):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("head_dim,rotary_dim,rows", [(32, 16, 7), (64, 32, 1), (48, 20, 5), (128, 64, 40)])
+def test_attention_part_with_a_rotation_of_the_first_dimensions_only(dtype, head_dim, rotary_dim, rows):
+    """A rotary part built with ``rotary_dim < head_dim`` turns the first ``rotary_dim`` dimensions of every
+    head (dimension i with i + rotary_dim / 2, angles of base ``theta`` over ``rotary_dim``) and lets the
+    rest pass: the plain rotation on that slice.  With few rows, too, where the projection's own kernel
+    would rotate whole heads: it must stand back."""
+    import math
+
+    from cie_amd.config import PartSpec
+    from cie_amd.parts.attention import Attention
+    from cie_amd.parts.position import RotaryHalf
+
+    with pytest.raises(ValueError):
+        RotaryHalf(head_dim=32, theta=1e4, max_position=8, rotary_dim=34)
+    with pytest.raises(ValueError):
+        RotaryHalf(head_dim=32, theta=1e4, max_position=8, rotary_dim=15)
+    hidden, heads, kv_heads = 64, 4, 2
+    position = PartSpec.of("rotary_half", head_dim=head_dim, theta=1e4, max_position=256, rotary_dim=rotary_dim)
+    attention = Attention(hidden, heads, kv_heads, head_dim, qkv_bias=True, out_bias=False, position=position)
+    w = bound(attention, "a.", dtype, 5, scale=0.3)
+    assert attention.cos.shape == (256, rotary_dim // 2)
+    total = rows + 3
+    manager, device_cache = harness([attention.cache_need()], [total],
+                                    dtype=torch.float32 if dtype == "float32" else torch.bfloat16, page_size=16)
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn((total, hidden), generator=g).to(attention.dtype)
+    # the plain parts, the rotation applied to the leading slice of every head
+    cos, sin = plain.rope_tables(rotary_dim, total, 1e4)
+    positions = torch.arange(total)
+
+    def heads_of(name):
+        return plain.linear(x.float(), w[f"a.{name}.weight"], w[f"a.{name}.bias"]).view(total, -1, head_dim)
+
+    def turned(t):
+        return torch.cat([plain.apply_rope(t[..., :rotary_dim], cos, sin, positions), t[..., rotary_dim:]], dim=-1)
+
+    context = plain.causal_attention(turned(heads_of("q_proj")), turned(heads_of("k_proj")), heads_of("v_proj"),
+                                     1.0 / math.sqrt(head_dim))
+    expected = plain.linear(context, w["a.o_proj.weight"])
+    view = device_cache.view(0)
+    first = attention.forward(x[:rows].cuda(), batch_of(manager, [(0, 0, rows)]), view)
+    manager.commit_lengths({"r0": rows})
+    rest = [attention.forward(x[i:i + 1].cuda(), batch_of(manager, [(0, i, 1)]), view) for i in range(rows, total)]
+    check(torch.cat([first] + rest).float().cpu(), expected, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_a_mixer_that_norms_its_heads_between_projection_and_rotation(dtype):
     """The seam between projection and rotation: a variant of the attention mixer, defined here, that
     divides every query and key head by its root mean square before the rotation overrides one method and
@@ -349,14 +396,75 @@ def register_toy():
                     view.state[slot] = state
             return out.to(x.dtype)
 
+    class RunningSumOnDevice(RunningSum):
+        """The same sum with every request's slot read on the device: what changes from step to step
+        comes from the batch's device tensors, the loops follow the step's shape alone, so a step that holds
+        it may be captured and replayed."""
+
+        graph_safe = True
+
+        def forward(self, x, batch, view, writes=True):
+            projected = x.float() @ self.weight.t()
+            slots = batch.seq_slot.long()
+            state = view.state.index_select(0, slots)
+            out = torch.empty_like(projected)
+            row, last = 0, []
+            for index, count in enumerate(batch.host_q_lens):
+                current = state[index]
+                for _ in range(count):
+                    current = self.decay * current + projected[row]
+                    out[row] = current
+                    row += 1
+                last.append(current)
+            if writes:
+                view.state.index_copy_(0, slots, torch.stack(last))
+            return out.to(x.dtype)
+
+    class TwoStates(Part):
+        """A mixer with two states of different shape and type beside each other: the two inputs before
+        this one (float32 [2, hidden]) and a count of the tokens seen (int32 [1]).
+        y_t = W (x_t + x_{t-1} / 2 + x_{t-2} / 4) / (1 + count_t / 8)."""
+
+        def __init__(self, hidden_size: int) -> None:
+            self.hidden_size = hidden_size
+
+        def cache_need(self):
+            return (FixedState((2, self.hidden_size), "float32"), FixedState((1,), "int32"))
+
+        def expected_tensors(self, prefix):
+            return {prefix + "in_proj.weight": TensorSpec((self.hidden_size, self.hidden_size))}
+
+        def bind(self, tensors, prefix, dtype, device):
+            super().bind(tensors, prefix, dtype, device)
+            self.weight = tensors[prefix + "in_proj.weight"].float()
+
+        def forward(self, x, batch, view, writes=True):
+            window, count = view
+            out = torch.empty((x.shape[0], self.hidden_size), dtype=torch.float32, device=x.device)
+            row = 0
+            for slot, tokens in zip(batch.host_slots, batch.host_q_lens):
+                before, seen = window.state[slot].clone(), int(count.state[slot])
+                for _ in range(tokens):
+                    current = x[row].float()
+                    out[row] = (self.weight @ (current + before[0] / 2 + before[1] / 4)) / (1 + seen / 8)
+                    before = torch.stack([current, before[0]])
+                    seen += 1
+                    row += 1
+                if writes:
+                    window.state[slot] = before
+                    count.state[slot] = seen
+            return out.to(x.dtype)
+
     class ToyConfig(Qwen2Config):
         architecture = "ToyRunningSumForCausalLM"
+        MIXER = "running_sum"
 
         def model_spec(self) -> ModelSpec:
             base = super().model_spec()
             attention_layer = base.layers[0]
             toy_layer = LayerSpec(
-                mixer=PartSpec.of("running_sum", hidden_size=self.hidden_size, decay=0.75),
+                mixer=(PartSpec.of(self.MIXER, hidden_size=self.hidden_size) if self.MIXER == "two_states"
+                       else PartSpec.of(self.MIXER, hidden_size=self.hidden_size, decay=0.75)),
                 feed_forward=attention_layer.feed_forward, norm1=attention_layer.norm1, norm2=attention_layer.norm2,
                 names=(("norm1", "input_layernorm"), ("mixer", "toy"), ("norm2", "post_attention_layernorm"),
                        ("feed_forward", "mlp")))
@@ -379,19 +487,35 @@ def register_toy():
                 layers=mixed.layers[:1], order=(LayerCall(0, 0), LayerCall(0, 1)),
                 final_norm=mixed.final_norm, tie_word_embeddings=True, max_position=self.max_position_embeddings)
 
+    class OnDeviceConfig(ToyConfig):
+        architecture = "ToyRunningSumOnDeviceForCausalLM"
+        MIXER = "running_sum_on_device"
+
+    class TwoStatesConfig(ToyConfig):
+        architecture = "ToyTwoStatesForCausalLM"
+        MIXER = "two_states"
+
     register_part("mixer", "running_sum", RunningSum)
+    register_part("mixer", "running_sum_on_device", RunningSumOnDevice)
+    register_part("mixer", "two_states", TwoStates)
+    register_architecture("ToyRunningSumOnDeviceForCausalLM", OnDeviceConfig)
+    register_architecture("ToyTwoStatesForCausalLM", TwoStatesConfig)
     register_architecture("ToyRunningSumForCausalLM", ToyConfig)
     register_architecture("ToyOnlyStateForCausalLM", OnlyStateConfig)
     return ToyConfig
 
 
-def toy_plain(raw, weights, tokens, order=(0, 1, 0)):
+def toy_plain(raw, weights, tokens, order=(0, 1, 0), two_states=False):
     """Whole-sequence reference of the toy model, from the plain parts."""
     eps = raw["rms_norm_eps"]
     h = weights["model.embed_tokens.weight"][torch.tensor(tokens)]
     cos, sin = plain.rope_tables(plain.head_dim_of(raw), len(tokens), raw["rope_theta"])
 
     def toy(x, p):
+        if two_states:
+            zero = torch.zeros_like(x[:1])
+            mixed = x + torch.cat([zero, x[:-1]]) / 2 + torch.cat([zero, zero, x[:-2]])[: len(x)] / 4
+            return (mixed @ weights[p + "toy.in_proj.weight"].t()) / (1 + torch.arange(len(x))[:, None] / 8)
         projected = x @ weights[p + "toy.in_proj.weight"].t()
         state = torch.zeros(raw["hidden_size"])
         rows = []
@@ -446,6 +570,60 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
         replay_util.compare(rows, reference, rtol=1e-4, atol=2e-5)
     # a slot handed to a new request starts from a cleared state (slots were reused above)
+    assert runner.cache.stats().slots_used == 0
+
+
+def _toy_runner(tmp_path, architecture, **options):
+    from cie_amd.config import build_engine_config, load_config
+    from cie_amd.engine import Runner, load_model
+    from cie_amd.parts.model import expected_tensors
+    from cie_amd.weights import RandomSource, write_tensors
+
+    register_toy()
+    raw = dict(architectures=[architecture], model_type="qwen2", hidden_size=32, num_hidden_layers=2,
+               num_attention_heads=2, num_key_value_heads=1, intermediate_size=56, vocab_size=64,
+               rms_norm_eps=1e-6, rope_theta=1e4, max_position_embeddings=128, tie_word_embeddings=True)
+    write_tensors(tmp_path, raw, {})
+    tensors = RandomSource(8, std=0.1).load(expected_tensors(load_config(tmp_path).model_spec()), "float32", "cpu")
+    write_tensors(tmp_path, raw, tensors)
+    model, _ = load_model(tmp_path, "float32")
+    runner = Runner(model, build_engine_config(dtype="float32", page_size=8, kv_tokens=256, max_running=4,
+                                               max_model_len=128, prefix_cache_pages=0, **options))
+    return raw, tensors, runner
+
+
+def test_a_stateful_mixer_that_reads_its_slots_on_the_device_runs_from_captured_steps(tmp_path):
+    """A mixer with a state per request that declares ``graph_safe`` advances its state at every run of its
+    ``forward``.  Captured steps, single tokens and portions alike, are made on rows of padding (the pad slot's
+    state), so a request's state moves once per token: at the replay.  Every replay against the plain toy."""
+    raw, tensors, runner = _toy_runner(tmp_path, "ToyRunningSumOnDeviceForCausalLM", graph_decode=True,
+                                       graph_mixed_steps=8)
+    assert runner.graphs is not None and runner.mixed_graphs is not None
+    requests = {f"t{i}": random_tokens(n, 64, 70 + i) for i, n in enumerate([61, 40, 53, 31, 47])}
+    reference = {rid: toy_plain(raw, tensors, tokens) for rid, tokens in requests.items()}
+    for schedule in (lambda r: replay_util.fixed_portions(r, portion=8, live=3, decode_tail=12),
+                     lambda r: replay_util.mixed(r, live=4, decode_tail=20, seed=3)):
+        steps = schedule(requests)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        replay_util.compare(rows, reference, every_position=False, rtol=1e-4, atol=2e-5)
+    assert runner.graph_replays >= 10 and runner.mixed_graph_captures >= 1 and runner.mixed_graph_replays >= 3
+    assert runner.cache.stats().slots_used == 0
+
+
+def test_a_mixer_with_two_states_of_different_shape(tmp_path):
+    """``cache_need`` may be a tuple: the mixer is handed a tuple of views in the same order, each state has its
+    own shape and type, both are cleared when a slot goes to a new request."""
+    raw, tensors, runner = _toy_runner(tmp_path, "ToyTwoStatesForCausalLM", graph_decode=False)
+    cache = runner.cache
+    assert cache.unit_cells == [(0, 1), 2, (3, 4)] and set(cache.state_units) == {0, 1, 3, 4} and cache.unit_group == {2: 0}
+    window, count = runner.device_cache.view(0)
+    assert window.state.shape[1:] == (2, 32) and count.state.dtype == torch.int32
+    requests = {f"t{i}": random_tokens(n, 64, 170 + i) for i, n in enumerate([23, 40, 9, 31, 17, 50])}
+    reference = {rid: toy_plain(raw, tensors, tokens, two_states=True) for rid, tokens in requests.items()}
+    for schedule in (replay_util.whole, replay_util.portions, lambda r: replay_util.mixed(r, live=3)):
+        steps = schedule(requests)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        replay_util.compare(rows, reference, rtol=1e-4, atol=2e-5)
     assert runner.cache.stats().slots_used == 0
 
 
@@ -710,6 +888,120 @@ def test_toy_window_layer_under_random_traces(tmp_path, seed):
         assert runner.cache.stats().pages_used == 0
     finally:
         config_class.WINDOW = 20
+
+
+def _window_case(raw, tensors, config_class, rng, length):
+    """Plant one channel in the windowed layer (its slowest rotating pair): token ``ask`` scores 22 on token
+    ``key`` and little on any other.  The request has keys at the very edge of the window of an asking token
+    (just inside: the furthest key it may see; just outside: the nearest it may not), so that a window cut
+    one key off moves that row's logits by most of the attention's share."""
+    d, hidden, window = plain.head_dim_of(raw), raw["hidden_size"], config_class.WINDOW
+    key, ask = raw["vocab_size"] - 1, raw["vocab_size"] - 2
+    p = "model.layers.0.self_attn."
+    low, high = d // 2 - 1, d - 1
+    heads = raw["num_attention_heads"]
+    for name, bases, column in (("k_proj", [0], 0), ("q_proj", [h * d for h in range(heads)], 1)):
+        for base in bases:
+            for row in (base + low, base + high):
+                tensors[p + name + ".weight"][row] = 0.0
+                tensors[p + name + ".bias"][row] = 0.0
+            tensors[p + name + ".weight"][base + high, column] = 2.0
+    embed = tensors["model.embed_tokens.weight"]
+    embed[key] = 0.0
+    embed[key, 0] = embed[key, 5] = 0.1
+    embed[ask] *= 0.1
+    embed[ask, 1] = 0.1
+    tokens = [rng.randrange(raw["vocab_size"] - 2) for _ in range(length)]
+    asking = []
+    place = rng.randint(0, 5)
+    inside = True
+    while place + window < length:
+        tokens[place] = key
+        query = place + window - 1 if inside else place + window
+        tokens[query] = ask
+        asking.append((query, inside))
+        inside = not inside
+        place = query + rng.randint(1, 9)
+    return tokens, asking
+
+
+@pytest.mark.parametrize("graph", [False, True])
+@pytest.mark.parametrize("page,window,head_dim", [(16, 37, 64), (64, 70, 64), (16, 100, 128), (64, 45, 128)])
+def test_toy_window_layer_in_bfloat16_with_pages_of_16_and_64(tmp_path, monkeypatch, page, window, head_dim, graph):
+    """The windowed layer in bfloat16 with pages that send it to the matrix-core forms of four and eight waves,
+    joined decode rows and captured decode steps, while the pages that the window has passed go back to the pool
+    and are handed out again (the device's block table keeps their numbers): windows that are no multiples of
+    the kernels' blocks of 32 keys, a dominating key just inside the window and just outside it."""
+    import random
+
+    from cie_amd.config import build_engine_config, load_config
+    from cie_amd.engine import Runner, load_model
+    from cie_amd.parts import attention
+    from cie_amd.parts.model import expected_tensors
+    from cie_amd.weights import RandomSource, write_tensors
+
+    rng = random.Random(1000 * page + window)
+    config_class = register_routed_toy()
+    config_class.EXPERTS, config_class.WINDOW = 1, window
+    monkeypatch.setattr(attention, "EIGHT_WAVE_TILES", 0)  # heads of 128: every prompt portion in tiles of eight waves
+    raw = dict(architectures=["ToyRoutedWindowForCausalLM"], model_type="qwen2", hidden_size=64, num_hidden_layers=2,
+               num_attention_heads=2, num_key_value_heads=1, head_dim=head_dim, intermediate_size=72, vocab_size=80,
+               rms_norm_eps=1e-5, rope_theta=1e4, max_position_embeddings=600, tie_word_embeddings=True)
+    try:
+        write_tensors(tmp_path, raw, {})
+        tensors = RandomSource(window, std=0.15).load(expected_tensors(load_config(tmp_path).model_spec()), "float32", "cpu")
+        long_tokens, asking = _window_case(raw, tensors, config_class, rng, 560)
+        tensors = {k: (v.to(torch.bfloat16).float() if v.is_floating_point() else v) for k, v in tensors.items()}
+        write_tensors(tmp_path, raw, tensors)
+        lengths = [560, rng.randint(150, 400), rng.randint(20, 120), rng.randint(150, 300)]
+        requests, steps = replay_util.random_trace(rng, lengths, raw["vocab_size"] - 2, page)
+        requests["r0"][:] = long_tokens
+        at: dict[str, int] = {}
+        for step in steps:  # the cuts stay, the long request's tokens are the planted ones, every position is wanted
+            for entry in step["entries"]:
+                first = at.get(entry["id"], 0)
+                entry["tokens"] = requests[entry["id"]][first: first + len(entry["tokens"])]
+                entry["want"] = list(range(len(entry["tokens"])))
+                at[entry["id"]] = first + len(entry["tokens"])
+        longest_portion = max(len(entry["tokens"]) for step in steps for entry in step["entries"])
+        model, _ = load_model(tmp_path, "bfloat16")
+        runner = Runner(model, build_engine_config(
+            dtype="bfloat16", page_size=page, kv_tokens=replay_util.max_live_tokens(steps, page=page), max_running=4,
+            max_model_len=raw["max_position_embeddings"], prefix_cache_pages=0, graph_decode=graph,
+            prefill_chunk=longest_portion))
+        windowed = next(g for g in runner.cache.groups if g.spec.window is not None)
+        passed, reused = set(), []  # pages the window has passed while their request lives, and those handed out again
+        free, allocate = windowed.allocator.free, windowed.allocator.allocate
+
+        def spy_free(pages, owner):
+            if runner.cache.has(owner):
+                passed.update(pages)
+            return free(pages, owner)
+
+        def spy_allocate(owner, count):
+            pages = allocate(owner, count)
+            reused.extend(page for page in pages if page in passed)
+            return pages
+
+        monkeypatch.setattr(windowed.allocator, "free", spy_free)
+        monkeypatch.setattr(windowed.allocator, "allocate", spy_allocate)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        assert reused, "no page that the window had passed was handed out again"
+        expected = {rid: routed_toy_plain(raw, tensors, tokens, config_class) for rid, tokens in requests.items()}
+        rough = {rid: routed_toy_plain(raw, {k: v.to(torch.bfloat16) for k, v in tensors.items()}, tokens, config_class).float()
+                 for rid, tokens in requests.items()}
+        rms, worst, plain_rms, plain_worst = replay_util.closer_than_plain_bfloat16(rows, expected, rough)
+        print(f"window {window} page {page}: rms {rms:.3e} worst {worst:.3e}, plain in bfloat16 {plain_rms:.3e} {plain_worst:.3e}",
+              flush=True)
+        # the yardstick: a window one key longer or shorter moves the asking rows by far more than that
+        for wrong in (window + 1, window - 1):
+            config_class.WINDOW = wrong
+            off = routed_toy_plain(raw, tensors, long_tokens, config_class)
+            moved = [float((off[q] - expected["r0"][q]).abs().max()) for q, inside in asking if inside == (wrong < window)]
+            assert moved and min(moved) > 4 * 1.5 * plain_worst, (wrong, min(moved), plain_worst)
+        assert runner.cache.stats().pages_used == 0
+    finally:
+        config_class.WINDOW, config_class.EXPERTS = 20, 3
 
 
 # ----------------------------------------------------------------------------------------------------

@@ -488,6 +488,9 @@ class ManagerRunner:
     def free_tokens(self) -> int:
         return self.cache.free_tokens()
 
+    def tokens_needed(self, request, upto: int) -> int:
+        return self.cache.tokens_missing(request.request_id, upto)
+
     def execute_batch(self, plan):
         need = {p.request.request_id: p.end for p in plan.portions}
         self.cache.ensure_capacity_batch(need)
@@ -530,6 +533,37 @@ def test_a_cache_without_pages_admits_side_by_side():
     assert len(scheduler.active) == 4
     scheduler.run_until_done(50)
     assert runner.most_side_by_side == 4 and all(r.output == [100, 101, 102, 103] for r in requests)
+
+
+def test_admission_asks_the_runner_what_a_request_costs():
+    """A cache whose only group keeps a window of 8 keys: a request of 40 tokens never holds more than four
+    pages of 4, so four of them run side by side in a pool of 16 pages, which by their length alone
+    (11 pages each) would hold one.  The scheduler takes the cost from the runner, not from the page size."""
+    from cie_amd.cache.manager import CacheManager, PagedKV
+
+    manager = CacheManager([PagedKV(1, 8, window=8)], page_size=4, kv_tokens=64, max_running=4, max_model_len=64,
+                           prefill_chunk=4)
+    assert manager.groups[0].allocator.total_pages == 16 and manager.groups[0].most_per_request == 4
+    assert manager.tokens_missing("nobody", 41) == 16 and manager.tokens_missing("nobody", 5) == 8
+    runner = ManagerRunner(manager)
+    scheduler = make(runner, max_model_len=64, max_running=4, token_budget=16, prefill_chunk=4, page_size=4,
+                     admit_within_pool=True)
+    requests = [scheduler.submit([i + 1] * 40, GenerationConfig(max_output_tokens=3)) for i in range(4)]
+    scheduler.step()
+    assert len(scheduler.active) == 4
+    scheduler.run_until_done(200)
+    assert runner.most_side_by_side == 4 and all(r.output == [100, 101, 102] and r.preemptions == 0 for r in requests)
+    manager.assert_invariants()
+    # a runner that does not say falls back on whole pages per token: one request at a time here
+    silent = ManagerRunner(CacheManager([PagedKV(1, 8, window=8)], page_size=4, kv_tokens=64, max_running=4,
+                                        max_model_len=64, prefill_chunk=4))
+    silent.tokens_needed = None
+    scheduler = make(silent, max_model_len=64, max_running=4, token_budget=16, prefill_chunk=4, page_size=4,
+                     admit_within_pool=True)
+    for i in range(4):
+        scheduler.submit([i + 1] * 40, GenerationConfig(max_output_tokens=3))
+    scheduler.step()
+    assert len(scheduler.active) == 1
 
 
 @pytest.mark.parametrize("seed", [3, 12, 21, 30])
