@@ -52,8 +52,9 @@ __host__ __device__ inline bool all_in_first_share(int first_begin, int hi, int 
     return hi <= first_begin + per_split;
 }
 
-// The prompt form of eight waves per 128-row tile (csrc/attention_prompt.hip); returns a CIE_* code.
-int launch_prompt_form(hipStream_t stream, const AttentionArgs& a, int head_dim);
+// The prompt form whose waves share a tile's keys and values through LDS (csrc/attention_prompt.hip): eight waves
+// per tile of 128 rows, or four per tile of 64; returns a CIE_* code.
+int launch_prompt_form(hipStream_t stream, const AttentionArgs& a, int head_dim, int waves);
 
 constexpr int kPromptWaves = 8;       // waves of a workgroup in that form
 constexpr int kPromptTileRows = 128;  // (token, head) rows of its tiles

@@ -833,8 +833,9 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     // product in one page
     if (tile_waves != 1 && ((tile_waves != kTileWaves && tile_waves != kPromptWaves) || !(scale > 0.f) || page_size < 16))
         return CIE_BAD_ARGUMENT;
-    // the form of eight waves has tiles of 128 rows, no fewer, and heads of up to 128 dimensions
-    if (tile_waves == kPromptWaves && (16 * row_tiles != kPromptTileRows || head_dim > 128)) return CIE_BAD_ARGUMENT;
+    // the form that shares keys and values through LDS has tiles of 128 rows (eight waves) or of 64 (four), and
+    // heads of up to 128 dimensions
+    if (tile_waves == kPromptWaves && ((row_tiles != 8 && row_tiles != 4) || head_dim > 128)) return CIE_BAD_ARGUMENT;
     if (n_splits > 1 && (!part_o || !part_ml ||
                          (!max_context_dev && (keys_per_split <= 0 || keys_per_split % kKeysPerBlock))))
         return CIE_BAD_ARGUMENT;
@@ -872,9 +873,9 @@ CIE_API int cie_paged_attention_mfma(void* stream, const void* q, int q_row_stri
     hipStream_t s = static_cast<hipStream_t>(stream);
     int rc;
     if (tile_waves == kPromptWaves) {
-        rc = launch_prompt_form(s, a, head_dim);
+        rc = launch_prompt_form(s, a, head_dim, row_tiles);
         if (rc != CIE_OK || n_splits == 1) return rc;
-        return launch_merge(s, a, n_tiles, head_dim, kPromptTileRows);
+        return launch_merge(s, a, n_tiles, head_dim, 16 * row_tiles);
     }
     switch (head_dim) {
         case 32: rc = launch_for_dim<32>(s, a, n_tiles, row_tiles, tile_waves); break;

@@ -30,7 +30,6 @@ using namespace cie_attention;
 
 namespace {
 
-constexpr int kThreadsP = 64 * kPromptWaves;
 constexpr int kKeysPerStage = 2 * kKeysPerBlock;  // 64: one block for each half of the waves
 
 // The largest of three or two numbers in one instruction each, and the largest over the four 16-lane rows of a
@@ -71,17 +70,22 @@ struct PromptLayout {
     }
 };
 
-template <int D>
-__global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(AttentionArgs a) {
+// WAVES = 8: tiles of 128 rows; WAVES = 4: the same with tiles of 64 rows, two such workgroups to a compute unit,
+// which then walk their keys independently of each other (one's matrix products beside the other's softmax).
+template <int D, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) paged_attention_prompt_kernel(AttentionArgs a) {
     using L = PromptLayout<D>;
     constexpr int NK = D / 32;
     constexpr int ND = D / 16;
     constexpr int RT = 2;  // 16-row tiles of a wave
+    constexpr int QUARTERS = WAVES / 2;        // sets of 32 rows of the tile
+    constexpr int kTileRows = 32 * QUARTERS;
+    constexpr int kLoaderThreads = 64 * QUARTERS;  // threads that fetch one group of 16 keys
     extern __shared__ __align__(16) unsigned char lds[];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const int quarter = wave & 3;   // which 32 rows of the tile
-    const int half = wave >> 2;     // which 32 of each 64 keys
+    const int quarter = wave % QUARTERS;   // which 32 rows of the tile
+    const int half = wave / QUARTERS;      // which 32 of each 64 keys
     const int r = lane & 15;
     const int g = lane >> 4;
 
@@ -96,7 +100,12 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
         tile_index = blockIdx.x / a.kv_heads;
     }
     if (tile_index >= a.n_tiles) return;  // padding of the grid; the whole workgroup leaves
-    const int tile = a.n_tiles - 1 - tile_index;  // the last tiles see the most keys: they start first
+    // The last tiles of a prompt see the most keys: they start first.  Where two workgroups share a compute
+    // unit (WAVES = 4) the first half of the launch are the longest tiles in falling order and the second half
+    // the shortest in rising order: the hardware fills the units' second places in the order of the first, so
+    // that a unit gets a long tile and a short one, every unit about as many keys.
+    int tile = a.n_tiles - 1 - tile_index;
+    if (WAVES == 4 && tile_index >= (a.n_tiles + 1) / 2) tile = tile_index - (a.n_tiles + 1) / 2;
     const int group = a.q_heads / a.kv_heads;
     const int seq = a.tile_seq ? a.tile_seq[tile] : tile;
     const int q0 = a.tile_seq ? a.tile_q0[tile] : 0;
@@ -126,8 +135,8 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
             range_begin += blockIdx.y * per_split;
             range_end = min(hi, range_begin + per_split);
             if (range_begin >= range_end) {  // no keys in this share: its statistics say so, its sums are never read
-                float* pml = a.part_ml + ((static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + blockIdx.y) * kPromptTileRows * 2;
-                if (threadIdx.x < kPromptTileRows) {
+                float* pml = a.part_ml + ((static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + blockIdx.y) * kTileRows * 2;
+                if (threadIdx.x < kTileRows) {
                     pml[threadIdx.x * 2] = -INFINITY;
                     pml[threadIdx.x * 2 + 1] = 0.f;
                 }
@@ -179,22 +188,31 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
     // (Where a group has fewer pieces than the 256 threads that share it, the threads left over fetch and
     // store a piece a second time: the same bytes to the same place.)
     const int loader = half;  // (the same split of the waves, used here for something else)
-    const int key_piece = (threadIdx.x & 255) % (16 * L::C);
-    const int piece_key = key_piece / L::C;           // which of the group's 16 keys
-    const int piece_chunk = key_piece - piece_key * L::C;
-    const int key_from = (piece_key * D + piece_chunk * 8) * 2;  // bytes from the group's first key
-    const int key_to = ((loader * 16 + piece_key) * L::CS + (piece_chunk ^ L::key_swizzle(piece_key))) * 16;  // + pair * 32 keys
-    const int value_piece = (threadIdx.x & 255) % (2 * D);
-    const int piece_d = value_piece >> 1;         // which dimension's row of values
-    const int piece_h = value_piece & 1;          // which 8 of the group's 16 keys
-    const int value_from = ((piece_d << a.page_shift) + piece_h * 8) * 2;  // bytes from the group's first key in row 0
-    // row d of the block (pair); the group's keys are the block's first 16 (loader 0) or second 16 (loader 1):
-    // the first or second 8 bytes of a chunk; keys h*8 .. +3 belong to lane group 2h, keys h*8+4 .. +7 to 2h+1
-    const int value_row = L::kKeyBytes + piece_d * 64 + loader * 8;  // + pair * kValueBlockBytes
-    const int value_sw = (piece_d >> 2) & 3;
-    const int value_to_a = value_row + (((2 * piece_h) ^ value_sw) << 4);
-    const int value_to_b = value_row + (((2 * piece_h + 1) ^ value_sw) << 4);
-    static_assert(16 * L::C <= 256 && 2 * D <= 256, "one piece of each kind per thread and group");
+    // (with four waves a loader's 128 threads take two pieces of each kind in a group: kPasses)
+    constexpr int kKeyPieces = 16 * L::C, kValuePieces = 2 * D;
+    constexpr int kPasses = (kKeyPieces > kValuePieces ? kKeyPieces : kValuePieces) > kLoaderThreads ? 2 : 1;
+    static_assert(kKeyPieces <= kPasses * kLoaderThreads && kValuePieces <= kPasses * kLoaderThreads,
+                  "at most two pieces of each kind per thread and group");
+    const int loader_thread = threadIdx.x % kLoaderThreads;
+    int key_from[kPasses], key_to[kPasses], value_from[kPasses], value_to_a[kPasses], value_to_b[kPasses];
+#pragma unroll
+    for (int pass = 0; pass < kPasses; ++pass) {
+        const int key_piece = (loader_thread + pass * kLoaderThreads) % kKeyPieces;
+        const int piece_key = key_piece / L::C;           // which of the group's 16 keys
+        const int piece_chunk = key_piece - piece_key * L::C;
+        key_from[pass] = (piece_key * D + piece_chunk * 8) * 2;  // bytes from the group's first key
+        key_to[pass] = ((loader * 16 + piece_key) * L::CS + (piece_chunk ^ L::key_swizzle(piece_key))) * 16;  // + pair * 32 keys
+        const int value_piece = (loader_thread + pass * kLoaderThreads) % kValuePieces;
+        const int piece_d = value_piece >> 1;         // which dimension's row of values
+        const int piece_h = value_piece & 1;          // which 8 of the group's 16 keys
+        value_from[pass] = ((piece_d << a.page_shift) + piece_h * 8) * 2;  // bytes from the group's first key in row 0
+        // row d of the block (pair); the group's keys are the block's first 16 (loader 0) or second 16 (loader 1):
+        // the first or second 8 bytes of a chunk; keys h*8 .. +3 belong to lane group 2h, keys h*8+4 .. +7 to 2h+1
+        const int value_row = L::kKeyBytes + piece_d * 64 + loader * 8;  // + pair * kValueBlockBytes
+        const int value_sw = (piece_d >> 2) & 3;
+        value_to_a[pass] = value_row + (((2 * piece_h) ^ value_sw) << 4);
+        value_to_b[pass] = value_row + (((2 * piece_h + 1) ^ value_sw) << 4);
+    }
 
     typedef const __attribute__((address_space(4))) int* const_int_ptr;
     const const_int_ptr table_c = (const_int_ptr)(uintptr_t)table;
@@ -208,31 +226,40 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
 #pragma unroll
         for (int pair = 0; pair < 2; ++pair) page[pair] = page_of(kb + (2 * pair + loader) * 16);
     };
-    uint4 key_regs0 = {0, 0, 0, 0}, key_regs1 = {0, 0, 0, 0}, value_regs0 = {0, 0, 0, 0}, value_regs1 = {0, 0, 0, 0};
-    auto fetch_pair = [&](int kb, int pair, int page_id, uint4& keys, uint4& values) {
-        const int first = min(kb + (2 * pair + loader) * 16, last_group);
-        const size_t page_head = static_cast<size_t>(page_id) * a.kv_heads + kv_head;
-        const char* key_base = reinterpret_cast<const char*>(
-            a.k_pool + ((page_head << a.page_shift) + (first & page_mask)) * D);
-        keys = *reinterpret_cast<const uint4*>(key_base + key_from);
-        const char* value_base = reinterpret_cast<const char*>(
-            a.v_pool + (page_head * D << a.page_shift) + (first & page_mask));
-        values = *reinterpret_cast<const uint4*>(value_base + value_from);
-    };
+    uint4 key_regs[2][kPasses], value_regs[2][kPasses];
+#pragma unroll
+    for (int pair = 0; pair < 2; ++pair)
+#pragma unroll
+        for (int pass = 0; pass < kPasses; ++pass) key_regs[pair][pass] = value_regs[pair][pass] = uint4{0, 0, 0, 0};
     auto fetch = [&](int kb, const int (&page)[2]) {
-        fetch_pair(kb, 0, page[0], key_regs0, value_regs0);
-        fetch_pair(kb, 1, page[1], key_regs1, value_regs1);
-    };
-    auto stash_pair = [&](unsigned char* base, int pair, const uint4& keys, const uint4& values) {
-        *reinterpret_cast<uint4*>(base + key_to + pair * (32 * L::CS * 16)) = keys;
-        unsigned char* block = base + pair * L::kValueBlockBytes;
-        *reinterpret_cast<uint2*>(block + value_to_a) = uint2{values.x, values.y};
-        *reinterpret_cast<uint2*>(block + value_to_b) = uint2{values.z, values.w};
+#pragma unroll
+        for (int pair = 0; pair < 2; ++pair) {
+            const int first = min(kb + (2 * pair + loader) * 16, last_group);
+            const size_t page_head = static_cast<size_t>(page[pair]) * a.kv_heads + kv_head;
+            const char* key_base = reinterpret_cast<const char*>(
+                a.k_pool + ((page_head << a.page_shift) + (first & page_mask)) * D);
+            const char* value_base = reinterpret_cast<const char*>(
+                a.v_pool + (page_head * D << a.page_shift) + (first & page_mask));
+#pragma unroll
+            for (int pass = 0; pass < kPasses; ++pass) {
+                key_regs[pair][pass] = *reinterpret_cast<const uint4*>(key_base + key_from[pass]);
+                value_regs[pair][pass] = *reinterpret_cast<const uint4*>(value_base + value_from[pass]);
+            }
+        }
     };
     auto stash = [&](int stage) {
         unsigned char* base = lds + stage * L::kStageBytes;
-        stash_pair(base, 0, key_regs0, value_regs0);
-        stash_pair(base, 1, key_regs1, value_regs1);
+#pragma unroll
+        for (int pair = 0; pair < 2; ++pair) {
+            unsigned char* block = base + pair * L::kValueBlockBytes;
+#pragma unroll
+            for (int pass = 0; pass < kPasses; ++pass) {
+                *reinterpret_cast<uint4*>(base + key_to[pass] + pair * (32 * L::CS * 16)) = key_regs[pair][pass];
+                const uint4 values = value_regs[pair][pass];
+                *reinterpret_cast<uint2*>(block + value_to_a[pass]) = uint2{values.x, values.y};
+                *reinterpret_cast<uint2*>(block + value_to_b[pass]) = uint2{values.z, values.w};
+            }
+        }
     };
 
     // ---- a lane's constant parts of its operand addresses in a stage
@@ -363,8 +390,8 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
     // ---- the two halves of the keys meet: the upper waves hand their sums to the lower ones through LDS,
     // one 16-row tile at a time (the references of the rows, then ND tiles of the output and one of the
     // probabilities' sums, each as the 4 x 64 numbers the lanes hold)
-    float* lds_m = reinterpret_cast<float*>(lds);             // [4 quarters][16 rows]
-    float* lds_o = reinterpret_cast<float*>(lds) + 4 * 16;    // [4 quarters][(ND + 1) * 4][64 lanes]
+    float* lds_m = reinterpret_cast<float*>(lds);                    // [quarters][16 rows]
+    float* lds_o = reinterpret_cast<float*>(lds) + QUARTERS * 16;    // [quarters][(ND + 1) * 4][64 lanes]
     constexpr int kMeetTile = (ND + 1) * 4;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
@@ -400,8 +427,8 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
                                lds_o[(quarter * kMeetTile + dt * 4 + i) * kWave + lane] * w_other_o[i];
         if (!whole) {  // this share's sums and statistics for the merge kernel
             const size_t unit = (static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + blockIdx.y;
-            float* po = a.part_o + unit * kPromptTileRows * D;
-            float* pml = a.part_ml + unit * kPromptTileRows * 2;
+            float* po = a.part_o + unit * kTileRows * D;
+            float* pml = a.part_ml + unit * kTileRows * 2;
             if (g == 0) pml[(wave_row0 + rt * 16 + r) * 2] = m_all;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -428,17 +455,17 @@ __global__ void __launch_bounds__(kThreadsP) paged_attention_prompt_kernel(Atten
     }
 }
 
-template <int D>
+template <int D, int WAVES>
 int launch(hipStream_t s, const AttentionArgs& a) {
     using L = PromptLayout<D>;
     // the stages, or the meeting place of the two halves at the end, whichever is larger
-    constexpr int kMeetBytes = (4 * 16 + 4 * ((D / 16 + 1) * 4) * kWave) * 4;
+    constexpr int kMeetBytes = ((WAVES / 2) * 16 + (WAVES / 2) * ((D / 16 + 1) * 4) * kWave) * 4;
     constexpr int kLdsBytes = 2 * L::kStageBytes > kMeetBytes ? 2 * L::kStageBytes : kMeetBytes;
     static_assert(kLdsBytes <= 64 * 1024, "a workgroup's LDS without asking for more");
     const dim3 grid = a.xcds_per_head > 0
                           ? dim3(kXcds * ((a.n_tiles + a.xcds_per_head - 1) / a.xcds_per_head), a.n_splits)
                           : dim3(static_cast<unsigned>(a.n_tiles) * a.kv_heads, a.n_splits);
-    paged_attention_prompt_kernel<D><<<grid, kThreadsP, kLdsBytes, s>>>(a);
+    paged_attention_prompt_kernel<D, WAVES><<<grid, 64 * WAVES, kLdsBytes, s>>>(a);
     return cie_after_launch();
 }
 
@@ -446,12 +473,21 @@ int launch(hipStream_t s, const AttentionArgs& a) {
 
 namespace cie_attention {
 
-int launch_prompt_form(hipStream_t stream, const AttentionArgs& a, int head_dim) {
+int launch_prompt_form(hipStream_t stream, const AttentionArgs& a, int head_dim, int waves) {
+    if (waves == 4) {
+        switch (head_dim) {
+            case 32: return launch<32, 4>(stream, a);
+            case 64: return launch<64, 4>(stream, a);
+            case 96: return launch<96, 4>(stream, a);
+            case 128: return launch<128, 4>(stream, a);
+            default: return CIE_BAD_ARGUMENT;
+        }
+    }
     switch (head_dim) {
-        case 32: return launch<32>(stream, a);
-        case 64: return launch<64>(stream, a);
-        case 96: return launch<96>(stream, a);
-        case 128: return launch<128>(stream, a);
+        case 32: return launch<32, 8>(stream, a);
+        case 64: return launch<64, 8>(stream, a);
+        case 96: return launch<96, 8>(stream, a);
+        case 128: return launch<128, 8>(stream, a);
         default: return CIE_BAD_ARGUMENT;  // wider heads: a wave's 32 rows of accumulators would not fit
     }
 }

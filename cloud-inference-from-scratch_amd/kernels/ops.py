@@ -331,9 +331,10 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
     (a multiple of 32; or, with ``max_context_dev``, derived on the device from the
     step's longest context) and merged through the workspaces.  ``tile_waves=4`` gives
     every tile (and every part of its keys) a workgroup of four waves that take the
-    blocks of 32 keys in turn; it needs pages of at least 16 keys.  ``tile_waves=8`` (with
-    ``row_tiles=8``: tiles of 128 rows, heads of up to 128 dimensions) gives every tile eight waves that
-    share the tile's keys and values through LDS."""
+    blocks of 32 keys in turn; it needs pages of at least 16 keys.  ``tile_waves=8`` (heads of up to
+    128 dimensions) is the form whose waves share the tile's keys and values through LDS: with
+    ``row_tiles=8`` tiles of 128 rows and eight waves, with ``row_tiles=4`` tiles of 64 rows and four
+    waves, two such workgroups to a compute unit."""
     if not (
         q.is_cuda and q.dtype == torch.bfloat16 and q.dim() == 2 and q.stride(1) == 1 and q.stride(0) == q_row_stride
     ):
@@ -373,7 +374,7 @@ def paged_attention_mfma(q: torch.Tensor, q_row_stride: int, k_pool: torch.Tenso
         (tile_waves == 1 and row_tiles <= 4)
         or (tile_waves == TILE_WAVES and scale > 0 and page_size >= 16 and row_tiles <= 4
             and (row_tiles == 1 or head_dim <= 128))
-        or (tile_waves == PROMPT_WAVES and scale > 0 and page_size >= 16 and row_tiles == 8 and head_dim <= 128)
+        or (tile_waves == PROMPT_WAVES and scale > 0 and page_size >= 16 and row_tiles in (4, 8) and head_dim <= 128)
     ):
         raise ValueError(f"tile_waves {tile_waves} with {n_splits} splits, {row_tiles} row tiles, head size {head_dim}, "
                          f"pages of {page_size}")

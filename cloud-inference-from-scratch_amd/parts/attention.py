@@ -145,13 +145,14 @@ SPLIT_DECODE_KEYS = 192  # contexts from which the keys of decode rows are cut i
 JOINED_DECODE_ROWS = 32  # up to this many single-token sequences beside prompt portions ride in the prompt form's launch
 PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's keys are cut
 # (cutting a prompt form's keys aims at as many workgroups as the GPU has compute units)
-# Tiles of 128 rows x kv heads from which prompt portions take the form of eight waves: enough to give most
-# compute units a workgroup without cutting the keys (whose parts, 64 KB of sums per tile and kv head, cost that
+# Tiles of 64 rows x kv heads (as a share of the compute units) from which prompt portions take the form that
+# shares keys and values through LDS: enough to give most compute units a workgroup without cutting the keys (whose parts, 64 KB of sums per tile and kv head, cost that
 # form more than they gain it: 512 tokens behind 1,536 keys, 7B heads, 60 us in two parts against 40 us in the form
 # of four waves).  Measured at head size 128 (us, four waves -> eight): 2,048 tokens of one prompt 55.7 -> 51.4
 # (3B heads), 101 -> 58 (7B), 144 -> 84 (14B); behind 2,048 keys 108 -> 91, 195 -> 135, 284 -> 201; beside 8 single
 # tokens 108 -> 64, 138 -> 75, 182 -> 111.
 EIGHT_WAVE_TILES = 0.75  # of the compute units
+LARGE_TILES_ABOVE = 1.0  # tiles of 128 rows x kv heads (as a share of the compute units) above which that form takes them
 
 
 def plan_splits(units: int, max_keys: int, target_waves: int = 1024, min_keys: int = 128) -> tuple[int, int]:
@@ -194,9 +195,14 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     bound = batch.static_plan.max_keys if batch.static_plan is not None else max_keys
     cuts = max(1, bound // PROMPT_SPLIT_KEYS) if wide and window is None else 1  # (a window's keys stay whole)
     big_tiles = -(-prompt_tokens * group // 128) * num_kv_heads
-    # (heads of 128 dimensions: with 64 the form of four waves is the faster one, 2,048 tokens behind 6,144
-    # keys 114 against 140 us, since the softmax arithmetic per key is the same and the products are half)
-    eight = wide and head_dim == 128 and group <= 128 and big_tiles >= max(1, EIGHT_WAVE_TILES * cus)
+    small_tiles = -(-prompt_tokens * group // 64) * num_kv_heads
+    # That form has tiles of 128 rows for eight waves, and tiles of 64 rows for four, two such workgroups to a
+    # compute unit, where the larger tiles would not give every unit more than one (isolated kernel, us, 128 rows
+    # -> 64: 2,048 tokens of one prompt, 3B heads, 256 large tiles: 50.8 -> 46.8, 1,024 tokens 27.5 -> 24.8; 7B
+    # heads, 456 large tiles: 55.3 -> 70.5; heads of 64 dimensions, where the softmax arithmetic per key is the same
+    # and the products are half: 2,048 tokens 40.2 -> 33.0, against 43.1 in the form of four waves without LDS).
+    eight = (wide and head_dim in (64, 128) and group <= 64 and small_tiles >= max(1, EIGHT_WAVE_TILES * cus))
+    lds_row_tiles = 8 if head_dim == 128 and big_tiles > LARGE_TILES_ABOVE * cus else 4
 
     def decode_form(bound: int, units: int) -> tuple[int, dict]:
         # Decode rows, `units` (sequence, kv head) pairs over up to `bound` keys.  Long contexts: four waves
@@ -264,7 +270,7 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         # short portion behind a long context also has its keys cut (256 tokens behind 3,840 keys, 2 kv heads:
         # 34 us with 64 rows per tile and four parts, 48 us with 16 rows per tile and the keys whole)
         if eight:
-            tile_waves, row_tiles = ops.PROMPT_WAVES, 8
+            tile_waves, row_tiles = ops.PROMPT_WAVES, lds_row_tiles
         else:
             tile_waves = ops.TILE_WAVES
             row_tiles = 4 if head_dim <= 128 else 1

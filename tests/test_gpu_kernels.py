@@ -231,7 +231,7 @@ MFMA_GEOMETRY = [(16, 2, 128, 16), (4, 2, 32, 8), (3, 1, 32, 8), (6, 6, 64, 4), 
 
 
 @pytest.mark.parametrize("geometry", MFMA_GEOMETRY)
-@pytest.mark.parametrize("row_tiles,tile_waves", [(1, 1), (2, 1), (4, 1), (1, 4), (2, 4), (4, 4), (8, 8)])
+@pytest.mark.parametrize("row_tiles,tile_waves", [(1, 1), (2, 1), (4, 1), (1, 4), (2, 4), (4, 4), (8, 8), (4, 8)])
 def test_paged_attention_mfma_ragged(ops, geometry, row_tiles, tile_waves):
     """The tiled forms (one wave per tile; four waves that share a tile's keys; eight waves per tile of
     128 rows with keys and values in LDS) on
@@ -298,12 +298,15 @@ def test_paged_attention_mfma_decode_splits(ops, geometry, splits, tile_waves):
 
 
 @pytest.mark.parametrize("geometry", [(16, 2, 128, 16), (6, 2, 32, 16), (5, 5, 64, 32)])
-@pytest.mark.parametrize("row_tiles", [1, 2, 4, 8])
+@pytest.mark.parametrize("row_tiles", [1, 2, 4, 8, -4])
 @pytest.mark.parametrize("splits", [(3, 512), (5, 256), (9, 128)])
 def test_paged_attention_mfma_prompt_portions_with_their_keys_cut(ops, geometry, row_tiles, splits):
     """Portions of prompts behind long contexts, tiles of 16 to 128 rows whose keys are cut into
-    parts (some of them empty for the shorter sequences, some ending inside the portion)."""
+    parts (some of them empty for the shorter sequences, some ending inside the portion); tiles of 128
+    rows, and of 64 where ``row_tiles`` is given as -4, in the form that shares keys and values through LDS."""
     q_heads, kv_heads, head_dim, page_size = geometry
+    through_lds = row_tiles in (8, -4)
+    row_tiles = abs(row_tiles)
     group = q_heads // kv_heads
     if group > 16 * row_tiles:
         pytest.skip("the group does not fit the tile")
@@ -321,7 +324,7 @@ def test_paged_attention_mfma_prompt_portions_with_their_keys_cut(ops, geometry,
     per_tile = (16 * row_tiles) // group
     out = run_mfma(ops, torch.cat(qs), contexts, q_lens, k_pool, v_pool, table, slots, q_heads, kv_heads, head_dim,
                    None, scale, per_tile, row_tiles, n_splits=n_splits, keys_per_split=per_split,
-                   tile_waves=8 if row_tiles == 8 else 4)
+                   tile_waves=8 if through_lds else 4)
     torch.testing.assert_close(out, torch.cat(expected), **tol(torch.bfloat16))
 
 
@@ -332,7 +335,7 @@ def test_paged_attention_mfma_window(ops, window):
     q_lens = [40, 1, 17, 1]
     lengths = [c + q for c, q in zip(contexts, q_lens)]
     scale = 1.0 / math.sqrt(head_dim)
-    for page_size, variants in ((8, ((1, 1),)), (16, ((4, 1), (4, 2), (8, 8))), (64, ((4, 4), (8, 8)))):
+    for page_size, variants in ((8, ((1, 1),)), (16, ((4, 1), (4, 2), (8, 8), (8, 4))), (64, ((4, 4), (8, 8), (8, 4)))):
         k_pool, v_pool, table, slots, dense = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=74)
         g = torch.Generator().manual_seed(75)
         qs, expected = [], []
@@ -444,9 +447,10 @@ def test_paged_attention_mfma_far_key(ops):
     q_many = torch.cat([torch.randn((39, q_heads, head_dim), generator=torch.Generator().manual_seed(77)), q])
     q_many = q_many.to(torch.bfloat16).float()
     expect = plain_qwen2.causal_attention(q_many, k, v, scale, past_len=length - 40)
-    for row_tiles in (1, 2, 4, 8):  # (tiles of 128 rows: the form of eight waves, whose two halves each see every other block)
+    # (tiles of 128 rows, and of 64 a second time: the form through LDS, whose two halves each see every other block)
+    for row_tiles, tile_waves in ((1, 4), (2, 4), (4, 4), (8, 8), (4, 8)):
         out = run_mfma(ops, q_many.reshape(40, -1), [length - 40], [40], k_pool, v_pool, table, slots, q_heads,
-                       kv_heads, head_dim, None, scale, 2 * row_tiles, row_tiles, tile_waves=8 if row_tiles == 8 else 4)
+                       kv_heads, head_dim, None, scale, 2 * row_tiles, row_tiles, tile_waves=tile_waves)
         torch.testing.assert_close(out, expect, **tol(torch.bfloat16))
         torch.testing.assert_close(out[-1].view(q_heads, head_dim), v[far].repeat_interleave(8, dim=0), rtol=0.05, atol=0.05)
 

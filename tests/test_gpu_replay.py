@@ -131,20 +131,25 @@ def test_replay_with_the_four_wave_prompt_attention(tiny_folders, plain, monkeyp
 
 @pytest.mark.parametrize("schedule", ["whole", "portions", "mixed"])
 @pytest.mark.parametrize("heads", [(16, 2), (28, 4), (10, 2)])
-def test_replay_with_the_eight_wave_prompt_attention(tmp_path, monkeypatch, schedule, heads):
-    """Prompt portions of many rows go to tiles of 128 rows and eight waves (heads of 128 dimensions).
-    The tiny requests here never have that many rows: the threshold is lowered so that every portion
-    takes that form, with groups of 8, 7 and 5 heads (tiles of 16, 18 and 25 tokens)."""
+@pytest.mark.parametrize("rows", [128, 64])
+def test_replay_with_the_prompt_attention_that_shares_keys_through_lds(tmp_path, monkeypatch, schedule, heads, rows):
+    """Prompt portions of many rows go to tiles of 128 rows and eight waves, or of 64 rows and four, whose keys
+    and values pass through LDS (heads of 128 dimensions).  The tiny requests here never have that many rows:
+    the thresholds are set so that every portion takes that form in the one size or the other, with groups of
+    8, 7 and 5 heads (tiles of 16, 18 and 25 tokens, or 8, 9 and 12)."""
     from conftest import TINY_C, make_folder
     from cie_amd.kernels import ops
     from cie_amd.parts import attention
 
     monkeypatch.setattr(attention, "EIGHT_WAVE_TILES", 0)  # (a share of the compute units: any tile at all)
+    monkeypatch.setattr(attention, "LARGE_TILES_ABOVE", -1 if rows == 128 else 1e9)
     seen = []
     real = ops.paged_attention_mfma
 
     def spy(*args, **kwargs):
         seen.append(kwargs.get("tile_waves", 1))
+        if kwargs.get("tile_waves", 1) == ops.PROMPT_WAVES:
+            assert 16 * kwargs["row_tiles"] == rows
         return real(*args, **kwargs)
 
     monkeypatch.setattr(ops, "paged_attention_mfma", spy)
