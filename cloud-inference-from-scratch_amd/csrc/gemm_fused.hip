@@ -42,7 +42,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes as one value (a struct is copied as memory)
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4, EPI_ROPE = 5, EPI_ROPE8 = 6 };
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_SILU = 2, EPI_RESID = 3, EPI_PARTIAL = 4, EPI_ROPE = 5, EPI_ROPE8 = 6, EPI_ATOMIC = 7 };
 
 // What the ROPE epilogue needs beside the product: where each row's token sits, and the cache.
 struct RopeArgs {
@@ -79,15 +79,11 @@ struct FusedArgs {
     const float* row_sumsq;    // SILU: [M, sumsq_parts] or null
     int sumsq_parts;
     float eps;
-    // ROPE with the norm in front of it folded in (a few rows): the rows of A are not read but made here, as
-    // bf16((fold_residual + the sum of fold_parts) * fold_weight), and the product is multiplied by each row's
-    // 1/rms; the first workgroup writes the summed stream to fold_residual_out (another buffer than
-    // fold_residual, which the other workgroups are still reading).
+    // ROPE with the norm in front of it folded in (up to 16 rows): the rows of A are not read but made here, as
+    // bf16(fold_residual * fold_weight), a lane making the very values its matrix operand holds, and the
+    // product is multiplied by each row's 1/rms, whose sums of squares the lanes gather on the way.
     const float* fold_residual;  // [M, K] float32 or null
-    const float* fold_parts;     // [fold_n_parts, M, K] float32
-    int fold_n_parts;
     const float* fold_weight;    // [K] float32
-    float* fold_residual_out;    // [M, K] float32
     RopeArgs rope;         // ROPE only
 };
 
@@ -129,6 +125,8 @@ __device__ __forceinline__ void store_tile(const FusedArgs& a, const floatx4& ac
             const float v = acc[i] + add;
             if (EPI == EPI_PARTIAL)
                 static_cast<float*>(a.c)[(static_cast<size_t>(blockIdx.z) * a.M + m) * a.N + n] = v;
+            else if (EPI == EPI_ATOMIC)  // every part of K adds its share into the stream (the hardware's own float add)
+                unsafeAtomicAdd(a.residual + static_cast<size_t>(m) * a.N + n, v);
             else if (EPI == EPI_F32)
                 static_cast<float*>(a.c)[static_cast<size_t>(m) * a.N + n] = v;
             else
@@ -373,8 +371,7 @@ __device__ __forceinline__ void store_rope8(const FusedArgs& a, const floatx4& a
 constexpr int kStageRow = 256 + 16;           // bytes of a row in a staging area: the padding spreads the rows over the banks
 constexpr int kStageTile = 16 * kStageRow;    // a wave's staging area
 
-constexpr int kFoldRows = 4;       // the most rows whose norm the q/k/v product makes itself
-constexpr int kFoldElems = 8192;   // rows x K it keeps in LDS for that (16 KB)
+constexpr int kFoldRows = 16;      // the most rows whose norm the q/k/v product makes itself: one row tile
 
 template <int WAVES, int EPI, int MT, int NT, bool FOLD = false>
 __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
@@ -393,9 +390,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     __shared__ __attribute__((aligned(16))) char shared[kSharedBytes + 16 * sizeof(float)];  // + the rows' scales
     float* reduce = reinterpret_cast<float*>(shared);
     char* stage = shared + (threadIdx.x / kWave) * kStageTile;
-    __shared__ __attribute__((aligned(16))) bf16_t fold_rows[FOLD ? kFoldElems : 8];  // [M][K]: the rows of A made here
-    __shared__ float fold_sq[FOLD ? WAVES * kFoldRows : 1];
-    __shared__ float fold_scale[FOLD ? kFoldRows : 1];
+    __shared__ float fold_sq[FOLD ? WAVES * kFoldRows : 1];  // the waves' shares of the rows' sums of squares
 
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
@@ -494,145 +489,8 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
 
     const int k_begin = blockIdx.z * a.k_per_part;
     const int k_end = min(a.K, k_begin + a.k_per_part);
-    if constexpr (FOLD) {
-        // The wave's first pieces of W are asked for, then the rows of A are made while they travel: the
-        // stream plus its pending partial sums, times the norm's weight, as bf16 into LDS (the rows' 1/rms
-        // multiplies the sums at the end: the product is linear in its rows).
-        uint4 b[U][NT][4];
-        auto load_w = [&](int kbase) __attribute__((always_inline)) {
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int k0 = kbase + u * WAVES * 128;
-#pragma unroll
-                for (int t = 0; t < NT; ++t)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        b[u][t][i] = (k0 + load_col < k_end) ? *reinterpret_cast<const uint4*>(w_rows[t][i] + k0) : uint4{0, 0, 0, 0};
-            }
-        };
-        int kbase = k_begin + wave * 128;
-        if (kbase < k_end) load_w(kbase);
-        if (rope_pending) {  // behind the wave's first loads of W
-            if (EPI == EPI_ROPE8)
-                rope8_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
-            else
-                rope_prefetch_rest(a, rope_head, rope_tile, lane, rope_rows);
-            rope_pending = false;
-        }
-        const bool writer = blockIdx.x == 0;
-        constexpr int kTogether = WAVES <= 4 ? 2 : 1;  // rows whose loads travel together
-        float sq[kFoldRows] = {0.f, 0.f, 0.f, 0.f};
-        for (int c = threadIdx.x * 8; c < a.K; c += WAVES * kWave * 8) {
-            const float4 w0 = *reinterpret_cast<const float4*>(a.fold_weight + c);
-            const float4 w1 = *reinterpret_cast<const float4*>(a.fold_weight + c + 4);
-#pragma unroll
-            for (int m2 = 0; m2 < kFoldRows; m2 += kTogether) {
-                if (m2 >= a.M) break;  // (uniform)
-                // two rows at a time where the registers allow it (up to four waves: 512 each), so that the loads
-                // of both are under way together (a second row past the last reads the last again; nothing of
-                // it is kept)
-                float4 x0[kTogether], x1[kTogether];
-                size_t at[kTogether];
-#pragma unroll
-                for (int h = 0; h < kTogether; ++h) {
-                    at[h] = static_cast<size_t>(min(m2 + h, a.M - 1)) * a.K + c;
-                    x0[h] = *reinterpret_cast<const float4*>(a.fold_residual + at[h]);
-                    x1[h] = *reinterpret_cast<const float4*>(a.fold_residual + at[h] + 4);
-                }
-                // eight parts at a time, their loads all under way before the first is added (a part past the
-                // last reads the last again and is not added)
-                for (int p0 = 0; p0 < a.fold_n_parts; p0 += 8) {
-                    float4 v[kTogether][8][2];
-#pragma unroll
-                    for (int h = 0; h < kTogether; ++h) {
-                        if (h > 0 && m2 + h >= a.M) {  // (uniform: a single row asks for nothing twice)
-#pragma unroll
-                            for (int j = 0; j < 8; ++j) v[h][j][0] = v[h][j][1] = float4{0.f, 0.f, 0.f, 0.f};
-                            continue;
-                        }
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            const int part = min(p0 + j, a.fold_n_parts - 1);
-                            const float* src = a.fold_parts + static_cast<size_t>(part) * a.M * a.K + at[h];
-                            v[h][j][0] = *reinterpret_cast<const float4*>(src);
-                            v[h][j][1] = *reinterpret_cast<const float4*>(src + 4);
-                        }
-                    }
-#pragma unroll
-                    for (int h = 0; h < kTogether; ++h)
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            // (a select, not a branch: behind a branch the compiler waits for each part's loads in turn)
-                            const bool real = p0 + j < a.fold_n_parts;
-                            x0[h].x += real ? v[h][j][0].x : 0.f; x0[h].y += real ? v[h][j][0].y : 0.f;
-                            x0[h].z += real ? v[h][j][0].z : 0.f; x0[h].w += real ? v[h][j][0].w : 0.f;
-                            x1[h].x += real ? v[h][j][1].x : 0.f; x1[h].y += real ? v[h][j][1].y : 0.f;
-                            x1[h].z += real ? v[h][j][1].z : 0.f; x1[h].w += real ? v[h][j][1].w : 0.f;
-                        }
-                }
-#pragma unroll
-                for (int h = 0; h < kTogether; ++h) {
-                    if (m2 + h >= a.M) break;  // (uniform)
-                    sq[m2 + h] += (x0[h].x * x0[h].x + x0[h].y * x0[h].y) + (x0[h].z * x0[h].z + x0[h].w * x0[h].w) +
-                                  (x1[h].x * x1[h].x + x1[h].y * x1[h].y) + (x1[h].z * x1[h].z + x1[h].w * x1[h].w);
-                    if (writer) {
-                        *reinterpret_cast<float4*>(a.fold_residual_out + at[h]) = x0[h];
-                        *reinterpret_cast<float4*>(a.fold_residual_out + at[h] + 4) = x1[h];
-                    }
-                    uint4 packed;
-                    packed.x = pack_bf16(x0[h].x * w0.x, x0[h].y * w0.y);
-                    packed.y = pack_bf16(x0[h].z * w0.z, x0[h].w * w0.w);
-                    packed.z = pack_bf16(x1[h].x * w1.x, x1[h].y * w1.y);
-                    packed.w = pack_bf16(x1[h].z * w1.z, x1[h].w * w1.w);
-                    *reinterpret_cast<uint4*>(fold_rows + at[h]) = packed;
-                }
-            }
-        }
-#pragma unroll
-        for (int m = 0; m < kFoldRows; ++m) {
-            float v = sq[m];
-#pragma unroll
-            for (int offset = kWave / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
-            if (lane == 0) fold_sq[wave * kFoldRows + m] = v;
-        }
-        __syncthreads();  // the rows and the waves' sums of squares are in LDS
-        if (threadIdx.x < kFoldRows) {
-            float total = 0.f;
-#pragma unroll
-            for (int w = 0; w < WAVES; ++w) total += fold_sq[w * kFoldRows + threadIdx.x];
-            fold_scale[threadIdx.x] = 1.0f / sqrtf(total / static_cast<float>(a.K) + a.eps);
-        }
-#pragma unroll 1
-        while (kbase < k_end) {
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int ka = kbase + u * WAVES * 128;
-                uint4 av[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int k_lane = ka + i * 32 + g * 8;
-                    av[i] = (r < a.M && k_lane < k_end)
-                                ? *reinterpret_cast<const uint4*>(fold_rows + static_cast<size_t>(r) * a.K + k_lane)
-                                : uint4{0, 0, 0, 0};
-                }
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        *reinterpret_cast<uint4*>(stage + (i * 4 + load_row) * kStageRow + load_col * 2) = b[u][t][i];
-                    uint4 bt[4];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) bt[j] = *reinterpret_cast<const uint4*>(stage + r * kStageRow + j * 64 + g * 16);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                            __builtin_bit_cast(bf16x8, av[j]), __builtin_bit_cast(bf16x8, bt[j]), acc[0][t], 0, 0, 0);
-                }
-            }
-            kbase += U * WAVES * 128;
-            if (kbase < k_end) load_w(kbase);
-        }
-    } else {
+    float fold_sq_lane = 0.f;  // FOLD: this lane's share of row r's sum of squares
+    {
 #pragma unroll 1
     for (int kbase = k_begin + wave * 128; kbase < k_end; kbase += U * WAVES * 128) {
         uint4 b[U][NT][4];
@@ -661,6 +519,34 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
             // the few rows of A come from the cache; their loads are issued slice by slice
             const int ka = kbase + u * WAVES * 128;
             uint4 av[MT][4];
+            if constexpr (FOLD) {
+                // lane (r, g) makes row r's k values i*32 + g*8 .. +7 from the float32 stream and the norm's
+                // weight (every load stands unconditionally; what lies past the end is dropped by a select)
+                const float* row = a.fold_residual + static_cast<size_t>(min(m0 + r, a.M - 1)) * a.K;
+                float4 x[4][2], nw[4][2];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int k_read = min(ka + i * 32 + g * 8, a.K - 8);
+                    x[i][0] = *reinterpret_cast<const float4*>(row + k_read);
+                    x[i][1] = *reinterpret_cast<const float4*>(row + k_read + 4);
+                    nw[i][0] = *reinterpret_cast<const float4*>(a.fold_weight + k_read);
+                    nw[i][1] = *reinterpret_cast<const float4*>(a.fold_weight + k_read + 4);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool inside = row_ok[0][i] && ka + i * 32 + g * 8 < k_end;
+                    const float4 lo = x[i][0], hi = x[i][1];
+                    const float sq = (lo.x * lo.x + lo.y * lo.y) + (lo.z * lo.z + lo.w * lo.w) +
+                                     (hi.x * hi.x + hi.y * hi.y) + (hi.z * hi.z + hi.w * hi.w);
+                    fold_sq_lane += inside ? sq : 0.f;
+                    uint4 packed;
+                    packed.x = pack_bf16(lo.x * nw[i][0].x, lo.y * nw[i][0].y);
+                    packed.y = pack_bf16(lo.z * nw[i][0].z, lo.w * nw[i][0].w);
+                    packed.z = pack_bf16(hi.x * nw[i][1].x, hi.y * nw[i][1].y);
+                    packed.w = pack_bf16(hi.z * nw[i][1].z, hi.w * nw[i][1].w);
+                    av[0][i] = inside ? packed : uint4{0, 0, 0, 0};
+                }
+            } else {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -669,6 +555,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
                     av[mt][i] = (row_ok[mt][i] && k_lane < k_end) ? *reinterpret_cast<const uint4*>(a_rows[mt][i] + ka)
                                                                   : uint4{0, 0, 0, 0};
                 }
+            }
             if (kStageA) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
@@ -715,6 +602,11 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) row_scale[i] = scale_lds[g * 4 + i];
         }
+    }
+    if constexpr (FOLD) {  // row r's sum of squares over this wave's slices: the lanes r, r + 16, r + 32, r + 48 hold it
+        fold_sq_lane += __shfl_xor(fold_sq_lane, 16, kWave);
+        fold_sq_lane += __shfl_xor(fold_sq_lane, 32, kWave);
+        if (lane < 16) fold_sq[wave * kFoldRows + lane] = fold_sq_lane;
     }
     // With more than one row tile the waves share the end of the work: row tile mt belongs to wave
     // mt % WAVES, which sums the other waves' partial tiles of that row tile and stores it (one wave
@@ -801,9 +693,13 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
         return;
     }
     if constexpr (FOLD) {  // the rows' 1/rms, which the rows of A were made without
+        // (wave 0, behind the barrier above if there are more; with one wave its LDS operations keep their order)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float scale = fold_scale[min(g * 4 + i, kFoldRows - 1)];  // (rows past the last are not stored)
+            float total = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) total += fold_sq[w * kFoldRows + g * 4 + i];
+            const float scale = 1.0f / sqrtf(total / static_cast<float>(a.K) + a.eps);
 #pragma unroll
             for (int t = 0; t < NT; ++t) acc[0][t][i] *= scale;
         }
@@ -891,7 +787,8 @@ struct SharedRowsLds {
 
 template <int EPI, int MT, int NT, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64) gemm_shared_rows_kernel(FusedArgs a) {
-    static_assert(EPI == EPI_SILU || EPI == EPI_PARTIAL || EPI == EPI_BF16 || EPI == EPI_F32, "epilogues of this form");
+    static_assert(EPI == EPI_SILU || EPI == EPI_PARTIAL || EPI == EPI_BF16 || EPI == EPI_F32 || EPI == EPI_ATOMIC,
+                  "epilogues of this form");
     static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
     constexpr int kWaves = WAVES;
     constexpr int kThreads = WAVES * 64;
@@ -1146,10 +1043,7 @@ CIE_API int cie_gemm_fused(void* stream, const void* a, int lda, const void* w, 
     f.sumsq_parts = sumsq_parts;
     f.eps = eps;
     f.fold_residual = nullptr;
-    f.fold_parts = nullptr;
-    f.fold_n_parts = 0;
     f.fold_weight = nullptr;
-    f.fold_residual_out = nullptr;
     f.rope = RopeArgs{};
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (epilogue) {
@@ -1174,11 +1068,8 @@ constexpr unsigned kSplitPairsBelow = 128;
 namespace {
 struct FoldedNorm {  // the norm in front of the q/k/v product, made by the product itself (see FusedArgs)
     const float* residual = nullptr;
-    const float* parts = nullptr;
-    int n_parts = 0;
     const float* weight = nullptr;
     float eps = 0.f;
-    float* residual_out = nullptr;
 };
 
 int qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bias, void* c,
@@ -1187,11 +1078,8 @@ int qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bi
              const int* block_table, int table_width, void* k_pool, void* v_pool, int q_heads,
              int kv_heads, int head_dim, int page_size, int rotate, int write_kv, const FoldedNorm* fold) {
     if (fold) {
-        if (M <= 0 || M > kFoldRows || K <= 0 || K % 8 || static_cast<long long>(M) * K > kFoldElems || !w || !c)
-            return CIE_BAD_ARGUMENT;
-        if (!fold->residual || !fold->parts || fold->n_parts < 1 || fold->n_parts > 64 || !fold->weight ||
-            !(fold->eps > 0.f) || !fold->residual_out || fold->residual_out == fold->residual)
-            return CIE_BAD_ARGUMENT;
+        if (M <= 0 || M > kFoldRows || K < 8 || K % 8 || !w || !c) return CIE_BAD_ARGUMENT;
+        if (!fold->residual || !fold->weight || !(fold->eps > 0.f)) return CIE_BAD_ARGUMENT;
         a = nullptr;
         lda = K;
     } else if (M <= 0 || (M + 63) / 64 > 65535 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) {
@@ -1222,10 +1110,7 @@ int qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bi
     f.sumsq_parts = 0;
     f.eps = 0.f;
     f.fold_residual = nullptr;
-    f.fold_parts = nullptr;
-    f.fold_n_parts = 0;
     f.fold_weight = nullptr;
-    f.fold_residual_out = nullptr;
     f.rope = RopeArgs{cos_table, sin_table, positions, seq_of_token, seq_slot, block_table, table_width,
                       static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_heads, kv_heads, head_dim,
                       page_size, rotate, write_kv};
@@ -1235,11 +1120,8 @@ int qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bi
     const bool one_tile = M <= 16 && grid.x < kSplitPairsBelow;  // few columns: one tile a workgroup, twice the workgroups
     if (fold) {
         f.fold_residual = fold->residual;
-        f.fold_parts = fold->parts;
-        f.fold_n_parts = fold->n_parts;
         f.fold_weight = fold->weight;
         f.eps = fold->eps;
-        f.fold_residual_out = fold->residual_out;
         if (one_tile) return launch_waves<EPI_ROPE8, 1, 1, true>(s, waves, twice, f);
         return launch_waves<EPI_ROPE, 1, 2, true>(s, waves, grid, f);
     }
@@ -1264,11 +1146,10 @@ CIE_API int cie_gemm_qkv_rope(void* stream, const void* a, int lda, const void* 
                     nullptr);
 }
 
-// The same for up to 4 rows (rows x K <= 8,192) whose RMSNorm the product makes itself: the rows are
-// (residual + the n_parts partial sums `parts` [n_parts, M, K]) * norm_weight * 1/rms, and the summed stream goes
-// to residual_out [M, K] (another buffer than residual).  A decode step of a few sequences saves the norm's kernel.
-CIE_API int cie_gemm_qkv_rope_folded_norm(void* stream, const float* residual, const float* parts, int n_parts,
-                                          const float* norm_weight, float eps, float* residual_out, const void* w,
+// The same for up to 16 rows whose RMSNorm the product makes itself: the rows are residual [M, K] (float32) *
+// norm_weight * 1/rms.  A decode step of a few sequences saves the norm's kernel.
+CIE_API int cie_gemm_qkv_rope_folded_norm(void* stream, const float* residual,
+                                          const float* norm_weight, float eps, const void* w,
                                           const void* bias, void* c, int M, int N, int K, int waves,
                                           const float* cos_table, const float* sin_table, const int* positions,
                                           const int* seq_of_token, const int* seq_slot, const int* block_table,
@@ -1276,11 +1157,8 @@ CIE_API int cie_gemm_qkv_rope_folded_norm(void* stream, const float* residual, c
                                           int head_dim, int page_size, int rotate, int write_kv) {
     FoldedNorm fold;
     fold.residual = residual;
-    fold.parts = parts;
-    fold.n_parts = n_parts;
     fold.weight = norm_weight;
     fold.eps = eps;
-    fold.residual_out = residual_out;
     return qkv_rope(stream, nullptr, K, w, bias, c, M, N, K, waves, cos_table, sin_table, positions, seq_of_token,
                     seq_slot, block_table, table_width, k_pool, v_pool, q_heads, kv_heads, head_dim, page_size, rotate,
                     write_kv, &fold);
@@ -1289,16 +1167,18 @@ CIE_API int cie_gemm_qkv_rope_folded_norm(void* stream, const float* residual, c
 // The form for 17 to 128 rows in which a workgroup's waves own columns and share the rows of A
 // through LDS (one workgroup row: M <= 128).  epilogue 0 (bf16, + bias), 1 (float32, + bias; two tiles a wave),
 // 2 (SiLU-gate; row_sumsq as in
-// cie_gemm_fused, for any number of rows here) or 4 (k_parts partial products).  column_tiles 1 or 2 tiles of
+// cie_gemm_fused, for any number of rows here), 4 (k_parts partial products) or 7 (k_parts parts of K, each of
+// which adds its products into `c`, float32 [M, N], with atomic adds: the order of the sums is not fixed).  column_tiles 1 or 2 tiles of
 // 16 columns per wave (SiLU: the gate tile and its up tile), 2 to 4 waves per workgroup.
 CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const void* w, const void* bias, void* c, int M,
                                  int N, int K, int epilogue, int column_tiles, int waves, int k_parts,
                                  const float* row_sumsq, int sumsq_parts, float eps) {
     if (M <= 0 || M > 128 || N <= 0 || K <= 0 || K % 8 || !a || !w || !c || lda < K || lda % 8) return CIE_BAD_ARGUMENT;
-    if (epilogue != EPI_BF16 && epilogue != EPI_F32 && epilogue != EPI_SILU && epilogue != EPI_PARTIAL) return CIE_BAD_ARGUMENT;
+    if (epilogue != EPI_BF16 && epilogue != EPI_F32 && epilogue != EPI_SILU && epilogue != EPI_PARTIAL && epilogue != EPI_ATOMIC)
+        return CIE_BAD_ARGUMENT;
     if (epilogue == EPI_SILU && (N % 2 || bias || column_tiles != 2)) return CIE_BAD_ARGUMENT;
     if (column_tiles != 1 && column_tiles != 2) return CIE_BAD_ARGUMENT;
-    if (k_parts < 1 || k_parts > 64 || (k_parts > 1 && epilogue != EPI_PARTIAL)) return CIE_BAD_ARGUMENT;
+    if (k_parts < 1 || k_parts > 64 || (k_parts > 1 && epilogue != EPI_PARTIAL && epilogue != EPI_ATOMIC)) return CIE_BAD_ARGUMENT;
     if (row_sumsq && (epilogue != EPI_SILU || sumsq_parts < 1 || !(eps > 0.f))) return CIE_BAD_ARGUMENT;
     FusedArgs f;
     f.a = static_cast<const bf16_t*>(a);
@@ -1306,7 +1186,7 @@ CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const voi
     f.w = static_cast<const bf16_t*>(w);
     f.bias = static_cast<const bf16_t*>(bias);
     f.c = c;
-    f.residual = nullptr;
+    f.residual = (epilogue == EPI_ATOMIC) ? static_cast<float*>(c) : nullptr;
     f.sumsq = nullptr;
     f.M = M;
     f.N = N;
@@ -1319,10 +1199,7 @@ CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const voi
     f.sumsq_parts = sumsq_parts;
     f.eps = eps;
     f.fold_residual = nullptr;
-    f.fold_parts = nullptr;
-    f.fold_n_parts = 0;
     f.fold_weight = nullptr;
-    f.fold_residual_out = nullptr;
     f.rope = RopeArgs{};
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (epilogue) {
@@ -1335,6 +1212,9 @@ CIE_API int cie_gemm_shared_rows(void* stream, const void* a, int lda, const voi
         case EPI_PARTIAL:
             return column_tiles == 2 ? launch_shared_rows<EPI_PARTIAL, 2>(s, waves, k_parts, f)
                                      : launch_shared_rows<EPI_PARTIAL, 1>(s, waves, k_parts, f);
+        case EPI_ATOMIC:
+            return column_tiles == 2 ? launch_shared_rows<EPI_ATOMIC, 2>(s, waves, k_parts, f)
+                                     : launch_shared_rows<EPI_ATOMIC, 1>(s, waves, k_parts, f);
     }
     return CIE_BAD_ARGUMENT;
 }

@@ -38,118 +38,6 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __rest
         dst[h] = from_float<T>((staged[h] * inv) * to_float(weight[h]));
 }
 
-// The same, with the branch given as `n_parts` float32 partial products [n_parts, rows_total, hidden]
-// (left by a product whose K was cut into parts): residual += sum of the parts, then the norm.
-template <typename W>
-__global__ void add_parts_rmsnorm_kernel(float* __restrict__ residual, const float* __restrict__ parts,
-                                         int n_parts, int rows_total, const W* __restrict__ weight,
-                                         bf16_t* __restrict__ out, const int* __restrict__ rows, int hidden,
-                                         float eps, int write_residual) {
-    extern __shared__ float staged[];
-    __shared__ float scratch[16];
-    const int out_row = blockIdx.x;
-    const int row = rows ? rows[out_row] : out_row;
-    float* res = residual + static_cast<size_t>(row) * hidden;
-    float sum_sq = 0.f;
-    for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
-        float x = res[h];
-        for (int p = 0; p < n_parts; ++p) x += parts[(static_cast<size_t>(p) * rows_total + row) * hidden + h];
-        if (write_residual) res[h] = x;
-        staged[h] = x;
-        sum_sq += x * x;
-    }
-    const float total = block_sum(sum_sq, scratch);
-    const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
-    bf16_t* dst = out + static_cast<size_t>(out_row) * hidden;
-    for (int h = threadIdx.x; h < hidden; h += blockDim.x)
-        dst[h] = from_float<bf16_t>((staged[h] * inv) * to_float(weight[h]));
-}
-
-// The same with four values per thread and 16-byte accesses (hidden a multiple of 4, bf16 norm weight):
-// a thread's loads of the residual and of all parts are independent and travel together.
-__global__ void add_parts_rmsnorm_vec4_kernel(float* __restrict__ residual, const float* __restrict__ parts,
-                                              int n_parts, int rows_total, const bf16_t* __restrict__ weight,
-                                              bf16_t* __restrict__ out, const int* __restrict__ rows, int hidden,
-                                              float eps, int write_residual) {
-    extern __shared__ float staged[];
-    __shared__ float scratch[16];
-    const int out_row = blockIdx.x;
-    const int row = rows ? rows[out_row] : out_row;
-    float* res = residual + static_cast<size_t>(row) * hidden;
-    const size_t part_stride = static_cast<size_t>(rows_total) * hidden;
-    const float* part0 = parts + static_cast<size_t>(row) * hidden;
-    float sum_sq = 0.f;
-    // One pass: the stream's four values and those of all parts, eight parts at a time with all their loads
-    // under way before the first is added.  No branch stands between the loads (behind one the compiler waits
-    // for each in turn): a part past the last reads the last again and is dropped by a select.
-    auto pass = [&](int h) __attribute__((always_inline)) {
-        float4 x = *reinterpret_cast<const float4*>(res + h);
-        for (int p0 = 0; p0 < n_parts; p0 += 8) {
-            float4 v[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                v[j] = *reinterpret_cast<const float4*>(part0 + min(p0 + j, n_parts - 1) * part_stride + h);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const bool real = p0 + j < n_parts;
-                x.x += real ? v[j].x : 0.f; x.y += real ? v[j].y : 0.f;
-                x.z += real ? v[j].z : 0.f; x.w += real ? v[j].w : 0.f;
-            }
-        }
-        if (write_residual) *reinterpret_cast<float4*>(res + h) = x;
-        *reinterpret_cast<float4*>(staged + h) = x;
-        sum_sq += (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
-    };
-    // The first pass (the only one of a row of up to 4,096 values on 1,024 threads) stands outside the loop (at a
-    // loop's head the compiler waits for every load that is under way), and the weight of its values is asked for
-    // with its other loads.
-    const int h_first = threadIdx.x * 4;
-    uint2 raw_first = uint2{0u, 0u};
-    if (h_first < hidden) {
-        raw_first = *reinterpret_cast<const uint2*>(weight + h_first);
-        pass(h_first);
-    }
-    for (int h = h_first + blockDim.x * 4; h < hidden; h += blockDim.x * 4) pass(h);
-    const float total = block_sum(sum_sq, scratch);
-    const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
-    bf16_t* dst = out + static_cast<size_t>(out_row) * hidden;
-    for (int h = threadIdx.x * 4; h < hidden; h += blockDim.x * 4) {
-        const float4 x = *reinterpret_cast<const float4*>(staged + h);
-        const uint2 raw = h == h_first ? raw_first : *reinterpret_cast<const uint2*>(weight + h);
-        uint2 packed;
-        packed.x = pack_bf16((x.x * inv) * __uint_as_float(raw.x << 16), (x.y * inv) * __uint_as_float(raw.x & 0xffff0000u));
-        packed.y = pack_bf16((x.z * inv) * __uint_as_float(raw.y << 16), (x.w * inv) * __uint_as_float(raw.y & 0xffff0000u));
-        *reinterpret_cast<uint2*>(dst + h) = packed;
-    }
-}
-
-CIE_API int cie_add_parts_rmsnorm(void* stream, int wdtype, float* residual, const float* parts, int n_parts,
-                                  int rows_total, const void* weight, void* out, const int* rows, int n_out,
-                                  int hidden, float eps, int write_residual) {
-    if (n_out < 0 || hidden <= 0 || hidden * sizeof(float) > 64 * 1024 || !(eps > 0.f) || n_parts < 1 || rows_total < 1)
-        return CIE_BAD_ARGUMENT;
-    if (rows && write_residual) return CIE_BAD_ARGUMENT;
-    if (n_out == 0) return CIE_OK;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    // few rows (a decode step): a row's loads are spread over 1024 threads so that they all travel at once
-    const int threads = n_out <= 64 ? 1024 : 256;
-    if (wdtype == CIE_BF16 && hidden % 4 == 0)
-        add_parts_rmsnorm_vec4_kernel<<<n_out, threads, hidden * sizeof(float), s>>>(
-            residual, parts, n_parts, rows_total, static_cast<const bf16_t*>(weight), static_cast<bf16_t*>(out), rows,
-            hidden, eps, write_residual);
-    else if (wdtype == CIE_BF16)
-        add_parts_rmsnorm_kernel<bf16_t><<<n_out, threads, hidden * sizeof(float), s>>>(
-            residual, parts, n_parts, rows_total, static_cast<const bf16_t*>(weight), static_cast<bf16_t*>(out), rows,
-            hidden, eps, write_residual);
-    else if (wdtype == CIE_F32)
-        add_parts_rmsnorm_kernel<float><<<n_out, threads, hidden * sizeof(float), s>>>(
-            residual, parts, n_parts, rows_total, static_cast<const float*>(weight), static_cast<bf16_t*>(out), rows,
-            hidden, eps, write_residual);
-    else
-        return CIE_BAD_ARGUMENT;
-    return cie_after_launch();
-}
-
 // bf16 activations and weight, hidden a multiple of 8: eight elements per thread, 16-byte accesses.
 __global__ void add_rmsnorm_vec8_kernel(float* __restrict__ residual, const bf16_t* __restrict__ branch,
                                         const bf16_t* __restrict__ weight, bf16_t* __restrict__ out,

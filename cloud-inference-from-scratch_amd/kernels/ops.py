@@ -162,29 +162,6 @@ def add_rmsnorm(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: 
     return out
 
 
-def add_parts_rmsnorm(residual: torch.Tensor, parts: torch.Tensor, weight: torch.Tensor, eps: float,
-                      rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``residual += parts.sum(0)`` (written back unless ``rows``), then bf16 RMSNorm; parts float32 [P, T, H]."""
-    _gpu("residual", residual, torch.float32, 2)
-    tokens, hidden = residual.shape
-    _gpu("parts", parts, torch.float32, 3)
-    if not (parts.shape[1:] == residual.shape):
-        raise ValueError(f"parts {tuple(parts.shape)} vs residual {tuple(residual.shape)}")
-    _gpu("weight", weight, dims=1)
-    if not (weight.shape[0] == hidden and weight.dtype in (torch.bfloat16, torch.float32)):
-        raise ValueError("norm weight does not fit")
-    if not (hidden <= MAX_NORM_WIDTH and eps > 0):
-        raise ValueError(f"hidden {hidden} or eps {eps} out of range")
-    if rows is not None:
-        _gpu("rows", rows, torch.int32, 1)
-    n_out = rows.shape[0] if rows is not None else tokens
-    out = torch.empty((n_out, hidden), dtype=torch.bfloat16, device=residual.device)
-    _run("cie_add_parts_rmsnorm", load_library().cie_add_parts_rmsnorm(
-        _stream(), _i(_code(weight.dtype)), _ptr(residual), _ptr(parts), _i(parts.shape[0]), _i(tokens), _ptr(weight),
-        _ptr(out), _ptr(rows), _i(n_out), _i(hidden), _f(eps), _i(0 if rows is not None else 1)))
-    return out
-
-
 def rmsnorm_from_sumsq(residual: torch.Tensor, sumsq: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """bf16 RMSNorm of float32 rows whose partial sums of squares ``sumsq`` [rows, parts] are known."""
     _gpu("residual", residual, torch.float32, 2)
@@ -426,6 +403,7 @@ def gemm_f32(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]
 
 
 EPI_BF16, EPI_F32, EPI_SILU, EPI_RESID, EPI_PARTIAL = 0, 1, 2, 3, 4
+EPI_ATOMIC = 7  # (the shared-rows form: parts of K add into a float32 stream with atomic adds)
 FUSED_TARGET_WAVES = 2048
 FUSED_MAX_ROWS = 64  # rows one workgroup of ``gemm_fused`` takes; more rows run as more workgroup rows
 FUSED_PAIR_WORKGROUPS = 256  # workgroups that must remain when workgroups of many rows take two column tiles
@@ -538,13 +516,16 @@ SHARED_ROWS_MAX = 128  # rows of the form whose waves share the rows of A
 
 def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias: Optional[torch.Tensor] = None,
                      column_tiles: int = 2, waves: int = 4, k_parts: int = 1,
-                     row_sumsq: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+                     row_sumsq: Optional[torch.Tensor] = None, eps: float = 0.0,
+                     add_into: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``a @ weight.T`` for 17 to 128 rows (it takes fewer too) in the form whose four waves per
     workgroup own columns and share each slice of ``a`` through LDS: ``EPI_BF16`` or ``EPI_F32`` (+ bias),
     ``EPI_SILU`` (weight = gate rows over up rows; with ``row_sumsq`` and ``eps`` the rows of ``a``
     lack their ``rsqrt(mean square + eps)``, as in :func:`gemm_fused`) or ``EPI_PARTIAL``
-    (``k_parts`` float32 partial products [k_parts, M, N], bias in part 0).  ``column_tiles``
-    tiles of 16 columns per wave, ``waves`` waves per workgroup."""
+    (``k_parts`` float32 partial products [k_parts, M, N], bias in part 0) or ``EPI_ATOMIC``
+    (each of the ``k_parts`` parts of K adds its products into ``add_into``, float32 [M, N], with the
+    hardware's atomic float add: no partial products to sum afterwards, and no fixed order of the sums;
+    ``add_into`` comes back).  ``column_tiles`` tiles of 16 columns per wave, ``waves`` waves per workgroup."""
     _gpu("weight", weight, torch.bfloat16, 2)
     n, k = weight.shape
     if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
@@ -555,12 +536,18 @@ def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias:
     lda = a.stride(0) if m > 1 else max(a.stride(0), k)
     if not (k % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0):
         raise ValueError(f"K and the row stride must be multiples of 8 (are {k}, {lda}) and the operands 16-byte aligned")
-    if epilogue not in (EPI_BF16, EPI_F32, EPI_SILU, EPI_PARTIAL):
+    if epilogue not in (EPI_BF16, EPI_F32, EPI_SILU, EPI_PARTIAL, EPI_ATOMIC):
         raise ValueError(f"epilogue {epilogue} is not one this form has")
     if epilogue == EPI_F32:
         column_tiles = 2
-    if not (1 <= k_parts <= 64 and (k_parts == 1 or epilogue == EPI_PARTIAL)):
+    if not (1 <= k_parts <= 64 and (k_parts == 1 or epilogue in (EPI_PARTIAL, EPI_ATOMIC))):
         raise ValueError(f"k_parts {k_parts} does not fit the epilogue")
+    if (epilogue == EPI_ATOMIC) != (add_into is not None):
+        raise ValueError("the atomic epilogue, and only it, adds into a stream that the caller gives")
+    if add_into is not None:
+        _gpu("add_into", add_into, torch.float32, 2)
+        if not (tuple(add_into.shape) == (m, n) and add_into.is_contiguous()):
+            raise ValueError(f"add_into is {tuple(add_into.shape)}, the product [{m}, {n}]")
     if epilogue == EPI_SILU:
         column_tiles = 2
         if n % 2 or bias is not None:
@@ -584,6 +571,8 @@ def gemm_shared_rows(weight: torch.Tensor, epilogue: int, a: torch.Tensor, bias:
         out = torch.empty((m, n), dtype=torch.float32, device=device)
     elif epilogue == EPI_SILU:
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=device)
+    elif epilogue == EPI_ATOMIC:
+        out = add_into
     else:
         out = torch.empty((k_parts, m, n), dtype=torch.float32, device=device)
     _run("cie_gemm_shared_rows", load_library().cie_gemm_shared_rows(
@@ -663,20 +652,31 @@ def gemm_library(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
 QKV_SPLIT_PAIRS_BELOW = 128  # (as in the kernel library: below this many pairs of tiles, one tile a workgroup)
 
 
-FOLDED_NORM_ROWS = 4      # the most rows whose norm the q/k/v product makes itself ...
-FOLDED_NORM_VALUES = 8192  # ... and the most values (rows x K) it keeps for that
+FOLDED_NORM_ROWS = 16      # the most rows whose norm the q/k/v product makes itself: one tile of rows
+# ... and the most values (rows x K) for which that is the faster way: every workgroup of the product makes
+# the rows anew, which costs it 1.8 to 2.8 us with the 3B shape's width and 4 to 6 us with the 14B shape's, where the
+# norm's own kernel takes 3.6 us (norm + product against the product that makes its norm, us: 3B 1 / 8 / 16 rows
+# 8.9 / 10.5 / 10.7 against 7.6 / 9.7 / 10.9; 7B 13.4 / 15.3 / 16.6 against 12.4 / 15.5 / 17.8; 14B 21.3 / 22.3 /
+# 23.4 against 21.4 / 24.7 / 27.5; 0.5B 7.0 / 8.4 / 8.5 against 6.3 / 8.1 / 9.3)
+FOLDED_NORM_VALUES = 16384
+FOLDED_NORM_WIDTH = 4096
 
 
 def folds_norm(rows: int, k: int) -> bool:
-    """Whether ``gemm_qkv_rope`` takes ``unsummed=`` for this many rows of ``k`` values."""
-    return 1 <= rows <= FOLDED_NORM_ROWS and rows * k <= FOLDED_NORM_VALUES and k % 8 == 0
+    """Whether ``gemm_qkv_rope`` takes ``folded=`` for this many rows of ``k`` values."""
+    return 1 <= rows <= FOLDED_NORM_ROWS and k >= 8 and k % 8 == 0
+
+
+def folding_norm_pays(rows: int, k: int) -> bool:
+    """Whether the product that makes its norm is the faster way for this many rows of ``k`` values."""
+    return folds_norm(rows, k) and rows * k <= FOLDED_NORM_VALUES and k <= FOLDED_NORM_WIDTH
 
 
 def gemm_qkv_rope(weight: torch.Tensor, a: Optional[torch.Tensor], bias: Optional[torch.Tensor], cos: torch.Tensor,
                   sin: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, seq_slot: torch.Tensor,
                   block_table: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, q_heads: int,
                   kv_heads: int, head_dim: int, rotate: bool = True, write_kv: bool = True,
-                  waves: Optional[int] = None, unsummed: Optional[tuple] = None):
+                  waves: Optional[int] = None, folded: Optional[tuple] = None) -> torch.Tensor:
     """The q/k/v product of a few rows (64 per workgroup) fused with what ``rope_kv_write`` does:
     ``a @ weight.T + bias`` for weight [(Hq+2Hkv)*D, K], queries and keys rotated
     by each row's position, keys and values written into the cache.  Returns the
@@ -684,27 +684,24 @@ def gemm_qkv_rope(weight: torch.Tensor, a: Optional[torch.Tensor], bias: Optiona
     and value columns are not written).  Same results as ``gemm_fused`` followed
     by ``rope_kv_write``.  Head sizes in steps of 32.
 
-    ``unsummed=(residual, parts, norm_weight, eps)`` instead of ``a`` (``folds_norm`` says for which sizes):
-    the rows are the RMSNorm of ``residual + parts.sum(0)`` (float32 [M, K] and [P, M, K], float32 weight),
-    made inside the product; returns ``(buffer, summed)`` with the summed stream in a tensor of its own."""
+    ``folded=(residual, norm_weight, eps)`` instead of ``a`` (``folds_norm`` says for which sizes): the rows
+    are the RMSNorm of ``residual`` (float32 [M, K], float32 weight), made inside the product: a lane makes
+    the values of its matrix operand from the stream, and the rows' 1/rms multiplies the sums."""
     _gpu("weight", weight, torch.bfloat16, 2)
     n, k = weight.shape
-    if unsummed is not None:
-        residual, parts, norm_weight, eps = unsummed
+    if folded is not None:
+        residual, norm_weight, eps = folded
         _gpu("residual", residual, torch.float32, 2)
-        _gpu("parts", parts, torch.float32, 3)
         _gpu("norm_weight", norm_weight, torch.float32, 1)
         m = residual.shape[0]
         if a is not None or not folds_norm(m, k):
-            raise ValueError(f"the product makes the norm of up to {FOLDED_NORM_ROWS} rows and {FOLDED_NORM_VALUES} "
-                             f"values itself, not of {m} rows of {k}; and then takes no rows")
-        if not (residual.shape == (m, k) and parts.shape[1:] == (m, k) and 1 <= parts.shape[0] <= 64
-                and norm_weight.shape == (k,) and eps > 0):
-            raise ValueError(f"residual {tuple(residual.shape)}, parts {tuple(parts.shape)}, weight "
-                             f"{tuple(norm_weight.shape)} do not fit rows of K={k}")
-        if not (residual.is_contiguous() and parts.is_contiguous() and norm_weight.is_contiguous()
-                and residual.data_ptr() % 16 == 0 and parts.data_ptr() % 16 == 0 and norm_weight.data_ptr() % 16 == 0):
-            raise ValueError("residual, parts and weight must be contiguous and 16-byte aligned")
+            raise ValueError(f"the product makes the norm of up to {FOLDED_NORM_ROWS} rows itself, not of {m} rows "
+                             f"of {k}; and then takes no rows")
+        if not (residual.shape == (m, k) and norm_weight.shape == (k,) and eps > 0):
+            raise ValueError(f"residual {tuple(residual.shape)}, weight {tuple(norm_weight.shape)} do not fit rows of K={k}")
+        if not (residual.is_contiguous() and norm_weight.is_contiguous()
+                and residual.data_ptr() % 16 == 0 and norm_weight.data_ptr() % 16 == 0):
+            raise ValueError("residual and weight must be contiguous and 16-byte aligned")
         lda = k
     else:
         if not (a.is_cuda and a.dtype == torch.bfloat16 and a.dim() == 2 and a.stride(1) == 1):
@@ -747,14 +744,13 @@ def gemm_qkv_rope(weight: torch.Tensor, a: Optional[torch.Tensor], bias: Optiona
     if not (waves in ((1, 2, 4, 8) if m <= 16 else (4, 8))):
         raise ValueError(f"{waves} waves per workgroup with {m} rows is not a form the kernel has")
     out = torch.empty((m, n), dtype=torch.bfloat16, device=weight.device)
-    if unsummed is not None:
-        summed = torch.empty_like(residual)
+    if folded is not None:
         _run("cie_gemm_qkv_rope_folded_norm", load_library().cie_gemm_qkv_rope_folded_norm(
-            _stream(), _ptr(residual), _ptr(parts), _i(parts.shape[0]), _ptr(norm_weight), _f(eps), _ptr(summed),
+            _stream(), _ptr(residual), _ptr(norm_weight), _f(eps),
             _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k), _i(waves), _ptr(cos), _ptr(sin), _ptr(positions),
             _ptr(seq_of_token), _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]), _ptr(k_pool), _ptr(v_pool),
             _i(q_heads), _i(kv_heads), _i(head_dim), _i(page_size), _i(1 if rotate else 0), _i(1 if write_kv else 0)))
-        return out, summed
+        return out
     _run("cie_gemm_qkv_rope", load_library().cie_gemm_qkv_rope(
         _stream(), _ptr(a), _i(lda), _ptr(weight), _ptr(bias), _ptr(out), _i(m), _i(n), _i(k), _i(waves), _ptr(cos),
         _ptr(sin), _ptr(positions), _ptr(seq_of_token), _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]),

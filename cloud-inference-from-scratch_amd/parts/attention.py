@@ -21,14 +21,14 @@ from ..config.specs import PartSpec
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, build_part, register_part
-from .linear import FUSED_ROWS, FUSED_SMALL_ROWS, FUSED_SMALL_WEIGHT, UnsummedRows, linear
+from .linear import FUSED_ROWS, FUSED_SMALL_ROWS, FUSED_SMALL_WEIGHT, RawRows, linear
 
 
 class Attention(Part):
     graph_safe = True
     adds_to_residual = True
     folds_next_norm = True  # its output product can leave the next norm's rows short of their scale
-    takes_unsummed_rows = True  # its first product can sum a few rows' pending parts and make their norm itself
+    takes_raw_rows = True  # its first product can make the norm of a few rows itself
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qkv_bias: bool, out_bias: bool, position: PartSpec, window: Optional[int] = None,
                  scale: Optional[float] = None) -> None:
@@ -105,15 +105,14 @@ class Attention(Part):
         rotary_dim = getattr(self.position, "rotary_dim", self.head_dim) if self.position.rotates else None
         untouched = (type(self).shape_projection is Attention.shape_projection
                      and rotary_dim in (None, self.head_dim))
-        if isinstance(x, UnsummedRows):
+        if isinstance(x, RawRows):
             if untouched and self.head_dim % 32 == 0 and self.w_qkv.dtype == torch.bfloat16:
-                # the product sums the stream's pending parts and makes the norm of its rows itself
-                qkv, x.residual = ops.gemm_qkv_rope(
+                # the product makes the norm of its rows itself
+                qkv = ops.gemm_qkv_rope(
                     self.w_qkv, None, self.b_qkv, self.cos, self.sin, batch.positions, batch.seq_of_token,
                     batch.seq_slot, view.block_table, view.k_pool, view.v_pool, self.num_heads, self.num_kv_heads,
                     self.head_dim, rotate=self.position.rotates, write_kv=writes,
-                    unsummed=(x.residual, x.parts, x.norm.weight_f32, x.norm.eps))
-                residual = x.residual if residual is not None else None
+                    folded=(x.residual, x.norm.weight_f32, x.norm.eps))
                 context = attend(qkv, batch, view, self.num_heads, self.num_kv_heads, self.head_dim,
                                  self.window, self.scale)
                 return linear(context, self.w_o, self.b_o, into=residual, then_norm=next_norm)

@@ -13,7 +13,7 @@ Interfaces (``x`` is ``[tokens, hidden]`` in the engine's activation dtype,
 ``Norm``        ``forward(residual, branch, out_dtype, rows=None) -> x``
                 adds ``branch`` into ``residual`` (in place, float32) and returns
                 the normalised rows.  A norm that sets ``takes_row_sumsq`` is
-                also handed the ``RowSumsq`` / ``PartialSum`` forms of a branch
+                also handed the ``RowSumsq`` / ``Added`` forms of a branch
                 (``parts/linear.py``); any other gets a tensor or ``None``.
 ``Position``    ``tables(device) -> (cos, sin)`` or whatever its mixer asks of it.
 ``Mixer``       ``cache_need() -> PagedKV | FixedState | None`` and
@@ -72,7 +72,7 @@ class Part:
 
     graph_safe = False
     # ``adds_to_residual``: ``forward`` takes ``residual=`` and may add its output there itself
-    # (returning a ``RowSumsq``) or leave partial products for the next norm (a ``PartialSum``).
+    # (returning a ``RowSumsq`` or an ``Added``).
     adds_to_residual = False
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:

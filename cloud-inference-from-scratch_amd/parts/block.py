@@ -5,8 +5,8 @@
 float32; a branch's output is added inside the next norm kernel, so the block
 returns the feed-forward output as ``pending`` instead of adding it.  A part
 that can add its output into the residual itself (the fused decode products do)
-returns a ``RowSumsq`` instead (or a ``PartialSum`` of partial products), and
-the next norm then runs its cheaper form (``parts/linear.py``).
+returns a ``RowSumsq`` or an ``Added`` instead, and the next norm then runs its
+cheaper form or rides along with the product behind it (``parts/linear.py``).
 """
 
 from __future__ import annotations
@@ -18,7 +18,7 @@ import torch
 from ..config.specs import LayerSpec
 from ..weights.tensors import TensorSpec
 from .base import build_part, register_part
-from .linear import PartialSum, RowSumsq, UnsummedRows
+from .linear import Added, RawRows, RowSumsq
 
 
 class PreNormBlock:
@@ -59,10 +59,10 @@ class PreNormBlock:
 
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], batch, view,
                 writes: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
-        if (isinstance(pending, PartialSum) and getattr(self.mixer, "takes_unsummed_rows", False)
-                and getattr(self.norm1, "folds_into_products", False) and UnsummedRows.fits(residual, self.dtype)):
-            # a few rows: the mixer's first product sums the parts and makes the norm itself (a kernel less)
-            x = UnsummedRows(residual, pending.parts, self.norm1, self.dtype)
+        if ((pending is None or isinstance(pending, Added)) and getattr(self.mixer, "takes_raw_rows", False)
+                and getattr(self.norm1, "folds_into_products", False) and RawRows.fits(residual, self.dtype)):
+            # a few rows, the stream complete: the mixer's first product makes the norm itself (a kernel less)
+            x = RawRows(residual, self.norm1, self.dtype)
         else:
             x = normalise(self.norm1, residual, pending, self.dtype)
         extra = {"residual": residual} if getattr(self.mixer, "adds_to_residual", False) else {}
@@ -70,8 +70,6 @@ class PreNormBlock:
                 and getattr(self.feed_forward, "takes_scaled_rows", False)):
             extra["next_norm"] = self.norm2  # the norm between the two rides along with their products
         mixed = self.mixer.forward(x, batch, view, writes, **extra)
-        if isinstance(x, UnsummedRows):
-            residual = x.residual  # the summed stream, where the mixer left it (and added its own output)
         x = normalise(self.norm2, residual, mixed, self.dtype)
         extra = {"residual": residual} if getattr(self.feed_forward, "adds_to_residual", False) else {}
         return residual, self.feed_forward.forward(x, **extra)
@@ -80,14 +78,9 @@ class PreNormBlock:
 def normalise(norm, residual: torch.Tensor, pending, dtype: torch.dtype, rows=None):
     """Run ``norm`` on the residual stream plus what is pending.  Only a norm that
     says so (``takes_row_sumsq``) is shown the fused forms of a branch; for any
-    other the partial products are added here and an already added branch
-    becomes ``None``."""
-    if not getattr(norm, "takes_row_sumsq", False):
-        if isinstance(pending, PartialSum):
-            residual.add_(pending.parts.sum(0))
-            pending = None
-        elif isinstance(pending, RowSumsq):
-            pending = None
+    other an already added branch becomes ``None``."""
+    if not getattr(norm, "takes_row_sumsq", False) and isinstance(pending, (RowSumsq, Added)):
+        pending = None
     if rows is not None:
         return norm.forward(residual, pending, dtype, rows=rows)
     return norm.forward(residual, pending, dtype)

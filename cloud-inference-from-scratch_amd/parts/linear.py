@@ -46,7 +46,7 @@ FUSED_SMALL_WEIGHT = 6 << 20
 # 64 rows; up to 64 rows it is one pass either way)
 FUSED_LOGIT_ROWS = 64
 # An ``into=`` product with fewer than this many 16-column tiles and a K of at least ``PART_MIN_K`` cuts K
-# into parts for more workgroups (partial products, summed by the next norm kernel; ``plan_shared_parts``).
+# into parts for more workgroups (each part adds its products into the stream with atomic adds; ``plan_shared_parts``).
 PART_BELOW_TILES = 512
 PART_MIN_K = 4096
 PART_K = 1024           # the shortest stretch of K a part takes
@@ -128,47 +128,35 @@ class ScaledRows:
 
 
 @dataclass
-class PartialSum:
-    """Stands where a branch output would: float32 partial products ``parts``
-    [P, rows, hidden] whose sum is the branch (a product whose K was cut)."""
-
-    parts: torch.Tensor
-
-
-# Rows up to which the q/k/v product sums the stream's pending parts and makes the norm itself.  Every workgroup
-# of the product then reads the rows and all their parts (3B shape, 8 parts: 72 KB a row through each compute
-# unit's cache) while its first weight loads travel, which costs it some 2 us where the norm's own kernel takes
-# 4.6.  Decode tokens/s without and with, at 1 / 2 / 4 sequences: 3B 435 -> 451, 860 -> 886, 1,665 -> 1,687;
-# 0.5B 1,013 -> 1,066, 1,994 -> 2,071, 3,792 -> 3,839; 7B 304 -> 308, 602 -> 605 (four rows of its width are
-# more than the kernel keeps).  (The parts' loads must not stand behind a branch: with one, the compiler waited
-# for each part in turn and the trade was even at two rows and lost 8 % at four.)
-UNSUMMED_ROWS = 4
+class Added:
+    """Stands where a branch output would: the branch was already added into the residual stream, and
+    nothing else is known of the stream's rows (a product whose K was cut into parts, each of which added
+    its share with atomic adds)."""
 
 
 @dataclass
-class UnsummedRows:
+class RawRows:
     """Stands where an RMSNorm's output would, before anything was computed: the rows are the norm ``norm``
-    of ``residual + parts.sum(0)``.  Only a mixer that says ``takes_unsummed_rows`` is shown it.  Whoever
-    sums the parts leaves the summed stream in ``residual`` (the same tensor, summed in place, or another
-    one): the block reads it there afterwards."""
+    of the float32 stream ``residual``.  Only a mixer that says ``takes_raw_rows`` is shown it (the attention
+    part's q/k/v product then makes its rows itself, with up to ``ops.FOLDED_NORM_ROWS`` rows: every workgroup
+    reads the few rows once, where a kernel of its own for the norm costs a decode layer 4.6 us)."""
 
     residual: torch.Tensor
-    parts: torch.Tensor
     norm: Any
     dtype: torch.dtype = torch.bfloat16
 
     @staticmethod
     def fits(residual: torch.Tensor, dtype: torch.dtype) -> bool:
         rows, width = residual.shape
-        return dtype == torch.bfloat16 and residual.is_cuda and rows <= UNSUMMED_ROWS and ops.folds_norm(rows, width)
+        return dtype == torch.bfloat16 and residual.is_cuda and ops.folding_norm_pays(rows, width)
 
     @property
     def shape(self):
         return self.residual.shape
 
     def complete(self) -> torch.Tensor:
-        """The norm's output after all (the parts are added into the stream in place)."""
-        return ops.add_parts_rmsnorm(self.residual, self.parts, self.norm.weight, self.norm.eps)
+        """The norm's output after all."""
+        return ops.add_rmsnorm(self.residual, None, self.norm.weight, self.norm.eps, self.dtype)
 
 
 _WIDENED: dict[int, tuple["weakref.ref", torch.Tensor]] = {}
@@ -191,14 +179,14 @@ def _fusable(rows: int, k: int, row_stride: int, weight: torch.Tensor) -> bool:
 
 def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None, epilogue: Optional[str] = None,
-           into: Optional[torch.Tensor] = None, then_norm: Any = None) -> Union[torch.Tensor, RowSumsq, PartialSum]:
+           into: Optional[torch.Tensor] = None, then_norm: Any = None) -> Union[torch.Tensor, RowSumsq, Added]:
     """``x @ weight.T + bias``.
 
     ``epilogue="silu"``: weight stacks gate rows over up rows; returns
     ``silu(gate) * up``.  ``into=residual``: the caller wants the result added to
-    the float32 residual stream; if a fused kernel runs, either it adds it in
-    place and a :class:`RowSumsq` comes back, or a :class:`PartialSum` of partial
-    products comes back that the next norm kernel adds; otherwise the plain
+    the float32 residual stream; if a fused kernel runs it adds it in place, and a
+    :class:`RowSumsq` comes back, or (a product whose K was cut into parts that
+    each add their share) an :class:`Added`; otherwise the plain
     result comes back and the caller adds it (the next norm kernel does).
     ``then_norm`` (with ``into``): the norm that follows, if it can be folded into
     this product and the next (``RMSNorm.folds_into_products``): the residual
@@ -226,11 +214,16 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     if rows == 0 and into is None:  # nothing to multiply: no kernel, and no widened copy of the weight
         return torch.empty((0, n // 2 if silu else n), dtype=torch.float32 if wants_f32 else x.dtype, device=x.device)
     fusable = _fusable(rows, k, x.stride(0) if rows > 1 else k, weight)
-    cut_k = into is not None and -(-n // 16) < PART_BELOW_TILES and k >= PART_MIN_K
+    cut_k = (into is not None and -(-n // 16) < PART_BELOW_TILES and k >= PART_MIN_K and into.is_contiguous()
+             and tuple(into.shape) == (rows, n))
     if fusable and cut_k and rows <= (FUSED_PARTS_ROWS_NARROW if -(-n // 16) < PARTS_NARROW_TILES else FUSED_PARTS_ROWS):
+        # (atomic adds cost the product nothing, measured against partial products written for the next norm
+        # kernel to sum: 10.3 us either way for the 3B shape's down product at 8 rows; and the kernel that summed
+        # them falls away)
         column_tiles, waves, parts = plan_shared_parts(-(-n // 16), k)
-        return PartialSum(ops.gemm_shared_rows(weight, ops.EPI_PARTIAL, x, bias=bias, column_tiles=column_tiles,
-                                               waves=waves, k_parts=parts))
+        ops.gemm_shared_rows(weight, ops.EPI_ATOMIC, x, bias=bias, column_tiles=column_tiles, waves=waves,
+                             k_parts=parts, add_into=into)
+        return Added()
     if fusable and silu and n % 2 == 0 and bias is None and into is None and not wants_f32 and rows <= SHARED_SILU_ROWS:
         waves, own_unit = plan_shared_silu(-(-n // 32))
         if rows > FUSED_ROWS or own_unit:

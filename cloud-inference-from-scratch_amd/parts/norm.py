@@ -15,7 +15,7 @@ import torch
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, register_part
-from .linear import PartialSum, RowSumsq, ScaledRows
+from .linear import Added, RowSumsq, ScaledRows
 
 
 class RMSNorm(Part):
@@ -43,12 +43,11 @@ class RMSNorm(Part):
 
     def forward(self, residual: torch.Tensor, branch, out_dtype: torch.dtype,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """``branch`` is a tensor still to be added into ``residual``, ``None``, a
-        ``PartialSum`` (float32 partial products still to be added) or a
-        ``RowSumsq`` (already added; the rows' sums of squares are known, so the
-        norm needs no reduction)."""
-        if isinstance(branch, PartialSum):
-            return ops.add_parts_rmsnorm(residual, branch.parts, self.weight, self.eps, rows=rows)
+        """``branch`` is a tensor still to be added into ``residual``, ``None``, an
+        ``Added`` (already added) or a ``RowSumsq`` (already added; the rows' sums
+        of squares are known, so the norm needs no reduction)."""
+        if isinstance(branch, Added):
+            branch = None
         if isinstance(branch, RowSumsq):
             if branch.scaled is not None and branch.norm is self and rows is None and out_dtype == torch.bfloat16:
                 return ScaledRows(branch.scaled, branch.sumsq, self.eps, residual, self)

@@ -586,29 +586,26 @@ def test_gemm_qkv_rope_equals_product_then_rotation(ops, geometry, rows, waves):
 
 @pytest.mark.parametrize("geometry", [(16, 2, 128, 16, 2048), (4, 2, 32, 8, 96), (3, 1, 64, 4, 328), (28, 4, 128, 16, 3584),
                                       (5, 5, 96, 32, 200), (64, 8, 128, 16, 8192)])
-@pytest.mark.parametrize("rows", [1, 2, 3, 4])
+@pytest.mark.parametrize("rows", [1, 3, 8, 13, 16, 17])
 @pytest.mark.parametrize("waves", [None, 1, 8])
-@pytest.mark.parametrize("n_parts", [1, 8, 11])
-def test_gemm_qkv_rope_that_sums_the_stream_and_makes_the_norm_itself(ops, geometry, rows, waves, n_parts):
-    """The q/k/v product of a few rows that is given the residual stream and its pending partial sums instead
-    of normalised rows: the summed stream, the rotated queries and the cache against float64 arithmetic on
-    the kernel's own operand rounding (rows are bf16(x * weight), their 1/rms multiplies the sums)."""
+def test_gemm_qkv_rope_that_makes_the_norm_itself(ops, geometry, rows, waves):
+    """The q/k/v product of up to 16 rows that is given the float32 residual stream instead of normalised rows:
+    the rotated queries and the cache against float64 arithmetic on the kernel's own operand rounding (rows are
+    bf16(x * weight), their 1/rms multiplies the sums), and against the two kernels it replaces."""
     q_heads, kv_heads, head_dim, page_size, hidden = geometry
     if not ops.folds_norm(rows, hidden):
         with pytest.raises(ValueError, match="makes the norm of up to"):
             ops.gemm_qkv_rope(rand(((q_heads + 2 * kv_heads) * head_dim, hidden), torch.bfloat16, 1), None, None,
                               *([torch.zeros(1, device="cuda")] * 8), q_heads, kv_heads, head_dim,
-                              unsummed=(torch.zeros((rows, hidden), device="cuda"), torch.zeros((1, rows, hidden), device="cuda"),
-                                        torch.ones(hidden, device="cuda"), 1e-6))
+                              folded=(torch.zeros((rows, hidden), device="cuda"), torch.ones(hidden, device="cuda"), 1e-6))
         return
     n = (q_heads + 2 * kv_heads) * head_dim
     eps = 1e-5
-    lengths = [40, 35, 100, 33][:rows]
+    lengths = [40, 35, 100, 33, 64, 1, 17, 90, 41, 36, 101, 34, 65, 2, 18, 91][:rows]
     k_pool, v_pool, table, slots, _ = build_cache(torch.bfloat16, lengths, kv_heads, head_dim, page_size, seed=61)
     k_two, v_two = k_pool.clone(), v_pool.clone()
     positions = [length - 1 for length in lengths]
-    residual = rand((rows, hidden), torch.float32, 62, 2.0)
-    parts = rand((n_parts, rows, hidden), torch.float32, 63, 0.7)
+    residual = rand((rows, hidden), torch.float32, 62, 2.0) * torch.linspace(0.2, 3.0, rows, device="cuda")[:, None]
     norm_weight = (1.0 + rand((hidden,), torch.float32, 64, 0.3)).contiguous()
     w, b = rand((n, hidden), torch.bfloat16, 65, 0.05), rand((n,), torch.bfloat16, 66)
     cos, sin = plain_qwen2.rope_tables(head_dim, 512, 1e6)
@@ -617,13 +614,11 @@ def test_gemm_qkv_rope_that_sums_the_stream_and_makes_the_norm_itself(ops, geome
     meta = (torch.tensor(positions, dtype=torch.int32).cuda(), torch.arange(rows, dtype=torch.int32).cuda(),
             torch.tensor(slots, dtype=torch.int32).cuda(), table)
     before = residual.clone()
-    fused, summed = ops.gemm_qkv_rope(w, None, b, cos, sin, *meta, k_pool, v_pool, q_heads, kv_heads, head_dim,
-                                      waves=waves, unsummed=(residual, parts, norm_weight, eps))
-    assert torch.equal(residual, before) and summed.data_ptr() != residual.data_ptr()  # the stream it read is left alone
-    want_sum = residual.double() + parts.double().sum(0)
-    torch.testing.assert_close(summed.double(), want_sum, rtol=1e-6, atol=1e-5)
-    scale = torch.rsqrt(want_sum.pow(2).mean(-1, keepdim=True) + eps)
-    operand = (summed * norm_weight).to(torch.bfloat16).double()  # the rows as the kernel rounds them
+    fused = ops.gemm_qkv_rope(w, None, b, cos, sin, *meta, k_pool, v_pool, q_heads, kv_heads, head_dim,
+                              waves=waves, folded=(residual, norm_weight, eps))
+    assert torch.equal(residual, before)  # the stream is read only
+    scale = torch.rsqrt(residual.double().pow(2).mean(-1, keepdim=True) + eps)
+    operand = (residual * norm_weight).to(torch.bfloat16).double()  # the rows as the kernel rounds them
     unrotated = ((operand @ w.double().t()) * scale + b.double()).to(torch.bfloat16)
     ops.rope_kv_write(unrotated, cos, sin, *meta, k_two, v_two, q_heads, kv_heads, head_dim)
     q_cols = q_heads * head_dim
@@ -633,7 +628,7 @@ def test_gemm_qkv_rope_that_sums_the_stream_and_makes_the_norm_itself(ops, geome
     torch.testing.assert_close(k_pool.float(), k_two.float(), **step)
     torch.testing.assert_close(v_pool.float(), v_two.float(), **step)
     # ... and it agrees with the two kernels it replaces to the rounding of their different order
-    normed = ops.add_parts_rmsnorm(residual.clone(), parts, norm_weight, eps)
+    normed = ops.add_rmsnorm(residual.clone(), None, norm_weight, eps, torch.bfloat16)
     two = ops.gemm_qkv_rope(w, normed, b, cos, sin, *meta, k_two, v_two, q_heads, kv_heads, head_dim)
     torch.testing.assert_close(fused[:, :q_cols].float(), two[:, :q_cols].float(), rtol=2 ** -5,
                                atol=2 ** -6 * float(unrotated.float().abs().max()))
@@ -812,8 +807,8 @@ def test_gemm_fused_random_shapes(ops):
                                    (128, 96, 328)])
 @pytest.mark.parametrize("k_parts", [1, 3, 4])
 def test_gemm_fused_partial_products_and_their_norm(ops, shape, k_parts):
-    """K cut into parts: the float32 partial products sum to the product (bias once), and the
-    add-parts norm kernel equals adding that product into the residual and normalising."""
+    """K cut into parts: the float32 partial products sum to the product (bias once); and the same parts added
+    into a float32 stream with atomic adds leave the stream plus the product there, twice in a row."""
     m, n, k = shape
     a, w, b = rand((m, k), torch.bfloat16, 94), rand((n, k), torch.bfloat16, 95, 0.3), rand((n,), torch.bfloat16, 96)
     parts = ops.gemm_shared_rows(w, ops.EPI_PARTIAL, a, bias=b, k_parts=k_parts)
@@ -821,17 +816,17 @@ def test_gemm_fused_partial_products_and_their_norm(ops, shape, k_parts):
     exact = a.double() @ w.double().t() + b.double()
     torch.testing.assert_close(parts.double().sum(0), exact, rtol=1e-4, atol=2e-4 * math.sqrt(k))
     residual = rand((m, n), torch.float32, 97, 2.0)
-    weight = rand((n,), torch.bfloat16, 98) + 1
-    want_residual = residual.double() + parts.double().sum(0)
-    want = plain_qwen2.rms_norm(want_residual.float().cpu(), weight.float().cpu(), 1e-6)
-    rows = torch.tensor([m - 1, 0], dtype=torch.int32).cuda()
-    before = residual.clone()
-    picked = ops.add_parts_rmsnorm(residual, parts, weight, 1e-6, rows=rows)
-    assert torch.equal(residual, before)
-    torch.testing.assert_close(picked.float().cpu(), want[rows.long().cpu()], **tol(torch.bfloat16))
-    out = ops.add_parts_rmsnorm(residual, parts, weight, 1e-6)
-    torch.testing.assert_close(residual.double(), want_residual, rtol=1e-5, atol=1e-5)
-    torch.testing.assert_close(out.float().cpu(), want, **tol(torch.bfloat16))
+    before = residual.double()
+    for turn in (1, 2):
+        out = ops.gemm_shared_rows(w, ops.EPI_ATOMIC, a, bias=b, k_parts=k_parts, add_into=residual)
+        assert out is residual
+        torch.testing.assert_close(residual.double(), before + turn * exact, rtol=1e-4, atol=turn * 2e-4 * math.sqrt(k))
+    with pytest.raises(ValueError):
+        ops.gemm_shared_rows(w, ops.EPI_ATOMIC, a, k_parts=k_parts)                       # nothing to add into
+    with pytest.raises(ValueError):
+        ops.gemm_shared_rows(w, ops.EPI_PARTIAL, a, k_parts=k_parts, add_into=residual)   # only the atomic form adds
+    with pytest.raises(ValueError):
+        ops.gemm_shared_rows(w, ops.EPI_ATOMIC, a, k_parts=k_parts, add_into=residual[:, : n - 8])
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

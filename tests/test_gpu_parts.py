@@ -36,7 +36,7 @@ def harness(needs, lengths, page_size=8, dtype=torch.float32):
     from cie_amd.cache import CacheManager
     from cie_amd.engine.device_cache import DeviceCache
 
-    manager = CacheManager(needs, page_size, kv_tokens=512, max_running=4, max_model_len=256)
+    manager = CacheManager(needs, page_size, kv_tokens=512, max_running=max(4, len(lengths)), max_model_len=256)
     device_cache = DeviceCache(manager, dtype, torch.device("cuda:0"))
     for i, n in enumerate(lengths):
         manager.admit(f"r{i}")
@@ -276,7 +276,8 @@ def test_a_mixer_that_norms_its_heads_between_projection_and_rotation(dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_block_part(dtype, rows, part_k, monkeypatch):
     """norm -> mixer -> add -> norm -> feed-forward, the add of the second branch left pending
-    (as a tensor, as partial products, or already done, depending on rows and dtype)."""
+    (as a tensor) or already done (by a product's epilogue, or by the atomic adds of a product whose K is
+    cut into parts), depending on rows and dtype."""
     if part_k is not None:
         from cie_amd.parts import linear
 
@@ -301,11 +302,11 @@ def test_block_part(dtype, rows, part_k, monkeypatch):
     mid = h + plain.attention_layer(a, w, p + "self_attn.", raw, cos, sin, torch.arange(rows))
     m = plain.rms_norm(mid, w[p + "post_attention_layernorm.weight"], 1e-5)
     branch = plain.swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
-    from cie_amd.parts.linear import PartialSum, RowSumsq
+    from cie_amd.parts.linear import Added, RowSumsq
 
-    if isinstance(pending, PartialSum):  # the last product left its K in parts for the next norm to add
-        check(out_residual.cpu(), mid, dtype)
-        check(pending.parts.sum(0).cpu(), branch, dtype)
+    if isinstance(pending, Added):  # the last product's parts of K added their shares into the stream
+        assert part_k is not None and dtype == "bfloat16"
+        check(out_residual.cpu(), mid + branch, dtype)
     elif isinstance(pending, RowSumsq):  # few rows in bfloat16: the fused products added both branches themselves
         check(out_residual.cpu(), mid + branch, dtype)
         check(pending.sumsq.sum(-1).cpu(), (mid + branch).pow(2).sum(-1), dtype)
@@ -314,48 +315,48 @@ def test_block_part(dtype, rows, part_k, monkeypatch):
         check(pending.float().cpu(), branch, dtype)
 
 
-def test_block_whose_first_product_sums_the_pending_parts_of_one_row():
-    """A decode row whose stream still lacks the partial products of the layer before: in bfloat16 the block
-    hands both to its mixer, whose q/k/v product sums them and makes the norm itself.  The stream that comes
-    back is another tensor (the one that went in is left as it was), and everything agrees with the plain
-    block on the summed stream."""
+@pytest.mark.parametrize("rows", [1, 5, 16])
+def test_block_whose_first_product_makes_the_norm_itself(rows, monkeypatch):
+    """Decode rows whose stream is complete (the layer before added its branch itself): in bfloat16 the block
+    hands the stream to its mixer, whose q/k/v product makes the norm of up to 16 rows itself, and no norm
+    kernel runs in front of the mixer.  Everything agrees with the plain block."""
     from cie_amd.config import Qwen2Config
+    from cie_amd.kernels import ops
     from cie_amd.parts.block import PreNormBlock
-    from cie_amd.parts.linear import PartialSum, RowSumsq
+    from cie_amd.parts.linear import Added, RowSumsq
 
     raw = dict(model_type="qwen2", hidden_size=96, num_hidden_layers=1, num_attention_heads=3,
                num_key_value_heads=1, intermediate_size=88, vocab_size=32, rms_norm_eps=1e-5, rope_theta=1e4,
                max_position_embeddings=128)
     block = PreNormBlock(Qwen2Config.from_hf_config(raw).model_spec().layers[0])
-    w = bound(block, "model.layers.0.", "bfloat16", 15, scale=0.3)
+    w = bound(block, "model.layers.0.", "bfloat16", 15, scale=0.2)  # (softmaxes that 16-bit keys still resolve)
     prompt = 12
-    manager, device_cache = harness([block.cache_need()], [prompt + 1], dtype=block.dtype)
+    manager, device_cache = harness([block.cache_need()], [prompt + 1] * rows, dtype=block.dtype)
     g = torch.Generator().manual_seed(16)
-    h = torch.randn((prompt + 1, 96), generator=g)
-    parts = torch.randn((5, 1, 96), generator=g) * 0.4
+    hs = [torch.randn((prompt + 1, 96), generator=g) * (0.5 + 0.25 * i) for i in range(rows)]
     view = device_cache.view(0)
-    block.forward(h[:prompt].clone().cuda(), None, batch_of(manager, [(0, 0, prompt)]), view)
-    manager.commit_lengths({"r0": prompt})
-    last = h[prompt:].clone().cuda()
-    kept = last.clone()
-    out_residual, pending = block.forward(last, PartialSum(parts.cuda()), batch_of(manager, [(0, prompt, 1)]), view)
-    assert out_residual.data_ptr() != last.data_ptr() and torch.equal(last, kept)
-    summed = h.clone()
-    summed[prompt] += parts.sum(0)[0]
+    block.forward(torch.cat([h[:prompt] for h in hs]).cuda(), None,
+                  batch_of(manager, [(i, 0, prompt) for i in range(rows)]), view)
+    manager.commit_lengths({f"r{i}": prompt for i in range(rows)})
+    norms = []
+    real = ops.add_rmsnorm
+    monkeypatch.setattr(ops, "add_rmsnorm", lambda *a, **k: (norms.append(1), real(*a, **k))[1])
+    last = torch.cat([h[prompt:] for h in hs]).cuda()
+    out_residual, pending = block.forward(last, Added(), batch_of(manager, [(i, prompt, 1) for i in range(rows)]), view)
+    assert not norms, "a norm kernel ran although the product could make the norm"
+    assert out_residual.data_ptr() == last.data_ptr()
     p = "model.layers.0."
     cos, sin = plain.rope_tables(32, prompt + 1, 1e4)
-    a = plain.rms_norm(summed, w[p + "input_layernorm.weight"], 1e-5)
-    mid = summed + plain.attention_layer(a, w, p + "self_attn.", raw, cos, sin, torch.arange(prompt + 1))
-    m = plain.rms_norm(mid, w[p + "post_attention_layernorm.weight"], 1e-5)
-    branch = plain.swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
-    if isinstance(pending, PartialSum):
-        check(out_residual.cpu(), mid[prompt:], "bfloat16")
-        check(pending.parts.sum(0).cpu(), branch[prompt:], "bfloat16")
-    elif isinstance(pending, RowSumsq):
-        check(out_residual.cpu(), (mid + branch)[prompt:], "bfloat16")
-    else:
-        check(out_residual.cpu(), mid[prompt:], "bfloat16")
-        check(pending.float().cpu(), branch[prompt:], "bfloat16")
+    for i, h in enumerate(hs):
+        a = plain.rms_norm(h, w[p + "input_layernorm.weight"], 1e-5)
+        mid = h + plain.attention_layer(a, w, p + "self_attn.", raw, cos, sin, torch.arange(prompt + 1))
+        m = plain.rms_norm(mid, w[p + "post_attention_layernorm.weight"], 1e-5)
+        branch = plain.swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        if isinstance(pending, (Added, RowSumsq)):
+            check(out_residual[i: i + 1].cpu(), (mid + branch)[prompt:], "bfloat16")
+        else:
+            check(out_residual[i: i + 1].cpu(), mid[prompt:], "bfloat16")
+            check(pending[i: i + 1].float().cpu(), branch[prompt:], "bfloat16")
 
 
 # -- a toy mixer with state of its own -----------------------------------------------------
