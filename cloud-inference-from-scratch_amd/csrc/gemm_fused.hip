@@ -373,9 +373,11 @@ constexpr int kStageTile = 16 * kStageRow;    // a wave's staging area
 
 constexpr int kFoldRows = 16;      // the most rows whose norm the q/k/v product makes itself: one row tile
 
-template <int WAVES, int EPI, int MT, int NT, bool FOLD = false>
+// FOLD: 0, or the groups of four rows (2 or 4) of the float32 stream from which the rows of A are made (see FusedArgs).
+template <int WAVES, int EPI, int MT, int NT, int FOLD = 0>
 __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
-    static_assert(!FOLD || (MT == 1 && (EPI == EPI_ROPE || EPI == EPI_ROPE8)), "the folded norm: q/k/v of one row tile");
+    static_assert(FOLD == 0 || ((FOLD == 2 || FOLD == 4) && MT == 1 && (EPI == EPI_ROPE || EPI == EPI_ROPE8)),
+                  "the folded norm: q/k/v of one row tile");
     static_assert(EPI != EPI_SILU || NT == 2, "the SiLU epilogue pairs a gate tile with its up tile");
     static_assert(EPI != EPI_ROPE || NT == 2, "the ROPE epilogue pairs the two halves of a head");
     static_assert(EPI != EPI_ROPE8 || NT == 1, "the one-tile ROPE epilogue: one column tile a workgroup");
@@ -390,7 +392,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     __shared__ __attribute__((aligned(16))) char shared[kSharedBytes + 16 * sizeof(float)];  // + the rows' scales
     float* reduce = reinterpret_cast<float*>(shared);
     char* stage = shared + (threadIdx.x / kWave) * kStageTile;
-    __shared__ float fold_sq[FOLD ? WAVES * kFoldRows : 1];  // the waves' shares of the rows' sums of squares
+    __shared__ float fold_sq[FOLD > 0 ? WAVES * kFoldRows : 1];  // the waves' shares of the rows' sums of squares
 
     const int lane = threadIdx.x % kWave;
     const int wave = threadIdx.x / kWave;
@@ -489,7 +491,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
 
     const int k_begin = blockIdx.z * a.k_per_part;
     const int k_end = min(a.K, k_begin + a.k_per_part);
-    float fold_sq_lane = 0.f;  // FOLD: this lane's share of row r's sum of squares
+    float fold_sq_lane[FOLD > 0 ? FOLD : 1] = {};  // FOLD: this lane's share of the sums of squares of rows i * 4 + load_row
     {
 #pragma unroll 1
     for (int kbase = k_begin + wave * 128; kbase < k_end; kbase += U * WAVES * 128) {
@@ -519,33 +521,39 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
             // the few rows of A come from the cache; their loads are issued slice by slice
             const int ka = kbase + u * WAVES * 128;
             uint4 av[MT][4];
-            if constexpr (FOLD) {
-                // lane (r, g) makes row r's k values i*32 + g*8 .. +7 from the float32 stream and the norm's
-                // weight (every load stands unconditionally; what lies past the end is dropped by a select)
-                const float* row = a.fold_residual + static_cast<size_t>(min(m0 + r, a.M - 1)) * a.K;
-                float4 x[4][2], nw[4][2];
+            if constexpr (FOLD > 0) {
+                // The piece of A (16 x 128) made from the float32 stream: sixteen neighbouring lanes read 256 bytes
+                // (64 values) of a row, four rows a load, FOLD such loads for each half of the slice (rows past
+                // the last are not read); times the norm's weight, as bf16 through the wave's staging area into
+                // the operand layout.  Every load stands unconditionally; what lies past an end is dropped by a select.
+                const int lc = lane & 15;
+                float4 x[2][FOLD], nw[2];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int k_read = min(ka + i * 32 + g * 8, a.K - 8);
-                    x[i][0] = *reinterpret_cast<const float4*>(row + k_read);
-                    x[i][1] = *reinterpret_cast<const float4*>(row + k_read + 4);
-                    nw[i][0] = *reinterpret_cast<const float4*>(a.fold_weight + k_read);
-                    nw[i][1] = *reinterpret_cast<const float4*>(a.fold_weight + k_read + 4);
+                for (int cb = 0; cb < 2; ++cb) {
+                    const int k_col = min(ka + cb * 64 + lc * 4, a.K - 4);
+                    nw[cb] = *reinterpret_cast<const float4*>(a.fold_weight + k_col);
+#pragma unroll
+                    for (int i = 0; i < FOLD; ++i)
+                        x[cb][i] = *reinterpret_cast<const float4*>(
+                            a.fold_residual + static_cast<size_t>(min(m0 + i * 4 + load_row, a.M - 1)) * a.K + k_col);
                 }
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const bool inside = row_ok[0][i] && ka + i * 32 + g * 8 < k_end;
-                    const float4 lo = x[i][0], hi = x[i][1];
-                    const float sq = (lo.x * lo.x + lo.y * lo.y) + (lo.z * lo.z + lo.w * lo.w) +
-                                     (hi.x * hi.x + hi.y * hi.y) + (hi.z * hi.z + hi.w * hi.w);
-                    fold_sq_lane += inside ? sq : 0.f;
-                    uint4 packed;
-                    packed.x = pack_bf16(lo.x * nw[i][0].x, lo.y * nw[i][0].y);
-                    packed.y = pack_bf16(lo.z * nw[i][0].z, lo.w * nw[i][0].w);
-                    packed.z = pack_bf16(hi.x * nw[i][1].x, hi.y * nw[i][1].y);
-                    packed.w = pack_bf16(hi.z * nw[i][1].z, hi.w * nw[i][1].w);
-                    av[0][i] = inside ? packed : uint4{0, 0, 0, 0};
-                }
+                for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                    for (int i = 0; i < FOLD; ++i) {
+                        const bool inside = m0 + i * 4 + load_row < a.M && ka + cb * 64 + lc * 4 < k_end;
+                        const float4 v = x[cb][i];
+                        fold_sq_lane[i] += inside ? (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w) : 0.f;
+                        uint2 packed;
+                        packed.x = pack_bf16(v.x * nw[cb].x, v.y * nw[cb].y);
+                        packed.y = pack_bf16(v.z * nw[cb].z, v.w * nw[cb].w);
+                        *reinterpret_cast<uint2*>(stage + (i * 4 + load_row) * kStageRow + (cb * 64 + lc * 4) * 2) =
+                            inside ? packed : uint2{0u, 0u};
+                    }
+#pragma unroll
+                for (int j = 0; j < 4; ++j)  // (rows the loads left out hold what the piece before left: not used)
+                    av[0][j] = r < 4 * FOLD ? *reinterpret_cast<const uint4*>(stage + r * kStageRow + j * 64 + g * 16)
+                                            : uint4{0, 0, 0, 0};
             } else {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
@@ -603,10 +611,16 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
             for (int i = 0; i < 4; ++i) row_scale[i] = scale_lds[g * 4 + i];
         }
     }
-    if constexpr (FOLD) {  // row r's sum of squares over this wave's slices: the lanes r, r + 16, r + 32, r + 48 hold it
-        fold_sq_lane += __shfl_xor(fold_sq_lane, 16, kWave);
-        fold_sq_lane += __shfl_xor(fold_sq_lane, 32, kWave);
-        if (lane < 16) fold_sq[wave * kFoldRows + lane] = fold_sq_lane;
+    if constexpr (FOLD > 0) {  // the rows' sums of squares over this wave's slices: sixteen lanes hold a row's
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float v = i < FOLD ? fold_sq_lane[i < FOLD ? i : 0] : 0.f;
+            v += __shfl_xor(v, 1, kWave);
+            v += __shfl_xor(v, 2, kWave);
+            v += __shfl_xor(v, 4, kWave);
+            v += __shfl_xor(v, 8, kWave);
+            if ((lane & 15) == 0) fold_sq[wave * kFoldRows + i * 4 + load_row] = v;
+        }
     }
     // With more than one row tile the waves share the end of the work: row tile mt belongs to wave
     // mt % WAVES, which sums the other waves' partial tiles of that row tile and stores it (one wave
@@ -692,7 +706,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
                 store_resid(a, acc[0][t], resid_rows[t], m0, (tile_first + t) * 16 + r, tile_first + t, lane);
         return;
     }
-    if constexpr (FOLD) {  // the rows' 1/rms, which the rows of A were made without
+    if constexpr (FOLD > 0) {  // the rows' 1/rms, which the rows of A were made without
         // (wave 0, behind the barrier above if there are more; with one wave its LDS operations keep their order)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -721,7 +735,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_rows_kernel(FusedArgs a) {
     }
 }
 
-template <int EPI, int MT, int NT, bool FOLD = false>
+template <int EPI, int MT, int NT, int FOLD = 0>
 int launch_waves(hipStream_t s, int waves, dim3 grid, const FusedArgs& a) {
     if constexpr (MT == 1) {
         switch (waves) {
@@ -1122,8 +1136,12 @@ int qkv_rope(void* stream, const void* a, int lda, const void* w, const void* bi
         f.fold_residual = fold->residual;
         f.fold_weight = fold->weight;
         f.eps = fold->eps;
-        if (one_tile) return launch_waves<EPI_ROPE8, 1, 1, true>(s, waves, twice, f);
-        return launch_waves<EPI_ROPE, 1, 2, true>(s, waves, grid, f);
+        if (M <= 8) {
+            if (one_tile) return launch_waves<EPI_ROPE8, 1, 1, 2>(s, waves, twice, f);
+            return launch_waves<EPI_ROPE, 1, 2, 2>(s, waves, grid, f);
+        }
+        if (one_tile) return launch_waves<EPI_ROPE8, 1, 1, 4>(s, waves, twice, f);
+        return launch_waves<EPI_ROPE, 1, 2, 4>(s, waves, grid, f);
     }
     if (one_tile) return launch_waves<EPI_ROPE8, 1, 1>(s, waves, twice, f);
     if (M <= 64 && grid.x < kSplitPairsBelow) {  // the same with more row tiles

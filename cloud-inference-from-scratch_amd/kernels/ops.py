@@ -653,23 +653,17 @@ QKV_SPLIT_PAIRS_BELOW = 128  # (as in the kernel library: below this many pairs 
 
 
 FOLDED_NORM_ROWS = 16      # the most rows whose norm the q/k/v product makes itself: one tile of rows
-# ... and the most values (rows x K) for which that is the faster way: every workgroup of the product makes
-# the rows anew, which costs it 1.8 to 2.8 us with the 3B shape's width and 4 to 6 us with the 14B shape's, where the
-# norm's own kernel takes 3.6 us (norm + product against the product that makes its norm, us: 3B 1 / 8 / 16 rows
-# 8.9 / 10.5 / 10.7 against 7.6 / 9.7 / 10.9; 7B 13.4 / 15.3 / 16.6 against 12.4 / 15.5 / 17.8; 14B 21.3 / 22.3 /
-# 23.4 against 21.4 / 24.7 / 27.5; 0.5B 7.0 / 8.4 / 8.5 against 6.3 / 8.1 / 9.3)
-FOLDED_NORM_VALUES = 16384
-FOLDED_NORM_WIDTH = 4096
+# (norm kernel + product against the product that makes its norm, us in a captured chain: 3B shape 1 / 8 / 16 rows
+# 9.0 / 10.6 / 10.9 against 7.1 / 7.9 / 8.9; 7B 13.3 / 15.2 / 16.0 against 11.3 / 12.8 / 14.2; 14B 21.1 / 22.3 /
+# 23.4 against 18.9 / 20.2 / 22.0; 0.5B 7.0 / 8.3 / 8.5 against 5.7 / 6.6 / 7.4.  Every workgroup makes the rows
+# anew, which costs it about 1 us: the rows are read in whole 256-byte segments, four rows a load, and pass through
+# the wave's staging area; with every lane reading the values of its own matrix operand it cost 2 to 6 us and lost
+# from the 7B width on.)
 
 
 def folds_norm(rows: int, k: int) -> bool:
     """Whether ``gemm_qkv_rope`` takes ``folded=`` for this many rows of ``k`` values."""
     return 1 <= rows <= FOLDED_NORM_ROWS and k >= 8 and k % 8 == 0
-
-
-def folding_norm_pays(rows: int, k: int) -> bool:
-    """Whether the product that makes its norm is the faster way for this many rows of ``k`` values."""
-    return folds_norm(rows, k) and rows * k <= FOLDED_NORM_VALUES and k <= FOLDED_NORM_WIDTH
 
 
 def gemm_qkv_rope(weight: torch.Tensor, a: Optional[torch.Tensor], bias: Optional[torch.Tensor], cos: torch.Tensor,

@@ -148,7 +148,7 @@ class RawRows:
     @staticmethod
     def fits(residual: torch.Tensor, dtype: torch.dtype) -> bool:
         rows, width = residual.shape
-        return dtype == torch.bfloat16 and residual.is_cuda and ops.folding_norm_pays(rows, width)
+        return dtype == torch.bfloat16 and residual.is_cuda and ops.folds_norm(rows, width)
 
     @property
     def shape(self):
