@@ -3,8 +3,8 @@
 (default: the 3B one) with random weights, plus prefill and roofline figures.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
-                    [--shape 0.5b|3b|7b|14b|32b|72b] [--layers N] [--long-contexts 16384,32768]
-                    [--mixed-portions 16,64,248]
+                    [--shape 0.5b|3b|7b|14b|32b|72b] [--layers N] [--long-contexts 32768]
+                    [--mixed-portions 16,64,248] [--other-shapes 7b,14b]
 
 A "step" is one decode step of the whole engine (scheduler iteration: plan,
 step function, sampling, token hand-over).  Protocol after the reference's
@@ -21,9 +21,12 @@ states ("2,048-token prefill, then decode to 4,096").  The whole range is
 measured beside it (``range``): prompts of ``--prefill-tokens``, then every
 decode step up to ``--context``, one warm-up run and three measured ones.
 ``prefill`` is one prompt of ``--prefill-tokens`` run to its first token.
-``--mixed-portions`` adds the time of the steps that chunked serving meets: the
-batch's decode tokens beside one portion of a further prompt (``mixed``).
-ONE JSON line is printed.
+``mixed`` is the time of the steps that chunked serving meets: the batch's decode
+tokens beside one portion of a further prompt (``--mixed-portions``).  ``points``
+holds decode at batch 1 and 64, at the main batch behind ``--long-contexts``
+tokens, and, for the ``--other-shapes`` of the family, decode at the main batch
+and context and the prefill, each with its share of the roofline in
+``points_frac`` (the bytes and flops of its own shape).  ONE JSON line is printed.
 """
 
 from __future__ import annotations
@@ -229,9 +232,11 @@ def main(argv=None) -> int:
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--no-range", action="store_true", help="skip the run over the whole range of contexts")
-    parser.add_argument("--long-contexts", default="", help="further decode points of the main batch, e.g. 16384,32768")
-    parser.add_argument("--mixed-portions", default="",
-                        help="also time steps of the batch's decode tokens beside a prompt portion of these sizes, e.g. 16,64,248")
+    parser.add_argument("--long-contexts", default="32768", help="further decode points of the main batch, e.g. 16384,32768")
+    parser.add_argument("--mixed-portions", default="16,64,248",
+                        help="also time steps of the batch's decode tokens beside a prompt portion of these sizes ('' for none)")
+    parser.add_argument("--other-shapes", default="7b,14b",
+                        help="further shapes whose decode at the main batch and context and whose prefill go into the points ('' for none)")
     args = parser.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not run (this engine is single-GPU)")
@@ -257,10 +262,10 @@ def main(argv=None) -> int:
     def say(text: str) -> None:
         print(f"[bench] {text}", file=sys.stderr, flush=True)
 
-    def point(batch: int, context: int):
+    def point(batch: int, context: int, config=config, layers=layers, label: str = ""):
         """(tokens/s of each measured window, the median window's ms per step and roofline share)."""
         context = min(context, config.max_position_embeddings - SLACK)  # (the last positions are the slack's)
-        say(f"decode, batch {batch}, context {context}")
+        say(f"decode{label}, batch {batch}, context {context}")
         engine = make_engine(config, args.dtype, batch, context, args.prefill_tokens)
         measured = decode_windows(engine, config, batch, context, steps, warmup, seed=batch)
         del engine
@@ -269,6 +274,15 @@ def main(argv=None) -> int:
         seconds, mean_context = sorted(measured)[len(measured) // 2]
         achieved = decode_bytes(config, layers, batch, mean_context, elem) / (seconds / steps) / 1e9
         return rates, seconds / steps * 1e3, achieved
+
+    def prefill_point(config=config, layers=layers, label: str = ""):
+        """(seconds of each measured run, the step's flops) of one prompt run to its first token."""
+        say(f"prefill{label} of {args.prefill_tokens} tokens")
+        engine = make_engine(config, args.dtype, 1, args.prefill_tokens + 1, args.prefill_tokens)
+        seconds = time_prefill(engine, config, args.prefill_tokens, seed=99)
+        del engine
+        release()
+        return seconds, prefill_flops(config, layers, args.prefill_tokens)
 
     rates, ms_per_step, achieved = point(args.batch, args.context)
     name = f"Qwen2.5-{args.shape.upper()} shape"
@@ -317,13 +331,8 @@ def main(argv=None) -> int:
             "ms_per_step": round(seconds / n * 1e3, 4), "frac": round(through / HBM_GBPS, 4),
         }
     if not args.no_prefill:
-        say(f"prefill of {args.prefill_tokens} tokens")
-        engine = make_engine(config, args.dtype, 1, args.prefill_tokens + 1, args.prefill_tokens)
-        seconds = time_prefill(engine, config, args.prefill_tokens, seed=99)
-        del engine
-        release()
+        seconds, flops = prefill_point()
         median = statistics.median(seconds)
-        flops = prefill_flops(config, layers, args.prefill_tokens)
         line["prefill"] = {
             "value": round(args.prefill_tokens / median, 1), "tokens": args.prefill_tokens,
             "ms": round(median * 1e3, 3), "frac": round(flops / median / PEAK_FLOPS[args.dtype], 4),
@@ -342,8 +351,26 @@ def main(argv=None) -> int:
         points[key] = round(statistics.median(rates), 2)
         fractions[key] = round(achieved / HBM_GBPS, 4)
         all_runs[key] = [round(r, 2) for r in rates]
+    # other shapes of the family, whole, at the main batch and context: their own bytes and flops
+    if not args.no_points and args.layers is None:
+        for other in [name for name in args.other_shapes.split(",") if name and name != args.shape]:
+            other_shape = SHAPES[other]
+            other_layers = other_shape["num_hidden_layers"]
+            other_config = Qwen2Config.from_hf_config(dict(other_shape))
+            rates, _, achieved = point(args.batch, args.context, other_config, other_layers, f" ({other} shape)")
+            key = f"decode_b{args.batch}_{other}"
+            points[key] = round(statistics.median(rates), 2)
+            fractions[key] = round(achieved / HBM_GBPS, 4)
+            all_runs[key] = [round(r, 2) for r in rates]
+            if not args.no_prefill:
+                seconds, flops = prefill_point(other_config, other_layers, f" ({other} shape)")
+                median = statistics.median(seconds)
+                key = f"prefill_{args.prefill_tokens}_{other}"
+                points[key] = round(args.prefill_tokens / median, 1)
+                fractions[key] = round(flops / median / PEAK_FLOPS[args.dtype], 4)
+                all_runs[key] = [round(args.prefill_tokens / s, 1) for s in seconds]
     portions = [int(c) for c in args.mixed_portions.split(",") if c]
-    if portions:
+    if portions and not args.no_points:
         say(f"steps of {args.batch} decode tokens beside a prompt portion of {portions}")
         longest = max(portions)
         engine = make_engine(config, args.dtype, args.batch + 1, max(args.context, 64 * longest), args.prefill_tokens)

@@ -23,7 +23,7 @@ def test_more_than_one_gpu_is_said_and_refused():
 def test_one_json_line_with_the_agreed_fields():
     """A short run of one layer of the default shape: the line's fields, and that its figures follow from one another."""
     command = [sys.executable, str(ROOT / "bench.py"), "--gpus", "1", "--steps", "4", "--warmup", "1", "--layers", "1",
-               "--context", "256", "--prefill-tokens", "64", "--mixed-portions", "6,20"]
+               "--context", "256", "--prefill-tokens", "64", "--mixed-portions", "6,20", "--long-contexts", ""]
     done = subprocess.run(command, capture_output=True, text=True, timeout=600)
     assert done.returncode == 0, done.stderr[-3000:]
     lines = done.stdout.strip().splitlines()
