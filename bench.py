@@ -233,8 +233,9 @@ def main(argv=None) -> int:
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--no-range", action="store_true", help="skip the run over the whole range of contexts")
     parser.add_argument("--long-contexts", default="32768", help="further decode points of the main batch, e.g. 16384,32768")
-    parser.add_argument("--mixed-portions", default="16,64,248",
-                        help="also time steps of the batch's decode tokens beside a prompt portion of these sizes ('' for none)")
+    parser.add_argument("--mixed-portions", default=None,
+                        help="also time steps of the batch's decode tokens beside a prompt portion of these sizes "
+                             "(default 16,64,248; '' for none, as with --no-points)")
     parser.add_argument("--other-shapes", default="7b,14b",
                         help="further shapes whose decode at the main batch and context and whose prefill go into the points ('' for none)")
     args = parser.parse_args(argv)
@@ -369,8 +370,9 @@ def main(argv=None) -> int:
                 points[key] = round(args.prefill_tokens / median, 1)
                 fractions[key] = round(flops / median / PEAK_FLOPS[args.dtype], 4)
                 all_runs[key] = [round(args.prefill_tokens / s, 1) for s in seconds]
-    portions = [int(c) for c in args.mixed_portions.split(",") if c]
-    if portions and not args.no_points:
+    mixed_portions = args.mixed_portions if args.mixed_portions is not None else ("" if args.no_points else "16,64,248")
+    portions = [int(c) for c in mixed_portions.split(",") if c]
+    if portions:
         say(f"steps of {args.batch} decode tokens beside a prompt portion of {portions}")
         longest = max(portions)
         engine = make_engine(config, args.dtype, args.batch + 1, max(args.context, 64 * longest), args.prefill_tokens)

@@ -184,7 +184,9 @@ class DecodeGraphs:
         if rows == list(range(len(entries))):
             view = bucket.logits[: len(entries)]
             return view if borrow else view.clone()
-        return bucket.logits[torch.tensor(rows, dtype=torch.long, device=runner.device)]
+        # (the index goes over as an asynchronous copy: a tensor made on the device from a list would wait for the replay)
+        index = to_device_staging(rows, runner.device).to(runner.device, non_blocking=True).long()
+        return bucket.logits.index_select(0, index)
 
 
 @dataclass
@@ -199,6 +201,9 @@ class _CapturedStep:
     batch: StepBatch
     graph: Any = None
     logits: torch.Tensor | None = None
+    # which rows of ``logits`` a step's entries want, as index tensors on the device, by the rows' numbers: made
+    # once each (a tensor made on the device from a host list waits for the stream, that is for the replay)
+    wanted_rows: dict = None
 
 
 class MixedGraphs:
@@ -297,7 +302,7 @@ class MixedGraphs:
             host_slots=[pad] * sequences, host_starts=[0] * sequences, host_q_lens=q_lens,
             static_plan=StaticPlan(None, None, view("max_context", 1), bound, decode_rows=decode_rows),
         )
-        return _CapturedStep(decode_rows, portions, host, dev, offsets, batch)
+        return _CapturedStep(decode_rows, portions, host, dev, offsets, batch, wanted_rows={})
 
     def _fill(self, step: _CapturedStep, single: Sequence[Any], portions: Sequence[Any]) -> None:
         """Real single-token rows first, padding up to the bucket (token 0 at position 0 of the pad slot),
@@ -373,5 +378,11 @@ class MixedGraphs:
         self.replays += 1
         row_of = {id(e): index for index, e in enumerate(single)}
         row_of.update({id(e): step.decode_rows + index for index, e in enumerate(portions)})
-        rows = [row_of[id(e)] for e in entries for _ in e.want]
-        return step.logits[torch.tensor(rows, dtype=torch.long, device=self.runner.device)]
+        rows = tuple(row_of[id(e)] for e in entries for _ in e.want)
+        index = step.wanted_rows.get(rows)
+        if index is None:
+            if len(step.wanted_rows) > 64:
+                step.wanted_rows.clear()
+            index = step.wanted_rows[rows] = to_device_staging(list(rows), self.runner.device).to(
+                self.runner.device, non_blocking=True).long()
+        return step.logits.index_select(0, index)
