@@ -232,7 +232,8 @@ def main(argv=None) -> int:
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points")
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--no-range", action="store_true", help="skip the run over the whole range of contexts")
-    parser.add_argument("--long-contexts", default="32768", help="further decode points of the main batch, e.g. 16384,32768")
+    parser.add_argument("--long-contexts", default=None,
+                        help="further decode points of the main batch, e.g. 16384,32768 (default: 32768; none with --no-points)")
     parser.add_argument("--mixed-portions", default=None,
                         help="also time steps of the batch's decode tokens beside a prompt portion of these sizes "
                              "(default 16,64,248; '' for none, as with --no-points)")
@@ -346,7 +347,8 @@ def main(argv=None) -> int:
             points[f"decode_b{batch}"] = round(statistics.median(rates), 2)
             fractions[f"decode_b{batch}"] = round(achieved / HBM_GBPS, 4)
             all_runs[f"decode_b{batch}"] = [round(r, 2) for r in rates]
-    for context in [int(c) for c in args.long_contexts.split(",") if c]:
+    long_contexts = args.long_contexts if args.long_contexts is not None else ("" if args.no_points else "32768")
+    for context in [int(c) for c in long_contexts.split(",") if c]:
         rates, _, achieved = point(args.batch, context)
         key = f"decode_b{args.batch}_ctx{context}"
         points[key] = round(statistics.median(rates), 2)

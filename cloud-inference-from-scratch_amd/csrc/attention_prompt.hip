@@ -311,7 +311,9 @@ __global__ void __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) paged_attentio
             // ---- running maxima; masks only in blocks that reach a row's edge
             const bool edge = kb + kKeysPerBlock - 1 > wave_first_pos || kb + kKeysPerBlock > range_end ||
                               (a.window > 0 && kb < wave_last_pos + 1 - a.window);
-            float m_use[RT];
+            // A row's reference moves only if one of its scores passes it by the margin, and each of the row's four
+            // lanes can tell that of its own eight scores: the common block needs no maximum across lanes at all.
+            float own_max[RT];
             bool moved = false;
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -327,22 +329,21 @@ __global__ void __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) paged_attentio
                             if (!(key <= pos && key >= row_lo)) s[rt][kt][i] = -INFINITY;
                         }
                 }
-                float block_max = max3(max3(s[rt][0][0], s[rt][0][1], s[rt][0][2]),
-                                       max3(s[rt][0][3], s[rt][1][0], s[rt][1][1]),
-                                       max3(s[rt][1][2], s[rt][1][3], s[rt][1][3]));
-                block_max = rows_max_lean(block_max) * scale_log2;  // maxima are kept in scaled base-2 units
-                const bool passes = block_max > m_run[rt] + kLazyRescale;
-                moved = moved || passes;
-                m_use[rt] = passes ? block_max : m_run[rt];
+                own_max[rt] = max3(max3(s[rt][0][0], s[rt][0][1], s[rt][0][2]),
+                                   max3(s[rt][0][3], s[rt][1][0], s[rt][1][1]),
+                                   max3(s[rt][1][2], s[rt][1][3], s[rt][1][3]));
+                moved = moved || own_max[rt] * scale_log2 > m_run[rt] + kLazyRescale;  // (the scale is positive)
             }
             if (__any(moved)) {
                 // some row's reference moves (rare once the first blocks have set every row's scale): what the
                 // row has summed so far is scaled down to the new reference
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    const float m_safe = (m_use[rt] == -INFINITY) ? 0.f : m_use[rt];
+                    const float block_max = rows_max_lean(own_max[rt]) * scale_log2;  // maxima are kept in scaled base-2 units
+                    const float m_new = (block_max > m_run[rt] + kLazyRescale) ? block_max : m_run[rt];
+                    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
                     const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_safe);  // m_run = -inf: 0, and the sums are 0 anyway
-                    m_run[rt] = m_use[rt];
+                    m_run[rt] = m_new;
                     float alpha_o[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha, g * 4 + i, kWave);
