@@ -998,6 +998,10 @@ int launch_shared_rows_waves(hipStream_t s, int k_parts, const FusedArgs& a) {
     if (a.M <= 16) return launch_shared_rows_tiles<EPI, 1, NT, WAVES>(s, grid, a);
     if (a.M <= 32) return launch_shared_rows_tiles<EPI, 2, NT, WAVES>(s, grid, a);
     if (a.M <= 64) return launch_shared_rows_tiles<EPI, 4, NT, WAVES>(s, grid, a);
+    // 65 to 96 rows (single tokens beside a prompt portion of 64): six row tiles instead of eight for the epilogues
+    // that the engine's steps meet there (a thread fetches and stores six pieces of the rows a slice instead of eight)
+    if constexpr (EPI == EPI_ATOMIC || EPI == EPI_SILU || EPI == EPI_F32)
+        if (a.M <= 96) return launch_shared_rows_tiles<EPI, 6, NT, WAVES>(s, grid, a);
     return launch_shared_rows_tiles<EPI, 8, NT, WAVES>(s, grid, a);
 }
 

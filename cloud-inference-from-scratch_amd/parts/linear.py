@@ -29,12 +29,11 @@ from ..kernels import ops
 # is long and is cut into parts (the down product: 17-20 us against the library's 27-32 us); its gate/up
 # product loses from 32 rows on (34 us against 26 + 5 us at 64 rows: every workgroup re-reads the rows of A).
 FUSED_ROWS = 16
-FUSED_PARTS_ROWS = 64
-# ... and up to 128 rows where the weight has few columns, which leave the library few tiles to spread (a step
-# of 72 rows: 3B shape, 128 column tiles, 4.38 -> 4.17 ms; 7B, 224 tiles, 7.5 -> 6.4 ms; 14B, 320 tiles,
-# 10.8 -> 11.6 ms: there the library stays)
-FUSED_PARTS_ROWS_NARROW = 128
-PARTS_NARROW_TILES = 256
+# ... and up to 128 rows (the down product alone, weight from memory, own kernel against the library, us: 3B shape at
+# 72 / 96 / 128 rows 18.3 / 19.9 / 24.2 against 27.7 / 28.4 / 28.4; 7B 41.6 / 45.8 / 54.4 against 96 / 95 / 84; 14B
+# 36.3 / 39.8 / 48.2 against 50.0 / 61.6 / 60.9: the library has no good algorithm for a long K and few rows, and at
+# row counts that do not recur it takes its heuristic's first choice)
+FUSED_PARTS_ROWS = 128
 # With 17 to 128 rows it also wins where the weight is small (q/k/v and o_proj of the 3B shape: 7-9 us against
 # the library's 12-18 us inside a step at up to 64 rows, 9.3 and 8.2 us against 9.5-12.4 and 9.1 us at 72 and 128
 # rows, where the weight is streamed twice; and the rotation, the cache write, the residual add and the next
@@ -54,9 +53,11 @@ PART_K = 1024           # the shortest stretch of K a part takes
 
 # SiLU-gate products of up to this many rows take the form whose waves own columns and share the rows of A
 # through LDS (gate/up of the 3B shape at 32 / 64 rows: 21 / 24 us against the library's 26 / 27 us and 5 us
-# for the SiLU kernel behind it; 14B: 50 / 56 against 55 / 62 + 6; 7B: level); from 65 rows on the library is
-# level or ahead (3B at 128 rows: 34 against 30 + 5 us).
-SHARED_SILU_ROWS = 64
+# for the SiLU kernel behind it; 14B: 50 / 56 against 55 / 62 + 6; 7B: level); from 65 to 96 rows, on six row tiles
+# (3B / 7B / 14B at 72 rows: 28.3 / 67.7 / 63.7 us against 31.4 / 75.2 / 70.4 for the library and its SiLU kernel,
+# at 96 rows 29.6 / 69.6 / 65.0 against 32.2 / 71.1 / 64.6); beyond that the library is level or ahead (3B at 128
+# rows: 35 against 30 + 5 us; 7B: 111 against 66).
+SHARED_SILU_ROWS = 96
 # float32 logits take that form up to this many rows (the head of the 3B / 7B / 14B shape, us: 64 rows 156 against
 # 173 in the form whose waves share K; 72 rows 165 / 239 / 333 against the library's 174 / 249 / 349; 96 rows
 # 172 / 255 / 346 against 174 / 238 / 338)
@@ -216,7 +217,7 @@ def linear(x: Union[torch.Tensor, ScaledRows], weight: torch.Tensor, bias: Optio
     fusable = _fusable(rows, k, x.stride(0) if rows > 1 else k, weight)
     cut_k = (into is not None and -(-n // 16) < PART_BELOW_TILES and k >= PART_MIN_K and into.is_contiguous()
              and tuple(into.shape) == (rows, n))
-    if fusable and cut_k and rows <= (FUSED_PARTS_ROWS_NARROW if -(-n // 16) < PARTS_NARROW_TILES else FUSED_PARTS_ROWS):
+    if fusable and cut_k and rows <= FUSED_PARTS_ROWS:
         # (atomic adds cost the product nothing, measured against partial products written for the next norm
         # kernel to sum: 10.3 us either way for the 3B shape's down product at 8 rows; and the kernel that summed
         # them falls away)
