@@ -12,6 +12,7 @@ switches, scale, position encoding and an optional window are parameters.
 from __future__ import annotations
 
 import math
+import warnings
 from typing import Optional
 
 import torch
@@ -47,9 +48,17 @@ class Attention(Part):
         self.window = window
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.position = build_part("position", position)
+        # A head size that the matrix-core attention does not take (80, 112, 40, ...) runs as the next one it does:
+        # the projections' rows of a head are padded with zero rows, which changes no score and no output (the keys'
+        # and values' extra dimensions are zeros in the cache, o_proj's extra columns are zeros), and costs that much
+        # more cache.  The generic kernel, which takes every size, is 20 (decode) to 180 (a 2,048-token prompt) times
+        # slower.  A variant that works on the projected heads (``shape_projection``) sees the heads as they are.
+        self.kernel_head_dim = head_dim
+        if type(self).shape_projection is Attention.shape_projection:
+            self.kernel_head_dim = next((size for size in ops.MFMA_HEAD_DIMS if size >= head_dim), head_dim)
 
     def cache_need(self) -> PagedKV:
-        return PagedKV(self.num_kv_heads, self.head_dim, self.window)
+        return PagedKV(self.num_kv_heads, self.kernel_head_dim, self.window)
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
         q_out = self.num_heads * self.head_dim
@@ -71,19 +80,30 @@ class Attention(Part):
     def bind(self, tensors, prefix, dtype, device) -> None:
         super().bind(tensors, prefix, dtype, device)
         names = ("q_proj", "k_proj", "v_proj")
-        self.w_qkv = torch.cat([tensors[f"{prefix}{n}.weight"] for n in names], dim=0).contiguous()
+        extra = self.kernel_head_dim - self.head_dim
+
+        def per_head(t: torch.Tensor) -> torch.Tensor:
+            # [heads * head_dim, ...] -> [heads * kernel_head_dim, ...], each head followed by zero rows
+            if not extra:
+                return t
+            heads = t.shape[0] // self.head_dim
+            padded = t.new_zeros((heads, self.kernel_head_dim) + tuple(t.shape[1:]))
+            padded[:, : self.head_dim] = t.reshape((heads, self.head_dim) + tuple(t.shape[1:]))
+            return padded.reshape((heads * self.kernel_head_dim,) + tuple(t.shape[1:]))
+
+        self.w_qkv = torch.cat([per_head(tensors[f"{prefix}{n}.weight"]) for n in names], dim=0).contiguous()
         self.b_qkv = (
-            torch.cat([tensors[f"{prefix}{n}.bias"] for n in names], dim=0).contiguous()
+            torch.cat([per_head(tensors[f"{prefix}{n}.bias"]) for n in names], dim=0).contiguous()
             if self.qkv_bias else None
         )
-        self.w_o = tensors[prefix + "o_proj.weight"].contiguous()
+        self.w_o = per_head(tensors[prefix + "o_proj.weight"].t()).t().contiguous()
         self.b_o = tensors[prefix + "o_proj.bias"].contiguous() if self.out_bias else None
         self.cos, self.sin = self.position.tables(device)
 
     def warm_up(self, rows: int) -> None:
         blank = lambda width: torch.zeros((rows, width), dtype=self.w_qkv.dtype, device=self.w_qkv.device)
         linear(blank(self.hidden_size), self.w_qkv, self.b_qkv)
-        linear(blank(self.num_heads * self.head_dim), self.w_o, self.b_o)
+        linear(blank(self.num_heads * self.kernel_head_dim), self.w_o, self.b_o)
 
     def shape_projection(self, qkv: torch.Tensor, batch) -> torch.Tensor:
         """The seam between projection and rotation: what a variant of this mixer does to the projected
@@ -101,35 +121,36 @@ class Attention(Part):
             )
         rows = x.shape[0]
         few = rows <= FUSED_ROWS or (rows <= FUSED_SMALL_ROWS and self.w_qkv.numel() <= FUSED_SMALL_WEIGHT)
+        head_dim = self.kernel_head_dim  # what the kernels and the cache see
         # the projection's own kernel rotates whole heads only, and only an untouched projection
         rotary_dim = getattr(self.position, "rotary_dim", self.head_dim) if self.position.rotates else None
         untouched = (type(self).shape_projection is Attention.shape_projection
-                     and rotary_dim in (None, self.head_dim))
+                     and rotary_dim in (None, head_dim) and head_dim == self.head_dim)
         if isinstance(x, RawRows):
-            if untouched and self.head_dim % 32 == 0 and self.w_qkv.dtype == torch.bfloat16:
+            if untouched and head_dim % 32 == 0 and self.w_qkv.dtype == torch.bfloat16:
                 # the product makes the norm of its rows itself
                 qkv = ops.gemm_qkv_rope(
                     self.w_qkv, None, self.b_qkv, self.cos, self.sin, batch.positions, batch.seq_of_token,
                     batch.seq_slot, view.block_table, view.k_pool, view.v_pool, self.num_heads, self.num_kv_heads,
-                    self.head_dim, rotate=self.position.rotates, write_kv=writes,
+                    head_dim, rotate=self.position.rotates, write_kv=writes,
                     folded=(x.residual, x.norm.weight_f32, x.norm.eps))
-                context = attend(qkv, batch, view, self.num_heads, self.num_kv_heads, self.head_dim,
+                context = attend(qkv, batch, view, self.num_heads, self.num_kv_heads, head_dim,
                                  self.window, self.scale)
                 return linear(context, self.w_o, self.b_o, into=residual, then_norm=next_norm)
             x = x.complete()
-        if (x.dtype == torch.bfloat16 and few and untouched and self.head_dim % 32 == 0
+        if (x.dtype == torch.bfloat16 and few and untouched and head_dim % 32 == 0
                 and x.shape[1] % 8 == 0 and (rows == 1 or x.stride(0) % 8 == 0)):
             # few rows (where the hand-written product is the faster one): its epilogue rotates and writes the cache
             qkv = ops.gemm_qkv_rope(self.w_qkv, x, self.b_qkv, self.cos, self.sin, batch.positions,
                                     batch.seq_of_token, batch.seq_slot, view.block_table, view.k_pool, view.v_pool,
-                                    self.num_heads, self.num_kv_heads, self.head_dim,
+                                    self.num_heads, self.num_kv_heads, head_dim,
                                     rotate=self.position.rotates, write_kv=writes)
         else:
             qkv = self.shape_projection(linear(x, self.w_qkv, self.b_qkv), batch)
             ops.rope_kv_write(qkv, self.cos, self.sin, batch.positions, batch.seq_of_token, batch.seq_slot,
                               view.block_table, view.k_pool, view.v_pool, self.num_heads, self.num_kv_heads,
-                              self.head_dim, rotate=self.position.rotates, write_kv=writes, rotary_dim=rotary_dim)
-        context = attend(qkv, batch, view, self.num_heads, self.num_kv_heads, self.head_dim,
+                              head_dim, rotate=self.position.rotates, write_kv=writes, rotary_dim=rotary_dim)
+        context = attend(qkv, batch, view, self.num_heads, self.num_kv_heads, head_dim,
                          self.window, self.scale)
         return linear(context, self.w_o, self.b_o, into=residual, then_norm=next_norm)
 
@@ -152,6 +173,9 @@ PROMPT_SPLIT_KEYS = 512  # the fewest keys of a part when a prompt portion's key
 # tokens 108 -> 64, 138 -> 75, 182 -> 111.
 EIGHT_WAVE_TILES = 0.75  # of the compute units
 LARGE_TILES_ABOVE = 1.0  # tiles of 128 rows x kv heads (as a share of the compute units) above which that form takes them
+
+
+_SAID_GENERIC: set = set()  # geometries whose bfloat16 attention was sent to the generic kernel, each said once
 
 
 def plan_splits(units: int, max_keys: int, target_waves: int = 1024, min_keys: int = 128) -> tuple[int, int]:
@@ -180,6 +204,13 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     cus = ops.compute_units()  # compute units of the GPU
     if (qkv.dtype != torch.bfloat16 or head_dim not in ops.MFMA_HEAD_DIMS or group > 16 or page_size < 4
             or page_size & (page_size - 1)):
+        if qkv.dtype == torch.bfloat16 and (head_dim, group, page_size) not in _SAID_GENERIC:
+            # right, and many times slower than the matrix-core forms: said once per geometry, not silently
+            _SAID_GENERIC.add((head_dim, group, page_size))
+            warnings.warn(f"bfloat16 attention with head size {head_dim}, {group} query heads per key head and pages of "
+                          f"{page_size} takes the generic kernel (the matrix-core forms take head sizes "
+                          f"{ops.MFMA_HEAD_DIMS}, up to 16 heads per key head and pages of a power of two >= 4)",
+                          RuntimeWarning, stacklevel=2)
         return ops.paged_attention_generic(
             qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, batch.positions,
             batch.seq_of_token, batch.seq_slot, batch.tokens, num_heads, num_kv_heads, head_dim, window, scale)

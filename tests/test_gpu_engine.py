@@ -390,7 +390,9 @@ def test_the_pool_is_sized_by_what_the_requests_can_use_or_by_the_memory_that_is
     folder, raw, _ = tiny_folders["A"]
     engine = Engine(folder, dtype="bfloat16", max_running=3, max_model_len=100, page_size=16, prefix_cache_pages=5)
     assert engine.runner.cache.stats().pages_total == 3 * 7 + 5  # 7 pages a request: 100 tokens
-    per_token = 2 * raw["num_hidden_layers"] * raw["num_key_value_heads"] * 16 * 2  # keys and values, bfloat16
+    head_width = engine.runner.model.cache_needs()[0].head_dim  # (heads of 16 lie in the cache as the heads of 32 the kernels take)
+    assert head_width == 32
+    per_token = 2 * raw["num_hidden_layers"] * raw["num_key_value_heads"] * head_width * 2  # keys and values, bfloat16
     engine = Engine(folder, dtype="bfloat16", max_running=3, max_model_len=100, page_size=16, kv_cache_bytes=40 * per_token)
     assert engine.runner.cache.stats().pages_total == 2  # 40 tokens' worth: two whole pages
     engine = Engine(folder, dtype="bfloat16", max_running=3, max_model_len=100, page_size=16, kv_tokens=64)

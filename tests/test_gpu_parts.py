@@ -177,6 +177,44 @@ def test_attention_part_whole_and_in_portions(dtype, rotary):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("head_dim,padded,rows", [(80, 96, 40), (40, 64, 5), (112, 128, 70), (24, 32, 1), (144, 256, 9)])
+def test_attention_part_with_a_head_size_between_those_of_the_matrix_core_kernels(dtype, head_dim, padded, rows):
+    """A head size that the matrix-core attention does not take runs as the next one it does: the cache and the
+    kernels see heads padded with zeros, the tensors of the checkpoint and the results are those of the head size
+    itself (the plain functions at that size), with a whole-head rotation, a portion and then single tokens, and in
+    bfloat16 without a word from the generic kernel."""
+    import warnings
+
+    from cie_amd.config import PartSpec
+    from cie_amd.parts.attention import Attention
+
+    hidden, heads, kv_heads = 64, 4, 2
+    position = PartSpec.of("rotary_half", head_dim=head_dim, theta=1e4, max_position=256)
+    attention = Attention(hidden, heads, kv_heads, head_dim, qkv_bias=True, out_bias=False, position=position)
+    assert attention.kernel_head_dim == padded and attention.cache_need().head_dim == padded
+    assert attention.expected_tensors("a.")["a.q_proj.weight"].shape == (heads * head_dim, hidden)
+    w = bound(attention, "a.", dtype, 7, scale=0.3)
+    assert attention.w_qkv.shape == ((heads + 2 * kv_heads) * padded, hidden) and attention.w_o.shape == (hidden, heads * padded)
+    total = rows + 3
+    manager, device_cache = harness([attention.cache_need()], [total],
+                                    dtype=torch.float32 if dtype == "float32" else torch.bfloat16, page_size=16)
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn((total, hidden), generator=g).to(attention.dtype)
+    config = {"hidden_size": hidden, "num_attention_heads": heads, "head_dim": head_dim, "attention_bias": True}
+    cos, sin = plain.rope_tables(head_dim, total, 1e4)
+    expected = plain.attention_layer(x.float(), w, "a.", config, cos, sin, torch.arange(total))
+    view = device_cache.view(0)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")  # the generic kernel would say so in bfloat16
+        first = attention.forward(x[:rows].cuda(), batch_of(manager, [(0, 0, rows)]), view)
+        manager.commit_lengths({"r0": rows})
+        rest = [attention.forward(x[i:i + 1].cuda(), batch_of(manager, [(0, i, 1)]), view) for i in range(rows, total)]
+    check(torch.cat([first] + rest).float().cpu(), expected, dtype)
+    # what the cache holds behind a head's own dimensions is zeros
+    assert float(view.k_pool[..., head_dim:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("head_dim,rotary_dim,rows", [(32, 16, 7), (64, 32, 1), (48, 20, 5), (128, 64, 40)])
 def test_attention_part_with_a_rotation_of_the_first_dimensions_only(dtype, head_dim, rotary_dim, rows):
     """A rotary part built with ``rotary_dim < head_dim`` turns the first ``rotary_dim`` dimensions of every
@@ -291,7 +329,9 @@ def test_block_part(dtype, rows, part_k, monkeypatch):
                max_position_embeddings=128)
     spec = Qwen2Config.from_hf_config(raw).model_spec().layers[0]
     block = PreNormBlock(spec)
-    w = bound(block, "model.layers.0.", dtype, 5, scale=0.3)
+    # (bfloat16: softmaxes that 16-bit queries and keys still resolve, as in the attention part's own test; the heads
+    # of 16 run on the matrix cores, as heads of 32, where the probabilities are rounded to bfloat16 too)
+    w = bound(block, "model.layers.0.", dtype, 5, scale=0.3 if dtype == "float32" else 0.2)
     manager, device_cache = harness([block.cache_need()], [rows], dtype=block.dtype)
     h = torch.randn((rows, 48), generator=torch.Generator().manual_seed(6))
     residual = h.clone().cuda()
