@@ -12,11 +12,13 @@ the caller, so trace replay and generation drive the same function.
 
 from __future__ import annotations
 
+import itertools
 from collections import deque
 from collections.abc import Sequence
 from dataclasses import dataclass, field
 from typing import Any
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, PagedKV
@@ -24,7 +26,7 @@ from ..config.engine_config import EngineConfig
 from ..kernels import ops
 from ..profiling import trace_range
 from ..sampling.sampler import Sampler
-from .batch import StepBatch, to_device_staging
+from .batch import StepBatch
 from .device_cache import DeviceCache
 from .graphs import DecodeGraphs, MixedGraphs
 
@@ -278,47 +280,53 @@ class Runner:
                 raise ValueError(
                     f"request {entry.request_id} continues at {entry.start_pos} but the cache holds {held} tokens"
                 )
-            for token in entry.tokens:
-                if not 0 <= token < vocab:
-                    raise ValueError(f"token id {token} outside the vocabulary of {vocab}")
+            if not (0 <= min(entry.tokens) and max(entry.tokens) < vocab):  # (two passes at C speed; a prompt portion has thousands)
+                token = next(t for t in entry.tokens if not 0 <= t < vocab)
+                raise ValueError(f"token id {token} outside the vocabulary of {vocab}")
             for place in entry.want:
                 if not 0 <= place < count:
                     raise ValueError(f"wanted place {place} outside the {count} tokens of {entry.request_id}")
 
     def pack(self, entries: Sequence[StepEntry]) -> StepBatch:
-        ids: list[int] = []
-        positions: list[int] = []
-        seq_of_token: list[int] = []
-        slots: list[int] = []
-        starts: list[int] = []
-        q_lens: list[int] = []
+        """The step's metadata, laid out in one page-locked buffer and copied to the device once.  What has an
+        entry per token (ids, positions, sequence of the token) is made by array operations, not token by token:
+        a prompt portion of 2,048 tokens took 0.4 ms of lists here, before the step's first kernel could start."""
+        count_of = [len(entry.tokens) for entry in entries]
+        sequences = len(entries)
+        total = sum(count_of)
+        slots = [self.cache.slot(entry.request_id) for entry in entries]
+        starts = [entry.start_pos for entry in entries]
         q_start_loc = [0]
-        logit_rows: list[int] = []
-        for index, entry in enumerate(entries):
-            count = len(entry.tokens)
-            base = len(ids)
-            ids.extend(entry.tokens)
-            positions.extend(range(entry.start_pos, entry.start_pos + count))
-            seq_of_token.extend([index] * count)
-            slots.append(self.cache.slot(entry.request_id))
-            starts.append(entry.start_pos)
-            q_lens.append(count)
-            q_start_loc.append(base + count)
-            logit_rows.extend(base + place for place in entry.want)
-        parts = [ids, positions, seq_of_token, slots, starts, q_lens, q_start_loc, logit_rows]
-        flat = [value for part in parts for value in part]
-        dev = self._stage(len(flat))
-        dev[: len(flat)].copy_(to_device_staging(flat, self.device), non_blocking=True)
-        views = []
-        offset = 0
-        for part in parts:
-            views.append(dev[offset: offset + len(part)])
-            offset += len(part)
+        for count in count_of:
+            q_start_loc.append(q_start_loc[-1] + count)
+        logit_rows = [q_start_loc[index] + place for index, entry in enumerate(entries) for place in entry.want]
+        sizes = [total, total, total, sequences, sequences, sequences, sequences + 1, len(logit_rows)]
+        staged = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=self.device.type == "cuda")
+        host = staged.numpy()
+        bounds = [0]
+        for size in sizes:
+            bounds.append(bounds[-1] + size)
+        part = [host[bounds[i]: bounds[i + 1]] for i in range(len(sizes))]
+        counts = np.asarray(count_of, dtype=np.int32)
+        part[0][:] = np.fromiter(itertools.chain.from_iterable(entry.tokens for entry in entries), dtype=np.int32,
+                                 count=total)
+        part[2][:] = np.repeat(np.arange(sequences, dtype=np.int32), counts)
+        # a token's position: its place on the flat axis, less its sequence's first place, plus the sequence's start
+        shift = np.asarray(starts, dtype=np.int32) - np.asarray(q_start_loc[:-1], dtype=np.int32)
+        part[1][:] = np.arange(total, dtype=np.int32) + np.repeat(shift, counts)
+        part[3][:] = slots
+        part[4][:] = starts
+        part[5][:] = count_of
+        part[6][:] = q_start_loc
+        part[7][:] = logit_rows
+        dev = self._stage(staged.numel())
+        dev[: staged.numel()].copy_(staged, non_blocking=True)
+        views = [dev[bounds[i]: bounds[i + 1]] for i in range(len(sizes))]
         return StepBatch(
-            tokens=len(ids), sequences=len(entries), token_ids=views[0], positions=views[1],
+            tokens=total, sequences=sequences, token_ids=views[0], positions=views[1],
             seq_of_token=views[2], seq_slot=views[3], seq_start=views[4], seq_q_len=views[5],
             q_start_loc=views[6], logit_rows=views[7], host_slots=slots, host_starts=starts,
-            host_q_lens=q_lens, request_ids=tuple(e.request_id for e in entries),
+            host_q_lens=count_of, request_ids=tuple(e.request_id for e in entries),
         )
 
     # -- the step ------------------------------------------------------------------
