@@ -199,8 +199,8 @@ bool agrees_with_first(Timing& timing, int i, size_t elements, bool f32_out) {
         (void)hipGetLastError();
         return false;
     }
-    unsigned* verdict = reinterpret_cast<unsigned*>(other + (bytes + 7) / 8 * 8);
-    bool good = hipMemsetAsync(verdict, 0, 8, timing.stream) == hipSuccess && timing.run(0, nullptr, true) &&
+    unsigned* outcome = reinterpret_cast<unsigned*>(other + (bytes + 7) / 8 * 8);
+    bool good = hipMemsetAsync(outcome, 0, 8, timing.stream) == hipSuccess && timing.run(0, nullptr, true) &&
                 timing.run(i, other, true);
     if (good) {
         // bf16 results: two roundings of the same sum lie an ulp (2^-8 of the value) apart, sums in another
@@ -208,19 +208,19 @@ bool agrees_with_first(Timing& timing, int i, size_t elements, bool f32_out) {
         const int blocks = 1024, threads = 256;
         if (f32_out) {
             const float* mine = static_cast<const float*>(timing.c);
-            results_size_kernel<float><<<blocks, threads, 0, timing.stream>>>(mine, elements, verdict);
+            results_size_kernel<float><<<blocks, threads, 0, timing.stream>>>(mine, elements, outcome);
             results_differ_kernel<float><<<blocks, threads, 0, timing.stream>>>(
-                mine, reinterpret_cast<const float*>(other), elements, 1.f / 1024.f, 1.f / 4096.f, verdict);
+                mine, reinterpret_cast<const float*>(other), elements, 1.f / 1024.f, 1.f / 4096.f, outcome);
         } else {
             const unsigned short* mine = static_cast<const unsigned short*>(timing.c);
-            results_size_kernel<unsigned short><<<blocks, threads, 0, timing.stream>>>(mine, elements, verdict);
+            results_size_kernel<unsigned short><<<blocks, threads, 0, timing.stream>>>(mine, elements, outcome);
             results_differ_kernel<unsigned short><<<blocks, threads, 0, timing.stream>>>(
-                mine, reinterpret_cast<const unsigned short*>(other), elements, 1.f / 64.f, 1.f / 256.f, verdict);
+                mine, reinterpret_cast<const unsigned short*>(other), elements, 1.f / 64.f, 1.f / 256.f, outcome);
         }
         good = hipGetLastError() == hipSuccess;
     }
     unsigned bits[2] = {0, 0};
-    good = good && hipMemcpyAsync(bits, verdict, 8, hipMemcpyDeviceToHost, timing.stream) == hipSuccess &&
+    good = good && hipMemcpyAsync(bits, outcome, 8, hipMemcpyDeviceToHost, timing.stream) == hipSuccess &&
            hipStreamSynchronize(timing.stream) == hipSuccess;
     hipStreamSynchronize(timing.stream);
     hipFree(other);
