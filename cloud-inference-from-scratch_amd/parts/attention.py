@@ -200,16 +200,19 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
     sizes, groups of more than 16 heads, pages of fewer than 4 tokens): the
     generic kernel."""
     group = num_heads // num_kv_heads
+    decode_tiles = 1 if group <= 16 else 2 if group <= 32 else 4  # 16-row tiles that hold one token's heads
     page_size = view.page_size
     cus = ops.compute_units()  # compute units of the GPU
-    if (qkv.dtype != torch.bfloat16 or head_dim not in ops.MFMA_HEAD_DIMS or group > 16 or page_size < 4
-            or page_size & (page_size - 1)):
+    # (a token's heads of one key head share a tile: up to 64 rows, 16 where the head has 256 dimensions)
+    if (qkv.dtype != torch.bfloat16 or head_dim not in ops.MFMA_HEAD_DIMS or group > (64 if head_dim <= 128 else 16)
+            or page_size < 4 or page_size & (page_size - 1)):
         if qkv.dtype == torch.bfloat16 and (head_dim, group, page_size) not in _SAID_GENERIC:
             # right, and many times slower than the matrix-core forms: said once per geometry, not silently
             _SAID_GENERIC.add((head_dim, group, page_size))
             warnings.warn(f"bfloat16 attention with head size {head_dim}, {group} query heads per key head and pages of "
                           f"{page_size} takes the generic kernel (the matrix-core forms take head sizes "
-                          f"{ops.MFMA_HEAD_DIMS}, up to 16 heads per key head and pages of a power of two >= 4)",
+                          f"{ops.MFMA_HEAD_DIMS}, up to 64 heads per key head, 16 at head size 256, and pages of a power "
+                          f"of two >= 4)",
                           RuntimeWarning, stacklevel=2)
         return ops.paged_attention_generic(
             qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, batch.positions,
@@ -270,9 +273,9 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
             n_splits, _ = plan_splits(decode_rows * num_kv_heads, max_keys, **split_options)
             part_o = part_ml = None
             if n_splits > 1:
-                part_o, part_ml = _workspaces(qkv.device, decode_rows * num_kv_heads * n_splits, 16, head_dim)
+                part_o, part_ml = _workspaces(qkv.device, decode_rows * num_kv_heads * n_splits, 16 * decode_tiles, head_dim)
             ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, None,
-                                     None, decode_rows, *common, tokens_per_tile=1, row_tiles=1,
+                                     None, decode_rows, *common, tokens_per_tile=1, row_tiles=decode_tiles,
                                      n_splits=n_splits, max_context_dev=longest_dev, part_o=part_o, part_ml=part_ml,
                                      tile_waves=decode_waves)
         if decode_rows == batch.sequences:
@@ -290,9 +293,9 @@ def attend(qkv: torch.Tensor, batch, view, num_heads: int, num_kv_heads: int, he
         n_splits, per_split = plan_splits(n_tiles * num_kv_heads, max_keys, **split_options)
         part_o = part_ml = None
         if n_splits > 1:
-            part_o, part_ml = _workspaces(qkv.device, n_tiles * num_kv_heads * n_splits, 16, head_dim)
+            part_o, part_ml = _workspaces(qkv.device, n_tiles * num_kv_heads * n_splits, 16 * decode_tiles, head_dim)
         ops.paged_attention_mfma(qkv, qkv.stride(0), view.k_pool, view.v_pool, view.block_table, tile_seq, tile_q0,
-                                 n_tiles, *common, tokens_per_tile=1, row_tiles=1, n_splits=n_splits,
+                                 n_tiles, *common, tokens_per_tile=1, row_tiles=decode_tiles, n_splits=n_splits,
                                  keys_per_split=per_split, part_o=part_o, part_ml=part_ml, tile_waves=decode_waves)
     if wide:
         # the prompt forms: waves share a tile's keys.  More rows per tile re-use each key more often,

@@ -214,6 +214,50 @@ def test_attention_part_with_a_head_size_between_those_of_the_matrix_core_kernel
     assert float(view.k_pool[..., head_dim:].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("page_size", [8, 16])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(24, 1, 32), (40, 1, 64), (34, 2, 128), (64, 1, 32)])
+def test_attention_part_with_more_than_sixteen_heads_on_a_key_head(heads, kv_heads, head_dim, page_size):
+    """Groups of 17 to 64 query heads on one key head in bfloat16: a token's heads fill two or four 16-row tiles of the
+    matrix-core kernels (no word from the generic kernel), as a prompt, as a portion behind context and as single
+    tokens over a context that is cut into parts."""
+    import warnings
+
+    from cie_amd.config import PartSpec
+    from cie_amd.parts.attention import Attention
+
+    hidden = 64
+    position = PartSpec.of("rotary_half", head_dim=head_dim, theta=1e4, max_position=512)
+    attention = Attention(hidden, heads, kv_heads, head_dim, qkv_bias=True, out_bias=False, position=position)
+    w = bound(attention, "a.", "bfloat16", 11, scale=0.2)
+    lengths = [245, 37]
+    manager, device_cache = harness([attention.cache_need()], lengths, dtype=torch.bfloat16, page_size=page_size)
+    g = torch.Generator().manual_seed(12)
+    xs = [torch.randn((n, hidden), generator=g).to(attention.dtype) for n in lengths]
+    config = {"hidden_size": hidden, "num_attention_heads": heads, "head_dim": head_dim, "attention_bias": True}
+    expected = []
+    for x, n in zip(xs, lengths):
+        cos, sin = plain.rope_tables(head_dim, n, 1e4)
+        expected.append(plain.attention_layer(x.float(), w, "a.", config, cos, sin, torch.arange(n)))
+    view = device_cache.view(0)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        # request 0: 230 tokens at once, then a portion of 8 beside the first 30 tokens of request 1
+        first = attention.forward(xs[0][:230].cuda(), batch_of(manager, [(0, 0, 230)]), view)
+        manager.commit_lengths({"r0": 230})
+        both = attention.forward(torch.cat([xs[0][230:238], xs[1][:30]]).cuda(), batch_of(manager, [(0, 230, 8), (1, 0, 30)]), view)
+        manager.commit_lengths({"r0": 238, "r1": 30})
+        got0, got1 = [first, both[:8]], [both[8:]]
+        # single tokens of both, one step each (request 0 over more than 192 keys: its keys are cut into parts)
+        for step in range(3):
+            out = attention.forward(torch.cat([xs[0][238 + step:239 + step], xs[1][30 + step:31 + step]]).cuda(),
+                                    batch_of(manager, [(0, 238 + step, 1), (1, 30 + step, 1)]), view)
+            manager.commit_lengths({"r0": 239 + step, "r1": 31 + step})
+            got0.append(out[:1])
+            got1.append(out[1:])
+    check(torch.cat(got0).float().cpu(), expected[0][:241], "bfloat16")
+    check(torch.cat(got1).float().cpu(), expected[1][:33], "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("head_dim,rotary_dim,rows", [(32, 16, 7), (64, 32, 1), (48, 20, 5), (128, 64, 40)])
 def test_attention_part_with_a_rotation_of_the_first_dimensions_only(dtype, head_dim, rotary_dim, rows):
