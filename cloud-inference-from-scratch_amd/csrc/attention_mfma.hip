@@ -409,7 +409,10 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                if (rt >= rt_used) break;  // (the same for the whole workgroup)
+                // (Every row tile is multiplied, also one without rows: a way out of this loop would be a short cut
+                // from a product to the first read of its result, and the compiler counts the wait between the two
+                // along the straight path only.  With that short cut a tile of one token read scores that were not
+                // finished, now and then.)
                 floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int j = 0; j < NK; ++j)
@@ -424,7 +427,10 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
 
         // ---- running maxima of all row tiles first; masks only in blocks that reach a row's edge
         const bool edge = kb + kKeysPerBlock - 1 > first_pos || (a.window > 0 && kb < last_pos + 1 - a.window);
-        float m_use[RT], alpha[RT];
+        // The reference of a row moves only when a score passes it by more than kLazyRescale: until then
+        // probabilities may reach 2^kLazyRescale, which float32 sums and bfloat16 products hold as well.  Each of
+        // a row's four lanes can tell that of its own eight scores, so the common block needs no maximum across lanes.
+        float own_max[RT], m_use[RT];
         bool moved = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
@@ -440,26 +446,24 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
                         if (!(key <= pos && key >= row_lo)) s[rt][kt][i] = -INFINITY;
                     }
             }
-            float block_max = fmaxf(fmaxf(fmaxf(s[rt][0][0], s[rt][0][1]), fmaxf(s[rt][0][2], s[rt][0][3])),
-                                    fmaxf(fmaxf(s[rt][1][0], s[rt][1][1]), fmaxf(s[rt][1][2], s[rt][1][3])));
-            block_max = rows_max(block_max) * scale_log2;  // maxima are kept in scaled base-2 units
-            // the reference of a row moves only when a score passes it by more than kLazyRescale: until then
-            // probabilities may reach 2^kLazyRescale, which float32 sums and bfloat16 products hold as well
-            const float m_new = (block_max > m_run[rt] + kLazyRescale) ? block_max : m_run[rt];
-            m_use[rt] = (m_new == -INFINITY) ? 0.f : m_new;
-            alpha[rt] = __builtin_amdgcn_exp2f(m_run[rt] - m_use[rt]);  // m_run = -inf: 0, and l, O are 0 anyway
-            moved = moved || (m_new != m_run[rt]);
-            m_run[rt] = m_new;
-            l_run[rt] *= alpha[rt];
+            own_max[rt] = fmaxf(fmaxf(fmaxf(s[rt][0][0], s[rt][0][1]), fmaxf(s[rt][0][2], s[rt][0][3])),
+                                fmaxf(fmaxf(s[rt][1][0], s[rt][1][1]), fmaxf(s[rt][1][2], s[rt][1][3])));
+            moved = moved || own_max[rt] * scale_log2 > m_run[rt] + kLazyRescale;  // (the scale is positive)
         }
         if (__any(moved)) {
             // the products that wrote these accumulators were issued a whole score phase ago
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 if (rt >= rt_used) break;
+                const float block_max = rows_max(own_max[rt]) * scale_log2;  // maxima are kept in scaled base-2 units
+                const float m_new = (block_max > m_run[rt] + kLazyRescale) ? block_max : m_run[rt];
+                const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+                const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_safe);  // m_run = -inf: 0, and l, O are 0 anyway
+                m_run[rt] = m_new;
+                l_run[rt] *= alpha;
                 float alpha_o[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha[rt], g * 4 + i, kWave);
+                for (int i = 0; i < 4; ++i) alpha_o[i] = __shfl(alpha, g * 4 + i, kWave);
 #pragma unroll
                 for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
@@ -467,6 +471,8 @@ __global__ void __launch_bounds__(64 * WAVES) paged_attention_tile_kernel(Attent
             }
             asm volatile("s_nop 7");  // before a product reads what was just written
         }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) m_use[rt] = (m_run[rt] == -INFINITY) ? 0.f : m_run[rt];
         // ---- probabilities (one fused multiply-add and one exp2 each) and O += P . V, row tile by row tile
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
